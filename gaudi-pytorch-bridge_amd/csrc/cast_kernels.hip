@@ -1,0 +1,624 @@
+// cast_to_fp8 / cast_from_fp8 / amax kernels for gfx950 and their C entry points.
+//
+// All three are HBM-bound streaming kernels: every lane moves 16-byte vectors,
+// a wave's accesses are contiguous, and each thread keeps several independent
+// loads in flight.  Rounding and saturation use the CDNA4 conversion
+// instructions (v_cvt_pk_{fp8,bf8}_f32, v_cvt_pk_f32_{fp8,bf8},
+// v_cvt_pk_bf16_f32); see device_common.h.
+#include "device_common.h"
+
+namespace mi355q {
+
+enum ScaleKind { SK_SCALAR = 0, SK_ROW = 1, SK_COL = 2, SK_FULL = 3 };
+
+constexpr int kThreads = 256;
+
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t v) { *p = v; }
+
+// Block-level max of abs-value bit patterns, then one atomicMax per block.
+// Bit patterns of non-negative floats order like the floats, and a NaN
+// pattern is larger than Inf, so NaN wins and the result reads back as NaN.
+__device__ __forceinline__ void block_amax_commit(uint32_t m, uint32_t* amax) {
+  __shared__ uint32_t wave_part[kThreads / 64];
+  m = wave_max_u32(m);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) wave_part[wave] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t r = wave_part[0];
+#pragma unroll
+    for (int w = 1; w < kThreads / 64; ++w) r = r > wave_part[w] ? r : wave_part[w];
+    if (r != 0) atomicMax(amax, r);
+  }
+}
+
+// ---------------------------------------------------------------- cast_to_fp8
+//
+// The input is viewed as [rows, vec_per_row] vectors of 8 elements.  Flat
+// modes use rows == 1.  A block owns blockDim*U consecutive vectors of one
+// row; U loads per thread are issued before any is consumed.
+//   SK_SCALAR  one scale for everything (host value or *scale)
+//   SK_ROW     scale[row % mid]
+//   SK_COL     scale[column]
+//   SK_FULL    scale[element]
+template <bool BF16_IN, int FMT, int SK, bool AMAX, int U>
+__global__ __launch_bounds__(kThreads) void cast_to_fp8_vec8(
+    const uint8_t* __restrict__ x, uint8_t* __restrict__ y, const float* __restrict__ scale,
+    float scale_host, int scale_is_dev, int64_t vec_per_row, int64_t blocks_per_row,
+    int64_t mid, uint32_t* __restrict__ amax) {
+  const int64_t row = blockIdx.x / blocks_per_row;
+  const int64_t bir = blockIdx.x - row * blocks_per_row;
+  const int64_t v0 = bir * (int64_t)(kThreads * U) + threadIdx.x;
+  const int64_t row_base = row * vec_per_row;
+
+  float s = 1.0f;
+  if constexpr (SK == SK_SCALAR) s = scale_is_dev ? scale[0] : scale_host;
+  if constexpr (SK == SK_ROW) s = scale[row % mid];
+  if constexpr (BF16_IN) s = round_to_bf16(s);
+
+  constexpr int IN_BYTES = BF16_IN ? 16 : 32;
+  u32x4 in[U][BF16_IN ? 1 : 2];
+  bool ok[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t vr = v0 + (int64_t)u * kThreads;
+    ok[u] = vr < vec_per_row;
+    if (ok[u]) {
+      const u32x4* p = reinterpret_cast<const u32x4*>(x + (row_base + vr) * IN_BYTES);
+      in[u][0] = __builtin_nontemporal_load(p);
+      if constexpr (!BF16_IN) in[u][1] = __builtin_nontemporal_load(p + 1);
+    }
+  }
+
+  uint32_t am = 0;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (!ok[u]) continue;
+    const int64_t vr = v0 + (int64_t)u * kThreads;
+    float v[8];
+    if constexpr (BF16_IN) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t w = in[u][0][i];
+        v[2 * i] = __uint_as_float(w << 16);
+        v[2 * i + 1] = __uint_as_float(w & 0xffff0000u);
+        if constexpr (AMAX) {
+          // packed 16-bit max over the two abs bit patterns of this dword
+          const u16x2 a = __builtin_bit_cast(u16x2, w & 0x7fff7fffu);
+          const u16x2 m = __builtin_elementwise_max(a, __builtin_bit_cast(u16x2, am));
+          am = __builtin_bit_cast(uint32_t, m);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t w = in[u][i >> 2][i & 3];
+        v[i] = __uint_as_float(w);
+        if constexpr (AMAX) {
+          const uint32_t a = w & 0x7fffffffu;
+          am = am > a ? am : a;
+        }
+      }
+    }
+    float sv[8];
+    if constexpr (SK == SK_COL || SK == SK_FULL) {
+      const int64_t si = (SK == SK_COL ? vr : row_base + vr) * 8;
+      const f32x4 s0 = *reinterpret_cast<const f32x4*>(scale + si);
+      const f32x4 s1 = *reinterpret_cast<const f32x4*>(scale + si + 4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        sv[i] = BF16_IN ? round_to_bf16(s0[i]) : s0[i];
+        sv[4 + i] = BF16_IN ? round_to_bf16(s1[i]) : s1[i];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sv[i] = s;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float p = v[i] * sv[i];
+      if constexpr (BF16_IN) p = round_to_bf16(p);
+      v[i] = p;
+    }
+    u32x2 out;
+    out.x = cvt_fp8x4<FMT>(v[0], v[1], v[2], v[3]);
+    out.y = cvt_fp8x4<FMT>(v[4], v[5], v[6], v[7]);
+    __builtin_nontemporal_store(out, reinterpret_cast<u32x2*>(y + (row_base + vr) * 8));
+  }
+
+  if constexpr (AMAX) {
+    if constexpr (BF16_IN) {
+      const uint32_t lo = am & 0xffffu, hi = am >> 16;
+      am = (lo > hi ? lo : hi) << 16;
+    }
+    block_amax_commit(am, amax);
+  }
+}
+
+// One element per thread, any alignment, any broadcast: tails and odd shapes.
+template <bool BF16_IN, int FMT>
+__global__ __launch_bounds__(kThreads) void cast_to_fp8_generic(
+    const uint8_t* __restrict__ x, uint8_t* __restrict__ y, const float* __restrict__ scale,
+    float scale_host, int mode, int64_t start, int64_t n, int64_t mid, int64_t inner,
+    uint32_t* __restrict__ amax) {
+  const int64_t i = start + (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  uint32_t am = 0;
+  if (i < n) {
+    float s = 1.0f;
+    if (mode == MI355Q_SCALE_HOST) s = scale_host;
+    else if (mode == MI355Q_SCALE_DEV) s = scale[0];
+    else if (mode == MI355Q_SCALE_MID) s = scale[(i / inner) % mid];
+    else if (mode == MI355Q_SCALE_FULL) s = scale[i];
+    float v, p;
+    if constexpr (BF16_IN) {
+      const uint32_t h = reinterpret_cast<const uint16_t*>(x)[i];
+      v = bf16_bits_to_f32(h);
+      p = round_to_bf16(v * round_to_bf16(s));
+    } else {
+      v = reinterpret_cast<const float*>(x)[i];
+      p = v * s;
+    }
+    am = __float_as_uint(v) & 0x7fffffffu;
+    y[i] = (uint8_t)(cvt_fp8x4<FMT>(p, p, p, p) & 0xffu);
+  }
+  if (amax != nullptr) block_amax_commit(am, amax);
+}
+
+// ---------------------------------------------------------------------- amax
+template <bool BF16_IN, int U>
+__global__ __launch_bounds__(kThreads) void amax_vec(const uint8_t* __restrict__ x, int64_t nvec,
+                                                     uint32_t* __restrict__ amax) {
+  // vectors of 16 bytes
+  const int64_t v0 = (int64_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+  u32x4 in[U];
+  bool ok[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t v = v0 + (int64_t)u * kThreads;
+    ok[u] = v < nvec;
+    if (ok[u]) in[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x) + v);
+  }
+  uint32_t am = 0;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (!ok[u]) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (BF16_IN) {
+        const u16x2 a = __builtin_bit_cast(u16x2, in[u][i] & 0x7fff7fffu);
+        am = __builtin_bit_cast(uint32_t,
+                                __builtin_elementwise_max(a, __builtin_bit_cast(u16x2, am)));
+      } else {
+        const uint32_t a = in[u][i] & 0x7fffffffu;
+        am = am > a ? am : a;
+      }
+    }
+  }
+  if constexpr (BF16_IN) {
+    const uint32_t lo = am & 0xffffu, hi = am >> 16;
+    am = (lo > hi ? lo : hi) << 16;
+  }
+  block_amax_commit(am, amax);
+}
+
+template <bool BF16_IN>
+__global__ __launch_bounds__(kThreads) void amax_generic(const uint8_t* __restrict__ x,
+                                                         int64_t start, int64_t n,
+                                                         uint32_t* __restrict__ amax) {
+  const int64_t i = start + (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  uint32_t am = 0;
+  if (i < n) {
+    if constexpr (BF16_IN) am = ((uint32_t)reinterpret_cast<const uint16_t*>(x)[i] & 0x7fffu) << 16;
+    else am = reinterpret_cast<const uint32_t*>(x)[i] & 0x7fffffffu;
+  }
+  block_amax_commit(am, amax);
+}
+
+// One block per row; rows are independent so no atomics and no pre-zeroing.
+template <bool BF16_IN>
+__global__ __launch_bounds__(kThreads) void rowwise_amax_kernel(const uint8_t* __restrict__ x,
+                                                               int64_t cols, int vec_ok,
+                                                               float* __restrict__ out) {
+  __shared__ uint32_t wave_part[kThreads / 64];
+  const int64_t row = blockIdx.x;
+  constexpr int ES = BF16_IN ? 2 : 4;
+  const uint8_t* xr = x + row * cols * ES;
+  uint32_t am = 0;
+  int64_t done = 0;
+  if (vec_ok) {
+    const int64_t nvec = cols * ES / 16;
+    for (int64_t v = threadIdx.x; v < nvec; v += kThreads) {
+      const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xr) + v);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if constexpr (BF16_IN) {
+          const u16x2 a = __builtin_bit_cast(u16x2, w[i] & 0x7fff7fffu);
+          am = __builtin_bit_cast(uint32_t,
+                                  __builtin_elementwise_max(a, __builtin_bit_cast(u16x2, am)));
+        } else {
+          const uint32_t a = w[i] & 0x7fffffffu;
+          am = am > a ? am : a;
+        }
+      }
+    }
+    if constexpr (BF16_IN) {
+      const uint32_t lo = am & 0xffffu, hi = am >> 16;
+      am = (lo > hi ? lo : hi) << 16;
+    }
+    done = nvec * (16 / ES);
+  }
+  for (int64_t c = done + threadIdx.x; c < cols; c += kThreads) {
+    uint32_t a;
+    if constexpr (BF16_IN) a = ((uint32_t)reinterpret_cast<const uint16_t*>(xr)[c] & 0x7fffu) << 16;
+    else a = reinterpret_cast<const uint32_t*>(xr)[c] & 0x7fffffffu;
+    am = am > a ? am : a;
+  }
+  am = wave_max_u32(am);
+  if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = am;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t r = wave_part[0];
+#pragma unroll
+    for (int w = 1; w < kThreads / 64; ++w) r = r > wave_part[w] ? r : wave_part[w];
+    out[row] = __uint_as_float(r);
+  }
+}
+
+// -------------------------------------------------------------- cast_from_fp8
+//
+// Vectors of 16 fp8 bytes in, 16 bf16 (2 x 16 B) or 16 fp32 (4 x 16 B) out.
+template <int FMT, bool BF16_OUT, int SK, int U>
+__global__ __launch_bounds__(kThreads) void cast_from_fp8_vec16(
+    const uint8_t* __restrict__ x, uint8_t* __restrict__ y, const float* __restrict__ scale,
+    float scale_host, int scale_is_dev, int has_scale, int64_t vec_per_row,
+    int64_t blocks_per_row, int64_t mid) {
+  const int64_t row = blockIdx.x / blocks_per_row;
+  const int64_t bir = blockIdx.x - row * blocks_per_row;
+  const int64_t v0 = bir * (int64_t)(kThreads * U) + threadIdx.x;
+  const int64_t row_base = row * vec_per_row;
+
+  float s = 1.0f;
+  if constexpr (SK == SK_SCALAR) s = scale_is_dev ? scale[0] : scale_host;
+  if constexpr (SK == SK_ROW) s = scale[row % mid];
+  if constexpr (BF16_OUT) s = round_to_bf16(s);
+
+  u32x4 in[U];
+  bool ok[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t vr = v0 + (int64_t)u * kThreads;
+    ok[u] = vr < vec_per_row;
+    if (ok[u]) in[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x) + row_base + vr);
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (!ok[u]) continue;
+    const int64_t vr = v0 + (int64_t)u * kThreads;
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      cvt_f32x4<FMT>(in[u][i], v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+    if (has_scale) {
+      if constexpr (SK == SK_COL || SK == SK_FULL) {
+        const int64_t si = (SK == SK_COL ? vr : row_base + vr) * 16;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const f32x4 sq = *reinterpret_cast<const f32x4*>(scale + si + 4 * q);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[4 * q + i] *= BF16_OUT ? round_to_bf16(sq[i]) : sq[i];
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] *= s;
+      }
+    }
+    if constexpr (BF16_OUT) {
+      u32x4* o = reinterpret_cast<u32x4*>(y + (row_base + vr) * 32);
+      u32x4 o0, o1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        o0[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+        o1[i] = pack_bf16x2(v[8 + 2 * i], v[8 + 2 * i + 1]);
+      }
+      __builtin_nontemporal_store(o0, o);
+      __builtin_nontemporal_store(o1, o + 1);
+    } else {
+      f32x4* o = reinterpret_cast<f32x4*>(y + (row_base + vr) * 64);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        f32x4 t = {v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+        __builtin_nontemporal_store(t, o + q);
+      }
+    }
+  }
+}
+
+template <int FMT, bool BF16_OUT>
+__global__ __launch_bounds__(kThreads) void cast_from_fp8_generic(
+    const uint8_t* __restrict__ x, uint8_t* __restrict__ y, const float* __restrict__ scale,
+    float scale_host, int mode, int64_t start, int64_t n, int64_t mid, int64_t inner) {
+  const int64_t i = start + (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= n) return;
+  float v = cvt_f32x1<FMT>(x[i]);
+  if (mode != MI355Q_SCALE_NONE) {
+    float s = 1.0f;
+    if (mode == MI355Q_SCALE_HOST) s = scale_host;
+    else if (mode == MI355Q_SCALE_DEV) s = scale[0];
+    else if (mode == MI355Q_SCALE_MID) s = scale[(i / inner) % mid];
+    else if (mode == MI355Q_SCALE_FULL) s = scale[i];
+    if constexpr (BF16_OUT) s = round_to_bf16(s);
+    v *= s;
+  }
+  if constexpr (BF16_OUT) reinterpret_cast<uint16_t*>(y)[i] = (uint16_t)(pack_bf16x2(v, v) & 0xffffu);
+  else reinterpret_cast<float*>(y)[i] = v;
+}
+
+__global__ __launch_bounds__(kThreads) void copy_bytes_kernel(const uint8_t* __restrict__ x,
+                                                              uint8_t* __restrict__ y, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i < n) y[i] = x[i];
+}
+
+__global__ __launch_bounds__(kThreads) void copy_vec16_kernel(const u32x4* __restrict__ x,
+                                                              u32x4* __restrict__ y, int64_t nvec) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i < nvec) __builtin_nontemporal_store(__builtin_nontemporal_load(x + i), y + i);
+}
+
+// --------------------------------------------------------------- host helpers
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+inline int launch_status() { return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH; }
+inline unsigned blocks_for(int64_t n, int64_t per) { return (unsigned)((n + per - 1) / per); }
+
+// Decide how the vector kernels see the problem.  Returns false when only the
+// generic kernel applies.
+struct VecPlan {
+  int sk;
+  int64_t rows, row_len, mid;
+};
+
+inline bool plan_vectors(int mode, int64_t outer, int64_t mid, int64_t inner, int64_t vec,
+                         VecPlan* p) {
+  const int64_t n = outer * mid * inner;
+  switch (mode) {
+    case MI355Q_SCALE_NONE:
+    case MI355Q_SCALE_HOST:
+    case MI355Q_SCALE_DEV:
+      *p = {SK_SCALAR, 1, n, 1};
+      return true;
+    case MI355Q_SCALE_FULL:
+      *p = {SK_FULL, 1, n, 1};
+      return true;
+    case MI355Q_SCALE_MID:
+      if (inner == 1) {  // per column of [outer, mid]
+        if (mid % vec != 0 || mid < 4 * vec) return false;
+        *p = {SK_COL, outer, mid, mid};
+        return true;
+      }
+      if (inner % vec != 0 || inner < 4 * vec) return false;
+      *p = {SK_ROW, outer * mid, inner, mid};
+      return true;
+    default:
+      return false;
+  }
+}
+
+template <bool BF16_IN, int FMT, bool AMAX>
+void launch_cast_to_vec(int sk, unsigned grid, hipStream_t st, const uint8_t* x, uint8_t* y,
+                        const float* scale, float sh, int is_dev, int64_t vpr, int64_t bpr,
+                        int64_t mid, uint32_t* amax) {
+  constexpr int U = 4;
+  switch (sk) {
+    case SK_SCALAR:
+      cast_to_fp8_vec8<BF16_IN, FMT, SK_SCALAR, AMAX, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, mid, amax);
+      break;
+    case SK_ROW:
+      cast_to_fp8_vec8<BF16_IN, FMT, SK_ROW, AMAX, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, mid, amax);
+      break;
+    case SK_COL:
+      cast_to_fp8_vec8<BF16_IN, FMT, SK_COL, AMAX, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, mid, amax);
+      break;
+    default:
+      cast_to_fp8_vec8<BF16_IN, FMT, SK_FULL, AMAX, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, mid, amax);
+      break;
+  }
+}
+
+template <bool BF16_IN, int FMT>
+int cast_to_dispatch(const uint8_t* x, uint8_t* y, const float* scale, float sh, int mode,
+                     int64_t outer, int64_t mid, int64_t inner, uint32_t* amax, hipStream_t st) {
+  constexpr int U = 4;
+  constexpr int IN_BYTES = BF16_IN ? 16 : 32;
+  const int64_t n = outer * mid * inner;
+  VecPlan p;
+  const bool vec = aligned(x, 16) && aligned(y, 8) &&
+                   (scale == nullptr || aligned(scale, 16)) && plan_vectors(mode, outer, mid, inner, 8, &p);
+  int64_t done = 0;
+  if (vec) {
+    const int64_t vpr = p.row_len / 8;
+    // In flat modes the row length need not be a multiple of 8: the tail goes
+    // to the generic kernel.  In 2-D modes plan_vectors has required it.
+    if (vpr > 0) {
+      const int64_t bpr = (vpr + kThreads * U - 1) / (kThreads * U);
+      const int64_t grid = bpr * p.rows;
+      if (grid > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+      const int is_dev = mode == MI355Q_SCALE_DEV;
+      if (amax) launch_cast_to_vec<BF16_IN, FMT, true>(p.sk, (unsigned)grid, st, x, y, scale, sh, is_dev, vpr, bpr, p.mid, amax);
+      else launch_cast_to_vec<BF16_IN, FMT, false>(p.sk, (unsigned)grid, st, x, y, scale, sh, is_dev, vpr, bpr, p.mid, amax);
+      done = p.rows == 1 ? vpr * 8 : n;
+    }
+    (void)IN_BYTES;
+  }
+  if (done < n) {
+    const int64_t rest = n - done;
+    const int64_t grid = (rest + kThreads - 1) / kThreads;
+    if (grid > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+    cast_to_fp8_generic<BF16_IN, FMT><<<(unsigned)grid, kThreads, 0, st>>>(x, y, scale, sh, mode, done, n, mid, inner, amax);
+  }
+  return launch_status();
+}
+
+template <int FMT, bool BF16_OUT>
+int cast_from_dispatch(const uint8_t* x, uint8_t* y, const float* scale, float sh, int mode,
+                       int64_t outer, int64_t mid, int64_t inner, hipStream_t st) {
+  constexpr int U = 2;
+  const int64_t n = outer * mid * inner;
+  VecPlan p;
+  const bool vec = aligned(x, 16) && aligned(y, 16) &&
+                   (scale == nullptr || aligned(scale, 16)) && plan_vectors(mode, outer, mid, inner, 16, &p);
+  int64_t done = 0;
+  if (vec) {
+    const int64_t vpr = p.row_len / 16;
+    if (vpr > 0) {
+      const int64_t bpr = (vpr + kThreads * U - 1) / (kThreads * U);
+      const int64_t grid64 = bpr * p.rows;
+      if (grid64 > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+      const unsigned grid = (unsigned)grid64;
+      const int is_dev = mode == MI355Q_SCALE_DEV;
+      const int has_scale = mode != MI355Q_SCALE_NONE;
+      switch (p.sk) {
+        case SK_SCALAR:
+          cast_from_fp8_vec16<FMT, BF16_OUT, SK_SCALAR, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+          break;
+        case SK_ROW:
+          cast_from_fp8_vec16<FMT, BF16_OUT, SK_ROW, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+          break;
+        case SK_COL:
+          cast_from_fp8_vec16<FMT, BF16_OUT, SK_COL, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+          break;
+        default:
+          cast_from_fp8_vec16<FMT, BF16_OUT, SK_FULL, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+          break;
+      }
+      done = p.rows == 1 ? vpr * 16 : n;
+    }
+  }
+  if (done < n) {
+    const int64_t grid = (n - done + kThreads - 1) / kThreads;
+    if (grid > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+    cast_from_fp8_generic<FMT, BF16_OUT><<<(unsigned)grid, kThreads, 0, st>>>(x, y, scale, sh, mode, done, n, mid, inner);
+  }
+  return launch_status();
+}
+
+inline bool scale_args_ok(const float* scale, int mode, int64_t outer, int64_t mid, int64_t inner) {
+  if (mode < MI355Q_SCALE_NONE || mode > MI355Q_SCALE_FULL) return false;
+  if (outer < 0 || mid < 0 || inner < 0) return false;
+  if ((mode == MI355Q_SCALE_DEV || mode == MI355Q_SCALE_MID || mode == MI355Q_SCALE_FULL) && scale == nullptr)
+    return false;
+  return true;
+}
+
+}  // namespace mi355q
+
+using namespace mi355q;
+
+extern "C" {
+
+int mi355q_amax(const void* x, int x_dtype, int64_t n, float* amax_out, void* stream) {
+  if (amax_out == nullptr || n < 0 || (n > 0 && x == nullptr)) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (x_dtype != MI355Q_F32 && x_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint32_t* am = reinterpret_cast<uint32_t*>(amax_out);
+  fill_u32_kernel<<<1, 1, 0, st>>>(am, 0u);
+  if (n == 0) return launch_status();
+  constexpr int U = 4;
+  const int es = x_dtype == MI355Q_BF16 ? 2 : 4;
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  int64_t done = 0;
+  if (aligned(x, 16)) {
+    const int64_t nvec = n * es / 16;
+    if (nvec > 0) {
+      const int64_t grid = (nvec + kThreads * U - 1) / (kThreads * U);
+      if (grid > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+      if (x_dtype == MI355Q_BF16) amax_vec<true, U><<<(unsigned)grid, kThreads, 0, st>>>(xb, nvec, am);
+      else amax_vec<false, U><<<(unsigned)grid, kThreads, 0, st>>>(xb, nvec, am);
+      done = nvec * (16 / es);
+    }
+  }
+  if (done < n) {
+    const int64_t grid = (n - done + kThreads - 1) / kThreads;
+    if (grid > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+    if (x_dtype == MI355Q_BF16) amax_generic<true><<<(unsigned)grid, kThreads, 0, st>>>(xb, done, n, am);
+    else amax_generic<false><<<(unsigned)grid, kThreads, 0, st>>>(xb, done, n, am);
+  }
+  return launch_status();
+}
+
+int mi355q_rowwise_amax(const void* x, int x_dtype, int64_t rows, int64_t cols, float* amax_out,
+                        void* stream) {
+  if (rows < 0 || cols < 0) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (rows == 0) return MI355Q_OK;
+  if (amax_out == nullptr || (cols > 0 && x == nullptr)) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (x_dtype != MI355Q_F32 && x_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (rows > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int es = x_dtype == MI355Q_BF16 ? 2 : 4;
+  const int vec_ok = aligned(x, 16) && (cols * es) % 16 == 0;
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  if (x_dtype == MI355Q_BF16) rowwise_amax_kernel<true><<<(unsigned)rows, kThreads, 0, st>>>(xb, cols, vec_ok, amax_out);
+  else rowwise_amax_kernel<false><<<(unsigned)rows, kThreads, 0, st>>>(xb, cols, vec_ok, amax_out);
+  return launch_status();
+}
+
+int mi355q_cast_to_fp8(const void* x, int x_dtype, void* y, int fp8_fmt, const float* scale_dev,
+                       float scale_host, int scale_mode, int64_t outer, int64_t mid, int64_t inner,
+                       float* amax_out, void* stream) {
+  if (fp8_fmt != MI355Q_E4M3FN && fp8_fmt != MI355Q_E5M2) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (!scale_args_ok(scale_dev, scale_mode, outer, mid, inner)) return MI355Q_ERR_INVALID_ARGUMENT;
+  const int64_t n = outer * mid * inner;
+  if (n > 0 && (x == nullptr || y == nullptr)) return MI355Q_ERR_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  uint8_t* yb = static_cast<uint8_t*>(y);
+
+  if (x_dtype == MI355Q_E4M3FN || x_dtype == MI355Q_E5M2) {
+    // fp8 in, same fp8 out: identity copy, no amax (fp8_ops.cpp:201-215)
+    if (x_dtype != fp8_fmt || amax_out != nullptr) return MI355Q_ERR_INVALID_ARGUMENT;
+    if (n == 0) return MI355Q_OK;
+    int64_t done = 0;
+    if (aligned(x, 16) && aligned(y, 16) && n >= 16) {
+      const int64_t nvec = n / 16;
+      copy_vec16_kernel<<<blocks_for(nvec, kThreads), kThreads, 0, st>>>(
+          reinterpret_cast<const u32x4*>(xb), reinterpret_cast<u32x4*>(yb), nvec);
+      done = nvec * 16;
+    }
+    if (done < n)
+      copy_bytes_kernel<<<blocks_for(n - done, kThreads), kThreads, 0, st>>>(xb + done, yb + done, n - done);
+    return launch_status();
+  }
+  if (x_dtype != MI355Q_F32 && x_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
+
+  uint32_t* am = reinterpret_cast<uint32_t*>(amax_out);
+  if (am) fill_u32_kernel<<<1, 1, 0, st>>>(am, 0u);
+  if (n == 0) return launch_status();
+  if (x_dtype == MI355Q_BF16) {
+    if (fp8_fmt == MI355Q_E4M3FN) return cast_to_dispatch<true, MI355Q_E4M3FN>(xb, yb, scale_dev, scale_host, scale_mode, outer, mid, inner, am, st);
+    return cast_to_dispatch<true, MI355Q_E5M2>(xb, yb, scale_dev, scale_host, scale_mode, outer, mid, inner, am, st);
+  }
+  if (fp8_fmt == MI355Q_E4M3FN) return cast_to_dispatch<false, MI355Q_E4M3FN>(xb, yb, scale_dev, scale_host, scale_mode, outer, mid, inner, am, st);
+  return cast_to_dispatch<false, MI355Q_E5M2>(xb, yb, scale_dev, scale_host, scale_mode, outer, mid, inner, am, st);
+}
+
+int mi355q_cast_from_fp8(const void* x, int fp8_fmt, void* y, int out_dtype, const float* scale_dev,
+                         float scale_host, int scale_mode, int64_t outer, int64_t mid,
+                         int64_t inner, void* stream) {
+  if (fp8_fmt != MI355Q_E4M3FN && fp8_fmt != MI355Q_E5M2) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (out_dtype != MI355Q_F32 && out_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (!scale_args_ok(scale_dev, scale_mode, outer, mid, inner)) return MI355Q_ERR_INVALID_ARGUMENT;
+  const int64_t n = outer * mid * inner;
+  if (n == 0) return MI355Q_OK;
+  if (x == nullptr || y == nullptr) return MI355Q_ERR_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  uint8_t* yb = static_cast<uint8_t*>(y);
+  if (fp8_fmt == MI355Q_E4M3FN) {
+    if (out_dtype == MI355Q_BF16) return cast_from_dispatch<MI355Q_E4M3FN, true>(xb, yb, scale_dev, scale_host, scale_mode, outer, mid, inner, st);
+    return cast_from_dispatch<MI355Q_E4M3FN, false>(xb, yb, scale_dev, scale_host, scale_mode, outer, mid, inner, st);
+  }
+  if (out_dtype == MI355Q_BF16) return cast_from_dispatch<MI355Q_E5M2, true>(xb, yb, scale_dev, scale_host, scale_mode, outer, mid, inner, st);
+  return cast_from_dispatch<MI355Q_E5M2, false>(xb, yb, scale_dev, scale_host, scale_mode, outer, mid, inner, st);
+}
+
+}  // extern "C"

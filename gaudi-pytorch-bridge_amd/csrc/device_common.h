@@ -1,0 +1,91 @@
+// Shared device-side helpers for the gfx950 kernels: vector types, fp8 / bf16
+// conversions built on the CDNA4 conversion instructions, wave reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mi355q.h"
+
+namespace mi355q {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kFp8Max[2] = {448.0f, 57344.0f};  // e4m3fn, e5m2
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// fp32 -> bf16 round-to-nearest-even (v_cvt_pk_bf16_f32), returned as fp32.
+__device__ __forceinline__ float round_to_bf16(float v) {
+  __bf16 h = (__bf16)v;
+  return (float)h;
+}
+
+// two fp32 -> packed bf16 pair (lo = a, hi = b)
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  bf16x2 r = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+// Clamp to the finite fp8 range.  minimum/maximum propagate NaN, so a NaN
+// input still converts to an fp8 NaN; +-Inf saturates like any overflow.
+template <int FMT>
+__device__ __forceinline__ float sat_fp8(float v) {
+  constexpr float mx = (FMT == MI355Q_E5M2) ? 57344.0f : 448.0f;
+  return __builtin_elementwise_minimum(__builtin_elementwise_maximum(v, -mx), mx);
+}
+
+// four fp32 -> four fp8 bytes (element 0 in the low byte), RNE, saturating.
+// The raw v_cvt_pk_{fp8,bf8}_f32 turns overflow into NaN/Inf, hence the clamp.
+template <int FMT>
+__device__ __forceinline__ uint32_t cvt_fp8x4(float a, float b, float c, float d) {
+  a = sat_fp8<FMT>(a);
+  b = sat_fp8<FMT>(b);
+  c = sat_fp8<FMT>(c);
+  d = sat_fp8<FMT>(d);
+  int r;
+  if constexpr (FMT == MI355Q_E5M2) {
+    r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+    r = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, r, true);
+  } else {
+    r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+  }
+  return (uint32_t)r;
+}
+
+// four fp8 bytes of one dword -> four fp32 (exact)
+template <int FMT>
+__device__ __forceinline__ void cvt_f32x4(uint32_t w, float& a, float& b, float& c, float& d) {
+  f32x2 lo, hi;
+  if constexpr (FMT == MI355Q_E5M2) {
+    lo = __builtin_amdgcn_cvt_pk_f32_bf8((int)w, false);
+    hi = __builtin_amdgcn_cvt_pk_f32_bf8((int)w, true);
+  } else {
+    lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+    hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+  }
+  a = lo.x; b = lo.y; c = hi.x; d = hi.y;
+}
+
+template <int FMT>
+__device__ __forceinline__ float cvt_f32x1(uint32_t byte) {
+  if constexpr (FMT == MI355Q_E5M2) return __builtin_amdgcn_cvt_f32_bf8((int)byte, 0);
+  else return __builtin_amdgcn_cvt_f32_fp8((int)byte, 0);
+}
+
+// max over the 64 lanes of a wave of a non-negative-float bit pattern
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    uint32_t o = (uint32_t)__shfl_xor((int)v, off, 64);
+    v = v > o ? v : o;
+  }
+  return v;
+}
+
+}  // namespace mi355q

@@ -1,0 +1,652 @@
+// torch.ops.hpu.* host layer on PyTorch-ROCm: schemas, argument checks, output
+// allocation and the calls into the mi355q C ABI.
+//
+// The schema strings are those of the reference
+// (habana_eager/eager_custom_op_register.cpp:2146-2171); the checks and error
+// strings follow CastToFp8V2::AddNode, CastFromFp8::AddNode, Fp8GemmV2::AddNode
+// (hpu_ops/backend/fp8_ops.cpp:29-53,192-308,403-496), Int4BaseOp
+// (hpu_ops/backend/int4_ops.cpp:22-56) and getBatchMatmulOutShape
+// (hpu_ops/common/batched_matmul_output_shape.cpp:33-85).  Output shapes and
+// dtypes for tracing follow dynamo/_custom_op_meta_registrations.py:56-217.
+//
+// Kernels are registered for the CUDA dispatch key (the key PyTorch-ROCm uses
+// for HIP tensors) and for Meta.  There is no CPU implementation: a CPU tensor
+// fails in the dispatcher.
+#include <ATen/ATen.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/library.h>
+
+#include <cstdlib>
+#include <iostream>
+#include <sstream>
+
+#include "../../include/mi355q.h"
+
+namespace {
+
+using at::Tensor;
+using c10::IValue;
+using OptShape = c10::optional<std::vector<int64_t>>;
+// PyTorch-ROCm presents HIP devices under the name "cuda".
+using DeviceGuard = c10::hip::HIPGuardMasqueradingAsCUDA;
+
+bool log_enabled() {
+  static const bool on = [] {
+    const char* e = std::getenv("MI355Q_LOG");
+    return e != nullptr && e[0] != '\0' && e[0] != '0';
+  }();
+  return on;
+}
+
+#define MI355Q_OP_INFO(...)                                   \
+  do {                                                        \
+    if (log_enabled()) {                                      \
+      std::ostringstream os__;                                \
+      os__ << "[mi355q] " << __VA_ARGS__ << "\n";             \
+      std::cerr << os__.str();                                \
+    }                                                         \
+  } while (0)
+
+void check_status(int st, const char* what) {
+  TORCH_CHECK(st == MI355Q_OK, what, " failed: ", mi355q_status_string(st));
+}
+
+bool is_fp8(at::ScalarType t) {
+  return t == at::kFloat8_e5m2 || t == at::kFloat8_e4m3fn;
+}
+
+int to_mi355q_dtype(at::ScalarType t) {
+  switch (t) {
+    case at::kFloat: return MI355Q_F32;
+    case at::kBFloat16: return MI355Q_BF16;
+    case at::kFloat8_e4m3fn: return MI355Q_E4M3FN;
+    case at::kFloat8_e5m2: return MI355Q_E5M2;
+    default: TORCH_CHECK(false, "mi355q: unsupported dtype ", t);
+  }
+}
+
+void* current_stream(const Tensor& t) {
+  return static_cast<void*>(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream());
+}
+
+int64_t prod(at::IntArrayRef v, size_t b, size_t e) {
+  int64_t p = 1;
+  for (size_t i = b; i < e; ++i) p *= v[i];
+  return p;
+}
+
+// ValidateScaleShape, hpu_ops/backend/fp8_ops.cpp:29-53
+void validate_scale_shape(const IValue& scale, const OptShape& scale_shape) {
+  if (scale.isNone() || scale.isDouble() || !scale_shape.has_value()) return;
+  int64_t scale_numel = 0;
+  if (scale.isTensor()) scale_numel = scale.toTensor().numel();
+  else if (scale.isDoubleList()) scale_numel = (int64_t)scale.toDoubleVector().size();
+  int64_t shape_numel = 1;
+  for (auto d : *scale_shape) shape_numel *= d;
+  TORCH_CHECK(scale_numel == shape_numel, "Number of scale elements (", scale_numel,
+              ") is not equal to number of scale_shape elements (", shape_numel, ").");
+}
+
+// A cast scale resolved against the input shape, ready for the C ABI.
+struct CastScale {
+  Tensor holder;  // keeps device memory alive
+  const float* dev = nullptr;
+  float host = 1.0f;
+  int mode = MI355Q_SCALE_NONE;
+  int64_t outer = 1, mid = 1, inner = 1;
+};
+
+Tensor list_to_device(const std::vector<double>& v, const Tensor& like) {
+  Tensor cpu = at::empty({(int64_t)v.size()}, at::TensorOptions().dtype(at::kFloat));
+  float* p = cpu.data_ptr<float>();
+  for (size_t i = 0; i < v.size(); ++i) p[i] = (float)v[i];
+  return cpu.to(like.device());
+}
+
+CastScale resolve_cast_scale(const IValue& scale, const OptShape& scale_shape, const Tensor& x) {
+  CastScale r;
+  const int64_t n = x.numel();
+  r.outer = n;
+  if (scale.isNone()) return r;
+  if (scale.isDouble()) {
+    r.mode = MI355Q_SCALE_HOST;
+    r.host = (float)scale.toDouble();
+    return r;
+  }
+  Tensor s;
+  if (scale.isDoubleList()) {
+    auto v = scale.toDoubleVector();
+    TORCH_CHECK(!v.empty(), "scale list must not be empty");
+    if (v.size() == 1) {
+      r.mode = MI355Q_SCALE_HOST;
+      r.host = (float)v[0];
+      return r;
+    }
+    s = list_to_device(v, x);
+  } else {
+    TORCH_CHECK(scale.isTensor(), "scale must be None, a Tensor, a float or a list of floats");
+    s = scale.toTensor();
+    TORCH_CHECK(s.device() == x.device(), "scale must be on the same device as input, got ",
+                s.device(), " and ", x.device());
+    s = s.to(at::kFloat).contiguous();
+  }
+  if (s.numel() == 1) {
+    r.holder = s;
+    r.dev = s.data_ptr<float>();
+    r.mode = MI355Q_SCALE_DEV;
+    return r;
+  }
+  std::vector<int64_t> shp = scale_shape.has_value() ? *scale_shape : s.sizes().vec();
+  const auto xs = x.sizes();
+  TORCH_CHECK(shp.size() <= xs.size(), "scale shape ", at::IntArrayRef(shp),
+              " is not broadcastable to input shape ", xs);
+  std::vector<int64_t> full(xs.size(), 1);
+  std::copy(shp.begin(), shp.end(), full.begin() + (xs.size() - shp.size()));
+  for (size_t i = 0; i < xs.size(); ++i)
+    TORCH_CHECK(full[i] == 1 || full[i] == xs[i], "scale shape ", at::IntArrayRef(shp),
+                " is not broadcastable to input shape ", xs);
+  // One contiguous run of dims where the scale is not broadcast -> [outer, mid, inner].
+  size_t a = 0;
+  while (a < full.size() && (full[a] == 1)) ++a;
+  size_t b = full.size();
+  while (b > a && (full[b - 1] == 1)) --b;
+  bool run = true;
+  for (size_t i = a; i < b; ++i) run = run && (full[i] == xs[i]);
+  if (run) {
+    r.holder = s;
+    r.dev = s.data_ptr<float>();
+    r.outer = prod(xs, 0, a);
+    r.mid = prod(xs, a, b);
+    r.inner = prod(xs, b, xs.size());
+    if (r.outer == 1 && r.inner == 1) {
+      r.mode = MI355Q_SCALE_FULL;
+      r.outer = n;
+      r.mid = r.inner = 1;
+    } else {
+      r.mode = MI355Q_SCALE_MID;
+    }
+    return r;
+  }
+  Tensor e = s.reshape(full).expand(xs).contiguous();
+  r.holder = e;
+  r.dev = e.data_ptr<float>();
+  r.mode = MI355Q_SCALE_FULL;
+  return r;
+}
+
+// ------------------------------------------------------------ cast_to_fp8_v2
+
+void check_cast_to_args(const Tensor& input, bool stochastic_rounding, bool is_amax,
+                        const IValue& dtype_iv, const IValue& scale, const OptShape& scale_shape) {
+  const auto src = input.scalar_type();
+  const bool fp8_in = is_fp8(src);
+  TORCH_CHECK(fp8_in || src == at::kFloat || src == at::kBFloat16,
+              "CastToFp8V2 input dtype must be one of [float, bfloat16, float8_e5m2, float8_e4m3fn].");
+  TORCH_CHECK(!dtype_iv.isNone(),
+              "cast_to_fp8_v2: dtype must be given (torch.float8_e4m3fn or torch.float8_e5m2)");
+  const auto dst = dtype_iv.toScalarType();
+  TORCH_CHECK(is_fp8(dst), "cast_to_fp8_v2: dtype must be torch.float8_e4m3fn or torch.float8_e5m2, got ", dst);
+  if (fp8_in) {
+    TORCH_CHECK(!is_amax, "CastToFp8V2 must have no amax for float8.");
+    TORCH_CHECK(src == dst, "CastToFp8V2 input and output must have the same dtype for float8, but are ",
+                src, " and ", dst);
+  }
+  validate_scale_shape(scale, scale_shape);
+  TORCH_CHECK(!stochastic_rounding,
+              "cast_to_fp8_v2: stochastic_rounding=True is not implemented in this build "
+              "(round-to-nearest-even only)");
+}
+
+OptShape shape_from_ivalue(const IValue& v) {
+  if (v.isNone()) return c10::nullopt;
+  return v.toIntVector();
+}
+
+// Stack layout (all three overloads): input, scale, stochastic_rounding,
+// is_amax, dtype, scale_shape.  The .scalar overload ignores scale_shape
+// (eager_custom_op_register.cpp:92-101).
+void cast_to_fp8_v2_boxed(const c10::OperatorHandle& op, c10::DispatchKeySet, torch::jit::Stack* stack) {
+  TORCH_CHECK(stack->size() >= 6, "cast_to_fp8_v2 expects 6 arguments");
+  const size_t base = stack->size() - 6;
+  Tensor input = (*stack)[base + 0].toTensor();
+  IValue scale = (*stack)[base + 1];
+  const bool sr = (*stack)[base + 2].toBool();
+  const bool is_amax = (*stack)[base + 3].toBool();
+  IValue dtype_iv = (*stack)[base + 4];
+  OptShape scale_shape = scale.isDouble() ? c10::nullopt : shape_from_ivalue((*stack)[base + 5]);
+  (void)op;
+
+  check_cast_to_args(input, sr, is_amax, dtype_iv, scale, scale_shape);
+  const auto dst = dtype_iv.toScalarType();
+  MI355Q_OP_INFO("cast_to_fp8_v2 : input=" << input.sizes() << " " << input.scalar_type()
+                                           << " is_amax=" << is_amax << " dtype=" << dst);
+
+  Tensor out, amax;
+  if (input.is_meta()) {
+    out = at::empty(input.sizes(), input.options().dtype(dst));
+    amax = at::empty(is_amax ? std::vector<int64_t>{} : std::vector<int64_t>{0},
+                     input.options().dtype(at::kFloat));
+  } else {
+    DeviceGuard guard(input.device());
+    Tensor x = input.contiguous();
+    out = at::empty(x.sizes(), x.options().dtype(dst));
+    amax = at::empty(is_amax ? std::vector<int64_t>{} : std::vector<int64_t>{0},
+                     x.options().dtype(at::kFloat));
+    CastScale cs;
+    if (is_fp8(x.scalar_type())) {
+      cs.outer = x.numel();  // fp8 -> same fp8: copy, scale plays no part
+    } else {
+      cs = resolve_cast_scale(scale, scale_shape, x);
+    }
+    check_status(mi355q_cast_to_fp8(x.data_ptr(), to_mi355q_dtype(x.scalar_type()), out.data_ptr(),
+                                    to_mi355q_dtype(dst), cs.dev, cs.host, cs.mode, cs.outer, cs.mid,
+                                    cs.inner, is_amax ? amax.data_ptr<float>() : nullptr,
+                                    current_stream(x)),
+                 "mi355q_cast_to_fp8");
+  }
+  torch::jit::drop(*stack, 6);
+  stack->emplace_back(std::move(out));
+  stack->emplace_back(std::move(amax));
+}
+
+// ------------------------------------------------------------- cast_from_fp8
+
+Tensor cast_from_fp8_impl(const Tensor& input, const IValue& scale, at::ScalarType out_dtype,
+                          const OptShape& scale_shape) {
+  validate_scale_shape(scale, scale_shape);
+  TORCH_CHECK(out_dtype == at::kFloat || out_dtype == at::kBFloat16,
+              "CastFromFp8 output dtype must be equal to float or bfloat16.");
+  TORCH_CHECK(is_fp8(input.scalar_type()), "CastFromFp8 input must be float8_e5m2 or float8_e4m3fn, got ",
+              input.scalar_type());
+  MI355Q_OP_INFO("cast_from_fp8 : input=" << input.sizes() << " " << input.scalar_type()
+                                          << " out_dtype=" << out_dtype);
+  if (input.is_meta()) return at::empty(input.sizes(), input.options().dtype(out_dtype));
+  DeviceGuard guard(input.device());
+  Tensor x = input.contiguous();
+  Tensor out = at::empty(x.sizes(), x.options().dtype(out_dtype));
+  CastScale cs = resolve_cast_scale(scale, scale_shape, x);
+  check_status(mi355q_cast_from_fp8(x.data_ptr(), to_mi355q_dtype(x.scalar_type()), out.data_ptr(),
+                                    to_mi355q_dtype(out_dtype), cs.dev, cs.host, cs.mode, cs.outer,
+                                    cs.mid, cs.inner, current_stream(x)),
+               "mi355q_cast_from_fp8");
+  return out;
+}
+
+OptShape to_opt_shape(at::OptionalIntArrayRef s) {
+  if (!s.has_value()) return c10::nullopt;
+  return s->vec();
+}
+
+Tensor cast_from_fp8(const Tensor& input, const c10::optional<Tensor>& scale, at::ScalarType out_dtype,
+                     at::OptionalIntArrayRef scale_shape) {
+  return cast_from_fp8_impl(input, scale.has_value() ? IValue(*scale) : IValue(), out_dtype,
+                            to_opt_shape(scale_shape));
+}
+Tensor cast_from_fp8_scalar(const Tensor& input, double scale, at::ScalarType out_dtype,
+                            at::OptionalIntArrayRef) {
+  return cast_from_fp8_impl(input, IValue(scale), out_dtype, c10::nullopt);
+}
+Tensor cast_from_fp8_scalar_list(const Tensor& input, c10::ArrayRef<double> scale,
+                                 at::ScalarType out_dtype, at::OptionalIntArrayRef scale_shape) {
+  return cast_from_fp8_impl(input, IValue(scale.vec()), out_dtype, to_opt_shape(scale_shape));
+}
+
+// --------------------------------------------------------------- fp8_gemm_v2
+
+// torch.matmul shape rule with optional transposes of the last two dims
+// (getBatchMatmulOutShape, hpu_ops/common/batched_matmul_output_shape.cpp:33-85).
+std::vector<int64_t> matmul_out_shape(at::IntArrayRef a, at::IntArrayRef b, bool ta, bool tb) {
+  const size_t ra = a.size(), rb = b.size();
+  TORCH_CHECK(ra >= 1 && rb >= 1, "fp8_gemm_v2 operands must have at least 1 dimension");
+  std::vector<int64_t> tail;
+  int64_t ka = a[0], kb = b[0];
+  if (ra > 1) {
+    tail.push_back(ta ? a[ra - 1] : a[ra - 2]);
+    ka = ta ? a[ra - 2] : a[ra - 1];
+  }
+  if (rb > 1) {
+    tail.push_back(tb ? b[rb - 2] : b[rb - 1]);
+    kb = tb ? b[rb - 1] : b[rb - 2];
+  }
+  TORCH_CHECK(ka == kb, "Common dimension sizes of matmul inputs should be the same. Got ", ka,
+              " and ", kb);
+  const size_t mr = std::max(ra, rb);
+  std::vector<int64_t> out;
+  for (size_t i = mr; i >= 3; --i) {
+    const int64_t da = i > ra ? 1 : a[ra - i];
+    const int64_t db = i > rb ? 1 : b[rb - i];
+    TORCH_CHECK(da == db || da == 1 || db == 1, "Batch dimension ", mr - i,
+                " of matmul inputs should be the same or at least one of them should be equal to 1. Got ",
+                da, " and ", db);
+    out.push_back(da == db ? da : da * db);
+  }
+  out.insert(out.end(), tail.begin(), tail.end());
+  return out;
+}
+
+struct GemmScale {
+  Tensor holder;
+  const float* dev = nullptr;
+  float host = 1.0f;
+  int mode = MI355Q_GS_NONE;
+};
+
+GemmScale resolve_gemm_scale(const IValue& scale, const OptShape& shape, int64_t M, int64_t N,
+                             const Tensor& like, const char* name) {
+  GemmScale r;
+  if (scale.isNone()) return r;
+  if (scale.isDouble()) {
+    r.mode = MI355Q_GS_HOST;
+    r.host = (float)scale.toDouble();
+    return r;
+  }
+  Tensor s;
+  if (scale.isDoubleList()) {
+    auto v = scale.toDoubleVector();
+    TORCH_CHECK(!v.empty(), name, " list must not be empty");
+    if (v.size() == 1) {
+      r.mode = MI355Q_GS_HOST;
+      r.host = (float)v[0];
+      return r;
+    }
+    s = list_to_device(v, like);
+  } else {
+    s = scale.toTensor();
+    TORCH_CHECK(s.device() == like.device(), name, " must be on the same device as A");
+    s = s.to(at::kFloat).contiguous();
+  }
+  r.holder = s;
+  r.dev = s.data_ptr<float>();
+  if (s.numel() == 1) {
+    r.mode = MI355Q_GS_DEV;
+    return r;
+  }
+  std::vector<int64_t> shp = shape.has_value() ? *shape : s.sizes().vec();
+  while (shp.size() > 2 && shp.front() == 1) shp.erase(shp.begin());
+  if (shp.size() == 1) shp.insert(shp.begin(), 1);
+  TORCH_CHECK(shp.size() == 2, name, " with shape ", at::IntArrayRef(shp),
+              " does not broadcast against the [M, N] output");
+  if (shp[0] == M && shp[1] == 1) r.mode = MI355Q_GS_PER_ROW;
+  else if (shp[0] == 1 && shp[1] == N) r.mode = MI355Q_GS_PER_COL;
+  else TORCH_CHECK(false, name, " with shape ", at::IntArrayRef(shp),
+                   " does not broadcast against the [", M, ", ", N, "] output as [M,1] or [1,N]");
+  return r;
+}
+
+Tensor fp8_gemm_v2_impl(const Tensor& A, bool trans_A, const Tensor& B, bool trans_B,
+                        const c10::optional<Tensor>& D, at::ScalarType out_dtype,
+                        const IValue& A_scale_inv, const IValue& B_scale_inv,
+                        const c10::optional<Tensor>& bias, bool accumulate,
+                        const OptShape& B_scale_shape) {
+  std::vector<int64_t> out_shape = matmul_out_shape(A.sizes(), B.sizes(), trans_A, trans_B);
+  validate_scale_shape(B_scale_inv, B_scale_shape);
+  TORCH_CHECK(!accumulate || D.has_value(),
+              "Accumulation tensor must be provided at index 4 for Fp8GemmV2, when accumulate is true");
+  TORCH_CHECK(out_dtype == at::kFloat || out_dtype == at::kBFloat16,
+              "fp8_gemm_v2 output dtype must be float or bfloat16, got ", out_dtype);
+  TORCH_CHECK(is_fp8(A.scalar_type()) && is_fp8(B.scalar_type()),
+              "fp8_gemm_v2 operands must be float8_e5m2 or float8_e4m3fn, got ", A.scalar_type(),
+              " and ", B.scalar_type());
+  MI355Q_OP_INFO("fp8_gemm_v2 : A=" << A.sizes() << " trans_A=" << trans_A << " B=" << B.sizes()
+                                    << " trans_B=" << trans_B << " out_dtype=" << out_dtype
+                                    << " accumulate=" << accumulate);
+  if (A.is_meta()) return at::empty(out_shape, A.options().dtype(out_dtype));
+  TORCH_CHECK(A.device() == B.device(), "fp8_gemm_v2 operands must be on the same device");
+  DeviceGuard guard(A.device());
+
+  // Reduce to batch x [M,K] x [K,N].
+  const bool a1 = A.dim() == 1, b1 = B.dim() == 1;
+  Tensor a = a1 ? A.unsqueeze(0) : A;  // [1, K]
+  Tensor b = b1 ? B.unsqueeze(1) : B;  // [K, 1]
+  const bool ta = a1 ? false : trans_A, tb = b1 ? false : trans_B;
+  const int64_t ar = a.size(-2), ac = a.size(-1), br = b.size(-2), bc = b.size(-1);
+  const int64_t M = ta ? ac : ar, K = ta ? ar : ac, N = tb ? br : bc;
+  std::vector<int64_t> batch_shape(out_shape.begin(),
+                                   out_shape.end() - ((a1 ? 0 : 1) + (b1 ? 0 : 1)));
+  int64_t batch = 1;
+  for (auto d : batch_shape) batch *= d;
+
+  auto prep = [&](const Tensor& t, int64_t rows, int64_t cols, int64_t* stride) {
+    int64_t tb_numel = t.numel() / std::max<int64_t>(rows * cols, 1);
+    if (rows * cols == 0) tb_numel = 1;
+    Tensor c;
+    if (tb_numel == 1) {
+      *stride = 0;
+      c = t.reshape({rows, cols}).contiguous();
+    } else {
+      std::vector<int64_t> full = batch_shape;
+      full.push_back(rows);
+      full.push_back(cols);
+      c = t.expand(full).contiguous();
+      *stride = rows * cols;
+    }
+    return c;
+  };
+  int64_t stride_a = 0, stride_b = 0;
+  Tensor ac_t = prep(a, ar, ac, &stride_a);
+  Tensor bc_t = prep(b, br, bc, &stride_b);
+
+  Tensor out = at::empty(out_shape, A.options().dtype(out_dtype));
+  if (out.numel() == 0) return out;
+
+  GemmScale sa = resolve_gemm_scale(A_scale_inv, c10::nullopt, M, N, A, "A_scale_inv");
+  GemmScale sb = resolve_gemm_scale(B_scale_inv, B_scale_shape, M, N, A, "B_scale_inv");
+
+  std::vector<int64_t> full_out = batch_shape;
+  full_out.push_back(M);
+  full_out.push_back(N);
+
+  Tensor bias_t, d_t;
+  int bias_mode = MI355Q_BIAS_NONE;
+  int64_t ldbias = 0, stride_bias = 0, stride_d = 0;
+  if (bias.has_value() && bias->defined()) {
+    bias_t = bias->to(out_dtype);
+    if (!b1 && bias_t.dim() <= 1 && bias_t.numel() == N) {
+      bias_t = bias_t.contiguous();
+      bias_mode = MI355Q_BIAS_ROW_VECTOR;
+    } else {
+      // broadcast against the output as torch would, then view as [batch, M, N]
+      bias_t = bias_t.expand(out_shape).reshape(full_out).contiguous();
+      bias_mode = MI355Q_BIAS_FULL;
+      ldbias = N;
+      stride_bias = M * N;
+    }
+  }
+  if (accumulate) {
+    d_t = D->to(out_dtype).expand(out_shape).reshape(full_out).contiguous();
+    stride_d = M * N;
+  }
+
+  check_status(
+      mi355q_fp8_gemm(ac_t.data_ptr(), to_mi355q_dtype(A.scalar_type()), ta ? 1 : 0, ac,
+                      bc_t.data_ptr(), to_mi355q_dtype(B.scalar_type()), tb ? 1 : 0, bc,
+                      out.data_ptr(), to_mi355q_dtype(out_dtype), N, M, N, K, sa.dev, sa.host, sa.mode,
+                      sb.dev, sb.host, sb.mode, bias_mode != MI355Q_BIAS_NONE ? bias_t.data_ptr() : nullptr,
+                      bias_mode, ldbias, accumulate ? d_t.data_ptr() : nullptr, N, batch, stride_a,
+                      stride_b, M * N, stride_d, stride_bias, current_stream(A)),
+      "mi355q_fp8_gemm");
+  return out;
+}
+
+IValue opt_tensor_iv(const c10::optional<Tensor>& t) {
+  return (t.has_value() && t->defined()) ? IValue(*t) : IValue();
+}
+
+Tensor fp8_gemm_v2(const Tensor& A, bool trans_A, const Tensor& B, bool trans_B,
+                   const c10::optional<Tensor>& D, at::ScalarType out_dtype,
+                   const c10::optional<Tensor>& A_scale_inv, const c10::optional<Tensor>& B_scale_inv,
+                   const c10::optional<Tensor>& bias, bool accumulate,
+                   at::OptionalIntArrayRef B_scale_shape) {
+  return fp8_gemm_v2_impl(A, trans_A, B, trans_B, D, out_dtype, opt_tensor_iv(A_scale_inv),
+                          opt_tensor_iv(B_scale_inv), bias, accumulate, to_opt_shape(B_scale_shape));
+}
+Tensor fp8_gemm_v2_scalar(const Tensor& A, bool trans_A, const Tensor& B, bool trans_B,
+                          const c10::optional<Tensor>& D, at::ScalarType out_dtype, double A_scale_inv,
+                          double B_scale_inv, const c10::optional<Tensor>& bias, bool accumulate,
+                          at::OptionalIntArrayRef) {
+  return fp8_gemm_v2_impl(A, trans_A, B, trans_B, D, out_dtype, IValue(A_scale_inv),
+                          IValue(B_scale_inv), bias, accumulate, c10::nullopt);
+}
+Tensor fp8_gemm_v2_scalar_list(const Tensor& A, bool trans_A, const Tensor& B, bool trans_B,
+                               const c10::optional<Tensor>& D, at::ScalarType out_dtype,
+                               c10::ArrayRef<double> A_scale_inv, c10::ArrayRef<double> B_scale_inv,
+                               const c10::optional<Tensor>& bias, bool accumulate,
+                               at::OptionalIntArrayRef B_scale_shape) {
+  return fp8_gemm_v2_impl(A, trans_A, B, trans_B, D, out_dtype, IValue(A_scale_inv.vec()),
+                          IValue(B_scale_inv.vec()), bias, accumulate, to_opt_shape(B_scale_shape));
+}
+
+// ------------------------------------------------- convert_from_int4 / uint4
+
+Tensor convert_from_int4_common(const char* op_name, bool is_signed, const Tensor& input,
+                                const Tensor& scale, const c10::optional<Tensor>& zero_point,
+                                at::ScalarType out_dtype) {
+  TORCH_CHECK(input.scalar_type() == at::kInt, op_name, " input must be int32 (8 nibbles per element), got ",
+              input.scalar_type());
+  TORCH_CHECK(input.dim() >= 1, op_name, " input must have at least 1 dimension");
+  TORCH_CHECK(out_dtype == at::kFloat || out_dtype == at::kBFloat16, op_name,
+              " output dtype must be float or bfloat16, got ", out_dtype);
+  std::vector<int64_t> out_shape = input.sizes().vec();
+  out_shape.back() *= 8;
+  MI355Q_OP_INFO(op_name << " : input=" << input.sizes() << " scale=" << scale.sizes()
+                         << " out_dtype=" << out_dtype);
+  if (input.is_meta()) return at::empty(out_shape, input.options().dtype(out_dtype));
+  DeviceGuard guard(input.device());
+
+  const int64_t pcols = input.size(-1);
+  const int64_t cols = pcols * 8;
+  const int64_t rows = pcols ? input.numel() / pcols : 0;
+  Tensor out = at::empty(out_shape, input.options().dtype(out_dtype));
+  if (out.numel() == 0) return out;
+
+  TORCH_CHECK(scale.device() == input.device(), op_name, " scale must be on the same device as input");
+  TORCH_CHECK(scale.numel() > 0 && scale.numel() % cols == 0 && scale.size(-1) == cols, op_name,
+              " scale last dimension must equal 8 * input last dimension (", cols, "), got ",
+              scale.sizes());
+  const int64_t srows = scale.numel() / cols;
+  TORCH_CHECK(rows % srows == 0, op_name, " scale rows (", srows, ") must divide input rows (", rows, ")");
+  const int64_t group = rows / srows;
+  TORCH_CHECK(group == 1 || input.dim() == 2, op_name,
+              " group-wise scales need a 2-D input, got ", input.sizes());
+  auto aligned16 = [](const Tensor& t) {
+    return t.is_contiguous() && (reinterpret_cast<uintptr_t>(t.data_ptr()) & 15u) == 0;
+  };
+  Tensor x = input.contiguous();
+  Tensor s = scale.to(out_dtype);
+  if (!aligned16(s)) s = s.clone(at::MemoryFormat::Contiguous);
+  Tensor z;
+  int zp_kind = MI355Q_ZP_NONE;
+  if (zero_point.has_value() && zero_point->defined()) {
+    TORCH_CHECK(zero_point->device() == input.device(), op_name,
+                " zero_point must be on the same device as input");
+    if (zero_point->scalar_type() == at::kInt) {
+      TORCH_CHECK(zero_point->numel() == srows * pcols, op_name,
+                  " packed zero_point must hold one nibble per scale element, got ",
+                  zero_point->sizes(), " for scale ", scale.sizes());
+      z = zero_point->contiguous();
+      zp_kind = MI355Q_ZP_PACKED;
+    } else {
+      TORCH_CHECK(zero_point->numel() == scale.numel(), op_name,
+                  " zero_point must have the shape of scale, got ", zero_point->sizes(), " and ",
+                  scale.sizes());
+      z = zero_point->to(out_dtype);
+      if (!aligned16(z)) z = z.clone(at::MemoryFormat::Contiguous);
+      zp_kind = MI355Q_ZP_FLOAT;
+    }
+  }
+  check_status(mi355q_dequant_4bit(x.data_ptr<int32_t>(), s.data_ptr(),
+                                   zp_kind != MI355Q_ZP_NONE ? z.data_ptr() : nullptr, zp_kind,
+                                   is_signed ? 1 : 0, to_mi355q_dtype(out_dtype), rows, pcols, group,
+                                   out.data_ptr(), current_stream(x)),
+               "mi355q_dequant_4bit");
+  return out;
+}
+
+Tensor convert_from_int4(const Tensor& input, const Tensor& scale,
+                         const c10::optional<Tensor>& zero_point, at::ScalarType out_dtype) {
+  return convert_from_int4_common("convert_from_int4", true, input, scale, zero_point, out_dtype);
+}
+Tensor convert_from_uint4(const Tensor& input, const Tensor& scale,
+                          const c10::optional<Tensor>& zero_point, at::ScalarType out_dtype) {
+  return convert_from_int4_common("convert_from_uint4", false, input, scale, zero_point, out_dtype);
+}
+
+// ------------------------------------------------------------- amax helpers
+
+Tensor amax_op(const Tensor& x) {
+  TORCH_CHECK(x.scalar_type() == at::kFloat || x.scalar_type() == at::kBFloat16,
+              "mi355q::amax input must be float or bfloat16");
+  if (x.is_meta()) return at::empty({}, x.options().dtype(at::kFloat));
+  DeviceGuard guard(x.device());
+  Tensor c = x.contiguous();
+  Tensor out = at::empty({}, c.options().dtype(at::kFloat));
+  check_status(mi355q_amax(c.data_ptr(), to_mi355q_dtype(c.scalar_type()), c.numel(),
+                           out.data_ptr<float>(), current_stream(c)),
+               "mi355q_amax");
+  return out;
+}
+
+Tensor rowwise_amax_op(const Tensor& x) {
+  TORCH_CHECK(x.scalar_type() == at::kFloat || x.scalar_type() == at::kBFloat16,
+              "mi355q::rowwise_amax input must be float or bfloat16");
+  TORCH_CHECK(x.dim() >= 1, "mi355q::rowwise_amax input must have at least 1 dimension");
+  std::vector<int64_t> shp(x.sizes().begin(), x.sizes().end() - 1);
+  if (x.is_meta()) return at::empty(shp, x.options().dtype(at::kFloat));
+  DeviceGuard guard(x.device());
+  Tensor c = x.contiguous();
+  Tensor out = at::empty(shp, c.options().dtype(at::kFloat));
+  const int64_t cols = c.size(-1);
+  const int64_t rows = out.numel();
+  check_status(mi355q_rowwise_amax(c.data_ptr(), to_mi355q_dtype(c.scalar_type()), rows, cols,
+                                   out.data_ptr<float>(), current_stream(c)),
+               "mi355q_rowwise_amax");
+  return out;
+}
+
+}  // namespace
+
+TORCH_LIBRARY(hpu, m) {
+  m.def("hpu::cast_from_fp8(Tensor input, Tensor? scale, ScalarType out_dtype, int[]? scale_shape=None) -> Tensor");
+  m.def("hpu::cast_from_fp8.scalar(Tensor input, float scale, ScalarType out_dtype, int[]? scale_shape=None) -> Tensor");
+  m.def("hpu::cast_from_fp8.scalar_list(Tensor input, float[] scale, ScalarType out_dtype, int[]? scale_shape=None) -> Tensor");
+  m.def("hpu::cast_to_fp8_v2(Tensor input, Tensor? scale=None, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)");
+  m.def("hpu::cast_to_fp8_v2.scalar(Tensor input, float scale, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)");
+  m.def("hpu::cast_to_fp8_v2.scalar_list(Tensor input, float[] scale, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)");
+  m.def("hpu::convert_from_int4(Tensor input, Tensor scale, Tensor? zero_point, ScalarType out_dtype) -> Tensor");
+  m.def("hpu::convert_from_uint4(Tensor input, Tensor scale, Tensor? zero_point, ScalarType out_dtype) -> Tensor");
+  m.def("hpu::fp8_gemm_v2(Tensor A, bool trans_A, Tensor B, bool trans_B, Tensor? D, ScalarType out_dtype, Tensor? A_scale_inv=None, Tensor? B_scale_inv=None, Tensor? bias=None, bool accumulate=False, int[]? B_scale_shape=None) -> Tensor");
+  m.def("hpu::fp8_gemm_v2.scalar(Tensor A, bool trans_A, Tensor B, bool trans_B, Tensor? D, ScalarType out_dtype, float A_scale_inv, float B_scale_inv, Tensor? bias=None, bool accumulate=False, int[]? B_scale_shape=None) -> Tensor");
+  m.def("hpu::fp8_gemm_v2.scalar_list(Tensor A, bool trans_A, Tensor B, bool trans_B, Tensor? D, ScalarType out_dtype, float[] A_scale_inv, float[] B_scale_inv, Tensor? bias=None, bool accumulate=False, int[]? B_scale_shape=None) -> Tensor");
+}
+
+// Helpers the reference has no op for: amax alone and per-row amax.
+TORCH_LIBRARY(mi355q, m) {
+  m.def("mi355q::amax(Tensor input) -> Tensor");
+  m.def("mi355q::rowwise_amax(Tensor input) -> Tensor");
+}
+
+#define MI355Q_REGISTER_HPU(m)                                                                 \
+  m.impl("cast_to_fp8_v2", torch::CppFunction::makeFromBoxedFunction<&cast_to_fp8_v2_boxed>()); \
+  m.impl("cast_to_fp8_v2.scalar", torch::CppFunction::makeFromBoxedFunction<&cast_to_fp8_v2_boxed>()); \
+  m.impl("cast_to_fp8_v2.scalar_list", torch::CppFunction::makeFromBoxedFunction<&cast_to_fp8_v2_boxed>()); \
+  m.impl("cast_from_fp8", cast_from_fp8);                                                      \
+  m.impl("cast_from_fp8.scalar", cast_from_fp8_scalar);                                        \
+  m.impl("cast_from_fp8.scalar_list", cast_from_fp8_scalar_list);                              \
+  m.impl("fp8_gemm_v2", fp8_gemm_v2);                                                          \
+  m.impl("fp8_gemm_v2.scalar", fp8_gemm_v2_scalar);                                            \
+  m.impl("fp8_gemm_v2.scalar_list", fp8_gemm_v2_scalar_list);                                  \
+  m.impl("convert_from_int4", convert_from_int4);                                              \
+  m.impl("convert_from_uint4", convert_from_uint4);
+
+TORCH_LIBRARY_IMPL(hpu, CUDA, m) { MI355Q_REGISTER_HPU(m) }
+TORCH_LIBRARY_IMPL(hpu, Meta, m) { MI355Q_REGISTER_HPU(m) }
+
+TORCH_LIBRARY_IMPL(mi355q, CUDA, m) {
+  m.impl("amax", amax_op);
+  m.impl("rowwise_amax", rowwise_amax_op);
+}
+TORCH_LIBRARY_IMPL(mi355q, Meta, m) {
+  m.impl("amax", amax_op);
+  m.impl("rowwise_amax", rowwise_amax_op);
+}

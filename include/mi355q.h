@@ -1,0 +1,171 @@
+/*
+ * mi355q: C ABI of the gfx950 kernels behind the hpu:: quantized-inference ops.
+ *
+ * Every entry point takes raw device pointers, sizes and a HIP stream
+ * (passed as void* so that this header needs no HIP include), launches
+ * asynchronously on that stream, never synchronises, never allocates and
+ * returns an mi355q_status.  All tensors are dense row-major unless a stride
+ * argument says otherwise.
+ *
+ * Each entry point names the reference interface it stands in for.  In the
+ * reference these are Synapse graph nodes identified by GUID strings; the
+ * arithmetic behind the GUIDs is not in the reference tree.
+ */
+#ifndef MI355Q_H
+#define MI355Q_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  MI355Q_OK = 0,
+  MI355Q_ERR_INVALID_ARGUMENT = 1, /* null pointer, bad enum, negative size */
+  MI355Q_ERR_UNSUPPORTED = 2,      /* valid request this build has no kernel for */
+  MI355Q_ERR_LAUNCH = 3,           /* hipLaunchKernel reported an error */
+  MI355Q_ERR_WORKSPACE = 4         /* workspace missing or too small */
+} mi355q_status;
+
+typedef enum {
+  MI355Q_F32 = 0,
+  MI355Q_BF16 = 1,
+  MI355Q_E4M3FN = 2, /* OCP fp8 e4m3fn, max 448, no Inf */
+  MI355Q_E5M2 = 3    /* OCP fp8 e5m2, max finite 57344 */
+} mi355q_dtype;
+
+/* How a cast scale is broadcast against the input
+ * (ValidateScaleShape / HandleScaleTensor / HandleScaleScalar,
+ * hpu_ops/backend/fp8_ops.cpp:29-100). */
+typedef enum {
+  MI355Q_SCALE_NONE = 0, /* scale == 1 */
+  MI355Q_SCALE_HOST = 1, /* one value, passed by value (the .scalar overloads) */
+  MI355Q_SCALE_DEV = 2,  /* one fp32 value in device memory */
+  MI355Q_SCALE_MID = 3,  /* input viewed as [outer, mid, inner]; scale is fp32[mid].
+                            inner == row length gives per-row scales,
+                            inner == 1 gives per-column scales */
+  MI355Q_SCALE_FULL = 4  /* one fp32 scale per element */
+} mi355q_scale_mode;
+
+/* GEMM scale / bias broadcast against the [M, N] output. */
+typedef enum {
+  MI355Q_GS_NONE = 0,
+  MI355Q_GS_HOST = 1,    /* scalar by value */
+  MI355Q_GS_DEV = 2,     /* one fp32 value in device memory */
+  MI355Q_GS_PER_ROW = 3, /* fp32[M]  (scale shape [M,1]) */
+  MI355Q_GS_PER_COL = 4  /* fp32[N]  (scale shape [1,N]) */
+} mi355q_gemm_scale_mode;
+
+typedef enum {
+  MI355Q_BIAS_NONE = 0,
+  MI355Q_BIAS_ROW_VECTOR = 1, /* [N], broadcast down the rows */
+  MI355Q_BIAS_FULL = 2        /* [M, N] with row stride ldbias */
+} mi355q_bias_mode;
+
+typedef enum {
+  MI355Q_ZP_NONE = 0,
+  MI355Q_ZP_FLOAT = 1, /* same dtype and shape as the scale */
+  MI355Q_ZP_PACKED = 2 /* int32, 8 nibbles per word, shape [rows/group, packed_cols] */
+} mi355q_zp_kind;
+
+/* ABI version: bumped when a signature below changes. */
+int mi355q_abi_version(void);
+const char* mi355q_status_string(int status);
+
+/*
+ * amax = max|x| over n elements of fp32 or bf16, written as one fp32.
+ * A NaN in x makes the result NaN.  Stands in for the amax output of the
+ * convert_to_fp8_* node (CastToFp8V2::AddNode, hpu_ops/backend/fp8_ops.cpp:
+ * 192-258, second output) when it is wanted without the cast.
+ */
+int mi355q_amax(const void* x, int x_dtype, int64_t n, float* amax_out, void* stream);
+
+/*
+ * Per-row amax of a [rows, cols] tensor -> fp32[rows].  The reference has no
+ * such op (its amax is always one scalar, fp8_ops.cpp:170-178); dynamic
+ * per-token quantisation needs it before cast_to_fp8 with per-row scales.
+ */
+int mi355q_rowwise_amax(const void* x, int x_dtype, int64_t rows, int64_t cols,
+                        float* amax_out, void* stream);
+
+/*
+ * y = saturating round-to-nearest-even fp8( x * scale ), optional amax of x.
+ * Replaces the convert_to_fp8_{f32,bf16} node built by CastToFp8V2::AddNode
+ * (hpu_ops/backend/fp8_ops.cpp:192-258; round mode CAST_ROUND_HALF_NE,
+ * GetCastParams :105-119).  For bf16 input the scale is rounded to bf16 and
+ * the product is rounded to bf16 before the fp8 rounding.
+ *   x          n = outer*mid*inner elements (for NONE/HOST/DEV/FULL pass
+ *              outer = n, mid = inner = 1)
+ *   scale_dev  fp32 device pointer for DEV / MID / FULL, else ignored
+ *   amax_out   NULL, or one fp32 that receives max|x| (of the unscaled input)
+ * x_dtype may also be an fp8 type equal to fp8_fmt: then y is a copy of x
+ * (fp8_ops.cpp:201-215) and amax_out must be NULL.
+ */
+int mi355q_cast_to_fp8(const void* x, int x_dtype, void* y, int fp8_fmt,
+                       const float* scale_dev, float scale_host, int scale_mode,
+                       int64_t outer, int64_t mid, int64_t inner,
+                       float* amax_out, void* stream);
+
+/*
+ * y = out_dtype(x_fp8) * scale, computed in out_dtype (fp32 or bf16).
+ * Replaces the convert_from_fp8_{f32,bf16} node of CastFromFp8::AddNode
+ * (hpu_ops/backend/fp8_ops.cpp:265-308).  Scale arguments as above.
+ */
+int mi355q_cast_from_fp8(const void* x, int fp8_fmt, void* y, int out_dtype,
+                         const float* scale_dev, float scale_host, int scale_mode,
+                         int64_t outer, int64_t mid, int64_t inner, void* stream);
+
+/*
+ * out[r, 8p+i] = (nibble_i(packed[r, p]) - z) * s, nibble i = bits [4i, 4i+4).
+ * Replaces the dequantize_4_bit_{f32,bf16} node of Int4BaseOp::AddNode
+ * (hpu_ops/backend/int4_ops.cpp:40-56); is_signed selects convert_from_int4
+ * (nibble >= 8 means nibble-16) over convert_from_uint4 (:58-62).
+ *   packed  int32 [rows, packed_cols]
+ *   scale   out_dtype [rows/group, 8*packed_cols]; group == 1 is the
+ *           elementwise form, group > 1 the group-wise (AutoGPTQ) form
+ *   zp      per zp_kind; a float zero-point is subtracted in out_dtype
+ *   out     out_dtype [rows, 8*packed_cols]
+ */
+int mi355q_dequant_4bit(const int32_t* packed, const void* scale, const void* zp,
+                        int zp_kind, int is_signed, int out_dtype, int64_t rows,
+                        int64_t packed_cols, int64_t group, void* out, void* stream);
+
+/*
+ * C[b] = out_dtype( (op(A[b]) @ op(B[b])) * sA * sB + bias + D[b] )
+ * with fp32 accumulation and one final rounding.  Replaces the
+ * fp8_gemm_{f32,bf16} node of Fp8GemmV2::AddNode
+ * (hpu_ops/backend/fp8_ops.cpp:403-496; synGEMMParams{trans_A, trans_B} :482).
+ *   A      fp8 (fmt_a); trans_a == 0: [M, K] with row stride lda,
+ *          trans_a != 0: [K, M] with row stride lda
+ *   B      fp8 (fmt_b); trans_b == 0: [K, N] with row stride ldb,
+ *          trans_b != 0: [N, K] with row stride ldb
+ *   C      out_dtype (fp32 or bf16) [M, N], row stride ldc
+ *   sa/sb  per mi355q_gemm_scale_mode (the *_scale_inv arguments of the op)
+ *   bias   out_dtype, per mi355q_bias_mode; D: out_dtype [M, N] stride ldd or NULL
+ *   batch  number of problems; stride_* are element strides between them
+ *          (0 broadcasts an operand)
+ * Leading dimensions and batch strides are in elements.
+ */
+int mi355q_fp8_gemm(const void* A, int fmt_a, int trans_a, int64_t lda,
+                    const void* B, int fmt_b, int trans_b, int64_t ldb,
+                    void* C, int out_dtype, int64_t ldc,
+                    int64_t M, int64_t N, int64_t K,
+                    const float* sa_dev, float sa_host, int sa_mode,
+                    const float* sb_dev, float sb_host, int sb_mode,
+                    const void* bias, int bias_mode, int64_t ldbias,
+                    const void* D, int64_t ldd,
+                    int64_t batch, int64_t stride_a, int64_t stride_b,
+                    int64_t stride_c, int64_t stride_d, int64_t stride_bias,
+                    void* stream);
+
+/* Name of the kernel variant mi355q_fp8_gemm would pick for a problem
+ * (for logs and profiles; static string). */
+const char* mi355q_fp8_gemm_variant(int trans_a, int64_t lda, int trans_b, int64_t ldb,
+                                    int64_t M, int64_t N, int64_t K);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355Q_H */

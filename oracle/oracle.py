@@ -1,0 +1,311 @@
+"""ctypes front-end of the C oracle plus a pure-PyTorch twin.
+
+TEST INFRASTRUCTURE ONLY: used by tests/, by __graft_entry__.smoke() as the
+checker, and by bench.py to time the CPU baseline.  Never imported by the
+product package.
+
+Two independent statements of the same semantics live here:
+  * ``c_*``     call oracle/mi355q_oracle.c (bit-level C, scalar loops);
+  * ``torch_*`` are the "PyTorch CPU float8 emulation" formulas: what the
+    reference's tests compute on the CPU to judge the device
+    (tests/pytest_working/any_mode/test_hpu_fp8_ops_any_mode.py:85-87,
+    any_mode/test_hpu_cast.py:35-55, any_mode/test_hpu_convert_from_int4.py:
+    104-131,224-247).  They run multi-threaded and serve as the CPU baseline.
+The tests check the two against each other and against the reference's
+known answers.
+"""
+import ctypes
+import os
+import subprocess
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libmi355q_oracle.so")
+
+F32, BF16, E4M3FN, E5M2 = 0, 1, 2, 3
+SCALE_NONE, SCALE_HOST, SCALE_DEV, SCALE_MID, SCALE_FULL = 0, 1, 2, 3, 4
+
+_DT = {torch.float32: F32, torch.bfloat16: BF16,
+       torch.float8_e4m3fn: E4M3FN, torch.float8_e5m2: E5M2}
+FP8_MAX = {torch.float8_e4m3fn: 448.0, torch.float8_e5m2: 57344.0}
+
+
+def build(force=False):
+    """Compile the C oracle with gcc (seconds)."""
+    src = os.path.join(_HERE, "mi355q_oracle.c")
+    if force or not os.path.exists(_LIB_PATH) or \
+            os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-s", "-C", _HERE, "-B", "libmi355q_oracle.so"])
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        c = ctypes
+        L.ora_f32_to_e4m3fn.argtypes = [c.c_float]
+        L.ora_f32_to_e4m3fn.restype = c.c_uint8
+        L.ora_f32_to_e5m2.argtypes = [c.c_float]
+        L.ora_f32_to_e5m2.restype = c.c_uint8
+        L.ora_f32_to_bf16.argtypes = [c.c_float]
+        L.ora_f32_to_bf16.restype = c.c_uint16
+        L.ora_e4m3fn_to_f32.argtypes = [c.c_uint8]
+        L.ora_e4m3fn_to_f32.restype = c.c_float
+        L.ora_e5m2_to_f32.argtypes = [c.c_uint8]
+        L.ora_e5m2_to_f32.restype = c.c_float
+        L.ora_cast_to_fp8.argtypes = [c.c_void_p, c.c_int, c.c_void_p, c.c_int, c.c_void_p,
+                                      c.c_float, c.c_int, c.c_int64, c.c_int64, c.c_int64,
+                                      c.c_void_p]
+        L.ora_cast_to_fp8.restype = None
+        L.ora_amax.argtypes = [c.c_void_p, c.c_int, c.c_int64, c.c_int64, c.c_void_p]
+        L.ora_amax.restype = None
+        L.ora_cast_from_fp8.argtypes = [c.c_void_p, c.c_int, c.c_void_p, c.c_int, c.c_void_p,
+                                        c.c_float, c.c_int, c.c_int64, c.c_int64, c.c_int64]
+        L.ora_cast_from_fp8.restype = None
+        L.ora_dequant_4bit.argtypes = [c.c_void_p, c.c_void_p, c.c_void_p, c.c_int, c.c_int,
+                                       c.c_int, c.c_int64, c.c_int64, c.c_int64, c.c_void_p]
+        L.ora_dequant_4bit.restype = None
+        L.ora_fp8_gemm.argtypes = [c.c_void_p, c.c_int, c.c_int64, c.c_int64,
+                                   c.c_void_p, c.c_int, c.c_int64, c.c_int64,
+                                   c.c_int64, c.c_int64, c.c_int64,
+                                   c.c_void_p, c.c_float, c.c_int,
+                                   c.c_void_p, c.c_float, c.c_int,
+                                   c.c_void_p, c.c_int, c.c_void_p, c.c_int, c.c_void_p]
+        L.ora_fp8_gemm.restype = None
+        _lib = L
+    return _lib
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _scale_args(x_shape, scale, scale_shape):
+    """Classify a scale the way the C ABI does.
+
+    Returns (tensor_or_None, host_value, mode, mid, inner).  ``scale`` may be
+    None, a python float, a list of floats or a tensor; ``scale_shape`` is the
+    optional broadcast shape (hpu_ops/backend/fp8_ops.cpp:29-100).
+    """
+    if scale is None:
+        return None, 1.0, SCALE_NONE, 1, 1
+    if isinstance(scale, (int, float)):
+        return None, float(scale), SCALE_HOST, 1, 1
+    if isinstance(scale, (list, tuple)):
+        scale = torch.tensor(scale, dtype=torch.float64).to(torch.float32)
+    scale = scale.detach().to("cpu", torch.float32).contiguous()
+    if scale.numel() == 1:
+        return scale.reshape(1), 0.0, SCALE_DEV, 1, 1
+    shape = list(scale_shape) if scale_shape is not None else list(scale.shape)
+    n = 1
+    for d in shape:
+        n *= d
+    if n != scale.numel():
+        raise ValueError(
+            f"Number of scale elements ({scale.numel()}) is not equal to number of "
+            f"scale_shape elements ({n}).")
+    full = scale.reshape(shape).expand(x_shape).contiguous().reshape(-1)
+    return full, 0.0, SCALE_FULL, 1, 1
+
+
+# ---------------------------------------------------------------- C oracle
+
+def c_cast_to_fp8(x, scale, out_dtype, is_amax=False, scale_shape=None):
+    """(fp8 tensor, amax) as hpu::cast_to_fp8_v2 defines them (RNE)."""
+    x = x.detach().cpu().contiguous()
+    st, host, mode, mid, inner = _scale_args(x.shape, scale, scale_shape)
+    y = torch.empty(x.shape, dtype=torch.uint8)
+    amax = torch.zeros((), dtype=torch.float32)
+    lib().ora_cast_to_fp8(_ptr(x), _DT[x.dtype], _ptr(y), _DT[out_dtype], _ptr(st), host, mode,
+                          x.numel(), mid, inner, _ptr(amax) if is_amax else None)
+    return y.view(out_dtype), (amax if is_amax else torch.empty(0, dtype=torch.float32))
+
+
+def c_amax(x, rowwise=False):
+    x = x.detach().cpu().contiguous()
+    rows = x.shape[0] if rowwise else 1
+    cols = x.numel() // max(rows, 1)
+    out = torch.zeros(rows, dtype=torch.float32)
+    lib().ora_amax(_ptr(x), _DT[x.dtype], rows, cols, _ptr(out))
+    return out if rowwise else out.reshape(())
+
+
+def c_cast_from_fp8(x8, scale, out_dtype, scale_shape=None):
+    x8 = x8.detach().cpu().contiguous()
+    st, host, mode, mid, inner = _scale_args(x8.shape, scale, scale_shape)
+    y = torch.empty(x8.shape, dtype=out_dtype)
+    lib().ora_cast_from_fp8(_ptr(x8), _DT[x8.dtype], _ptr(y), _DT[out_dtype], _ptr(st), host,
+                            mode, x8.numel(), mid, inner)
+    return y
+
+
+def c_dequant_4bit(packed, scale, zero_point, out_dtype, signed):
+    """hpu::convert_from_int4 / convert_from_uint4 on CPU tensors."""
+    packed = packed.detach().cpu().contiguous()
+    pcols = packed.shape[-1]
+    rows = packed.numel() // max(pcols, 1)
+    scale = scale.detach().cpu().to(out_dtype).contiguous()
+    srows = scale.numel() // (pcols * 8)
+    group = rows // srows
+    zp_kind = 0
+    zp = None
+    if zero_point is not None:
+        zero_point = zero_point.detach().cpu().contiguous()
+        if zero_point.dtype == torch.int32:
+            zp_kind, zp = 2, zero_point
+        else:
+            zp_kind, zp = 1, zero_point.to(out_dtype).contiguous()
+    out = torch.empty(list(packed.shape[:-1]) + [pcols * 8], dtype=out_dtype)
+    lib().ora_dequant_4bit(_ptr(packed), _ptr(scale), _ptr(zp), zp_kind, int(signed),
+                           _DT[out_dtype], rows, pcols, group, _ptr(out))
+    return out
+
+
+def _gemm_scale(s, M, N, shape=None):
+    if s is None:
+        return None, 1.0, 0
+    if isinstance(s, (int, float)):
+        return None, float(s), 1
+    if isinstance(s, (list, tuple)):
+        s = torch.tensor(s, dtype=torch.float64).to(torch.float32)
+    s = s.detach().cpu().to(torch.float32).contiguous()
+    if s.numel() == 1:
+        return s.reshape(1), 0.0, 2
+    shp = list(shape) if shape is not None else list(s.shape)
+    while len(shp) > 2 and shp[0] == 1:
+        shp = shp[1:]
+    if len(shp) == 1:
+        shp = [1] + shp
+    if shp == [M, 1]:
+        return s.reshape(-1), 0.0, 3
+    if shp == [1, N]:
+        return s.reshape(-1), 0.0, 4
+    raise ValueError(f"unsupported gemm scale shape {shp} for output [{M},{N}]")
+
+
+def c_fp8_gemm(A, trans_A, B, trans_B, out_dtype, A_scale_inv=None, B_scale_inv=None,
+               bias=None, D=None, B_scale_shape=None):
+    """One 2-D fp8 GEMM through the C oracle (small sizes only: scalar loops)."""
+    A = A.detach().cpu()
+    B = B.detach().cpu()
+    a = A.t() if trans_A else A
+    b = B.t() if trans_B else B
+    M, K = a.shape
+    K2, N = b.shape
+    assert K == K2
+    sa, sah, sam = _gemm_scale(A_scale_inv, M, N)
+    sb, sbh, sbm = _gemm_scale(B_scale_inv, M, N, B_scale_shape)
+    bias_mode = 0
+    if bias is not None:
+        bias = bias.detach().cpu().to(out_dtype).contiguous()
+        bias_mode = 1 if bias.numel() == N and bias.dim() <= 1 or list(bias.shape) == [1, N] else 2
+        if bias_mode == 2:
+            bias = bias.expand(M, N).contiguous()
+    if D is not None:
+        D = D.detach().cpu().to(out_dtype).expand(M, N).contiguous()
+    C = torch.empty(M, N, dtype=out_dtype)
+    lib().ora_fp8_gemm(_ptr(a), _DT[A.dtype], a.stride(0), a.stride(1),
+                       _ptr(b), _DT[B.dtype], b.stride(0), b.stride(1), M, N, K,
+                       _ptr(sa), sah, sam, _ptr(sb), sbh, sbm,
+                       _ptr(bias), bias_mode, _ptr(D), _DT[out_dtype], _ptr(C))
+    return C
+
+
+# ------------------------------------------------------------ PyTorch twin
+
+def _as_tensor_scale(scale, scale_shape):
+    if scale is None:
+        return None
+    if isinstance(scale, (int, float)):
+        return torch.tensor(float(scale), dtype=torch.float32)
+    if isinstance(scale, (list, tuple)):
+        scale = torch.tensor(scale, dtype=torch.float64).to(torch.float32)
+    scale = scale.detach().cpu().to(torch.float32)
+    if scale_shape is not None and scale.numel() > 1:
+        scale = scale.reshape(list(scale_shape))
+    return scale
+
+
+def torch_cast_to_fp8(x, scale, out_dtype, is_amax=False, scale_shape=None):
+    """(x * scale.to(x.dtype)) clamped to the finite fp8 range, PyTorch CPU RNE cast."""
+    x = x.detach().cpu()
+    s = _as_tensor_scale(scale, scale_shape)
+    p = x if s is None else x * s.to(x.dtype)
+    mx = FP8_MAX[out_dtype]
+    y = p.clamp(-mx, mx).to(out_dtype)
+    amax = x.abs().max().float() if is_amax else torch.empty(0, dtype=torch.float32)
+    return y, amax
+
+
+def torch_cast_from_fp8(x8, scale, out_dtype, scale_shape=None):
+    s = _as_tensor_scale(scale, scale_shape)
+    v = x8.detach().cpu().to(out_dtype)
+    return v if s is None else v * s.to(out_dtype)
+
+
+def torch_unpack_nibbles(packed, signed):
+    """int32 [..., P] -> int32 [..., 8P]; element 8p+i sits in bits [4i, 4i+4)."""
+    shifts = torch.arange(0, 32, 4, dtype=torch.int32)
+    q = (packed.detach().cpu().unsqueeze(-1) >> shifts) & 0xF
+    if signed:
+        q = torch.where(q > 7, q - 16, q)
+    return q.reshape(*packed.shape[:-1], packed.shape[-1] * 8)
+
+
+def torch_dequant_4bit(packed, scale, zero_point, out_dtype, signed):
+    q = torch_unpack_nibbles(packed, signed)
+    scale = scale.detach().cpu().to(out_dtype)
+    cols = q.shape[-1]
+    rows = q.numel() // cols
+    srows = scale.numel() // cols
+    group = rows // srows
+    q2 = q.reshape(srows, group, cols)
+    s2 = scale.reshape(srows, 1, cols)
+    if zero_point is None:
+        d = q2.to(out_dtype)
+    elif zero_point.dtype == torch.int32:
+        z = torch_unpack_nibbles(zero_point, signed).reshape(srows, 1, cols)
+        d = (q2 - z).to(out_dtype)
+    else:
+        d = q2.to(out_dtype) - zero_point.detach().cpu().to(out_dtype).reshape(srows, 1, cols)
+    return (d * s2).reshape(q.shape)
+
+
+def torch_fp8_gemm(A, trans_A, B, trans_B, out_dtype, A_scale_inv=None, B_scale_inv=None,
+                   bias=None, D=None, B_scale_shape=None):
+    """fp32-accumulated GEMM of the dequantised operands, torch.matmul batching."""
+    a = A.detach().cpu().float()
+    b = B.detach().cpu().float()
+    if trans_A and a.dim() > 1:
+        a = a.transpose(-2, -1)
+    if trans_B and b.dim() > 1:
+        b = b.transpose(-2, -1)
+    v = torch.matmul(a, b)
+    sa = _as_tensor_scale(A_scale_inv, None)
+    sb = _as_tensor_scale(B_scale_inv, B_scale_shape)
+    if sa is not None:
+        v = v * sa
+    if sb is not None:
+        v = v * sb
+    if bias is not None:
+        v = v + bias.detach().cpu().float()
+    if D is not None:
+        v = v + D.detach().cpu().float()
+    return v.to(out_dtype)
+
+
+def pack_nibbles(q):
+    """int tensor [..., 8P] with values in -8..15 -> packed int32 [..., P]."""
+    q = q.detach().cpu().to(torch.int64) & 0xF
+    q = q.reshape(*q.shape[:-1], q.shape[-1] // 8, 8)
+    shifts = torch.arange(0, 32, 4, dtype=torch.int64)
+    w = (q << shifts).sum(-1)
+    w = torch.where(w >= 2 ** 31, w - 2 ** 32, w)
+    return w.to(torch.int32)
