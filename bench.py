@@ -1,0 +1,367 @@
+"""Benchmark of the fp8 / int4 op family on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME[,NAME...]] [--no-cpu]
+
+A step is one call of the primary workload, BASELINE config 3: fp8_gemm_v2 on
+8192 x 4096 x 14336 (e4m3fn x e4m3fn -> bf16, per-tensor inverse scales, bf16
+bias), with all operands resident in HBM.  The single JSON line printed at the
+end carries that as ``value`` (TFLOP/s) with its MFMA roofline, and under
+``ops`` the HBM-bound members of the family (amax, cast_to_fp8_v2,
+cast_from_fp8, convert_from_uint4 / int4, the decode-shaped GEMMs) and the MLP
+block, each with its own roofline entry.
+
+Timing: W untimed warm-up calls, then K calls bracketed by HIP events on the
+stream the kernels are launched on (torch's current stream), divided by K.
+The streaming kernels rotate through enough distinct buffer sets to exceed the
+256 MiB Infinity Cache, so reads come from HBM.
+
+The CPU baseline is the PyTorch-CPU float8 emulation of the same semantics
+(oracle/oracle.py torch_* functions) timed on this host's cores on a bounded
+sample; it is reported next to the GPU figure and is not the target.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+FP8_PEAK_TFLOPS = 5000.0     # MI355X dense OCP fp8 MFMA, published
+E4 = torch.float8_e4m3fn
+SEED = 0xC001A1
+MALL_BYTES = 256 << 20
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (see profiles/); None where no counter run has been committed.
+MEASURED_TRAFFIC = {}
+
+
+def time_gpu(fn, steps, warmup):
+    """Average milliseconds per call of fn(i), HIP events on the current stream."""
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        fn(warmup + i)
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def time_cpu(fn, min_seconds=3.0, max_runs=5):
+    """Median seconds of fn() over up to max_runs runs (at least one)."""
+    ts = []
+    t_total = 0.0
+    while len(ts) < max_runs and (not ts or t_total < min_seconds):
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        ts.append(dt)
+        t_total += dt
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def hbm_entry(name, workload, bytes_per_call, ms, steps, kernel, cpu=None, extra=None):
+    gbs = bytes_per_call / (ms * 1e-3) / 1e9
+    e = {"name": name, "workload": workload, "metric": "GB/s", "value": round(gbs, 1), "unit": "GB/s",
+         "ms_per_call": round(ms, 5), "steps": steps,
+         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                      "algorithmic_bytes": bytes_per_call, "traffic": MEASURED_TRAFFIC.get(name)}}
+    if cpu is not None:
+        e["cpu_baseline"] = cpu
+    if extra:
+        e.update(extra)
+    return e
+
+
+def n_sets(bytes_per_set):
+    return max(2, -(-int(1.5 * MALL_BYTES) // bytes_per_set))
+
+
+def c1_input(gen, rows=4096, cols=4096):
+    x = torch.randn(rows, cols, generator=gen) * 3
+    n = x.numel()
+    k = -(-n // 1000)
+    pos = torch.randperm(n, generator=gen)[:k]
+    sign = torch.randint(0, 2, (k,), generator=gen).float() * 2 - 1
+    x.view(-1)[pos] = sign * 1e4
+    return x.bfloat16()
+
+
+def bench_cast(ops, oracle, dev, steps, warmup, cpu):
+    """BASELINE config 1: amax pass, cast_to_fp8_v2 (scale given), cast_from_fp8."""
+    out = []
+    gen = torch.Generator().manual_seed(SEED)
+    x = c1_input(gen)
+    n = x.numel()
+    amax = x.abs().max().float()
+    scale = (448.0 / amax).reshape(())
+    sets = n_sets(3 * n)
+    xs = [x.to(dev).clone() for _ in range(sets)]
+    sd, sinv = scale.to(dev), scale.reciprocal().to(dev)
+    cores = torch.get_num_threads()
+
+    ms = time_gpu(lambda i: torch.ops.mi355q.amax(xs[i % sets]), steps, warmup)
+    c = None
+    if cpu:
+        t = time_cpu(lambda: x.abs().max().float())
+        c = {"value": round(2 * n / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+             "sample": "full 4096x4096 bf16 tensor, x.abs().max()"}
+    out.append(hbm_entry("amax", "C1a amax of bf16 [4096,4096]", 2 * n, ms, steps, "amax_vec<bf16>", c))
+
+    ring = [None] * sets  # keeps the last `sets` outputs alive so that outputs rotate as well
+
+    def keep(i, v):
+        ring[i % sets] = v
+
+    ms = time_gpu(lambda i: keep(i, ops.cast_to_fp8_v2(xs[i % sets], sd, False, False, E4)), steps, warmup)
+    c = None
+    if cpu:
+        t = time_cpu(lambda: oracle.torch_cast_to_fp8(x, scale, E4))
+        c = {"value": round(3 * n / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+             "sample": "full 4096x4096 bf16 tensor, (x*s.to(bf16)).clamp(-448,448).to(float8_e4m3fn)"}
+    out.append(hbm_entry("cast_to_fp8_v2", "C1b cast_to_fp8_v2 bf16 [4096,4096] -> e4m3fn, per-tensor scale",
+                         3 * n, ms, steps, "cast_to_fp8_vec8<bf16,e4m3fn,scalar>", c))
+
+    ms = time_gpu(lambda i: keep(i, ops.cast_to_fp8_v2(xs[i % sets], sd, False, True, E4)), steps, warmup)
+    out.append(hbm_entry("cast_to_fp8_v2+amax", "C1 cast_to_fp8_v2 with is_amax=True (one pass)", 3 * n + 4, ms, steps,
+                         "cast_to_fp8_vec8<bf16,e4m3fn,scalar,amax>"))
+
+    y8 = [ops.cast_to_fp8_v2(xs[i], sd, False, False, E4)[0] for i in range(sets)]
+    del xs
+    ring = [None] * sets
+    ms = time_gpu(lambda i: keep(i, ops.cast_from_fp8(y8[i % sets], sinv, torch.bfloat16)), steps, warmup)
+    c = None
+    if cpu:
+        y_cpu = y8[0].cpu()
+        t = time_cpu(lambda: oracle.torch_cast_from_fp8(y_cpu, scale.reciprocal(), torch.bfloat16))
+        c = {"value": round(3 * n / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+             "sample": "full 4096x4096 e4m3fn tensor, x8.to(bf16) * s_inv.to(bf16)"}
+    out.append(hbm_entry("cast_from_fp8", "C1c cast_from_fp8 e4m3fn [4096,4096] -> bf16", 3 * n, ms, steps,
+                         "cast_from_fp8_vec16<e4m3fn,bf16,scalar>", c))
+    return out
+
+
+def bench_int4(ops, oracle, dev, steps, warmup, cpu):
+    """BASELINE config 2: K = N = 4096, group 128."""
+    out = []
+    gen = torch.Generator().manual_seed(SEED)
+    K = N = 4096
+    q = torch.randint(0, 16, (K, N), generator=gen)
+    packed = oracle.pack_nibbles(q)
+    s = (torch.rand(K // 128, N, generator=gen) * 0.019 + 0.001).bfloat16()
+    zp = oracle.pack_nibbles(torch.randint(0, 16, (K // 128, N), generator=gen))
+    b_u = K * N // 2 + s.numel() * 2 + zp.numel() * 4 + K * N * 2
+    b_i = K * N // 2 + s.numel() * 2 + K * N * 2
+    sets = n_sets(K * N // 2 + K * N * 2)
+    ps = [packed.to(dev).clone() for _ in range(sets)]
+    sd, zd = s.to(dev), zp.to(dev)
+    cores = torch.get_num_threads()
+    ring = [None] * sets
+
+    def keep(i, v):
+        ring[i % sets] = v
+
+    ms = time_gpu(lambda i: keep(i, ops.convert_from_uint4(ps[i % sets], sd, zd, torch.bfloat16)), steps, warmup)
+    c = None
+    if cpu:
+        t = time_cpu(lambda: oracle.torch_dequant_4bit(packed, s, zp, torch.bfloat16, False), max_runs=3)
+        c = {"value": round(b_u / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+             "sample": "full K=N=4096 problem, shift/mask unpack + (q - z) * s in torch"}
+    out.append(hbm_entry("convert_from_uint4", "C2 convert_from_uint4 K=N=4096 group 128, packed zero-points -> bf16",
+                         b_u, ms, steps, "dequant_4bit_kernel<unsigned,bf16,packed zp>", c))
+    ms = time_gpu(lambda i: keep(i, ops.convert_from_int4(ps[i % sets], sd, None, torch.bfloat16)), steps, warmup)
+    out.append(hbm_entry("convert_from_int4", "C2 convert_from_int4 K=N=4096 group 128, no zero-point -> bf16",
+                         b_i, ms, steps, "dequant_4bit_kernel<signed,bf16,no zp>"))
+    return out
+
+
+def quant_per_tensor(ops, x_dev):
+    amax = torch.ops.mi355q.amax(x_dev)
+    s = 448.0 / amax
+    return ops.cast_to_fp8_v2(x_dev, s, False, False, E4)[0], (1.0 / s)
+
+
+def bench_gemm_c3(ops, oracle, pkg, dev, steps, warmup, cpu):
+    gen = torch.Generator().manual_seed(SEED)
+    M, K, N = 8192, 4096, 14336
+    a = torch.randn(M, K, generator=gen).bfloat16().to(dev)
+    w = (torch.randn(K, N, generator=gen) * 0.02).bfloat16().to(dev)
+    bias = (torch.randn(N, generator=gen) * 0.01).bfloat16().to(dev)
+    a8, sa_inv = quant_per_tensor(ops, a)
+    w8, sw_inv = quant_per_tensor(ops, w)
+    del a, w
+    flop = 2.0 * M * N * K
+    ms = time_gpu(lambda i: ops.fp8_gemm_v2(a8, False, w8, False, None, torch.bfloat16, sa_inv, sw_inv, bias, False),
+                  steps, warmup)
+    tflops = flop / (ms * 1e-3) / 1e12
+    variant = pkg.capi().mi355q_fp8_gemm_variant(0, K, 0, N, M, N, K).decode()
+    cpu_entry = None
+    if cpu:
+        rows = 1024
+        a_cpu, w_cpu, b_cpu = a8[:rows].cpu(), w8.cpu(), bias.cpu()
+        sa_c, sw_c = sa_inv.cpu(), sw_inv.cpu()
+        t = time_cpu(lambda: oracle.torch_fp8_gemm(a_cpu, False, w_cpu, False, torch.bfloat16, sa_c, sw_c, bias=b_cpu),
+                     min_seconds=8.0, max_runs=3)
+        cpu_entry = {"value": round(2.0 * rows * N * K / t / 1e12, 4), "unit": "TFLOP/s",
+                     "cores": torch.get_num_threads(), "kind": "port",
+                     "sample": f"first {rows} of 8192 rows of A against the full B: "
+                               "((A8.float() @ B8.float()) * sA * sB + bias).bfloat16()"}
+    return {"ms": ms, "tflops": tflops, "flop": flop, "variant": variant, "cpu": cpu_entry}
+
+
+def bench_gemm_decode(ops, oracle, dev, steps, warmup):
+    """BASELINE config 4: per-token x per-channel scales, K = 8192, N = 28672."""
+    out = []
+    gen = torch.Generator().manual_seed(SEED)
+    K, N = 8192, 28672
+    w = (torch.randn(K, N, generator=gen) * 0.02).bfloat16().to(dev)
+    amax_c = w.abs().amax(dim=0).float()
+    s_col = 448.0 / amax_c
+    w8 = ops.cast_to_fp8_v2(w, s_col, False, False, E4, [1, N])[0]
+    sw_inv = (1.0 / s_col).contiguous()
+    del w
+    # two copies of the weights exceed the Infinity Cache: alternate between them
+    w8s = [w8, w8.clone()]
+    cols = torch.randperm(K, generator=gen)[:82]
+    for M in (16, 64, 256):
+        x = torch.randn(M, K, generator=gen)
+        x[:, cols] *= 20
+        x = x.bfloat16().to(dev)
+        amax_r = torch.ops.mi355q.rowwise_amax(x)
+        s_row = (448.0 / amax_r).reshape(M, 1)
+        x8 = ops.cast_to_fp8_v2(x, s_row, False, False, E4, [M, 1])[0]
+        sx_inv = (1.0 / s_row).contiguous()
+        ms = time_gpu(lambda i: ops.fp8_gemm_v2(x8, False, w8s[i % 2], False, None, torch.bfloat16, sx_inv, sw_inv,
+                                                None, False, [1, N]), steps, warmup)
+        nbytes = K * N + M * K + 2 * M * N + 4 * (M + N)
+        flop = 2.0 * M * N * K
+        out.append(hbm_entry(f"fp8_gemm_v2_decode_M{M}",
+                             f"C4 fp8_gemm_v2 M={M} K=8192 N=28672 per-token x per-channel scales -> bf16",
+                             nbytes, ms, steps, "fp8_gemm_tile_kernel",
+                             extra={"tflops": round(flop / (ms * 1e-3) / 1e12, 2)}))
+    return out
+
+
+def bench_mlp(ops, dev, steps, warmup):
+    """BASELINE config 5: fp8 decoder MLP block, Llama-3-8B dims, 4096 tokens."""
+    gen = torch.Generator().manual_seed(SEED)
+    T, d, ff = 4096, 4096, 14336
+
+    def qweight(k, n):
+        w = (torch.randn(k, n, generator=gen) * 0.02).bfloat16().to(dev)
+        s = 448.0 / w.abs().amax(dim=0).float()
+        return ops.cast_to_fp8_v2(w, s, False, False, E4, [1, n])[0], (1.0 / s).contiguous()
+
+    wg, sg = qweight(d, ff)
+    wu, su = qweight(d, ff)
+    wd, sdn = qweight(ff, d)
+    x = torch.randn(T, d, generator=gen).bfloat16().to(dev)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(8)]
+
+    def quant_rows(t):
+        amax = torch.ops.mi355q.rowwise_amax(t)
+        s = (448.0 / amax).reshape(-1, 1)
+        return ops.cast_to_fp8_v2(t, s, False, False, E4, [t.shape[0], 1])[0], (1.0 / s)
+
+    def block(record=False):
+        if record: ev[0].record()
+        x8, sx = quant_rows(x)
+        if record: ev[1].record()
+        g = ops.fp8_gemm_v2(x8, False, wg, False, None, torch.bfloat16, sx, sg, None, False, [1, ff])
+        u = ops.fp8_gemm_v2(x8, False, wu, False, None, torch.bfloat16, sx, su, None, False, [1, ff])
+        if record: ev[2].record()
+        h = torch.nn.functional.silu(g) * u
+        if record: ev[3].record()
+        h8, sh = quant_rows(h)
+        if record: ev[4].record()
+        y = ops.fp8_gemm_v2(h8, False, wd, False, None, torch.bfloat16, sh, sdn, None, False, [1, d])
+        if record: ev[5].record()
+        return y
+
+    ms = time_gpu(lambda i: block(), steps, warmup)
+    block(record=True)
+    torch.cuda.synchronize()
+    parts = [ev[i].elapsed_time(ev[i + 1]) for i in range(5)]
+    flop = 3 * 2.0 * T * d * ff
+    return {"name": "mlp_block", "workload": "C5 fp8 MLP block T=4096 d=4096 ff=14336, per-token x per-channel",
+            "metric": "tokens/s", "value": round(T / (ms * 1e-3), 1), "unit": "tokens/s",
+            "ms_per_call": round(ms, 4), "steps": steps, "gemm_tflops": round(flop / (ms * 1e-3) / 1e12, 1),
+            "breakdown_ms": {"quant_x": round(parts[0], 4), "gemm_gate_up": round(parts[1], 4),
+                             "silu_mul_torch": round(parts[2], 4), "quant_h": round(parts[3], 4),
+                             "gemm_down": round(parts[4], 4)}}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,cast,int4,decode,mlp")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus 1); nothing here uses a second GPU.",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the kernels have no CPU fallback.", file=sys.stderr)
+        sys.exit(1)
+
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    from oracle import oracle
+    ops = torch.ops.hpu
+    dev = torch.device("cuda:0")
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    which = set(args.only.split(",")) if args.only else {"gemm", "cast", "int4", "decode", "mlp"}
+    cpu = not args.no_cpu
+    k_stream = max(args.steps, 50)      # the microsecond-scale kernels need more calls for a stable mean
+    w_stream = max(args.warmup, 10)
+
+    ops_out = []
+    if "cast" in which:
+        ops_out += bench_cast(ops, oracle, dev, k_stream, w_stream, cpu)
+    if "int4" in which:
+        ops_out += bench_int4(ops, oracle, dev, k_stream, w_stream, cpu)
+    if "decode" in which:
+        ops_out += bench_gemm_decode(ops, oracle, dev, args.steps, args.warmup)
+    if "mlp" in which:
+        ops_out.append(bench_mlp(ops, dev, max(args.steps // 2, 5), args.warmup))
+
+    line = {"metric": "cast/dequant GB/s (% HBM peak); fp8_gemm_v2 TFLOP/s (% fp8 MFMA peak)",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3fn x fp8_e4m3fn -> f32 accumulate -> bf16",
+            "data": "synthetic"}
+    if "gemm" in which:
+        g = bench_gemm_c3(ops, oracle, pkg, dev, args.steps, args.warmup, cpu)
+        line.update({"value": round(g["tflops"], 1), "unit": "TFLOP/s", "ms_per_step": round(g["ms"], 4),
+                     "config": {"workload": "C3 fp8_gemm_v2 M=8192 K=4096 N=14336 e4m3fn, per-tensor scales, bf16 bias",
+                                "kernel_variant": g["variant"]},
+                     "roofline": {"bound": "mfma", "kernel": "fp8_gemm_tile_kernel", "achieved": round(g["tflops"], 1),
+                                  "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(g["tflops"] / FP8_PEAK_TFLOPS, 4),
+                                  "algorithmic_flop": g["flop"], "traffic": MEASURED_TRAFFIC.get("fp8_gemm_v2")}})
+        if g["cpu"]:
+            line["cpu_baseline"] = g["cpu"]
+    else:
+        first = ops_out[0]
+        line.update({"value": first["value"], "unit": first["unit"], "ms_per_step": first["ms_per_call"],
+                     "config": {"workload": first["workload"]}, "roofline": first.get("roofline")})
+        if "cpu_baseline" in first:
+            line["cpu_baseline"] = first["cpu_baseline"]
+    line["ops"] = ops_out
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,243 @@
+"""GPU parity: cast_to_fp8_v2 / cast_from_fp8 / amax against the CPU oracle, bit exact."""
+import ctypes
+
+import pytest
+import torch
+
+from helpers import E4, E5, FP8_DTYPES, assert_bits_equal, assert_fp8_equal, c1_input
+
+pytestmark = pytest.mark.gpu
+ops = torch.ops.hpu
+
+
+def all_bf16_patterns():
+    return (torch.arange(65536, dtype=torch.int32) << 16).view(torch.float32)
+
+
+@pytest.mark.parametrize("out_dtype", FP8_DTYPES)
+@pytest.mark.parametrize("in_dtype", [torch.float32, torch.bfloat16])
+def test_exhaustive_bf16_patterns(oracle, dev, in_dtype, out_dtype):
+    """All 65536 bf16 bit patterns (NaN, Inf, subnormals, both zeros included)."""
+    x = all_bf16_patterns().to(in_dtype)
+    for scale in (None, 1.0, 0.37, 3.0):
+        got, _ = ops.cast_to_fp8_v2(x.to(dev), scale, False, False, out_dtype)
+        ref, _ = oracle.c_cast_to_fp8(x, scale, out_dtype)
+        assert_fp8_equal(got, ref, out_dtype, f"scale={scale}")
+
+
+@pytest.mark.parametrize("out_dtype", FP8_DTYPES)
+def test_random_fp32_bit_patterns(oracle, dev, out_dtype):
+    g = torch.Generator().manual_seed(11)
+    x = torch.randint(-2 ** 31, 2 ** 31 - 1, ((1 << 20) + 5,), generator=g, dtype=torch.int64).to(torch.int32).view(torch.float32)
+    x = torch.where(torch.isnan(x), torch.zeros_like(x), x)
+    got, amax = ops.cast_to_fp8_v2(x.to(dev), torch.tensor(0.75).to(dev), False, True, out_dtype)
+    ref, amax_ref = oracle.c_cast_to_fp8(x, 0.75, out_dtype, True)
+    assert_fp8_equal(got, ref, out_dtype)
+    assert amax.cpu().item() == amax_ref.item()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("is_amax", [True, False])
+@pytest.mark.parametrize("out_dtype", FP8_DTYPES)
+def test_cast_to_fp8_v2_round_trip(oracle, dev, dtype, is_amax, out_dtype):
+    """test_hpu_fp8_ops_any_mode.py:53-147 (RNE cases), shape (64, 48) doubled by the sign cat."""
+    pos = torch.rand(64, 48).to(dtype) * 30 + 10
+    x = torch.cat((pos, -pos))
+    scale = torch.tensor(1.3)
+    casted, amax = ops.cast_to_fp8_v2(x.to(dev), scale.to(dev), False, is_amax, out_dtype)
+    uncasted = ops.cast_from_fp8(casted, scale.reciprocal().to(dev), dtype, None)
+    ref8, ref_amax = oracle.c_cast_to_fp8(x, scale, out_dtype, is_amax)
+    assert_fp8_equal(casted, ref8, out_dtype)
+    assert_bits_equal(uncasted, oracle.c_cast_from_fp8(ref8, scale.reciprocal(), dtype), "round trip")
+    if is_amax:
+        assert amax.cpu() == torch.max(x.abs()) and amax.dim() == 0
+    else:
+        assert amax.numel() == 0 and tuple(amax.shape) == (0,)
+
+
+@pytest.mark.parametrize("dtype", FP8_DTYPES)
+@pytest.mark.parametrize("scale", [None, 1.0])
+def test_cast_to_fp8_v2_from_fp8_is_identity(dev, dtype, scale):
+    """test :150-176, plus all 256 codes."""
+    pos = torch.rand(64, 48) * 30 + 10
+    x = torch.cat((pos, -pos)).to(dtype)
+    out, _ = ops.cast_to_fp8_v2(x.to(dev), scale, False, False, dtype)
+    assert torch.equal(out.cpu().view(torch.uint8), x.view(torch.uint8))
+    codes = torch.arange(256, dtype=torch.uint8).view(dtype)
+    out, _ = ops.cast_to_fp8_v2(codes.to(dev), scale, False, False, dtype)
+    assert torch.equal(out.cpu().view(torch.uint8), codes.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", FP8_DTYPES)
+@pytest.mark.parametrize("dst_dtype", FP8_DTYPES)
+@pytest.mark.parametrize("is_amax", [False, True])
+def test_cast_to_fp8_v2_from_fp8_exception(dev, dtype, dst_dtype, is_amax):
+    """test :179-202."""
+    x = torch.rand(16, 24, 8).to(dtype).to(dev)
+    if is_amax:
+        with pytest.raises(RuntimeError, match="CastToFp8V2 must have no amax for float8."):
+            ops.cast_to_fp8_v2(x, None, False, is_amax, dst_dtype)
+    elif dtype != dst_dtype:
+        with pytest.raises(RuntimeError, match="CastToFp8V2 input and output must have the same dtype for float8, but are"):
+            ops.cast_to_fp8_v2(x, 1.0, False, is_amax, dst_dtype)
+    else:
+        ops.cast_to_fp8_v2(x, 1.0, False, is_amax, dst_dtype)
+
+
+@pytest.mark.parametrize("mode", ["scalar", "tensor_channel", "scalar_channel"])
+@pytest.mark.parametrize("axis", [0, 1])
+@pytest.mark.parametrize("out_dtype", FP8_DTYPES)
+def test_cast_to_fp8_v2_scales(oracle, dev, mode, axis, out_dtype):
+    """test :205-217: scalar, per-channel tensor and per-channel list scales on (16, 24, 8)."""
+    pos = torch.rand(16, 24, 8).bfloat16() * 30 + 10
+    x = torch.cat((pos, -pos))
+    if mode == "scalar":
+        s_cpu, s_arg, s_inv_arg, shape = 1.3, 1.3, 1 / 1.3, None
+    else:
+        vals = (torch.rand(x.shape[-1 - axis]) * 2.0 + 0.5)
+        shape = list(vals.unsqueeze(axis).shape)
+        s_cpu = vals
+        if mode == "tensor_channel":
+            s_arg, s_inv_arg = vals.to(dev), vals.reciprocal().to(dev)
+        else:
+            s_arg, s_inv_arg = vals.tolist(), vals.reciprocal().tolist()
+    casted, amax = ops.cast_to_fp8_v2(x.to(dev), s_arg, False, True, out_dtype, shape)
+    ref8, _ = oracle.c_cast_to_fp8(x, s_cpu, out_dtype, scale_shape=shape)
+    assert_fp8_equal(casted, ref8, out_dtype)
+    assert amax.cpu() == x.abs().max()
+    back = ops.cast_from_fp8(casted, s_inv_arg, torch.bfloat16, shape)
+    inv_cpu = (1 / 1.3) if mode == "scalar" else (vals.reciprocal() if mode == "tensor_channel" else torch.tensor(s_inv_arg))
+    assert_bits_equal(back, oracle.c_cast_from_fp8(ref8, inv_cpu, torch.bfloat16, scale_shape=shape), "back")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("big_tensor", [True, False])
+def test_cast_to_fp8_v2_out_of_range(dev, dtype, big_tensor):
+    """test :220-243: saturation, never Inf/NaN."""
+    for out_dtype, vals, mx in ((E5, [100000, 60000, -60000, -100000], 57344.0), (E4, [1000, 500, -500, -1000], 448.0)):
+        x = torch.tensor(vals, dtype=dtype)
+        expected = torch.tensor([mx, mx, -mx, -mx])
+        if big_tensor:
+            x = x.expand(800, 4).reshape(80, 40)
+            expected = expected.expand(800, 4).reshape(80, 40)
+        out, _ = ops.cast_to_fp8_v2(x.to(dev), torch.tensor(1.0).to(dev), False, False, out_dtype)
+        assert torch.equal(out.cpu().float(), expected)
+
+
+@pytest.mark.parametrize("in_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("out_dtype", FP8_DTYPES)
+@pytest.mark.parametrize("shape,scale_shape", [
+    ((257, 1024), (257, 1)),      # per row, vector kernel
+    ((64, 2048), (1, 2048)),      # per column, vector kernel
+    ((33, 40), (33, 1)),          # per row, generic kernel
+    ((33, 40), (1, 40)),          # per column, generic kernel
+    ((3, 5, 64), (3, 1, 64)),     # two separate runs -> expanded to full
+    ((6, 50), (6, 50)),           # elementwise
+    ((1031,), None),              # ragged flat tail
+    ((0, 8), None),               # empty
+])
+def test_scale_broadcast_forms(oracle, dev, in_dtype, out_dtype, shape, scale_shape):
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(shape, generator=g) * 40).to(in_dtype)
+    if scale_shape is None:
+        s = torch.tensor(0.9)
+    else:
+        s = torch.rand(scale_shape, generator=g) * 2 + 0.25
+    got, amax = ops.cast_to_fp8_v2(x.to(dev), s.to(dev), False, True, out_dtype, list(scale_shape) if scale_shape else None)
+    ref, amax_ref = oracle.c_cast_to_fp8(x, s, out_dtype, True, scale_shape=list(scale_shape) if scale_shape else None)
+    assert_fp8_equal(got, ref, out_dtype)
+    assert amax.cpu().item() == amax_ref.item()
+    for back_dtype in (torch.float32, torch.bfloat16):
+        back = ops.cast_from_fp8(got, s.to(dev), back_dtype, list(scale_shape) if scale_shape else None)
+        back_ref = oracle.c_cast_from_fp8(ref, s, back_dtype, scale_shape=list(scale_shape) if scale_shape else None)
+        assert_bits_equal(back, back_ref, f"cast_from {back_dtype}")
+
+
+@pytest.mark.parametrize("fmt", FP8_DTYPES)
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_cast_from_fp8_all_codes(oracle, dev, fmt, out_dtype):
+    codes = torch.arange(256, dtype=torch.uint8).repeat(37).view(fmt)  # 9472 = not a multiple of 16*256
+    for scale in (None, 1.0, 0.3, 1.0 / 448 * 7.5):
+        got = ops.cast_from_fp8(codes.to(dev), scale, out_dtype)
+        assert_bits_equal(got, oracle.c_cast_from_fp8(codes, scale, out_dtype), f"scale={scale}")
+
+
+def test_unaligned_views(oracle, dev):
+    """A contiguous view that starts 2 bytes off a 16-byte boundary takes the generic kernels."""
+    base = (torch.randn(4099) * 20).bfloat16()
+    xd = base.to(dev)[1:]
+    got, amax = ops.cast_to_fp8_v2(xd, 1.7, False, True, E4)
+    ref, amax_ref = oracle.c_cast_to_fp8(base[1:], 1.7, E4, True)
+    assert_fp8_equal(got, ref, E4)
+    assert amax.cpu().item() == amax_ref.item()
+    back = ops.cast_from_fp8(got[3:], 0.5, torch.bfloat16)
+    assert_bits_equal(back, oracle.c_cast_from_fp8(ref[3:], 0.5, torch.bfloat16), "unaligned cast_from")
+
+
+def test_amax_nan_propagates(dev):
+    x = torch.randn(5000).bfloat16()
+    x[1234] = float("nan")
+    _, amax = ops.cast_to_fp8_v2(x.to(dev), None, False, True, E4)
+    assert torch.isnan(amax.cpu())
+    assert torch.isnan(torch.ops.mi355q.amax(x.float().to(dev)).cpu())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_amax_ops(oracle, dev, dtype):
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(300, 1000, generator=g) * 7).to(dtype)
+    assert torch.ops.mi355q.amax(x.to(dev)).cpu() == oracle.c_amax(x)
+    assert torch.equal(torch.ops.mi355q.rowwise_amax(x.to(dev)).cpu(), oracle.c_amax(x, rowwise=True))
+    y = x[:, :777].contiguous()
+    assert torch.equal(torch.ops.mi355q.rowwise_amax(y.to(dev)).cpu(), oracle.c_amax(y, rowwise=True))
+    assert torch.ops.mi355q.amax(y.to(dev)).cpu() == oracle.c_amax(y)
+
+
+def test_config1_full_size(oracle, dev):
+    """BASELINE config 1 at full size: amax, scale = 448/amax, cast, cast back.
+    Checked bit-exactly against the PyTorch-CPU twin (multi-threaded; the C
+    oracle is pinned to it on smaller inputs) and on a 1/16 slice against C."""
+    x = c1_input()
+    xd = x.to(dev)
+    amax = torch.ops.mi355q.amax(xd)
+    assert amax.cpu() == x.abs().max().float()
+    scale = (448.0 / amax.cpu()).reshape(())
+    y, amax2 = ops.cast_to_fp8_v2(xd, scale.to(dev), False, True, E4)
+    assert amax2.cpu() == amax.cpu()
+    ref, _ = oracle.torch_cast_to_fp8(x, scale, E4)
+    assert_fp8_equal(y, ref, E4, "full size vs torch twin")
+    cref, _ = oracle.c_cast_to_fp8(x[:256], scale, E4)
+    assert_fp8_equal(y[:256], cref, E4, "slice vs C oracle")
+    back = ops.cast_from_fp8(y, scale.reciprocal().to(dev), torch.bfloat16)
+    assert_bits_equal(back, oracle.torch_cast_from_fp8(ref, scale.reciprocal(), torch.bfloat16), "cast back")
+    # saturation was exercised: the +-1e4 outliers sit at +-448
+    assert (y.cpu().float().abs() == 448).sum().item() >= 16778
+
+
+def test_c_abi_direct(oracle, pkg, dev):
+    """Straight through the C ABI with raw device pointers, no torch op in between."""
+    lib = pkg.capi()
+    x = (torch.randn(128, 512) * 5).bfloat16()
+    xd = x.to(dev)
+    y = torch.empty(128, 512, dtype=torch.uint8, device=dev)
+    amax = torch.full((1,), -1.0, device=dev)
+    scale = torch.rand(128) + 0.5
+    sd = scale.to(dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    st = lib.mi355q_cast_to_fp8(xd.data_ptr(), pkg.BF16, y.data_ptr(), pkg.E4M3FN, sd.data_ptr(), 0.0,
+                                pkg.SCALE_MID, 1, 128, 512, amax.data_ptr(), stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    ref, aref = oracle.c_cast_to_fp8(x, scale, E4, True, scale_shape=[128, 1])
+    assert_fp8_equal(y.view(E4), ref, E4)
+    assert amax.cpu().item() == aref.item()
+    out = torch.empty(128, 512, dtype=torch.float32, device=dev)
+    st = lib.mi355q_cast_from_fp8(y.data_ptr(), pkg.E4M3FN, out.data_ptr(), pkg.F32, sd.data_ptr(), 0.0,
+                                  pkg.SCALE_MID, 1, 128, 512, stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    assert_bits_equal(out, oracle.c_cast_from_fp8(ref, scale, torch.float32, scale_shape=[128, 1]))
+    ra = torch.empty(128, device=dev)
+    assert lib.mi355q_rowwise_amax(xd.data_ptr(), pkg.BF16, 128, 512, ra.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(ra.cpu(), x.abs().amax(1).float())

@@ -1,0 +1,211 @@
+"""Host layer without a GPU: the C-ABI library loads and exports what
+include/mi355q.h declares, the hpu:: schemas are the reference's, and shapes,
+dtypes and error strings follow the reference (exercised on meta tensors)."""
+import os
+import re
+
+import pytest
+import torch
+
+from helpers import E4, E5
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# habana_eager/eager_custom_op_register.cpp:2146-2171
+REFERENCE_SCHEMAS = {
+    ("cast_from_fp8", ""): "hpu::cast_from_fp8(Tensor input, Tensor? scale, ScalarType out_dtype, int[]? scale_shape=None) -> Tensor",
+    ("cast_from_fp8", "scalar"): "hpu::cast_from_fp8.scalar(Tensor input, float scale, ScalarType out_dtype, int[]? scale_shape=None) -> Tensor",
+    ("cast_from_fp8", "scalar_list"): "hpu::cast_from_fp8.scalar_list(Tensor input, float[] scale, ScalarType out_dtype, int[]? scale_shape=None) -> Tensor",
+    ("cast_to_fp8_v2", ""): "hpu::cast_to_fp8_v2(Tensor input, Tensor? scale=None, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)",
+    ("cast_to_fp8_v2", "scalar"): "hpu::cast_to_fp8_v2.scalar(Tensor input, float scale, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)",
+    ("cast_to_fp8_v2", "scalar_list"): "hpu::cast_to_fp8_v2.scalar_list(Tensor input, float[] scale, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)",
+    ("convert_from_int4", ""): "hpu::convert_from_int4(Tensor input, Tensor scale, Tensor? zero_point, ScalarType out_dtype) -> Tensor",
+    ("convert_from_uint4", ""): "hpu::convert_from_uint4(Tensor input, Tensor scale, Tensor? zero_point, ScalarType out_dtype) -> Tensor",
+    ("fp8_gemm_v2", ""): "hpu::fp8_gemm_v2(Tensor A, bool trans_A, Tensor B, bool trans_B, Tensor? D, ScalarType out_dtype, Tensor? A_scale_inv=None, Tensor? B_scale_inv=None, Tensor? bias=None, bool accumulate=False, int[]? B_scale_shape=None) -> Tensor",
+    ("fp8_gemm_v2", "scalar"): "hpu::fp8_gemm_v2.scalar(Tensor A, bool trans_A, Tensor B, bool trans_B, Tensor? D, ScalarType out_dtype, float A_scale_inv, float B_scale_inv, Tensor? bias=None, bool accumulate=False, int[]? B_scale_shape=None) -> Tensor",
+    ("fp8_gemm_v2", "scalar_list"): "hpu::fp8_gemm_v2.scalar_list(Tensor input, float[] A_scale_inv, float[] B_scale_inv)".replace(
+        "Tensor input, float[] A_scale_inv, float[] B_scale_inv",
+        "Tensor A, bool trans_A, Tensor B, bool trans_B, Tensor? D, ScalarType out_dtype, float[] A_scale_inv, float[] B_scale_inv, Tensor? bias=None, bool accumulate=False, int[]? B_scale_shape=None") + " -> Tensor",
+}
+
+
+def meta(shape, dtype):
+    return torch.empty(shape, device="meta", dtype=dtype)
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    header = open(os.path.join(ROOT, "include", "mi355q.h")).read()
+    declared = set(re.findall(r"^(?:int|const char\*)\s+(mi355q_[a-z0-9_]+)\s*\(", header, flags=re.M))
+    assert declared == set(pkg.EXPORTED_SYMBOLS)
+    lib = pkg.capi()
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.mi355q_abi_version() == 1
+    assert lib.mi355q_status_string(0) == b"ok"
+    assert b"invalid" in lib.mi355q_status_string(1)
+
+
+def test_no_compute_entry_point_accepts_bad_enums(pkg):
+    """Argument validation happens before any launch, so it runs without a GPU."""
+    lib = pkg.capi()
+    assert lib.mi355q_cast_to_fp8(None, 0, None, 7, None, 1.0, 0, 1, 1, 1, None, None) == 1
+    assert lib.mi355q_cast_to_fp8(None, 0, None, pkg.E4M3FN, None, 1.0, pkg.SCALE_DEV, 1, 1, 1, None, None) == 1
+    assert lib.mi355q_cast_from_fp8(None, pkg.E4M3FN, None, pkg.E5M2, None, 1.0, 0, 1, 1, 1, None) == 1
+    assert lib.mi355q_dequant_4bit(None, None, None, 0, 0, pkg.BF16, 4, 4, 0, None, None) == 1
+    assert lib.mi355q_fp8_gemm(None, 0, 0, 0, None, 2, 0, 0, None, 1, 0, 1, 1, 1, None, 1.0, 0, None, 1.0, 0,
+                               None, 0, 0, None, 0, 1, 0, 0, 0, 0, 0, None) == 1
+    # empty problems succeed without touching the device
+    assert lib.mi355q_cast_from_fp8(None, pkg.E4M3FN, None, pkg.BF16, None, 1.0, 0, 0, 1, 1, None) == 0
+    assert lib.mi355q_fp8_gemm(None, 2, 0, 0, None, 2, 0, 0, None, 1, 0, 0, 16, 16, None, 1.0, 0, None, 1.0, 0,
+                               None, 0, 0, None, 0, 1, 0, 0, 0, 0, 0, None) == 0
+
+
+def test_variant_names(pkg):
+    lib = pkg.capi()
+    assert b"256x256" in lib.mi355q_fp8_gemm_variant(0, 4096, 0, 14336, 8192, 14336, 4096)
+    assert lib.mi355q_fp8_gemm_variant(0, 24, 0, 36, 12, 36, 24) == b"simple"
+
+
+@pytest.mark.parametrize("key", sorted(REFERENCE_SCHEMAS))
+def test_schemas_are_the_references(pkg, key):
+    name, overload = key
+    packet = getattr(torch.ops.hpu, name)
+    op = getattr(packet, overload or "default")
+    assert str(op._schema) == REFERENCE_SCHEMAS[key]
+
+
+def test_no_cpu_implementation(pkg):
+    with pytest.raises((RuntimeError, NotImplementedError), match="CPU"):
+        torch.ops.hpu.cast_to_fp8_v2(torch.zeros(4), None, False, False, E4)
+    with pytest.raises((RuntimeError, NotImplementedError), match="CPU"):
+        torch.ops.hpu.convert_from_int4(torch.zeros(4, dtype=torch.int32), torch.ones(32), None, torch.bfloat16)
+
+
+@pytest.mark.parametrize("is_amax", [True, False])
+@pytest.mark.parametrize("dtype", [E4, E5])
+def test_cast_to_fp8_v2_meta(pkg, is_amax, dtype):
+    """dynamo/_custom_op_meta_registrations.py:56-76 and fp8_ops.cpp:170-178."""
+    x = meta((16, 24, 8), torch.bfloat16)
+    for scale in (None, meta((), torch.float32), 1.3, [1.0] * 8):
+        args = [x, scale, False, is_amax, dtype] + ([[1, 8]] if isinstance(scale, list) else [])
+        out, amax = torch.ops.hpu.cast_to_fp8_v2(*args)
+        assert out.shape == x.shape and out.dtype == dtype
+        assert amax.dtype == torch.float32
+        assert tuple(amax.shape) == (() if is_amax else (0,))
+
+
+def test_cast_to_fp8_v2_errors(pkg):
+    """Strings of fp8_ops.cpp:46-52,203-215 (test_hpu_fp8_ops_any_mode.py:179-202)."""
+    for src in (E4, E5):
+        for dst in (E4, E5):
+            x = meta((16, 24, 8), src)
+            with pytest.raises(RuntimeError, match="CastToFp8V2 must have no amax for float8."):
+                torch.ops.hpu.cast_to_fp8_v2(x, None, False, True, dst)
+            if src != dst:
+                msg = ("CastToFp8V2 input and output must have the same dtype for float8, but are "
+                       f"{str(src).replace('torch.f', 'F')} and {str(dst).replace('torch.f', 'F')}")
+                with pytest.raises(RuntimeError, match=re.escape(msg)):
+                    torch.ops.hpu.cast_to_fp8_v2(x, 1.0, False, False, dst)
+            else:
+                out, _ = torch.ops.hpu.cast_to_fp8_v2(x, None, False, False, dst)
+                assert out.dtype == dst
+    with pytest.raises(RuntimeError, match=re.escape(
+            "CastToFp8V2 input dtype must be one of [float, bfloat16, float8_e5m2, float8_e4m3fn].")):
+        torch.ops.hpu.cast_to_fp8_v2(meta((4,), torch.float16), None, False, False, E4)
+    with pytest.raises(RuntimeError, match=re.escape(
+            "Number of scale elements (8) is not equal to number of scale_shape elements (24).")):
+        torch.ops.hpu.cast_to_fp8_v2(meta((16, 24, 8), torch.bfloat16), meta((8,), torch.float32), False, False, E4, [24, 1])
+    with pytest.raises(RuntimeError, match="dtype must be given"):
+        torch.ops.hpu.cast_to_fp8_v2(meta((4,), torch.float32))
+    with pytest.raises(RuntimeError, match="stochastic_rounding=True is not implemented"):
+        torch.ops.hpu.cast_to_fp8_v2(meta((4,), torch.float32), None, True, False, E4)
+
+
+def test_cast_from_fp8_meta_and_errors(pkg):
+    x = meta((8, 16), E4)
+    for dt in (torch.float32, torch.bfloat16):
+        for scale in (None, meta((1,), torch.float32)):
+            out = torch.ops.hpu.cast_from_fp8(x, scale, dt)
+            assert out.shape == x.shape and out.dtype == dt
+        assert torch.ops.hpu.cast_from_fp8(x, 0.5, dt).dtype == dt
+        assert torch.ops.hpu.cast_from_fp8(x, [0.5] * 16, dt, [1, 16]).dtype == dt
+    with pytest.raises(RuntimeError, match="CastFromFp8 output dtype must be equal to float or bfloat16."):
+        torch.ops.hpu.cast_from_fp8(x, None, torch.float16)
+    with pytest.raises(RuntimeError, match="Number of scale elements"):
+        torch.ops.hpu.cast_from_fp8(x, [0.5] * 16, torch.float32, [1, 8])
+
+
+GEMM_SHAPES = [
+    ((24, 12), (24, 36), True, False),
+    ((2, 1, 4, 2), (1, 3, 4, 8), True, False),
+    ((2, 1, 4, 2), (4, 8), True, False),
+    ((4, 2), (3, 4, 8), True, False),
+    ((10,), (10,), False, False),
+    ((2, 10), (10,), False, False),
+    ((10,), (10, 2), False, False),
+    ((4, 8, 16), (16,), False, False),
+    ((8,), (2, 4, 8, 16), False, False),
+    ((5, 7, 3), (5, 3, 9), False, False),
+    ((5, 7, 3), (5, 9, 3), False, True),
+]
+
+
+@pytest.mark.parametrize("sa, sb, ta, tb", GEMM_SHAPES)
+def test_fp8_gemm_v2_shape_rule_is_torch_matmul(pkg, sa, sb, ta, tb):
+    """batched_matmul_output_shape.cpp:33-85; tests :504-514,534-596."""
+    A, B = meta(sa, E4), meta(sb, E4)
+    a = torch.empty(sa).transpose(-2, -1) if ta else torch.empty(sa)
+    b = torch.empty(sb).transpose(-2, -1) if tb else torch.empty(sb)
+    expect = torch.matmul(a, b).shape
+    for dt in (torch.bfloat16, torch.float32):
+        out = torch.ops.hpu.fp8_gemm_v2(A, ta, B, tb, None, dt)
+        assert out.shape == expect and out.dtype == dt
+    assert torch.ops.hpu.fp8_gemm_v2(A, ta, B, tb, None, torch.bfloat16, 1.0, 2.0).shape == expect
+    assert torch.ops.hpu.fp8_gemm_v2(A, ta, B, tb, None, torch.bfloat16, [1.0], [2.0]).shape == expect
+
+
+def test_fp8_gemm_v2_errors(pkg):
+    A, B = meta((12, 24), E4), meta((25, 36), E4)
+    with pytest.raises(RuntimeError, match=re.escape(
+            "Common dimension sizes of matmul inputs should be the same. Got 24 and 25")):
+        torch.ops.hpu.fp8_gemm_v2(A, False, B, False, None, torch.bfloat16)
+    with pytest.raises(RuntimeError, match=re.escape(
+            "Batch dimension 0 of matmul inputs should be the same or at least one of them should be equal to 1. Got 2 and 3")):
+        torch.ops.hpu.fp8_gemm_v2(meta((2, 4, 8), E4), False, meta((3, 8, 4), E4), False, None, torch.bfloat16)
+    B = meta((24, 36), E4)
+    with pytest.raises(RuntimeError, match=re.escape(
+            "Accumulation tensor must be provided at index 4 for Fp8GemmV2, when accumulate is true")):
+        torch.ops.hpu.fp8_gemm_v2(A, False, B, False, None, torch.bfloat16, None, None, None, True)
+    with pytest.raises(RuntimeError, match="Number of scale elements"):
+        torch.ops.hpu.fp8_gemm_v2(A, False, B, False, None, torch.bfloat16, [1.0], [1.0] * 36, None, False, [1, 12])
+    with pytest.raises(RuntimeError, match="output dtype"):
+        torch.ops.hpu.fp8_gemm_v2(A, False, B, False, None, torch.float16)
+    with pytest.raises(RuntimeError, match="operands must be float8"):
+        torch.ops.hpu.fp8_gemm_v2(meta((12, 24), torch.bfloat16), False, B, False, None, torch.bfloat16)
+
+
+@pytest.mark.parametrize("variant", ["int4", "uint4"])
+def test_convert_from_int4_meta(pkg, variant):
+    """int4_ops.cpp:22-30: last dim times 8, dtype = out_dtype."""
+    fn = getattr(torch.ops.hpu, "convert_from_" + variant)
+    for shape in ((10,), (4, 6, 4), (64, 8)):
+        real = list(shape)
+        real[-1] *= 8
+        for dt in (torch.float32, torch.bfloat16):
+            out = fn(meta(shape, torch.int32), meta(real, dt), None, dt)
+            assert list(out.shape) == real and out.dtype == dt
+    with pytest.raises(RuntimeError, match="must be int32"):
+        fn(meta((4, 4), torch.int64), meta((4, 32), torch.float32), None, torch.float32)
+    with pytest.raises(RuntimeError, match="output dtype must be float or bfloat16"):
+        fn(meta((4, 4), torch.int32), meta((4, 32), torch.float32), None, E4)
+
+
+def test_ops_trace_under_fake_tensors(pkg):
+    """The Meta kernels are what lets torch.compile / export trace the ops."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    with FakeTensorMode():
+        x = torch.empty(32, 64, dtype=torch.bfloat16, device="cuda")
+        w = torch.empty(64, 48, dtype=E4, device="cuda")
+        x8, amax = torch.ops.hpu.cast_to_fp8_v2(x, None, False, True, E4)
+        y = torch.ops.hpu.fp8_gemm_v2(x8, False, w, False, None, torch.bfloat16, 0.5, 0.25)
+        assert x8.dtype == E4 and amax.shape == () and y.shape == (32, 48) and y.device.type == "cuda"
