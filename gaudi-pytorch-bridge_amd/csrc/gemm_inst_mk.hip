@@ -1,0 +1,8 @@
+// fp8 GEMM tile kernels for one operand layout: A MN-major, B K-major.
+#include "gemm_tile.h"
+
+namespace mi355q {
+void launch_gemm_mk(const GemmArgs& g, int fmt_a, int fmt_b, int64_t batch, hipStream_t st) {
+  launch_by_format<false, true>(g, fmt_a, fmt_b, batch, st);
+}
+}  // namespace mi355q
