@@ -24,7 +24,7 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed fp32 VALU ops are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+    "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-Wno-inline-asm",
 ]
 
 

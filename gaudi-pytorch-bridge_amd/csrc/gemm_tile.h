@@ -1,11 +1,17 @@
 // fp8 x fp8 -> fp32-accumulate -> bf16/fp32 GEMM for gfx950 (fp8_gemm_v2).
 //
 // Tiled kernel: a 256-thread workgroup (4 waves, 2x2) owns a BM x BN tile of C
-// and walks K in steps of 128 bytes.  Operand tiles are staged in LDS in 16-byte
-// chunks whose position inside a row is XOR-swizzled with the row number, which
-// makes the 128-bit fragment reads bank-conflict free.  Each wave computes its
-// (BM/2) x (BN/2) sub-tile with v_mfma_f32_32x32x64_f8f6f4 (fp8/bf8 operands,
-// 64 k per instruction).
+// and walks K in steps of 128 bytes.  Operand tiles travel from global memory
+// straight into LDS (buffer_load_dwordx4 ... lds: no staging registers, and the
+// buffer descriptor's bounds check zero-fills rows past the matrix edge) into
+// one of two LDS stages, so the loads of step k+2 fly while step k computes.
+// Inside a stage, the 16-byte chunks of a row are XOR-swizzled with the row
+// number, which keeps the 128-bit and transposing fragment reads free of bank
+// conflicts; since a DMA load places lane l's chunk at LDS offset 16 l, the
+// swizzle is applied by choosing which global chunk each lane fetches.  Each
+// wave computes its (BM/2) x (BN/2) sub-tile with v_mfma_f32_32x32x64_f8f6f4
+// (fp8/bf8 operands, 64 k per instruction), reading the fragments of the next
+// half-step while the MFMAs of the current one run.
 //
 // Operand layouts.  An operand whose K index is contiguous in memory (A with
 // trans_a == 0, B with trans_b != 0) is "K-major": a lane's 32-byte MFMA
@@ -27,6 +33,7 @@ namespace mi355q {
 
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define LDS_AS __attribute__((address_space(3)))
 
@@ -74,82 +81,6 @@ struct TileGeom {
   }
 };
 
-// Loads one operand tile from global memory into registers.
-//   KMAJOR: rows index m/n (clamped to the last valid row), chunks walk k
-//           (chunks at or beyond K read as zero)
-//   else  : rows index k (rows at or beyond K read as zero), chunks walk m/n
-//           (chunks at or beyond the extent read as zero)
-template <bool KMAJOR, int EXT>  // EXT: tile extent along m/n
-struct TileLoader {
-  using G = TileGeom<KMAJOR ? EXT : kBK, KMAJOR ? kBK : EXT>;
-  u32x4 regs[G::kPerThread];
-
-  __device__ __forceinline__ void load(const uint8_t* base, int64_t ld, int mn0, int mn_extent,
-                                       int k0, int K) {
-#pragma unroll
-    for (int i = 0; i < G::kPerThread; ++i) {
-      const int q = threadIdx.x + i * kGemmThreads;
-      const int row = q / G::kChunksPerRow, c = q % G::kChunksPerRow;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if constexpr (KMAJOR) {
-        int r = mn0 + row;
-        r = r < mn_extent ? r : mn_extent - 1;
-        const int k = k0 + c * 16;
-        if (k < K) v = *reinterpret_cast<const u32x4*>(base + (int64_t)r * ld + k);
-      } else {
-        const int k = k0 + row;
-        const int mn = mn0 + c * 16;
-        if (k < K && mn < mn_extent) v = *reinterpret_cast<const u32x4*>(base + (int64_t)k * ld + mn);
-      }
-      regs[i] = v;
-    }
-  }
-
-  __device__ __forceinline__ void store(uint8_t* lds) const {
-#pragma unroll
-    for (int i = 0; i < G::kPerThread; ++i) {
-      const int q = threadIdx.x + i * kGemmThreads;
-      const int row = q / G::kChunksPerRow, c = q % G::kChunksPerRow;
-      *reinterpret_cast<u32x4*>(lds + G::lds_offset(row, c)) = regs[i];
-    }
-  }
-};
-
-// 32-byte MFMA fragment (32 rows of m/n x 32 k for this lane's k-half) from LDS.
-template <bool KMAJOR, int EXT>
-__device__ __forceinline__ i32x8 read_fragment(const uint8_t* lds, int mn_base, int ksub) {
-  using G = TileGeom<KMAJOR ? EXT : kBK, KMAJOR ? kBK : EXT>;
-  const int lane = threadIdx.x & 63;
-  i32x8 f;
-  if constexpr (KMAJOR) {
-    const int row = mn_base + (lane & 31);
-    const int c0 = ksub * 4 + (lane >> 5) * 2;
-    const u32x4 lo = *reinterpret_cast<const u32x4*>(lds + G::lds_offset(row, c0));
-    const u32x4 hi = *reinterpret_cast<const u32x4*>(lds + G::lds_offset(row, c0 + 1));
-    f[0] = lo[0]; f[1] = lo[1]; f[2] = lo[2]; f[3] = lo[3];
-    f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
-  } else {
-    // Within each group of 16 lanes, lanes 2r and 2r+1 point at the two 8-byte
-    // halves of k-row r; after the transposing read lane i of the group holds
-    // column i for those 8 k-rows.
-    const int blk = lane >> 4, i = lane & 15;
-    const int r = i >> 1, h = i & 1;
-    const int col = mn_base + (blk & 1) * 16;  // first column of this 16-lane group
-    const int kb = ksub * 64 + (blk >> 1) * 32;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const int krow = kb + kk * 8 + r;
-      const int off = G::lds_offset(krow, col >> 4) + h * 8;
-      const i32x2 t = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-          (LDS_AS i32x2*)((LDS_AS uint8_t*)lds + off));
-      f[2 * kk] = t[0];
-      f[2 * kk + 1] = t[1];
-    }
-  }
-  return f;
-}
-
-// ------------------------------------------------------------------- epilogue
 template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {
   if constexpr (N > 0) {
@@ -158,6 +89,126 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
+// Global -> LDS loader for one operand tile, one 16-byte chunk per lane per
+// instruction.  A wave-wide load fills a 1 KiB region of the LDS tile (lane l
+// lands at byte 16 l of the region), i.e. 64 / chunks-per-row consecutive rows;
+// the four waves split the regions of a tile evenly.
+//   KMAJOR: rows index m/n, chunks walk k.  Rows past the matrix end fall
+//           outside the buffer descriptor and read as zero; chunks at or beyond
+//           K are redirected outside it.
+//   else  : rows index k, chunks walk m/n.  Rows at or beyond K fall outside the
+//           descriptor; columns past the extent only feed outputs that are
+//           never stored.
+template <bool KMAJOR, int EXT>  // EXT: tile extent along m/n
+struct DmaLoader {
+  using G = TileGeom<KMAJOR ? EXT : kBK, KMAJOR ? kBK : EXT>;
+  static constexpr int kCPR = G::kChunksPerRow;
+  static constexpr int kRowsPerRegion = 64 / kCPR;
+  static constexpr int kRegions = G::kChunks / 64;
+  static constexpr int kPerWave = kRegions / 4;
+  static_assert(kRegions % 4 == 0 && 64 % kCPR == 0, "tile does not split over 4 waves");
+
+  i32x4 rsrc;  // raw buffer descriptor: base, stride 0, num_records (bytes), dword 3 flags
+  int voff[kPerWave];
+  int step;  // voffset increment per K stage
+  int kc;    // K-major: byte offset of this lane's chunk inside a stage row
+  int wave;
+
+  // base: first element of this batch's matrix; mn0: first row (K-major) or
+  // column (MN-major) of the tile; extent: matrix extent along m/n.
+  __device__ __forceinline__ void init(const uint8_t* base, int64_t ld, int mn0, int extent, int K) {
+    const int lane = threadIdx.x & 63;
+    wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rin = lane / kCPR, p = lane % kCPR;
+    int64_t records;
+    if constexpr (KMAJOR) {
+      base += (int64_t)mn0 * ld;
+      records = (int64_t)(extent - mn0 - 1) * ld + K;
+      step = kBK;
+    } else {
+      base += mn0;
+      records = (int64_t)(K - 1) * ld + (extent - mn0);
+      step = kBK * (int)ld;
+    }
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    rsrc[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    rsrc[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((b >> 32) & 0xffffu));
+    rsrc[2] = __builtin_amdgcn_readfirstlane((int)records);
+    rsrc[3] = 0x00020000;
+    kc = 0;
+#pragma unroll
+    for (int i = 0; i < kPerWave; ++i) {
+      const int row = (wave * kPerWave + i) * kRowsPerRegion + rin;
+      const int c = p ^ (row & G::kSwzMask);
+      voff[i] = row * (int)ld + c * 16;
+      if (i == 0) kc = c * 16;  // the same for every i: kRowsPerRegion is a multiple of the swizzle period or the row term cancels
+    }
+  }
+
+  // Issues load I of this wave's share of the stage that starts at k0.
+  template <int I>
+  __device__ __forceinline__ void issue_one(uint8_t* lds_tile, int k0, int K) const {
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)lds_tile;
+    {
+      constexpr int i = I;
+      int vo = voff[i];
+      if constexpr (KMAJOR) vo = (k0 + kc < K) ? vo : 0x7fffffff;
+      const uint32_t dst = lds_base + (uint32_t)((wave * kPerWave + i) * 1024);
+      // m0 holds the LDS address of the region; lane l's 16 bytes land at m0 + 16 l.
+      // Written as asm so that the compiler, which would otherwise make every later
+      // LDS read wait for all outstanding global->LDS loads, leaves the waiting to
+      // the explicit vmcnt drain before each barrier.
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                   :
+                   : "s"(dst), "v"(vo), "s"(rsrc)
+                   : "memory", "m0");
+    }
+  }
+
+  __device__ __forceinline__ void issue(uint8_t* lds_tile, int k0, int K) const {
+    static_for<kPerWave>([&](auto ic) { issue_one<decltype(ic)::value>(lds_tile, k0, K); });
+  }
+
+  __device__ __forceinline__ void advance() {
+#pragma unroll
+    for (int i = 0; i < kPerWave; ++i) voff[i] += step;
+  }
+};
+
+// A 32-byte MFMA fragment (32 rows of m/n x 32 k for this lane's k-half) is
+// read from LDS in parts: two ds_read_b128 for a K-major operand, four
+// ds_read_b64_tr_b8 for an MN-major one.
+template <bool KMAJOR>
+constexpr int frag_parts() { return KMAJOR ? 2 : 4; }
+
+template <bool KMAJOR, int EXT, int PART>
+__device__ __forceinline__ void read_fragment_part(const uint8_t* lds, int mn_base, int ksub, i32x8& f) {
+  using G = TileGeom<KMAJOR ? EXT : kBK, KMAJOR ? kBK : EXT>;
+  const int lane = threadIdx.x & 63;
+  if constexpr (KMAJOR) {
+    const int row = mn_base + (lane & 31);
+    const int c = ksub * 4 + (lane >> 5) * 2 + PART;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(lds + G::lds_offset(row, c));
+    f[4 * PART + 0] = v[0];
+    f[4 * PART + 1] = v[1];
+    f[4 * PART + 2] = v[2];
+    f[4 * PART + 3] = v[3];
+  } else {
+    // Within each group of 16 lanes, lanes 2r and 2r+1 point at the two 8-byte
+    // halves of k-row r; after the transposing read lane i of the group holds
+    // column i for those 8 k-rows.
+    const int blk = lane >> 4, i = lane & 15;
+    const int r = i >> 1, h = i & 1;
+    const int col = mn_base + (blk & 1) * 16;  // first column of this 16-lane group
+    const int krow = ksub * 64 + (blk >> 1) * 32 + PART * 8 + r;
+    const int off = G::lds_offset(krow, col >> 4) + h * 8;
+    const i32x2 t = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LDS_AS i32x2*)((LDS_AS uint8_t*)lds + off));
+    f[2 * PART] = t[0];
+    f[2 * PART + 1] = t[1];
+  }
+}
+
+// ------------------------------------------------------------------- epilogue
 __device__ __forceinline__ float load_out_as_f32(const uint8_t* p, int64_t idx, int bf16) {
   return bf16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[idx])
               : reinterpret_cast<const float*>(p)[idx];
@@ -294,14 +345,145 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
 }
 
 // --------------------------------------------------------------------- kernel
+// Per-wave state of the K loop: accumulators, two sets of fragments, loaders.
+template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
+struct TileCore {
+  static constexpr int TM = BM / 2, TN = BN / 2;
+  static constexpr int MT = TM / 32, NT = TN / 32;
+  f32x16 acc[MT][NT];
+  i32x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];
+  DmaLoader<A_KMAJOR, BM> la;
+  DmaLoader<B_KMAJOR, BN> lb;
+  int wm, wn, K;
+
+  __device__ __forceinline__ void init(const GemmArgs& g, int64_t batch, int m0, int n0, int wm_, int wn_) {
+    wm = wm_;
+    wn = wn_;
+    K = g.K;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+    la.init(g.A + batch * g.stride_a, g.lda, m0, g.M, g.K);
+    lb.init(g.B + batch * g.stride_b, g.ldb, n0, g.N, g.K);
+  }
+
+  static constexpr int kPartsA = frag_parts<A_KMAJOR>(), kPartsB = frag_parts<B_KMAJOR>();
+  static constexpr int kReadOps = MT * kPartsA + NT * kPartsB;  // LDS reads per half-step
+  static constexpr int kMfmas = MT * NT;
+  static constexpr int kDmaOps = DmaLoader<A_KMAJOR, BM>::kPerWave + DmaLoader<B_KMAJOR, BN>::kPerWave;
+
+  // Read op OP of a half-step, in the order the next MFMA block needs the
+  // fragments: A0, B0 .. B(NT-1), A1 .. A(MT-1).
+  template <int OP>
+  __device__ __forceinline__ void read_op(const uint8_t* stage, int ks, i32x8 (&fa)[MT], i32x8 (&fb)[NT]) {
+    if constexpr (OP < kPartsA) {
+      read_fragment_part<A_KMAJOR, BM, OP>(stage, wm, ks, fa[0]);
+    } else if constexpr (OP < kPartsA + NT * kPartsB) {
+      constexpr int o = OP - kPartsA;
+      read_fragment_part<B_KMAJOR, BN, o % kPartsB>(stage + BM * kBK, wn + (o / kPartsB) * 32, ks, fb[o / kPartsB]);
+    } else {
+      constexpr int o = OP - kPartsA - NT * kPartsB;
+      read_fragment_part<A_KMAJOR, BM, o % kPartsA>(stage, wm + (1 + o / kPartsA) * 32, ks, fa[1 + o / kPartsA]);
+    }
+  }
+
+  __device__ __forceinline__ void read_frags(const uint8_t* __restrict__ stage, int ks, i32x8 (&fa)[MT],
+                                             i32x8 (&fb)[NT]) {
+    static_for<kReadOps>([&](auto oc) { read_op<decltype(oc)::value>(stage, ks, fa, fb); });
+  }
+
+  template <int OP>
+  __device__ __forceinline__ void dma_op(uint8_t* stage, int kt) {
+    constexpr int na = DmaLoader<A_KMAJOR, BM>::kPerWave;
+    if constexpr (OP < na) la.template issue_one<OP>(stage, kt * kBK, K);
+    else lb.template issue_one<OP - na>(stage + BM * kBK, kt * kBK, K);
+  }
+
+  __device__ __forceinline__ void issue_stage(uint8_t* __restrict__ stage, int kt) {
+    static_for<kDmaOps>([&](auto oc) { dma_op<decltype(oc)::value>(stage, kt); });
+    la.advance();
+    lb.advance();
+  }
+
+  // One MFMA block (every tile of the wave, 64 k) on the fragments (ca, cb),
+  // with the LDS reads of the next block's fragments (na, nb) and, when
+  // WITH_DMA, this wave's global->LDS loads of a later stage dealt out between
+  // the MFMAs.  The matrix pipe is busy 16 passes per MFMA; the reads and loads
+  // issue in its shadow.  sched_barrier(0) after each group pins the written
+  // order (left alone, the scheduler gathers the reads after the MFMAs).
+  template <bool WITH_DMA>
+  __device__ __forceinline__ void block(const i32x8 (&ca)[MT], const i32x8 (&cb)[NT], i32x8 (&na)[MT],
+                                        i32x8 (&nb)[NT], const uint8_t* __restrict__ rd_stage, int rd_ks,
+                                        uint8_t* __restrict__ dma_stage, int dma_kt) {
+    // all reads within the first 3/4 of the MFMAs, so that they have landed when the next block starts
+    constexpr int kReadGroups = (kMfmas * 3 + 3) / 4;
+    constexpr int kReadsPerGroup = (kReadOps + kReadGroups - 1) / kReadGroups;
+    constexpr int kDmaPerGroup = (kDmaOps + kMfmas - 1) / kMfmas;
+    static_for<kMfmas>([&](auto gc) {
+      constexpr int gi = decltype(gc)::value;
+      constexpr int i = gi / NT, j = gi % NT;
+      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+          cb[j], ca[i], acc[i][j], mfma_code<FMT_B>(), mfma_code<FMT_A>(), 0, 0, 0, 0);
+      if constexpr (WITH_DMA) {
+        static_for<kDmaPerGroup>([&](auto dc) {
+          constexpr int op = gi * kDmaPerGroup + decltype(dc)::value;
+          if constexpr (op < kDmaOps) dma_op<op>(dma_stage, dma_kt);
+        });
+      }
+      static_for<kReadsPerGroup>([&](auto rc) {
+        constexpr int op = gi * kReadsPerGroup + decltype(rc)::value;
+        if constexpr (op < kReadOps) read_op<op>(rd_stage, rd_ks, na, nb);
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    if constexpr (WITH_DMA) {
+      la.advance();
+      lb.advance();
+    }
+  }
+
+  // A workgroup barrier orders LDS traffic but does not wait for this wave's
+  // outstanding global->LDS loads: drain them first (vmcnt(0)), so that after
+  // the barrier every wave sees every wave's share of the stage.
+  __device__ __forceinline__ static void wait_loads_then_barrier() {
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+  }
+
+  __device__ __forceinline__ void prologue(uint8_t* __restrict__ s0, uint8_t* __restrict__ s1) {
+    issue_stage(s0, 0);
+    issue_stage(s1, 1);
+    wait_loads_then_barrier();
+    read_frags(s0, 0, fa0, fb0);
+  }
+
+  // Two K stages: stage kt sits in s0, stage kt+1 in s1 (or is still landing
+  // there).  After each barrier every wave is done with the stage just
+  // consumed, so the stage two ahead starts to overwrite it while the second
+  // half of the current stage and the whole next stage compute.
+  __device__ __forceinline__ void k_pair(uint8_t* __restrict__ s0, uint8_t* __restrict__ s1, int kt) {
+    block<false>(fa0, fb0, fa1, fb1, s0, 1, nullptr, 0);
+    wait_loads_then_barrier();
+    block<true>(fa1, fb1, fa0, fb0, s1, 0, s0, kt + 2);
+    block<false>(fa0, fb0, fa1, fb1, s1, 1, nullptr, 0);
+    wait_loads_then_barrier();
+    block<true>(fa1, fb1, fa0, fb0, s0, 0, s1, kt + 3);
+  }
+};
+
 template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
 __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g) {
   constexpr int TM = BM / 2, TN = BN / 2;   // per-wave tile
   constexpr int MT = TM / 32, NT = TN / 32; // MFMA tiles per wave
   static_assert(BM == BN, "the epilogue staging area assumes square tiles");
-  __shared__ __attribute__((aligned(16))) uint8_t lds[(BM + BN) * kBK];
-  uint8_t* const lds_a = lds;
-  uint8_t* const lds_b = lds + BM * kBK;
+  constexpr int kStageBytes = (BM + BN) * kBK;
+  // Two stages as two separate arrays, so that loads into one and reads from
+  // the other are provably disjoint.
+  __shared__ __attribute__((aligned(1024))) uint8_t lds0[kStageBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds1[kStageBytes];
 
   // Tile order.  Workgroups are dealt to the 8 XCDs round-robin by id; give
   // each XCD a contiguous range of tiles, and walk tiles in column groups of
@@ -323,56 +505,26 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g)
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int64_t batch = blockIdx.y;
-  const uint8_t* A = g.A + batch * g.stride_a;
-  const uint8_t* B = g.B + batch * g.stride_b;
-
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = (wave >> 1) * TM, wn = (wave & 1) * TN;
 
-  f32x16 acc[MT][NT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-
-  TileLoader<A_KMAJOR, BM> la;
-  TileLoader<B_KMAJOR, BN> lb;
+  TileCore<BM, BN, A_KMAJOR, B_KMAJOR, FMT_A, FMT_B> core;
+  core.init(g, batch, m0, n0, wm, wn);
   const int KT = (g.K + kBK - 1) / kBK;
-  la.load(A, g.lda, m0, g.M, 0, g.K);
-  lb.load(B, g.ldb, n0, g.N, 0, g.K);
 
-  for (int kt = 0; kt < KT; ++kt) {
-    la.store(lds_a);
-    lb.store(lds_b);
-    __syncthreads();
-    if (kt + 1 < KT) {
-      la.load(A, g.lda, m0, g.M, (kt + 1) * kBK, g.K);
-      lb.load(B, g.ldb, n0, g.N, (kt + 1) * kBK, g.K);
-    }
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      i32x8 fa[MT], fb[NT];
-#pragma unroll
-      for (int i = 0; i < MT; ++i) fa[i] = read_fragment<A_KMAJOR, BM>(lds_a, wm + i * 32, ks);
-#pragma unroll
-      for (int j = 0; j < NT; ++j) fb[j] = read_fragment<B_KMAJOR, BN>(lds_b, wn + j * 32, ks);
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-              fb[j], fa[i], acc[i][j], mfma_code<FMT_B>(), mfma_code<FMT_A>(), 0, 0, 0, 0);
-    }
-    __syncthreads();
-  }
+  // Stages at or beyond K are loaded all the same: they fall outside the buffer
+  // descriptors and arrive as zeros.  The loop therefore runs an even number of
+  // branch-free steps, and an odd stage count costs one step of zero products
+  // instead of a second copy of the MFMA block.
+  core.prologue(lds0, lds1);
+  for (int kt = 0; kt < KT; kt += 2) core.k_pair(lds0, lds1, kt);
+  core.wait_loads_then_barrier();
 
-  // The operand tiles are dead (the K loop ends with a barrier); the general
-  // epilogue reuses the LDS as per-wave staging: 4 waves x 16 NT x 64 floats.
-  static_assert((BM + BN) * kBK >= 4 * 16 * NT * 64 * 4, "staging area does not fit");
-  float* stage = reinterpret_cast<float*>(lds) + wave * (16 * NT * 64);
-  epilogue<MT, NT>(g, batch, acc, m0 + wm + (lane & 31), n0 + wn + (lane >> 5) * 4, stage);
+  // The operand tiles are dead (barrier above); the general epilogue reuses
+  // stage 0 as per-wave staging: 4 waves x 16 NT x 64 floats.
+  static_assert(kStageBytes >= 4 * 16 * NT * 64 * 4, "staging area does not fit");
+  float* stage = reinterpret_cast<float*>(lds0) + wave * (16 * NT * 64);
+  epilogue<MT, NT>(g, batch, core.acc, m0 + wm + (lane & 31), n0 + wn + (lane >> 5) * 4, stage);
 }
 
 template <int BM, int BN, bool AK, bool BK_, int FA, int FB>
