@@ -1,6 +1,6 @@
 // fp8 x fp8 -> fp32-accumulate -> bf16/fp32 GEMM for gfx950 (fp8_gemm_v2).
 //
-// Tiled kernel: a 256-thread workgroup (4 waves, 2x2) owns a BM x BN tile of C
+// Tiled kernel: a 512-thread workgroup (8 waves, 2 x 4, two per SIMD) owns a BM x BN tile of C
 // and walks K in steps of 128 bytes.  Operand tiles travel from global memory
 // straight into LDS (buffer_load_dwordx4 ... lds: no staging registers, and the
 // buffer descriptor's bounds check zero-fills rows past the matrix edge) into
@@ -37,8 +37,25 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define LDS_AS __attribute__((address_space(3)))
 
-constexpr int kGemmThreads = 256;
+// Two waves per SIMD: a memory instruction of one wave (LDS fragment read,
+// global->LDS load) holds up that wave's next MFMA for tens of cycles, and only
+// a second resident wave lets the matrix pipe run meanwhile.
+constexpr int kGemmThreads = 512;
+constexpr int kWaves = kGemmThreads / 64;
+constexpr int kWavesM = 2, kWavesN = 4;  // wave grid over the tile
 constexpr int kBK = 128;  // bytes (= fp8 elements) of K per LDS stage
+
+// Number of compute units of the current device (workgroups of the persistent kernel).
+inline int compute_units() {
+  static const int n = [] {
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0)
+      cu = 256;
+    return cu;
+  }();
+  return n;
+}
 
 struct GemmArgs {
   const uint8_t* A;
@@ -107,7 +124,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 // Global -> LDS loader for one operand tile, one 16-byte chunk per lane per
 // instruction.  A wave-wide load fills a 1 KiB region of the LDS tile (lane l
 // lands at byte 16 l of the region), i.e. 64 / chunks-per-row consecutive rows;
-// the four waves split the regions of a tile evenly.
+// the waves split the regions of a tile evenly.
 //   KMAJOR: rows index m/n, chunks walk k.  Rows past the matrix end fall
 //           outside the buffer descriptor and read as zero; chunks at or beyond
 //           K are redirected outside it.
@@ -120,8 +137,8 @@ struct DmaLoader {
   static constexpr int kCPR = G::kChunksPerRow;
   static constexpr int kRowsPerRegion = 64 / kCPR;
   static constexpr int kRegions = G::kChunks / 64;
-  static constexpr int kPerWave = kRegions / 4;
-  static_assert(kRegions % 4 == 0 && 64 % kCPR == 0, "tile does not split over 4 waves");
+  static constexpr int kPerWave = kRegions / kWaves;
+  static_assert(kRegions % kWaves == 0 && 64 % kCPR == 0, "tile does not split over the waves");
 
   i32x4 rsrc;  // raw buffer descriptor: base, stride 0, num_records (bytes), dword 3 flags
   int voff[kPerWave];
@@ -166,7 +183,9 @@ struct DmaLoader {
     {
       constexpr int i = I;
       int vo = voff[i];
+#ifndef MI355Q_DBG_NO_KPRED
       if constexpr (KMAJOR) vo = (k0 + kc[i] < K) ? vo : 0x7fffffff;
+#endif
       const uint32_t dst = lds_base + (uint32_t)((wave * kPerWave + i) * 1024);
       // m0 holds the LDS address of the region; lane l's 16 bytes land at m0 + 16 l.
       // Written as asm so that the compiler, which would otherwise make every later
@@ -232,16 +251,24 @@ __device__ __forceinline__ float load_out_as_f32(const uint8_t* p, int64_t idx, 
 //   acc[i][j][e] on this lane is C[m][n] with
 //     m = m_wave + 32 i + lane % 32
 //     n = n_wave + 32 j + 8 (e / 4) + 4 (lane / 32) + e % 4
-// The accumulators of one row of tiles (32 rows x 32 NT columns per wave) are
-// written to a row-major fp32 copy in LDS (`stage`, rows padded by 16 bytes so
-// that both the 16-byte writes and the 16-byte reads are bank-conflict free)
-// and read back with a lane owning 4 consecutive columns of a row.  The
-// arithmetic then runs in one small runtime loop over the rows, whatever the
-// scale / bias / accumulate forms, and a wave-wide store writes whole rows of
-// the sub-tile (complete 128-byte lines).  Keeping this loop rolled matters:
-// unrolled over the 16 tiles the epilogue is tens of KiB of straight-line code
-// that every wave runs exactly once, which costs more in instruction fetch than
-// in memory traffic.
+// The accumulators pass through a small row-major fp32 staging area in LDS
+// (`stage`: kEpiRows rows of the wave's 32 NT columns, rows padded by 16 bytes)
+// eight rows at a time: the lanes that own those rows write their 4-column
+// pieces, and the data comes back with a lane owning 4 consecutive columns of
+// a row, so that a wave-wide store writes whole 128-byte lines.  The
+// arithmetic runs in one small runtime loop over the rows, whatever the scale
+// / bias / accumulate forms.  Two things keep it cheap: the loop is rolled
+// (unrolled over all tiles the epilogue is tens of KiB of straight-line code
+// that every wave runs once, and instruction fetch dominates), and its common
+// form holds no global load (loads and stores share one counter, vmcnt, so a
+// loop that may load makes every pass wait for the previous pass's store).
+// The staging area is separate from the operand stages, which at that time
+// already receive the first stages of the workgroup's next tile.
+constexpr int kEpiRows = 8;
+
+template <int MT, int NT>
+constexpr int epilogue_stage_floats() { return kEpiRows * (32 * NT + 4) + 2 * 32 * MT; }
+
 template <int MT, int NT>
 __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x16 (&acc)[MT][NT],
                                          int m_wave, int n_wave, float* stage) {
@@ -274,18 +301,18 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
                       ((reinterpret_cast<uintptr_t>(C) + (size_t)n * es) % (4 * es) == 0);
 
   // Per-row scales of the wave's 32 MT rows go to LDS once, so that the row
-  // loop below holds no global load: on gfx950 loads and stores share one
-  // counter (vmcnt), and a loop that may load makes every pass wait for the
-  // previous pass's store to complete.
-  float* row_sa = stage + 32 * kRowFloats;
+  // loop below holds no global load.
+  float* row_sa = stage + kEpiRows * kRowFloats;
   float* row_sb = row_sa + 32 * MT;
-  for (int t = lane; t < 32 * MT; t += 64) {
-    const int m = m_wave + t;
-    row_sa[t] = (g.sa_mode == MI355Q_GS_PER_ROW && m < g.M) ? g.sa[m] : 1.0f;
-    row_sb[t] = (g.sb_mode == MI355Q_GS_PER_ROW && m < g.M) ? g.sb[m] : 1.0f;
+  const bool row_scales = g.sa_mode == MI355Q_GS_PER_ROW || g.sb_mode == MI355Q_GS_PER_ROW;
+  if (row_scales) {
+    for (int t = lane; t < 32 * MT; t += 64) {
+      const int m = m_wave + t;
+      row_sa[t] = (g.sa_mode == MI355Q_GS_PER_ROW && m < g.M) ? g.sa[m] : 1.0f;
+      row_sb[t] = (g.sb_mode == MI355Q_GS_PER_ROW && m < g.M) ? g.sb[m] : 1.0f;
+    }
   }
   const bool general = g.bias_mode == MI355Q_BIAS_FULL || D != nullptr;
-  const bool row_scales = g.sa_mode == MI355Q_GS_PER_ROW || g.sb_mode == MI355Q_GS_PER_ROW;
 
   uint8_t* const c_col = C + (int64_t)n * es;   // this lane's columns in row 0
   const int64_t row_pitch = g.ldc * es;
@@ -295,7 +322,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
       uint16_t* cp = reinterpret_cast<uint16_t*>(rowp);
       if (vec_ok) {
         u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-        *reinterpret_cast<u32x2*>(cp) = o;
+        __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(cp));  // streamed: keep the operand panels in L2
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
@@ -305,7 +332,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
       float* cp = reinterpret_cast<float*>(rowp);
       if (vec_ok) {
         f32x4 o = {v[0], v[1], v[2], v[3]};
-        *reinterpret_cast<f32x4*>(cp) = o;
+        __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(cp));
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
@@ -316,123 +343,135 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
 
   static_for<MT>([&](auto ic) {
     constexpr int i = decltype(ic)::value;
-    static_for<NT>([&](auto jc) {
-      constexpr int j = decltype(jc)::value;
-      static_for<4>([&](auto qc) {
-        constexpr int q = decltype(qc)::value;
-        const f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-        *reinterpret_cast<f32x4*>(stage + (lane & 31) * kRowFloats + 32 * j + 8 * q + 4 * (lane >> 5)) = v;
-      });
-    });
-    if (!general && !row_scales) {
-      // scales and bias depend on the column only: two VALU ops per element;
-      // unrolled by 4 so that four LDS reads are in flight per wait
-#pragma unroll 4
-      for (int r = r_in; r < 32; r += kRowsPerPass) {
-        const f32x4 a = *reinterpret_cast<const f32x4*>(stage + r * kRowFloats + (lane % kLanesPerRow) * 4);
-        const int m = m_wave + 32 * i + r;
-        if (m < g.M && n < g.N) {
-          float v[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float t = a[e] * sa_c[e];
-            t = t * sb_c[e];
-            v[e] = t + bias_c[e];
-          }
-          store_row4(m, v);
-        }
-      }
-    } else if (!general) {
-#pragma unroll 4
-      for (int r = r_in; r < 32; r += kRowsPerPass) {
-        const f32x4 a = *reinterpret_cast<const f32x4*>(stage + r * kRowFloats + (lane % kLanesPerRow) * 4);
-        const float ra = row_sa[32 * i + r], rb = row_sb[32 * i + r];
-        const int m = m_wave + 32 * i + r;
-        if (m < g.M && n < g.N) {
-          float v[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            // one of (ra, sa_c) is exactly 1, likewise (rb, sb_c): the products are the scales themselves
-            float t = a[e] * (ra * sa_c[e]);
-            t = t * (rb * sb_c[e]);
-            v[e] = t + bias_c[e];
-          }
-          store_row4(m, v);
-        }
-      }
-    } else {
 #pragma unroll 1
-      for (int r = r_in; r < 32; r += kRowsPerPass) {
-        const f32x4 a = *reinterpret_cast<const f32x4*>(stage + r * kRowFloats + (lane % kLanesPerRow) * 4);
-        const float ra = row_sa[32 * i + r], rb = row_sb[32 * i + r];
-        const int m = m_wave + 32 * i + r;
-        if (m < g.M && n < g.N) {
-          float v[4];
+    for (int sub = 0; sub < 32 / kEpiRows; ++sub) {
+      if (((lane & 31) / kEpiRows) == sub) {
+        static_for<NT>([&](auto jc) {
+          constexpr int j = decltype(jc)::value;
+          static_for<4>([&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            const f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+            *reinterpret_cast<f32x4*>(stage + (lane & (kEpiRows - 1)) * kRowFloats + 32 * j + 8 * q + 4 * (lane >> 5)) = v;
+          });
+        });
+      }
+      const int row0 = 32 * i + kEpiRows * sub;  // first of these rows within the wave tile
+      if (!general && !row_scales) {
+        // scales and bias depend on the column only: two VALU ops per element
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int ne = (n + e) < g.N ? (n + e) : g.N - 1;
-            float t = a[e] * (ra * sa_c[e]);
-            t = t * (rb * sb_c[e]);
-            t += bias_c[e];
-            if (g.bias_mode == MI355Q_BIAS_FULL) t += load_out_as_f32(bias, (int64_t)m * g.ldbias + ne, g.out_bf16);
-            if (D) t += load_out_as_f32(D, (int64_t)m * g.ldd + ne, g.out_bf16);
-            v[e] = t;
+        for (int r = r_in; r < kEpiRows; r += kRowsPerPass) {
+          const f32x4 a = *reinterpret_cast<const f32x4*>(stage + r * kRowFloats + (lane % kLanesPerRow) * 4);
+          const int m = m_wave + row0 + r;
+          if (m < g.M && n < g.N) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              float t = a[e] * sa_c[e];
+              t = t * sb_c[e];
+              v[e] = t + bias_c[e];
+            }
+            store_row4(m, v);
           }
-          store_row4(m, v);
+        }
+      } else if (!general) {
+#pragma unroll
+        for (int r = r_in; r < kEpiRows; r += kRowsPerPass) {
+          const f32x4 a = *reinterpret_cast<const f32x4*>(stage + r * kRowFloats + (lane % kLanesPerRow) * 4);
+          const float ra = row_sa[row0 + r], rb = row_sb[row0 + r];
+          const int m = m_wave + row0 + r;
+          if (m < g.M && n < g.N) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              // one of (ra, sa_c) is exactly 1, likewise (rb, sb_c): the products are the scales themselves
+              float t = a[e] * (ra * sa_c[e]);
+              t = t * (rb * sb_c[e]);
+              v[e] = t + bias_c[e];
+            }
+            store_row4(m, v);
+          }
+        }
+      } else {
+#pragma unroll 1
+        for (int r = r_in; r < kEpiRows; r += kRowsPerPass) {
+          const f32x4 a = *reinterpret_cast<const f32x4*>(stage + r * kRowFloats + (lane % kLanesPerRow) * 4);
+          const float ra = row_scales ? row_sa[row0 + r] : 1.0f, rb = row_scales ? row_sb[row0 + r] : 1.0f;
+          const int m = m_wave + row0 + r;
+          if (m < g.M && n < g.N) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int ne = (n + e) < g.N ? (n + e) : g.N - 1;
+              float t = a[e] * (ra * sa_c[e]);
+              t = t * (rb * sb_c[e]);
+              t += bias_c[e];
+              if (g.bias_mode == MI355Q_BIAS_FULL) t += load_out_as_f32(bias, (int64_t)m * g.ldbias + ne, g.out_bf16);
+              if (D) t += load_out_as_f32(D, (int64_t)m * g.ldd + ne, g.out_bf16);
+              v[e] = t;
+            }
+            store_row4(m, v);
+          }
         }
       }
     }
   });
 }
 
-// Per-wave state of the K loop: accumulators, two sets of fragments, loaders.
+// Per-wave state of the K loop: accumulators, fragments, loaders.
+//
+// Register budget.  Two waves per SIMD leave 256 registers per lane: 128 hold
+// the accumulators of the (BM/2) x (BN/4) wave tile, so the fragments get 64:
+// the B fragments are double-buffered (the next half-step's set is read while
+// the current one is in use), the A fragments are single-buffered and rolled:
+// MFMAs run row by row, A_i is dead after the last MFMA of row i, and the next
+// half-step's A_i is read into the same registers right then.
 template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
 struct TileCore {
-  static constexpr int TM = BM / 2, TN = BN / 2;
+  static constexpr int TM = BM / kWavesM, TN = BN / kWavesN;
   static constexpr int MT = TM / 32, NT = TN / 32;
   f32x16 acc[MT][NT];
-  i32x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];
+  i32x8 fa[MT], fb0[NT], fb1[NT];
   DmaLoader<A_KMAJOR, BM> la;
   DmaLoader<B_KMAJOR, BN> lb;
   int wm, wn, K;
 
-  __device__ __forceinline__ void init(const GemmArgs& g, int64_t batch, int m0, int n0, int wm_, int wn_) {
+  __device__ __forceinline__ void init(const GemmArgs& g, int wm_, int wn_) {
     wm = wm_;
     wn = wn_;
     K = g.K;
+  }
+
+  __device__ __forceinline__ void zero_acc() {
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
       for (int j = 0; j < NT; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-    la.init(g.A + batch * g.stride_a, g.lda, m0, g.M, g.K);
-    lb.init(g.B + batch * g.stride_b, g.ldb, n0, g.N, g.K);
   }
 
-  static constexpr int kPartsA = frag_parts<A_KMAJOR>(), kPartsB = frag_parts<B_KMAJOR>();
-  static constexpr int kReadOps = MT * kPartsA + NT * kPartsB;  // LDS reads per half-step
-  static constexpr int kMfmas = MT * NT;
-  static constexpr int kDmaOps = DmaLoader<A_KMAJOR, BM>::kPerWave + DmaLoader<B_KMAJOR, BN>::kPerWave;
-
-  // Read op OP of a half-step, in the order the next MFMA block needs the
-  // fragments: A0, B0 .. B(NT-1), A1 .. A(MT-1).
-  template <int OP>
-  __device__ __forceinline__ void read_op(const uint8_t* stage, int ks, i32x8 (&fa)[MT], i32x8 (&fb)[NT]) {
-    if constexpr (OP < kPartsA) {
-      read_fragment_part<A_KMAJOR, BM, OP>(stage, wm, ks, fa[0]);
-    } else if constexpr (OP < kPartsA + NT * kPartsB) {
-      constexpr int o = OP - kPartsA;
-      read_fragment_part<B_KMAJOR, BN, o % kPartsB>(stage + BM * kBK, wn + (o / kPartsB) * 32, ks, fb[o / kPartsB]);
-    } else {
-      constexpr int o = OP - kPartsA - NT * kPartsB;
-      read_fragment_part<A_KMAJOR, BM, o % kPartsA>(stage, wm + (1 + o / kPartsA) * 32, ks, fa[1 + o / kPartsA]);
+  // Points the loaders at tile (m0, n0); `valid` false makes every load of the
+  // tile fall outside the descriptors (used past the workgroup's last tile).
+  __device__ __forceinline__ void retarget(const GemmArgs& g, int64_t batch, int m0, int n0, bool valid) {
+    la.init(g.A + batch * g.stride_a, g.lda, m0, g.M, g.K);
+    lb.init(g.B + batch * g.stride_b, g.ldb, n0, g.N, g.K);
+    if (!valid) {
+      la.rsrc[2] = 0;
+      lb.rsrc[2] = 0;
     }
   }
 
-  __device__ __forceinline__ void read_frags(const uint8_t* __restrict__ stage, int ks, i32x8 (&fa)[MT],
-                                             i32x8 (&fb)[NT]) {
-    static_for<kReadOps>([&](auto oc) { read_op<decltype(oc)::value>(stage, ks, fa, fb); });
+  static constexpr int kPartsA = frag_parts<A_KMAJOR>(), kPartsB = frag_parts<B_KMAJOR>();
+  static constexpr int kMfmas = MT * NT;
+  static constexpr int kDmaOps = DmaLoader<A_KMAJOR, BM>::kPerWave + DmaLoader<B_KMAJOR, BN>::kPerWave;
+
+  template <int I, int PART>
+  __device__ __forceinline__ void read_a(const uint8_t* stage, int ks) {
+    read_fragment_part<A_KMAJOR, BM, PART>(stage, wm + I * 32, ks, fa[I]);
+  }
+  template <int J, int PART>
+  __device__ __forceinline__ void read_b(const uint8_t* stage, int ks, i32x8 (&fb)[NT]) {
+    read_fragment_part<B_KMAJOR, BN, PART>(stage + BM * kBK, wn + J * 32, ks, fb[J]);
   }
 
   template <int OP>
@@ -448,25 +487,23 @@ struct TileCore {
     lb.advance();
   }
 
-  // One MFMA block (every tile of the wave, 64 k) on the fragments (ca, cb),
-  // with the LDS reads of the next block's fragments (na, nb) and, when
-  // WITH_DMA, this wave's global->LDS loads of a later stage dealt out between
-  // the MFMAs.  The matrix pipe is busy 16 passes per MFMA; the reads and loads
-  // issue in its shadow.  sched_barrier(0) after each group pins the written
-  // order (left alone, the scheduler gathers the reads after the MFMAs).
+  // One MFMA block (every tile of the wave, 64 k) on the fragments (fa, cb),
+  // with the LDS reads of the next block's fragments and, when WITH_DMA, this
+  // wave's global->LDS loads of a later stage dealt out between the MFMAs.
+  // sched_barrier(0) after each group pins the written order (left alone, the
+  // scheduler gathers the reads after the MFMAs).
   template <bool WITH_DMA>
-  __device__ __forceinline__ void block(const i32x8 (&ca)[MT], const i32x8 (&cb)[NT], i32x8 (&na)[MT],
-                                        i32x8 (&nb)[NT], const uint8_t* __restrict__ rd_stage, int rd_ks,
+  __device__ __forceinline__ void block(const i32x8 (&cb)[NT], i32x8 (&nb)[NT],
+                                        const uint8_t* __restrict__ rd_stage, int rd_ks,
                                         uint8_t* __restrict__ dma_stage, int dma_kt) {
-    // all reads within the first 3/4 of the MFMAs, so that they have landed when the next block starts
-    constexpr int kReadGroups = (kMfmas * 3 + 3) / 4;
-    constexpr int kReadsPerGroup = (kReadOps + kReadGroups - 1) / kReadGroups;
+    constexpr int kBOps = NT * kPartsB;
+    constexpr int kBPerGroup = (kBOps + kMfmas - 1) / kMfmas;
     constexpr int kDmaPerGroup = (kDmaOps + kMfmas - 1) / kMfmas;
     static_for<kMfmas>([&](auto gc) {
       constexpr int gi = decltype(gc)::value;
       constexpr int i = gi / NT, j = gi % NT;
       acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-          cb[j], ca[i], acc[i][j], mfma_code<FMT_B>(), mfma_code<FMT_A>(), 0, 0, 0, 0);
+          cb[j], fa[i], acc[i][j], mfma_code<FMT_B>(), mfma_code<FMT_A>(), 0, 0, 0, 0);
       if constexpr (WITH_DMA) {
         static_for<kDmaPerGroup>([&](auto dc) {
           constexpr int op = gi * kDmaPerGroup + decltype(dc)::value;
@@ -475,12 +512,16 @@ struct TileCore {
 #endif
         });
       }
-      static_for<kReadsPerGroup>([&](auto rc) {
-        constexpr int op = gi * kReadsPerGroup + decltype(rc)::value;
 #ifndef MI355Q_DBG_SKIP_READS
-        if constexpr (op < kReadOps) read_op<op>(rd_stage, rd_ks, na, nb);
-#endif
+      static_for<kBPerGroup>([&](auto rc) {
+        constexpr int op = gi * kBPerGroup + decltype(rc)::value;
+        if constexpr (op < kBOps) read_b<op / kPartsB, op % kPartsB>(rd_stage, rd_ks, nb);
       });
+      if constexpr (j == NT - 1) {
+        // row i of MFMAs is done: its A fragment is dead, fetch the next half-step's
+        static_for<kPartsA>([&](auto pc) { read_a<i, decltype(pc)::value>(rd_stage, rd_ks); });
+      }
+#endif
       __builtin_amdgcn_sched_barrier(0);
     });
     if constexpr (WITH_DMA) {
@@ -494,16 +535,29 @@ struct TileCore {
   // the barrier every wave sees every wave's share of the stage.
   __device__ __forceinline__ static void wait_loads_then_barrier() {
 #ifndef MI355Q_DBG_SKIP_BARRIER
+#ifdef MI355Q_DBG_NO_VMWAIT
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0) only: timing experiment, results are wrong
+#else
     __builtin_amdgcn_s_waitcnt(0);
+#endif
     __syncthreads();
 #endif
   }
 
-  __device__ __forceinline__ void prologue(uint8_t* __restrict__ s0, uint8_t* __restrict__ s1) {
-    issue_stage(s0, 0);
-    issue_stage(s1, 1);
+  // First fragments of a tile whose stages 0 and 1 have been issued.
+  __device__ __forceinline__ void first_fragments(uint8_t* __restrict__ s0) {
     wait_loads_then_barrier();
-    read_frags(s0, 0, fa0, fb0);
+    static_for<MT>([&](auto ic) {
+      static_for<kPartsA>([&](auto pc) { read_a<decltype(ic)::value, decltype(pc)::value>(s0, 0); });
+    });
+    static_for<NT>([&](auto jc) {
+      static_for<kPartsB>([&](auto pc) { read_b<decltype(jc)::value, decltype(pc)::value>(s0, 0, fb0); });
+    });
+#ifdef MI355Q_DBG_SKIP_READS
+    static_for<NT>([&](auto jc) {
+      static_for<kPartsB>([&](auto pc) { read_b<decltype(jc)::value, decltype(pc)::value>(s0, 1, fb1); });
+    });
+#endif
   }
 
   // Two K stages: stage kt sits in s0, stage kt+1 in s1 (or is still landing
@@ -511,75 +565,102 @@ struct TileCore {
   // consumed, so the stage two ahead starts to overwrite it while the second
   // half of the current stage and the whole next stage compute.
   __device__ __forceinline__ void k_pair(uint8_t* __restrict__ s0, uint8_t* __restrict__ s1, int kt) {
-    block<false>(fa0, fb0, fa1, fb1, s0, 1, nullptr, 0);
+    block<false>(fb0, fb1, s0, 1, nullptr, 0);
     wait_loads_then_barrier();
-    block<true>(fa1, fb1, fa0, fb0, s1, 0, s0, kt + 2);
-    block<false>(fa0, fb0, fa1, fb1, s1, 1, nullptr, 0);
+    block<true>(fb1, fb0, s1, 0, s0, kt + 2);
+    block<false>(fb0, fb1, s1, 1, nullptr, 0);
     wait_loads_then_barrier();
-    block<true>(fa1, fb1, fa0, fb0, s0, 0, s1, kt + 3);
+    block<true>(fb1, fb0, s0, 0, s1, kt + 3);
   }
 };
 
-template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
-__global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g) {
-  constexpr int TM = BM / 2, TN = BN / 2;   // per-wave tile
-  constexpr int MT = TM / 32, NT = TN / 32; // MFMA tiles per wave
-  static_assert(BM == BN, "the epilogue staging area assumes square tiles");
-  constexpr int kStageBytes = (BM + BN) * kBK;
-  // Two stages as two separate arrays, so that loads into one and reads from
-  // the other are provably disjoint.
-  __shared__ __attribute__((aligned(1024))) uint8_t lds0[kStageBytes];
-  __shared__ __attribute__((aligned(1024))) uint8_t lds1[kStageBytes];
-
-  // Tile order.  Workgroups are dealt to the 8 XCDs round-robin by id; give
-  // each XCD a contiguous range of tiles, and walk tiles in column groups of
-  // kGroupM rows so that the tiles resident on one XCD share A and B panels in
-  // its L2.
-  const int nb = gridDim.x;
-  const int bid = blockIdx.x;
-  const int per = nb >> 3, rem = nb & 7;
-  const int xcd = bid & 7, idx = bid >> 3;
-  const int logical = xcd < rem ? xcd * (per + 1) + idx : rem * (per + 1) + (xcd - rem) * per + idx;
+// Logical tile index -> (tile_m, tile_n), walking the tile grid in column
+// groups of kGroupM rows so that consecutive indices share A and B panels.
+__device__ __forceinline__ void tile_coords(int logical, int tiles_m, int tiles_n, int* tile_m, int* tile_n) {
   constexpr int kGroupM = 8;
-  const int group_size = kGroupM * g.tiles_n;
+  const int group_size = kGroupM * tiles_n;
   const int grp = logical / group_size;
   const int first_m = grp * kGroupM;
-  const int gm = (g.tiles_m - first_m) < kGroupM ? (g.tiles_m - first_m) : kGroupM;
+  const int gm = (tiles_m - first_m) < kGroupM ? (tiles_m - first_m) : kGroupM;
   const int in_grp = logical - grp * group_size;
-  const int tile_m = first_m + in_grp % gm;
-  const int tile_n = in_grp / gm;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  *tile_m = first_m + in_grp % gm;
+  *tile_n = in_grp / gm;
+}
+
+// Persistent kernel: gridDim.x workgroups (at most one per CU) each walk a list
+// of tiles.  Workgroups are dealt to the 8 XCDs round-robin by id; each XCD owns
+// a contiguous range of the tile order, and in round r its workgroups take the
+// next gridDim.x / 8 tiles of that range, so that the tiles in flight on one
+// XCD form a compact patch that shares A and B panels in its L2.
+template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
+__global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g) {
+  constexpr int TM = BM / kWavesM, TN = BN / kWavesN;   // per-wave tile
+  constexpr int MT = TM / 32, NT = TN / 32;             // MFMA tiles per wave
+  constexpr int kStageBytes = (BM + BN) * kBK;
+  // Two stages as two separate arrays, so that loads into one and reads from
+  // the other are provably disjoint; the epilogue has its own staging area.
+  __shared__ __attribute__((aligned(1024))) uint8_t lds0[kStageBytes];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds1[kStageBytes];
+  __shared__ __attribute__((aligned(16))) float lds_epi[kWaves * epilogue_stage_floats<MT, NT>()];
+
+  const int nb = gridDim.x, bid = blockIdx.x;
+  const int tiles = g.tiles_m * g.tiles_n;
+  const int xcd = bid & 7, slot = bid >> 3;
+  const int slots = (nb - xcd + 7) >> 3;              // workgroups on this XCD
+  const int per = tiles >> 3, rem = tiles & 7;
+  const int first = xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per;
+  const int count = per + (xcd < rem ? 1 : 0);        // tiles of this XCD
 
   const int64_t batch = blockIdx.y;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = (wave >> 1) * TM, wn = (wave & 1) * TN;
+  const int wave = threadIdx.x >> 6;
+  const int wm = (wave / kWavesN) * TM, wn = (wave % kWavesN) * TN;
+  float* stage = lds_epi + wave * epilogue_stage_floats<MT, NT>();
 
   TileCore<BM, BN, A_KMAJOR, B_KMAJOR, FMT_A, FMT_B> core;
-  core.init(g, batch, m0, n0, wm, wn);
+  core.init(g, wm, wn);
   const int KT = (g.K + kBK - 1) / kBK;
+  const int KT2 = (KT + 1) & ~1;
 
   // Stages at or beyond K are loaded all the same: they fall outside the buffer
-  // descriptors and arrive as zeros.  The loop therefore runs an even number of
-  // branch-free steps, and an odd stage count costs one step of zero products
-  // instead of a second copy of the MFMA block.
-  core.prologue(lds0, lds1);
-  for (int kt = 0; kt < KT; kt += 2) core.k_pair(lds0, lds1, kt);
-  core.wait_loads_then_barrier();
-
-  // The operand tiles are dead (barrier above): the epilogue reuses the stage
-  // arrays for the per-wave fp32 copies, two waves per array.
-  constexpr int kWaveStageBytes = 32 * (32 * NT + 4) * 4 + 2 * 32 * MT * 4;  // fp32 copy + per-row scales
-  static_assert(kStageBytes >= 2 * kWaveStageBytes, "epilogue staging does not fit");
-  float* stage = reinterpret_cast<float*>((wave < 2 ? lds0 : lds1) + (wave & 1) * kWaveStageBytes);
+  // descriptors and arrive as zeros.  The K loop therefore runs an even number
+  // of branch-free steps, and an odd stage count costs one step of zero
+  // products instead of a second copy of the MFMA block.  The loads that the
+  // last two steps of a tile issue are the first two stages of the workgroup's
+  // next tile, which land while the epilogue runs.
+  int idx = slot;
+  if (idx >= count) return;
+  int tile_m, tile_n;
+  tile_coords(first + idx, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+  core.retarget(g, batch, tile_m * BM, tile_n * BN, true);
+  core.issue_stage(lds0, 0);
+  core.issue_stage(lds1, 1);
+  for (;;) {
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    core.zero_acc();
+    core.first_fragments(lds0);
+    for (int kt = 0; kt < KT2; kt += 2) {
+      if (kt + 2 == KT2) {
+        idx += slots;
+        const bool more = idx < count;
+        if (more) tile_coords(first + idx, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+        core.retarget(g, batch, tile_m * BM, tile_n * BN, more);
+      }
+      // stage numbers restart at 0 for the next tile
+      core.k_pair(lds0, lds1, kt + 2 == KT2 ? -2 : kt);
+    }
 #ifdef MI355Q_DBG_SKIP_EPILOGUE
-  {
-    float t = 0.f;
-    for (int i = 0; i < MT; ++i) for (int j = 0; j < NT; ++j) for (int e = 0; e < 16; ++e) t += core.acc[i][j][e];
-    if (t == 12345.678f) reinterpret_cast<float*>(g.C)[0] = t;
-  }
+    {
+      float t = 0.f;
+      for (int i = 0; i < MT; ++i) for (int j = 0; j < NT; ++j) for (int e = 0; e < 16; ++e) t += core.acc[i][j][e];
+      if (t == 12345.678f) reinterpret_cast<float*>(g.C)[0] = t;
+    }
 #else
-  epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
+    epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
 #endif
+    if (idx >= count) break;
+  }
+  // drain the (out-of-range) loads issued for the tile that does not exist
+  __builtin_amdgcn_s_waitcnt(0);
 }
 
 template <int BM, int BN, bool AK, bool BK_, int FA, int FB>
@@ -587,7 +668,9 @@ void launch_tile(const GemmArgs& g, int64_t batch, hipStream_t st) {
   GemmArgs a = g;
   a.tiles_m = (g.M + BM - 1) / BM;
   a.tiles_n = (g.N + BN - 1) / BN;
-  dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch);
+  const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
+  const int cus = compute_units();
+  dim3 grid((unsigned)(tiles < cus ? tiles : cus), (unsigned)batch);
   fp8_gemm_tile_kernel<BM, BN, AK, BK_, FA, FB><<<grid, kGemmThreads, 0, st>>>(a);
 }
 
