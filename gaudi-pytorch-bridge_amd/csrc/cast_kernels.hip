@@ -15,20 +15,31 @@ constexpr int kThreads = 256;
 
 __global__ void fill_u32_kernel(uint32_t* p, uint32_t v) { *p = v; }
 
+// Kernels that reduce an amax run as at most kAmaxBlocks fat workgroups that
+// stride over the data: the number of same-address atomics, not the streaming,
+// is what bounds them otherwise (2048 blocks: ~30 us; 256 blocks: ~7 us for
+// 32 MiB).
+constexpr int kAmaxThreads = 1024;
+constexpr int kAmaxBlocks = 256;
+
 // Block-level max of abs-value bit patterns, then one atomicMax per block.
 // Bit patterns of non-negative floats order like the floats, and a NaN
 // pattern is larger than Inf, so NaN wins and the result reads back as NaN.
 __device__ __forceinline__ void block_amax_commit(uint32_t m, uint32_t* amax) {
-  __shared__ uint32_t wave_part[kThreads / 64];
+  __shared__ uint32_t wave_part[16];
   m = wave_max_u32(m);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (lane == 0) wave_part[wave] = m;
   __syncthreads();
   if (threadIdx.x == 0) {
     uint32_t r = wave_part[0];
-#pragma unroll
-    for (int w = 1; w < kThreads / 64; ++w) r = r > wave_part[w] ? r : wave_part[w];
-    if (r != 0) atomicMax(amax, r);
+    const int nwaves = (int)(blockDim.x >> 6);
+    for (int w = 1; w < nwaves; ++w) r = r > wave_part[w] ? r : wave_part[w];
+    // Atomics on one address serialise in L2.  The running maximum only grows,
+    // so a block whose maximum does not beat the value already there has
+    // nothing to add: read it first (device-scope load, not from L1) and skip
+    // the atomic.  After the first few blocks almost every block skips.
+    if (r != 0 && r > __hip_atomic_load(amax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(amax, r);
   }
 }
 
@@ -42,13 +53,18 @@ __device__ __forceinline__ void block_amax_commit(uint32_t m, uint32_t* amax) {
 //   SK_COL     scale[column]
 //   SK_FULL    scale[element]
 template <bool BF16_IN, int FMT, int SK, bool AMAX, int U>
-__global__ __launch_bounds__(kThreads) void cast_to_fp8_vec8(
+__global__ __launch_bounds__(AMAX ? kAmaxThreads : kThreads) void cast_to_fp8_vec8(
     const uint8_t* __restrict__ x, uint8_t* __restrict__ y, const float* __restrict__ scale,
     float scale_host, int scale_is_dev, int64_t vec_per_row, int64_t blocks_per_row,
-    int64_t mid, uint32_t* __restrict__ amax) {
-  const int64_t row = blockIdx.x / blocks_per_row;
-  const int64_t bir = blockIdx.x - row * blocks_per_row;
-  const int64_t v0 = bir * (int64_t)(kThreads * U) + threadIdx.x;
+    int64_t total_blocks, int64_t mid, uint32_t* __restrict__ amax) {
+  constexpr int THREADS = AMAX ? kAmaxThreads : kThreads;
+  uint32_t am = 0;
+  // a logical block is THREADS * U consecutive vectors of one row; without amax
+  // the grid holds one workgroup per logical block and this loop runs once
+  for (int64_t lb = blockIdx.x; lb < total_blocks; lb += gridDim.x) {
+  const int64_t row = lb / blocks_per_row;
+  const int64_t bir = lb - row * blocks_per_row;
+  const int64_t v0 = bir * (int64_t)(THREADS * U) + threadIdx.x;
   const int64_t row_base = row * vec_per_row;
 
   float s = 1.0f;
@@ -61,7 +77,7 @@ __global__ __launch_bounds__(kThreads) void cast_to_fp8_vec8(
   bool ok[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    const int64_t vr = v0 + (int64_t)u * kThreads;
+    const int64_t vr = v0 + (int64_t)u * THREADS;
     ok[u] = vr < vec_per_row;
     if (ok[u]) {
       const u32x4* p = reinterpret_cast<const u32x4*>(x + (row_base + vr) * IN_BYTES);
@@ -70,11 +86,10 @@ __global__ __launch_bounds__(kThreads) void cast_to_fp8_vec8(
     }
   }
 
-  uint32_t am = 0;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (!ok[u]) continue;
-    const int64_t vr = v0 + (int64_t)u * kThreads;
+    const int64_t vr = v0 + (int64_t)u * THREADS;
     float v[8];
     if constexpr (BF16_IN) {
 #pragma unroll
@@ -125,6 +140,7 @@ __global__ __launch_bounds__(kThreads) void cast_to_fp8_vec8(
     out.y = cvt_fp8x4<FMT>(v[4], v[5], v[6], v[7]);
     __builtin_nontemporal_store(out, reinterpret_cast<u32x2*>(y + (row_base + vr) * 8));
   }
+  }
 
   if constexpr (AMAX) {
     if constexpr (BF16_IN) {
@@ -166,19 +182,20 @@ __global__ __launch_bounds__(kThreads) void cast_to_fp8_generic(
 
 // ---------------------------------------------------------------------- amax
 template <bool BF16_IN, int U>
-__global__ __launch_bounds__(kThreads) void amax_vec(const uint8_t* __restrict__ x, int64_t nvec,
-                                                     uint32_t* __restrict__ amax) {
-  // vectors of 16 bytes
-  const int64_t v0 = (int64_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+__global__ __launch_bounds__(kAmaxThreads) void amax_vec(const uint8_t* __restrict__ x, int64_t nvec,
+                                                         uint32_t* __restrict__ amax) {
+  // vectors of 16 bytes; the grid strides over the data
+  uint32_t am = 0;
+  const int64_t stride = (int64_t)gridDim.x * kAmaxThreads;
+  for (int64_t v0 = (int64_t)blockIdx.x * kAmaxThreads + threadIdx.x; v0 < nvec; v0 += stride * U) {
   u32x4 in[U];
   bool ok[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    const int64_t v = v0 + (int64_t)u * kThreads;
+    const int64_t v = v0 + (int64_t)u * stride;
     ok[u] = v < nvec;
     if (ok[u]) in[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x) + v);
   }
-  uint32_t am = 0;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (!ok[u]) continue;
@@ -193,6 +210,7 @@ __global__ __launch_bounds__(kThreads) void amax_vec(const uint8_t* __restrict__
         am = am > a ? am : a;
       }
     }
+  }
   }
   if constexpr (BF16_IN) {
     const uint32_t lo = am & 0xffffu, hi = am >> 16;
@@ -404,23 +422,27 @@ inline bool plan_vectors(int mode, int64_t outer, int64_t mid, int64_t inner, in
   }
 }
 
+constexpr int kCastU = 4;  // 16-byte loads in flight per thread
+
 template <bool BF16_IN, int FMT, bool AMAX>
-void launch_cast_to_vec(int sk, unsigned grid, hipStream_t st, const uint8_t* x, uint8_t* y,
-                        const float* scale, float sh, int is_dev, int64_t vpr, int64_t bpr,
-                        int64_t mid, uint32_t* amax) {
-  constexpr int U = 4;
+void launch_cast_to_vec(int sk, hipStream_t st, const uint8_t* x, uint8_t* y, const float* scale,
+                        float sh, int is_dev, int64_t vpr, int64_t bpr, int64_t total, int64_t mid,
+                        uint32_t* amax) {
+  constexpr int U = kCastU;
+  constexpr int T = AMAX ? kAmaxThreads : kThreads;
+  const unsigned grid = (unsigned)(AMAX && total > kAmaxBlocks ? kAmaxBlocks : total);
   switch (sk) {
     case SK_SCALAR:
-      cast_to_fp8_vec8<BF16_IN, FMT, SK_SCALAR, AMAX, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, mid, amax);
+      cast_to_fp8_vec8<BF16_IN, FMT, SK_SCALAR, AMAX, U><<<grid, T, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, total, mid, amax);
       break;
     case SK_ROW:
-      cast_to_fp8_vec8<BF16_IN, FMT, SK_ROW, AMAX, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, mid, amax);
+      cast_to_fp8_vec8<BF16_IN, FMT, SK_ROW, AMAX, U><<<grid, T, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, total, mid, amax);
       break;
     case SK_COL:
-      cast_to_fp8_vec8<BF16_IN, FMT, SK_COL, AMAX, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, mid, amax);
+      cast_to_fp8_vec8<BF16_IN, FMT, SK_COL, AMAX, U><<<grid, T, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, total, mid, amax);
       break;
     default:
-      cast_to_fp8_vec8<BF16_IN, FMT, SK_FULL, AMAX, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, mid, amax);
+      cast_to_fp8_vec8<BF16_IN, FMT, SK_FULL, AMAX, U><<<grid, T, 0, st>>>(x, y, scale, sh, is_dev, vpr, bpr, total, mid, amax);
       break;
   }
 }
@@ -428,8 +450,7 @@ void launch_cast_to_vec(int sk, unsigned grid, hipStream_t st, const uint8_t* x,
 template <bool BF16_IN, int FMT>
 int cast_to_dispatch(const uint8_t* x, uint8_t* y, const float* scale, float sh, int mode,
                      int64_t outer, int64_t mid, int64_t inner, uint32_t* amax, hipStream_t st) {
-  constexpr int U = 4;
-  constexpr int IN_BYTES = BF16_IN ? 16 : 32;
+  constexpr int U = kCastU;
   const int64_t n = outer * mid * inner;
   VecPlan p;
   const bool vec = aligned(x, 16) && aligned(y, 8) &&
@@ -440,15 +461,15 @@ int cast_to_dispatch(const uint8_t* x, uint8_t* y, const float* scale, float sh,
     // In flat modes the row length need not be a multiple of 8: the tail goes
     // to the generic kernel.  In 2-D modes plan_vectors has required it.
     if (vpr > 0) {
-      const int64_t bpr = (vpr + kThreads * U - 1) / (kThreads * U);
-      const int64_t grid = bpr * p.rows;
-      if (grid > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+      const int64_t per_block = (int64_t)(amax ? kAmaxThreads : kThreads) * U;
+      const int64_t bpr = (vpr + per_block - 1) / per_block;
+      const int64_t total = bpr * p.rows;
+      if (total > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
       const int is_dev = mode == MI355Q_SCALE_DEV;
-      if (amax) launch_cast_to_vec<BF16_IN, FMT, true>(p.sk, (unsigned)grid, st, x, y, scale, sh, is_dev, vpr, bpr, p.mid, amax);
-      else launch_cast_to_vec<BF16_IN, FMT, false>(p.sk, (unsigned)grid, st, x, y, scale, sh, is_dev, vpr, bpr, p.mid, amax);
+      if (amax) launch_cast_to_vec<BF16_IN, FMT, true>(p.sk, st, x, y, scale, sh, is_dev, vpr, bpr, total, p.mid, amax);
+      else launch_cast_to_vec<BF16_IN, FMT, false>(p.sk, st, x, y, scale, sh, is_dev, vpr, bpr, total, p.mid, amax);
       done = p.rows == 1 ? vpr * 8 : n;
     }
-    (void)IN_BYTES;
   }
   if (done < n) {
     const int64_t rest = n - done;
@@ -530,10 +551,10 @@ int mi355q_amax(const void* x, int x_dtype, int64_t n, float* amax_out, void* st
   if (aligned(x, 16)) {
     const int64_t nvec = n * es / 16;
     if (nvec > 0) {
-      const int64_t grid = (nvec + kThreads * U - 1) / (kThreads * U);
-      if (grid > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
-      if (x_dtype == MI355Q_BF16) amax_vec<true, U><<<(unsigned)grid, kThreads, 0, st>>>(xb, nvec, am);
-      else amax_vec<false, U><<<(unsigned)grid, kThreads, 0, st>>>(xb, nvec, am);
+      int64_t grid = (nvec + kAmaxThreads * U - 1) / (kAmaxThreads * U);
+      if (grid > kAmaxBlocks) grid = kAmaxBlocks;
+      if (x_dtype == MI355Q_BF16) amax_vec<true, U><<<(unsigned)grid, kAmaxThreads, 0, st>>>(xb, nvec, am);
+      else amax_vec<false, U><<<(unsigned)grid, kAmaxThreads, 0, st>>>(xb, nvec, am);
       done = nvec * (16 / es);
     }
   }
