@@ -98,8 +98,15 @@ def c1_input(gen, rows=4096, cols=4096):
     return x.bfloat16()
 
 
-def bench_cast(ops, oracle, dev, steps, warmup, cpu):
-    """BASELINE config 1: amax pass, cast_to_fp8_v2 (scale given), cast_from_fp8."""
+def bench_cast(pkg, oracle, dev, steps, warmup, cpu):
+    """BASELINE config 1: amax pass, cast_to_fp8_v2 (scale given), cast_from_fp8.
+
+    These kernels run for about ten microseconds, less than the host needs to
+    dispatch a torch op, so they are timed through the C ABI (ctypes, outputs
+    allocated up front): the figure is the kernels' rate, not the dispatcher's.
+    """
+    import ctypes
+    lib = pkg.capi()
     out = []
     gen = torch.Generator().manual_seed(SEED)
     x = c1_input(gen)
@@ -108,23 +115,32 @@ def bench_cast(ops, oracle, dev, steps, warmup, cpu):
     scale = (448.0 / amax).reshape(())
     sets = n_sets(3 * n)
     xs = [x.to(dev).clone() for _ in range(sets)]
+    y8 = [torch.empty(x.shape, dtype=E4, device=dev) for _ in range(sets)]
+    yb = [torch.empty(x.shape, dtype=torch.bfloat16, device=dev) for _ in range(sets)]
+    am = torch.zeros((), device=dev)
     sd, sinv = scale.to(dev), scale.reciprocal().to(dev)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     cores = torch.get_num_threads()
 
-    ms = time_gpu(lambda i: torch.ops.mi355q.amax(xs[i % sets]), steps, warmup)
+    def ok(status):
+        if status != 0:
+            raise RuntimeError(lib.mi355q_status_string(status).decode())
+
+    ms = time_gpu(lambda i: ok(lib.mi355q_amax(xs[i % sets].data_ptr(), pkg.BF16, n, am.data_ptr(), st)), steps, warmup)
+    assert am.cpu() == amax
     c = None
     if cpu:
         t = time_cpu(lambda: x.abs().max().float())
         c = {"value": round(2 * n / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
              "sample": "full 4096x4096 bf16 tensor, x.abs().max()"}
-    out.append(hbm_entry("amax", "C1a amax of bf16 [4096,4096]", 2 * n, ms, steps, "amax_vec<bf16>", c))
+    out.append(hbm_entry("amax", "C1a amax of bf16 [4096,4096]", 2 * n, ms, steps, "fill_u32 + amax_vec<bf16>", c))
 
-    ring = [None] * sets  # keeps the last `sets` outputs alive so that outputs rotate as well
+    def cast_to(i, with_amax):
+        j = i % sets
+        ok(lib.mi355q_cast_to_fp8(xs[j].data_ptr(), pkg.BF16, y8[j].data_ptr(), pkg.E4M3FN, sd.data_ptr(), 0.0,
+                                  pkg.SCALE_DEV, n, 1, 1, am.data_ptr() if with_amax else None, st))
 
-    def keep(i, v):
-        ring[i % sets] = v
-
-    ms = time_gpu(lambda i: keep(i, ops.cast_to_fp8_v2(xs[i % sets], sd, False, False, E4)), steps, warmup)
+    ms = time_gpu(lambda i: cast_to(i, False), steps, warmup)
     c = None
     if cpu:
         t = time_cpu(lambda: oracle.torch_cast_to_fp8(x, scale, E4))
@@ -133,14 +149,13 @@ def bench_cast(ops, oracle, dev, steps, warmup, cpu):
     out.append(hbm_entry("cast_to_fp8_v2", "C1b cast_to_fp8_v2 bf16 [4096,4096] -> e4m3fn, per-tensor scale",
                          3 * n, ms, steps, "cast_to_fp8_vec8<bf16,e4m3fn,scalar>", c))
 
-    ms = time_gpu(lambda i: keep(i, ops.cast_to_fp8_v2(xs[i % sets], sd, False, True, E4)), steps, warmup)
+    ms = time_gpu(lambda i: cast_to(i, True), steps, warmup)
     out.append(hbm_entry("cast_to_fp8_v2+amax", "C1 cast_to_fp8_v2 with is_amax=True (one pass)", 3 * n + 4, ms, steps,
-                         "cast_to_fp8_vec8<bf16,e4m3fn,scalar,amax>"))
+                         "fill_u32 + cast_to_fp8_vec8<bf16,e4m3fn,scalar,amax>"))
 
-    y8 = [ops.cast_to_fp8_v2(xs[i], sd, False, False, E4)[0] for i in range(sets)]
-    del xs
-    ring = [None] * sets
-    ms = time_gpu(lambda i: keep(i, ops.cast_from_fp8(y8[i % sets], sinv, torch.bfloat16)), steps, warmup)
+    ms = time_gpu(lambda i: ok(lib.mi355q_cast_from_fp8(y8[i % sets].data_ptr(), pkg.E4M3FN, yb[i % sets].data_ptr(),
+                                                        pkg.BF16, sinv.data_ptr(), 0.0, pkg.SCALE_DEV, n, 1, 1, st)),
+                  steps, warmup)
     c = None
     if cpu:
         y_cpu = y8[0].cpu()
@@ -149,11 +164,25 @@ def bench_cast(ops, oracle, dev, steps, warmup, cpu):
              "sample": "full 4096x4096 e4m3fn tensor, x8.to(bf16) * s_inv.to(bf16)"}
     out.append(hbm_entry("cast_from_fp8", "C1c cast_from_fp8 e4m3fn [4096,4096] -> bf16", 3 * n, ms, steps,
                          "cast_from_fp8_vec16<e4m3fn,bf16,scalar>", c))
+    del xs, y8, yb
+
+    # the same cast on a tensor 16x larger: the C1 kernels are so short that launch ramp-up
+    # is a visible share of them; this shows the streaming rate without it
+    big = torch.randn(16384, 16384, generator=gen).bfloat16().to(dev) * 3
+    nb = big.numel()
+    big8 = [torch.empty(big.shape, dtype=E4, device=dev) for _ in range(2)]
+    ms = time_gpu(lambda i: ok(lib.mi355q_cast_to_fp8(big.data_ptr(), pkg.BF16, big8[i % 2].data_ptr(), pkg.E4M3FN,
+                                                      sd.data_ptr(), 0.0, pkg.SCALE_DEV, nb, 1, 1, None, st)),
+                  max(steps // 5, 5), 3)
+    out.append(hbm_entry("cast_to_fp8_v2_large", "cast_to_fp8_v2 bf16 [16384,16384] -> e4m3fn (not a BASELINE config)",
+                         3 * nb, ms, max(steps // 5, 5), "cast_to_fp8_vec8<bf16,e4m3fn,scalar>"))
     return out
 
 
-def bench_int4(ops, oracle, dev, steps, warmup, cpu):
-    """BASELINE config 2: K = N = 4096, group 128."""
+def bench_int4(pkg, oracle, dev, steps, warmup, cpu):
+    """BASELINE config 2: K = N = 4096, group 128 (timed through the C ABI, see bench_cast)."""
+    import ctypes
+    lib = pkg.capi()
     out = []
     gen = torch.Generator().manual_seed(SEED)
     K = N = 4096
@@ -165,14 +194,20 @@ def bench_int4(ops, oracle, dev, steps, warmup, cpu):
     b_i = K * N // 2 + s.numel() * 2 + K * N * 2
     sets = n_sets(K * N // 2 + K * N * 2)
     ps = [packed.to(dev).clone() for _ in range(sets)]
+    outs = [torch.empty(K, N, dtype=torch.bfloat16, device=dev) for _ in range(sets)]
     sd, zd = s.to(dev), zp.to(dev)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     cores = torch.get_num_threads()
-    ring = [None] * sets
 
-    def keep(i, v):
-        ring[i % sets] = v
+    def run(i, signed):
+        j = i % sets
+        status = lib.mi355q_dequant_4bit(ps[j].data_ptr(), sd.data_ptr(), None if signed else zd.data_ptr(),
+                                         pkg.ZP_NONE if signed else pkg.ZP_PACKED, int(signed), pkg.BF16, K, N // 8, 128,
+                                         outs[j].data_ptr(), st)
+        if status != 0:
+            raise RuntimeError(lib.mi355q_status_string(status).decode())
 
-    ms = time_gpu(lambda i: keep(i, ops.convert_from_uint4(ps[i % sets], sd, zd, torch.bfloat16)), steps, warmup)
+    ms = time_gpu(lambda i: run(i, False), steps, warmup)
     c = None
     if cpu:
         t = time_cpu(lambda: oracle.torch_dequant_4bit(packed, s, zp, torch.bfloat16, False), max_runs=3)
@@ -180,7 +215,7 @@ def bench_int4(ops, oracle, dev, steps, warmup, cpu):
              "sample": "full K=N=4096 problem, shift/mask unpack + (q - z) * s in torch"}
     out.append(hbm_entry("convert_from_uint4", "C2 convert_from_uint4 K=N=4096 group 128, packed zero-points -> bf16",
                          b_u, ms, steps, "dequant_4bit_kernel<unsigned,bf16,packed zp>", c))
-    ms = time_gpu(lambda i: keep(i, ops.convert_from_int4(ps[i % sets], sd, None, torch.bfloat16)), steps, warmup)
+    ms = time_gpu(lambda i: run(i, True), steps, warmup)
     out.append(hbm_entry("convert_from_int4", "C2 convert_from_int4 K=N=4096 group 128, no zero-point -> bf16",
                          b_i, ms, steps, "dequant_4bit_kernel<signed,bf16,no zp>"))
     return out
@@ -208,14 +243,14 @@ def bench_gemm_c3(ops, oracle, pkg, dev, steps, warmup, cpu):
     variant = pkg.capi().mi355q_fp8_gemm_variant(0, K, 0, N, M, N, K).decode()
     cpu_entry = None
     if cpu:
-        rows = 1024
+        rows = M
         a_cpu, w_cpu, b_cpu = a8[:rows].cpu(), w8.cpu(), bias.cpu()
         sa_c, sw_c = sa_inv.cpu(), sw_inv.cpu()
         t = time_cpu(lambda: oracle.torch_fp8_gemm(a_cpu, False, w_cpu, False, torch.bfloat16, sa_c, sw_c, bias=b_cpu),
-                     min_seconds=8.0, max_runs=3)
+                     min_seconds=10.0, max_runs=5)
         cpu_entry = {"value": round(2.0 * rows * N * K / t / 1e12, 4), "unit": "TFLOP/s",
                      "cores": torch.get_num_threads(), "kind": "port",
-                     "sample": f"first {rows} of 8192 rows of A against the full B: "
+                     "sample": f"the full problem ({rows} rows of A), median of up to 5 runs / 10 s: "
                                "((A8.float() @ B8.float()) * sA * sB + bias).bfloat16()"}
     return {"ms": ms, "tflops": tflops, "flop": flop, "variant": variant, "cpu": cpu_entry}
 
@@ -331,9 +366,9 @@ def main():
 
     ops_out = []
     if "cast" in which:
-        ops_out += bench_cast(ops, oracle, dev, k_stream, w_stream, cpu)
+        ops_out += bench_cast(pkg, oracle, dev, k_stream, w_stream, cpu)
     if "int4" in which:
-        ops_out += bench_int4(ops, oracle, dev, k_stream, w_stream, cpu)
+        ops_out += bench_int4(pkg, oracle, dev, k_stream, w_stream, cpu)
     if "decode" in which:
         ops_out += bench_gemm_decode(ops, oracle, dev, args.steps, args.warmup)
     if "mlp" in which:

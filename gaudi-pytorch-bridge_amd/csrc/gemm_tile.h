@@ -183,9 +183,7 @@ struct DmaLoader {
     {
       constexpr int i = I;
       int vo = voff[i];
-#ifndef MI355Q_DBG_NO_KPRED
       if constexpr (KMAJOR) vo = (k0 + kc[i] < K) ? vo : 0x7fffffff;
-#endif
       const uint32_t dst = lds_base + (uint32_t)((wave * kPerWave + i) * 1024);
       // m0 holds the LDS address of the region; lane l's 16 bytes land at m0 + 16 l.
       // Written as asm so that the compiler, which would otherwise make every later
@@ -507,12 +505,9 @@ struct TileCore {
       if constexpr (WITH_DMA) {
         static_for<kDmaPerGroup>([&](auto dc) {
           constexpr int op = gi * kDmaPerGroup + decltype(dc)::value;
-#ifndef MI355Q_DBG_SKIP_DMA
           if constexpr (op < kDmaOps) dma_op<op>(dma_stage, dma_kt);
-#endif
         });
       }
-#ifndef MI355Q_DBG_SKIP_READS
       static_for<kBPerGroup>([&](auto rc) {
         constexpr int op = gi * kBPerGroup + decltype(rc)::value;
         if constexpr (op < kBOps) read_b<op / kPartsB, op % kPartsB>(rd_stage, rd_ks, nb);
@@ -521,7 +516,6 @@ struct TileCore {
         // row i of MFMAs is done: its A fragment is dead, fetch the next half-step's
         static_for<kPartsA>([&](auto pc) { read_a<i, decltype(pc)::value>(rd_stage, rd_ks); });
       }
-#endif
       __builtin_amdgcn_sched_barrier(0);
     });
     if constexpr (WITH_DMA) {
@@ -534,14 +528,8 @@ struct TileCore {
   // outstanding global->LDS loads: drain them first (vmcnt(0)), so that after
   // the barrier every wave sees every wave's share of the stage.
   __device__ __forceinline__ static void wait_loads_then_barrier() {
-#ifndef MI355Q_DBG_SKIP_BARRIER
-#ifdef MI355Q_DBG_NO_VMWAIT
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0) only: timing experiment, results are wrong
-#else
     __builtin_amdgcn_s_waitcnt(0);
-#endif
     __syncthreads();
-#endif
   }
 
   // First fragments of a tile whose stages 0 and 1 have been issued.
@@ -553,11 +541,6 @@ struct TileCore {
     static_for<NT>([&](auto jc) {
       static_for<kPartsB>([&](auto pc) { read_b<decltype(jc)::value, decltype(pc)::value>(s0, 0, fb0); });
     });
-#ifdef MI355Q_DBG_SKIP_READS
-    static_for<NT>([&](auto jc) {
-      static_for<kPartsB>([&](auto pc) { read_b<decltype(jc)::value, decltype(pc)::value>(s0, 1, fb1); });
-    });
-#endif
   }
 
   // Two K stages: stage kt sits in s0, stage kt+1 in s1 (or is still landing
@@ -648,15 +631,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g)
       // stage numbers restart at 0 for the next tile
       core.k_pair(lds0, lds1, kt + 2 == KT2 ? -2 : kt);
     }
-#ifdef MI355Q_DBG_SKIP_EPILOGUE
-    {
-      float t = 0.f;
-      for (int i = 0; i < MT; ++i) for (int j = 0; j < NT; ++j) for (int e = 0; e < 16; ++e) t += core.acc[i][j][e];
-      if (t == 12345.678f) reinterpret_cast<float*>(g.C)[0] = t;
-    }
-#else
     epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
-#endif
     if (idx >= count) break;
   }
   // drain the (out-of-range) loads issued for the tile that does not exist
