@@ -163,7 +163,13 @@ def bench_cast(pkg, oracle, dev, steps, warmup, cpu):
         c = {"value": round(3 * n / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
              "sample": "full 4096x4096 e4m3fn tensor, x8.to(bf16) * s_inv.to(bf16)"}
     out.append(hbm_entry("cast_from_fp8", "C1c cast_from_fp8 e4m3fn [4096,4096] -> bf16", 3 * n, ms, steps,
-                         "cast_from_fp8_vec16<e4m3fn,bf16,scalar>", c))
+                         "cast_from_fp8_vec<e4m3fn,bf16,scalar>", c))
+    # fp8 -> fp8 is a plain copy (the reference forwards an fp8 input unchanged): the copy
+    # kernel of known size that hardware byte counters are calibrated against
+    ms = time_gpu(lambda i: ok(lib.mi355q_cast_to_fp8(y8[i % sets].data_ptr(), pkg.E4M3FN, yb[i % sets].data_ptr(),
+                                                      pkg.E4M3FN, None, 0.0, pkg.SCALE_NONE, n, 1, 1, None, st)),
+                  steps, warmup)
+    out.append(hbm_entry("copy_fp8", "cast_to_fp8_v2 of an fp8 tensor: copy of 16 MiB", 2 * n, ms, steps, "copy_vec16"))
     del xs, y8, yb
 
     # the same cast on a tensor 16x larger: the C1 kernels are so short that launch ramp-up

@@ -284,12 +284,19 @@ __global__ __launch_bounds__(kThreads) void rowwise_amax_kernel(const uint8_t* _
 
 // -------------------------------------------------------------- cast_from_fp8
 //
-// Vectors of 16 fp8 bytes in, 16 bf16 (2 x 16 B) or 16 fp32 (4 x 16 B) out.
+// A lane produces one 16-byte store: 8 fp8 bytes in for bf16 output, 4 for
+// fp32 output.  A wave's store then covers 1 KiB of whole cache lines; wider
+// loads would leave each lane with several stores that each touch only part
+// of a line, and those partial-line writes cost HBM bandwidth.
+template <bool BF16_OUT>
+constexpr int from_vec() { return BF16_OUT ? 8 : 4; }
+
 template <int FMT, bool BF16_OUT, int SK, int U>
-__global__ __launch_bounds__(kThreads) void cast_from_fp8_vec16(
+__global__ __launch_bounds__(kThreads) void cast_from_fp8_vec(
     const uint8_t* __restrict__ x, uint8_t* __restrict__ y, const float* __restrict__ scale,
     float scale_host, int scale_is_dev, int has_scale, int64_t vec_per_row,
     int64_t blocks_per_row, int64_t mid) {
+  constexpr int V = from_vec<BF16_OUT>();
   const int64_t row = blockIdx.x / blocks_per_row;
   const int64_t bir = blockIdx.x - row * blocks_per_row;
   const int64_t v0 = bir * (int64_t)(kThreads * U) + threadIdx.x;
@@ -300,53 +307,53 @@ __global__ __launch_bounds__(kThreads) void cast_from_fp8_vec16(
   if constexpr (SK == SK_ROW) s = scale[row % mid];
   if constexpr (BF16_OUT) s = round_to_bf16(s);
 
-  u32x4 in[U];
+  uint32_t in[U][V / 4];
   bool ok[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int64_t vr = v0 + (int64_t)u * kThreads;
     ok[u] = vr < vec_per_row;
-    if (ok[u]) in[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x) + row_base + vr);
+    if (ok[u]) {
+      if constexpr (V == 8) {
+        const u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(x) + row_base + vr);
+        in[u][0] = t[0];
+        in[u][1] = t[1];
+      } else {
+        in[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(x) + row_base + vr);
+      }
+    }
   }
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (!ok[u]) continue;
     const int64_t vr = v0 + (int64_t)u * kThreads;
-    float v[16];
+    float v[V];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < V / 4; ++i)
       cvt_f32x4<FMT>(in[u][i], v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
     if (has_scale) {
       if constexpr (SK == SK_COL || SK == SK_FULL) {
-        const int64_t si = (SK == SK_COL ? vr : row_base + vr) * 16;
+        const int64_t si = (SK == SK_COL ? vr : row_base + vr) * V;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < V / 4; ++q) {
           const f32x4 sq = *reinterpret_cast<const f32x4*>(scale + si + 4 * q);
 #pragma unroll
           for (int i = 0; i < 4; ++i) v[4 * q + i] *= BF16_OUT ? round_to_bf16(sq[i]) : sq[i];
         }
       } else {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) v[i] *= s;
+        for (int i = 0; i < V; ++i) v[i] *= s;
       }
     }
+    u32x4* o = reinterpret_cast<u32x4*>(y) + row_base + vr;
     if constexpr (BF16_OUT) {
-      u32x4* o = reinterpret_cast<u32x4*>(y + (row_base + vr) * 32);
-      u32x4 o0, o1;
+      u32x4 t;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        o0[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
-        o1[i] = pack_bf16x2(v[8 + 2 * i], v[8 + 2 * i + 1]);
-      }
-      __builtin_nontemporal_store(o0, o);
-      __builtin_nontemporal_store(o1, o + 1);
+      for (int i = 0; i < 4; ++i) t[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+      __builtin_nontemporal_store(t, o);
     } else {
-      f32x4* o = reinterpret_cast<f32x4*>(y + (row_base + vr) * 64);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        f32x4 t = {v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
-        __builtin_nontemporal_store(t, o + q);
-      }
+      u32x4 t = {__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])};
+      __builtin_nontemporal_store(t, o);
     }
   }
 }
@@ -483,14 +490,15 @@ int cast_to_dispatch(const uint8_t* x, uint8_t* y, const float* scale, float sh,
 template <int FMT, bool BF16_OUT>
 int cast_from_dispatch(const uint8_t* x, uint8_t* y, const float* scale, float sh, int mode,
                        int64_t outer, int64_t mid, int64_t inner, hipStream_t st) {
-  constexpr int U = 2;
+  constexpr int U = 4;
+  constexpr int V = from_vec<BF16_OUT>();
   const int64_t n = outer * mid * inner;
   VecPlan p;
-  const bool vec = aligned(x, 16) && aligned(y, 16) &&
-                   (scale == nullptr || aligned(scale, 16)) && plan_vectors(mode, outer, mid, inner, 16, &p);
+  const bool vec = aligned(x, V) && aligned(y, 16) &&
+                   (scale == nullptr || aligned(scale, 16)) && plan_vectors(mode, outer, mid, inner, V, &p);
   int64_t done = 0;
   if (vec) {
-    const int64_t vpr = p.row_len / 16;
+    const int64_t vpr = p.row_len / V;
     if (vpr > 0) {
       const int64_t bpr = (vpr + kThreads * U - 1) / (kThreads * U);
       const int64_t grid64 = bpr * p.rows;
@@ -500,19 +508,19 @@ int cast_from_dispatch(const uint8_t* x, uint8_t* y, const float* scale, float s
       const int has_scale = mode != MI355Q_SCALE_NONE;
       switch (p.sk) {
         case SK_SCALAR:
-          cast_from_fp8_vec16<FMT, BF16_OUT, SK_SCALAR, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+          cast_from_fp8_vec<FMT, BF16_OUT, SK_SCALAR, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
           break;
         case SK_ROW:
-          cast_from_fp8_vec16<FMT, BF16_OUT, SK_ROW, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+          cast_from_fp8_vec<FMT, BF16_OUT, SK_ROW, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
           break;
         case SK_COL:
-          cast_from_fp8_vec16<FMT, BF16_OUT, SK_COL, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+          cast_from_fp8_vec<FMT, BF16_OUT, SK_COL, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
           break;
         default:
-          cast_from_fp8_vec16<FMT, BF16_OUT, SK_FULL, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+          cast_from_fp8_vec<FMT, BF16_OUT, SK_FULL, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
           break;
       }
-      done = p.rows == 1 ? vpr * 16 : n;
+      done = p.rows == 1 ? vpr * V : n;
     }
   }
   if (done < n) {
