@@ -265,7 +265,11 @@ __device__ __forceinline__ float load_out_as_f32(const uint8_t* p, int64_t idx, 
 constexpr int kEpiRows = 8;
 
 template <int MT, int NT>
-constexpr int epilogue_stage_floats() { return kEpiRows * (32 * NT + 4) + 2 * 32 * MT; }
+constexpr int epilogue_stage_floats() {
+  constexpr int general = kEpiRows * (32 * NT + 4) + 2 * 32 * MT;  // fp32 rows + row scales
+  constexpr int fast = 32 * NT * 16;                               // 32 rows of 32 NT bf16
+  return general > fast ? general : fast;
+}
 
 template <int MT, int NT>
 __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x16 (&acc)[MT][NT],
@@ -409,6 +413,137 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
             }
             store_row4(m, v);
           }
+        }
+      }
+    }
+  });
+}
+
+// The forms the fast bf16 epilogue serves: bf16 output through 16-byte stores,
+// A scale a scalar or one value per row, B scale a scalar or one value per
+// column, bias none or a row vector, no accumulate input.
+__device__ __forceinline__ bool epilogue_fast_ok(const GemmArgs& g, int64_t batch) {
+  if (!g.out_bf16 || g.D != nullptr || g.bias_mode == MI355Q_BIAS_FULL) return false;
+  if (g.sa_mode == MI355Q_GS_PER_COL || g.sb_mode == MI355Q_GS_PER_ROW) return false;
+  const uintptr_t c = reinterpret_cast<uintptr_t>(g.C) + (size_t)(batch * g.stride_c) * 2;
+  return (c & 15u) == 0 && (g.ldc & 7) == 0;
+}
+
+// Four fp32 column values starting at column n (clamped reads past N).
+__device__ __forceinline__ void load_col4_f32(const float* p, int n, int N, float (&out)[4]) {
+  if (n + 3 < N && (reinterpret_cast<uintptr_t>(p + n) & 15u) == 0) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(p + n);
+    out[0] = v[0]; out[1] = v[1]; out[2] = v[2]; out[3] = v[3];
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out[e] = p[(n + e) < N ? (n + e) : N - 1];
+  }
+}
+__device__ __forceinline__ void load_col4_bf16(const uint16_t* p, int n, int N, float (&out)[4]) {
+  if (n + 3 < N && (reinterpret_cast<uintptr_t>(p + n) & 7u) == 0) {
+    const u32x2 v = *reinterpret_cast<const u32x2*>(p + n);
+    out[0] = __uint_as_float(v[0] << 16); out[1] = __uint_as_float(v[0] & 0xffff0000u);
+    out[2] = __uint_as_float(v[1] << 16); out[3] = __uint_as_float(v[1] & 0xffff0000u);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out[e] = bf16_bits_to_f32(p[(n + e) < N ? (n + e) : N - 1]);
+  }
+}
+
+// bf16 epilogue for the common forms.  Scales and bias are applied in the
+// accumulator layout (a lane holds one row m and runs of 4 columns), the
+// rounded bf16 values of 32 rows pass through a per-wave LDS area of 32 rows x
+// (32 NT) bf16, and come back with a lane owning 8 consecutive columns of a
+// row: a wave stores whole rows of its tile, 16 bytes per lane.
+// LDS layout: 8-byte slots of a row are XORed with f(row) so that the 32 lanes
+// of a write cycle (32 rows, one logical slot) and the 16 lanes of a read cycle
+// (rows of equal f, consecutive 16-byte chunks) touch distinct banks; an odd f
+// swaps the two halves of a 16-byte chunk, undone after the read.
+template <int MT, int NT>
+__device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t batch, f32x16 (&acc)[MT][NT],
+                                                   int m_wave, int n_wave, float* stage_f) {
+  constexpr int kRowBytes = 64 * NT;
+  constexpr int kSlotMask = 8 * NT - 1;
+  constexpr int kFShift = 3 - NT;            // NT == 1: rows r, r+4 share banks; NT == 2: rows r, r+2
+  static_assert(NT == 1 || NT == 2, "swizzle defined for 64- and 128-byte rows");
+  constexpr int kLanesPerRow = 4 * NT;       // a lane reads back 16 bytes
+  constexpr int kRowsPerPass = 64 / kLanesPerRow;
+  constexpr int kPasses = 32 / kRowsPerPass;
+  LDS_AS uint8_t* stage = (LDS_AS uint8_t*)stage_f;
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 31, h = lane >> 5;
+  uint16_t* C = reinterpret_cast<uint16_t*>(g.C) + batch * g.stride_c;
+
+  float sa_s = 1.0f, sb_s = 1.0f;
+  if (g.sa_mode == MI355Q_GS_HOST) sa_s = g.sa_host;
+  else if (g.sa_mode == MI355Q_GS_DEV) sa_s = g.sa[0];
+  if (g.sb_mode == MI355Q_GS_HOST) sb_s = g.sb_host;
+  else if (g.sb_mode == MI355Q_GS_DEV) sb_s = g.sb[0];
+
+  // per-column factors of the columns this lane holds in the accumulator layout
+  float cs[NT][4][4], cb[NT][4][4];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n_wave + 32 * j + 8 * q + 4 * h;
+      if (g.sb_mode == MI355Q_GS_PER_COL) load_col4_f32(g.sb, n, g.N, cs[j][q]);
+      else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) cs[j][q][e] = sb_s;
+      }
+      if (g.bias_mode == MI355Q_BIAS_ROW_VECTOR)
+        load_col4_bf16(reinterpret_cast<const uint16_t*>(g.bias) + batch * g.stride_bias, n, g.N, cb[j][q]);
+      else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) cb[j][q][e] = 0.0f;
+      }
+    }
+  float ra[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    const int m = m_wave + 32 * i + r;
+    ra[i] = g.sa_mode == MI355Q_GS_PER_ROW ? g.sa[m < g.M ? m : g.M - 1] : sa_s;
+  }
+
+  const int f_w = (r >> kFShift) & kSlotMask;
+  // read-back coordinates
+  const int row_in_pass = lane / kLanesPerRow, chunk = lane % kLanesPerRow;
+  const int n_out = n_wave + 8 * chunk;
+  const bool full = n_out + 7 < g.N;
+
+  static_for<MT>([&](auto ic) {
+    constexpr int i = decltype(ic)::value;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float t = acc[i][j][4 * q + e] * ra[i];
+          t = t * cs[j][q][e];
+          v[e] = t + cb[j][q][e];
+        }
+        const u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        const int slot = (8 * j + 2 * q + h) ^ f_w;
+        *reinterpret_cast<LDS_AS u32x2*>(stage + r * kRowBytes + slot * 8) = o;
+      }
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) {
+      const int row = p * kRowsPerPass + row_in_pass;
+      const int f = (row >> kFShift) & kSlotMask;
+      u32x4 o = *reinterpret_cast<LDS_AS u32x4*>(stage + row * kRowBytes + ((chunk ^ (f >> 1)) << 4));
+      if (f & 1) o = u32x4{o[2], o[3], o[0], o[1]};
+      const int m = m_wave + 32 * i + row;
+      if (m < g.M) {
+        uint16_t* cp = C + (int64_t)m * g.ldc + n_out;
+        if (full) {
+          __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(cp));  // streamed: keep the operand panels in L2
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (n_out + e < g.N) cp[e] = (uint16_t)(o[e >> 1] >> (16 * (e & 1)));
         }
       }
     }
@@ -599,6 +734,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g)
   const int wm = (wave / kWavesN) * TM, wn = (wave % kWavesN) * TN;
   float* stage = lds_epi + wave * epilogue_stage_floats<MT, NT>();
 
+  const bool fast_epilogue = epilogue_fast_ok(g, batch);
+
   TileCore<BM, BN, A_KMAJOR, B_KMAJOR, FMT_A, FMT_B> core;
   core.init(g, wm, wn);
   const int KT = (g.K + kBK - 1) / kBK;
@@ -631,7 +768,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g)
       // stage numbers restart at 0 for the next tile
       core.k_pair(lds0, lds1, kt + 2 == KT2 ? -2 : kt);
     }
-    epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
+    if (fast_epilogue) epilogue_bf16_fast<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
+    else epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
     if (idx >= count) break;
   }
   // drain the (out-of-range) loads issued for the tile that does not exist
