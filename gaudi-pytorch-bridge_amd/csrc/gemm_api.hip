@@ -1,6 +1,6 @@
 // fp8_gemm_v2 C entry point: argument checks, kernel choice, and the any-shape
 // fallback kernel.  The MFMA tile kernels live in gemm_tile.h.
-#include "gemm_tile.h"
+#include "gemm_pp.h"
 
 namespace mi355q {
 
@@ -73,7 +73,9 @@ extern "C" {
 const char* mi355q_fp8_gemm_variant(int trans_a, int64_t lda, int trans_b, int64_t ldb, int64_t M,
                                     int64_t N, int64_t K) {
   if (lda % 16 || ldb % 16 || (trans_a ? M : K) % 16 || (trans_b ? K : N) % 16) return "simple";
-  return (M > 128 && N > 128) ? "tile256x256x128_mfma32x32x64" : "tile128x128x128_mfma32x32x64";
+  if (M > 128 && N > 128)
+    return mi355q::use_pp_kernel(M, N, 1) ? "tile256x128x64_two_workgroups_mfma32x32x64" : "tile256x256x128_mfma32x32x64";
+  return "tile128x128x128_mfma32x32x64";
 }
 
 int mi355q_fp8_gemm(const void* A, int fmt_a, int trans_a, int64_t lda, const void* B, int fmt_b,

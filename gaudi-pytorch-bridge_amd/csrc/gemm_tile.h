@@ -97,14 +97,15 @@ constexpr int mfma_code() { return FMT == MI355Q_E5M2 ? 1 : 0; }
 //     times two adjacent chunks; XORing with (row & 7) << 1 sends the 8 rows to
 //     8 slots of one parity and leaves the other parity to the adjacent chunk.
 //   MN-major, 128-byte rows: two rows per 256 bytes, so (row >> 1 & 3) << 1.
+//   K-major, 64-byte rows: four rows per 256 bytes, so (row >> 2) & 3.
 template <bool KMAJOR, int ROWS, int ROW_BYTES>
 struct TileGeom {
   static constexpr int kChunksPerRow = ROW_BYTES / 16;
   static constexpr int kChunks = ROWS * kChunksPerRow;
-  static_assert(kChunks % kGemmThreads == 0, "tile must split evenly over the block");
-  static_assert(KMAJOR ? ROW_BYTES == 128 : (ROW_BYTES == 256 || ROW_BYTES == 128), "no swizzle defined");
+  static_assert(KMAJOR ? (ROW_BYTES == 128 || ROW_BYTES == 64) : (ROW_BYTES == 256 || ROW_BYTES == 128), "no swizzle defined");
   __device__ static __forceinline__ int swizzle(int row) {
-    if constexpr (KMAJOR) return (row >> 1) & 7;
+    if constexpr (KMAJOR && ROW_BYTES == 128) return (row >> 1) & 7;
+    else if constexpr (KMAJOR) return (row >> 2) & 3;
     else if constexpr (ROW_BYTES == 256) return (row & 7) << 1;
     else return ((row >> 1) & 3) << 1;
   }
@@ -131,14 +132,15 @@ __device__ __forceinline__ void static_for(F&& f) {
 //   else  : rows index k, chunks walk m/n.  Rows at or beyond K fall outside the
 //           descriptor; columns past the extent only feed outputs that are
 //           never stored.
-template <bool KMAJOR, int EXT>  // EXT: tile extent along m/n
+// EXT: tile extent along m/n; BK: bytes of K per stage; WAVES: waves of the workgroup
+template <bool KMAJOR, int EXT, int BK = kBK, int WAVES = kWaves>
 struct DmaLoader {
-  using G = TileGeom<KMAJOR, KMAJOR ? EXT : kBK, KMAJOR ? kBK : EXT>;
+  using G = TileGeom<KMAJOR, KMAJOR ? EXT : BK, KMAJOR ? BK : EXT>;
   static constexpr int kCPR = G::kChunksPerRow;
   static constexpr int kRowsPerRegion = 64 / kCPR;
   static constexpr int kRegions = G::kChunks / 64;
-  static constexpr int kPerWave = kRegions / kWaves;
-  static_assert(kRegions % kWaves == 0 && 64 % kCPR == 0, "tile does not split over the waves");
+  static constexpr int kPerWave = kRegions / WAVES;
+  static_assert(kRegions % WAVES == 0 && 64 % kCPR == 0, "tile does not split over the waves");
 
   i32x4 rsrc;  // raw buffer descriptor: base, stride 0, num_records (bytes), dword 3 flags
   int voff[kPerWave];
@@ -156,11 +158,11 @@ struct DmaLoader {
     if constexpr (KMAJOR) {
       base += (int64_t)mn0 * ld;
       records = (int64_t)(extent - mn0 - 1) * ld + K;
-      step = kBK;
+      step = BK;
     } else {
       base += mn0;
       records = (int64_t)(K - 1) * ld + (extent - mn0);
-      step = kBK * (int)ld;
+      step = BK * (int)ld;
     }
     const uint64_t b = reinterpret_cast<uint64_t>(base);
     rsrc[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
@@ -212,9 +214,9 @@ struct DmaLoader {
 template <bool KMAJOR>
 constexpr int frag_parts() { return KMAJOR ? 2 : 4; }
 
-template <bool KMAJOR, int EXT, int PART>
+template <bool KMAJOR, int EXT, int PART, int BK = kBK>
 __device__ __forceinline__ void read_fragment_part(const uint8_t* lds, int mn_base, int ksub, i32x8& f) {
-  using G = TileGeom<KMAJOR, KMAJOR ? EXT : kBK, KMAJOR ? kBK : EXT>;
+  using G = TileGeom<KMAJOR, KMAJOR ? EXT : BK, KMAJOR ? BK : EXT>;
   const int lane = threadIdx.x & 63;
   if constexpr (KMAJOR) {
     const int row = mn_base + (lane & 31);
@@ -277,7 +279,8 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
   constexpr int kRowFloats = 32 * NT + 4;
   constexpr int kLanesPerRow = 8 * NT;           // a lane owns 4 columns
   constexpr int kRowsPerPass = 64 / kLanesPerRow;
-  const int lane = threadIdx.x & 63;
+  int lane = threadIdx.x & 63;
+  asm volatile("" : "+v"(lane));  // keeps lane-derived values out of the registers of the K loop
   const int es = g.out_bf16 ? 2 : 4;
   uint8_t* C = g.C + batch * g.stride_c * es;
   const uint8_t* D = g.D ? g.D + batch * g.stride_d * es : nullptr;
@@ -459,7 +462,7 @@ __device__ __forceinline__ void load_col4_bf16(const uint16_t* p, int n, int N, 
 // of a write cycle (32 rows, one logical slot) and the 16 lanes of a read cycle
 // (rows of equal f, consecutive 16-byte chunks) touch distinct banks; an odd f
 // swaps the two halves of a 16-byte chunk, undone after the read.
-template <int MT, int NT>
+template <int MT, int NT, bool PER_COL>
 __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t batch, f32x16 (&acc)[MT][NT],
                                                    int m_wave, int n_wave, float* stage_f) {
   constexpr int kRowBytes = 64 * NT;
@@ -470,7 +473,13 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
   constexpr int kRowsPerPass = 64 / kLanesPerRow;
   constexpr int kPasses = 32 / kRowsPerPass;
   LDS_AS uint8_t* stage = (LDS_AS uint8_t*)stage_f;
-  const int lane = threadIdx.x & 63;
+  // The epilogue sits inside the persistent tile loop, and everything below
+  // that depends only on the lane number is invariant in that loop: left
+  // alone, the compiler computes it all once before the K loop, where no
+  // register is free, and spills it to scratch memory.  Routing the lane number through an empty
+  // volatile asm keeps those few integer operations here.
+  int lane = threadIdx.x & 63;
+  asm volatile("" : "+v"(lane));
   const int r = lane & 31, h = lane >> 5;
   uint16_t* C = reinterpret_cast<uint16_t*>(g.C) + batch * g.stride_c;
 
@@ -480,18 +489,17 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
   if (g.sb_mode == MI355Q_GS_HOST) sb_s = g.sb_host;
   else if (g.sb_mode == MI355Q_GS_DEV) sb_s = g.sb[0];
 
-  // per-column factors of the columns this lane holds in the accumulator layout
-  float cs[NT][4][4], cb[NT][4][4];
+  // Per-column values of the columns this lane holds in the accumulator layout.
+  // A scalar B scale is folded into the row factor instead, which leaves one
+  // fused multiply-add per element.
+  constexpr bool per_col = PER_COL;
+  float cs[PER_COL ? NT : 1][4][4], cb[NT][4][4];
 #pragma unroll
   for (int j = 0; j < NT; ++j)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int n = n_wave + 32 * j + 8 * q + 4 * h;
-      if (g.sb_mode == MI355Q_GS_PER_COL) load_col4_f32(g.sb, n, g.N, cs[j][q]);
-      else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) cs[j][q][e] = sb_s;
-      }
+      if constexpr (per_col) load_col4_f32(g.sb, n, g.N, cs[j][q]);
       if (g.bias_mode == MI355Q_BIAS_ROW_VECTOR)
         load_col4_bf16(reinterpret_cast<const uint16_t*>(g.bias) + batch * g.stride_bias, n, g.N, cb[j][q]);
       else {
@@ -504,6 +512,7 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
   for (int i = 0; i < MT; ++i) {
     const int m = m_wave + 32 * i + r;
     ra[i] = g.sa_mode == MI355Q_GS_PER_ROW ? g.sa[m < g.M ? m : g.M - 1] : sa_s;
+    if (!per_col) ra[i] *= sb_s;
   }
 
   const int f_w = (r >> kFShift) & kSlotMask;
@@ -519,11 +528,12 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         float v[4];
+        if constexpr (per_col) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float t = acc[i][j][4 * q + e] * ra[i];
-          t = t * cs[j][q][e];
-          v[e] = t + cb[j][q][e];
+          for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf(acc[i][j][4 * q + e] * ra[i], cs[j][q][e], cb[j][q][e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf(acc[i][j][4 * q + e], ra[i], cb[j][q][e]);
         }
         const u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
         const int slot = (8 * j + 2 * q + h) ^ f_w;
@@ -768,8 +778,12 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g)
       // stage numbers restart at 0 for the next tile
       core.k_pair(lds0, lds1, kt + 2 == KT2 ? -2 : kt);
     }
-    if (fast_epilogue) epilogue_bf16_fast<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
-    else epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
+    if (fast_epilogue) {
+      if (g.sb_mode == MI355Q_GS_PER_COL) epilogue_bf16_fast<MT, NT, true>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
+      else epilogue_bf16_fast<MT, NT, false>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
+    } else {
+      epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
+    }
     if (idx >= count) break;
   }
   // drain the (out-of-range) loads issued for the tile that does not exist
@@ -785,21 +799,6 @@ void launch_tile(const GemmArgs& g, int64_t batch, hipStream_t st) {
   const int cus = compute_units();
   dim3 grid((unsigned)(tiles < cus ? tiles : cus), (unsigned)batch);
   fp8_gemm_tile_kernel<BM, BN, AK, BK_, FA, FB><<<grid, kGemmThreads, 0, st>>>(a);
-}
-
-template <bool AK, bool BK_, int FA, int FB>
-void launch_by_size(const GemmArgs& g, int64_t batch, hipStream_t st) {
-  if (g.M > 128 && g.N > 128) launch_tile<256, 256, AK, BK_, FA, FB>(g, batch, st);
-  else launch_tile<128, 128, AK, BK_, FA, FB>(g, batch, st);
-}
-
-// One translation unit per operand layout instantiates this (gemm_inst_*.hip).
-template <bool AK, bool BK_>
-void launch_by_format(const GemmArgs& g, int fmt_a, int fmt_b, int64_t batch, hipStream_t st) {
-  if (fmt_a == MI355Q_E4M3FN && fmt_b == MI355Q_E4M3FN) launch_by_size<AK, BK_, MI355Q_E4M3FN, MI355Q_E4M3FN>(g, batch, st);
-  else if (fmt_a == MI355Q_E4M3FN) launch_by_size<AK, BK_, MI355Q_E4M3FN, MI355Q_E5M2>(g, batch, st);
-  else if (fmt_b == MI355Q_E4M3FN) launch_by_size<AK, BK_, MI355Q_E5M2, MI355Q_E4M3FN>(g, batch, st);
-  else launch_by_size<AK, BK_, MI355Q_E5M2, MI355Q_E5M2>(g, batch, st);
 }
 
 // A K-major / B K-major etc.; defined in gemm_inst_*.hip
