@@ -75,6 +75,7 @@ const char* mi355q_fp8_gemm_variant(int trans_a, int64_t lda, int trans_b, int64
   if (lda % 16 || ldb % 16 || (trans_a ? M : K) % 16 || (trans_b ? K : N) % 16) return "simple";
   if (M > 128 && N > 128)
     return mi355q::use_pp_kernel(M, N, 1) ? "tile256x128x64_two_workgroups_mfma32x32x64" : "tile256x256x128_mfma32x32x64";
+  if (M <= 128) return "strip_Mx128x128_ring_mfma32x32x64";
   return "tile128x128x128_mfma32x32x64";
 }
 

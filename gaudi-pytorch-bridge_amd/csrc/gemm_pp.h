@@ -16,6 +16,7 @@
 // area overlays the stage ring, which is idle by then; nothing is prefetched
 // across tiles, the other workgroup covers that gap.
 #pragma once
+#include "gemm_skinny.h"
 #include "gemm_tile.h"
 
 namespace mi355q {
@@ -233,6 +234,8 @@ void launch_by_size(const GemmArgs& g, int64_t batch, hipStream_t st) {
   if (g.M > 128 && g.N > 128) {
     if (use_pp_kernel(g.M, g.N, batch)) launch_pp<256, 128, AK, BK_, FA, FB>(g, batch, st);
     else launch_tile<256, 256, AK, BK_, FA, FB>(g, batch, st);
+  } else if (g.M <= 128) {
+    launch_skinny_by_m<AK, BK_, FA, FB>(g, batch, st);
   } else {
     launch_tile<128, 128, AK, BK_, FA, FB>(g, batch, st);
   }

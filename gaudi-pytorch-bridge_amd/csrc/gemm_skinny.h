@@ -1,0 +1,134 @@
+// fp8 GEMM for few rows of A (M <= 128: decode-shaped calls).
+//
+// These problems are bound by streaming B from HBM once: what matters is how
+// many bytes each compute unit keeps in flight, not the MFMA schedule.  One
+// 4-wave workgroup owns a strip of 128 columns of C for all M rows and walks K
+// in 128-byte stages through a ring of S LDS buffers, S as large as the 160 KB
+// of LDS allow (8 for BM = 32: up to seven stages, 112 KB of B per compute
+// unit, are on their way from memory while one is being multiplied).  Each wave
+// multiplies the whole A tile by its own 32 columns; fragments are read right
+// before use (the matrix pipes are mostly idle anyway).
+//
+// The global->LDS loads, LDS geometry, fragment reads and epilogues are those
+// of the large-tile kernel (gemm_tile.h).
+#pragma once
+#include "gemm_tile.h"
+
+namespace mi355q {
+
+constexpr int kSkThreads = 256;
+constexpr int kSkWaves = 4;
+constexpr int kSkBN = 128;
+
+template <int BM>
+constexpr int skinny_stages() {
+  constexpr int stage = (BM + kSkBN) * kBK;
+  constexpr int s = (160 * 1024) / stage;
+  return s > 8 ? 8 : s;
+}
+
+template <int BM, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
+__global__ __launch_bounds__(kSkThreads) void fp8_gemm_skinny_kernel(GemmArgs g) {
+  constexpr int MT = BM / 32;
+  constexpr int S = skinny_stages<BM>();
+  constexpr int kStageBytes = (BM + kSkBN) * kBK;
+  using LA = DmaLoader<A_KMAJOR, BM, kBK, kSkWaves>;
+  using LB = DmaLoader<B_KMAJOR, kSkBN, kBK, kSkWaves>;
+  constexpr int kOps = LA::kPerWave + LB::kPerWave;
+  constexpr int kInFlight = (S - 2) * kOps;  // loads that may stay outstanding while stage kt is consumed
+  static_assert(S >= 3 && kInFlight <= 63, "vmcnt holds 6 bits");
+  static_assert(kSkWaves * epilogue_stage_floats<MT, 1>() * 4 <= S * kStageBytes, "epilogue area overlays the ring");
+  constexpr int kPartsA = frag_parts<A_KMAJOR>(), kPartsB = frag_parts<B_KMAJOR>();
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[S * kStageBytes];
+
+  const int64_t batch = blockIdx.y;
+  const int n0 = blockIdx.x * kSkBN;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wn = wave * 32;
+
+  LA la;
+  LB lb;
+  la.init(g.A + batch * g.stride_a, g.lda, 0, g.M, g.K);
+  lb.init(g.B + batch * g.stride_b, g.ldb, n0, g.N, g.K);
+  auto issue_stage = [&](int off, int kt) {
+    static_for<LA::kPerWave>([&](auto ic) { la.template issue_one<decltype(ic)::value>(lds + off, kt * kBK, g.K); });
+    static_for<LB::kPerWave>([&](auto ic) { lb.template issue_one<decltype(ic)::value>(lds + off + BM * kBK, kt * kBK, g.K); });
+    la.advance();
+    lb.advance();
+  };
+
+  f32x16 acc[MT][1];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[i][0][e] = 0.0f;
+
+  const int KT = (g.K + kBK - 1) / kBK;
+  // stages 0 .. S-2 go out first; stages at or beyond K fall outside the
+  // buffer descriptors and arrive as zeros, so every step issues and waits alike
+#pragma unroll
+  for (int s = 0; s < S - 1; ++s) issue_stage(s * kStageBytes, s);
+
+  int rd_off = 0;                        // buffer of stage kt
+  int wr_off = (S - 1) * kStageBytes;    // buffer of stage kt + S - 1 (the one stage kt - 1 used)
+  for (int kt = 0; kt < KT; ++kt) {
+    // this wave's part of stage kt has landed once only the later stages' loads are outstanding
+    __builtin_amdgcn_s_waitcnt((kInFlight & 15) | ((kInFlight >> 4) << 14) | 0x0070);
+    __syncthreads();  // everyone's part has; and everyone is done with the buffer of stage kt - 1
+    issue_stage(wr_off, kt + S - 1);
+    const uint8_t* st = lds + rd_off;
+#pragma unroll
+    for (int ks = 0; ks < kBK / 64; ++ks) {
+      i32x8 fb, fa[MT];
+      static_for<kPartsB>([&](auto pc) {
+        read_fragment_part<B_KMAJOR, kSkBN, decltype(pc)::value>(st + BM * kBK, wn, ks, fb);
+      });
+      static_for<MT>([&](auto ic) {
+        static_for<kPartsA>([&](auto pc) {
+          read_fragment_part<A_KMAJOR, BM, decltype(pc)::value>(st, decltype(ic)::value * 32, ks, fa[decltype(ic)::value]);
+        });
+      });
+      static_for<MT>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        acc[i][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+            fb, fa[i], acc[i][0], mfma_code<FMT_B>(), mfma_code<FMT_A>(), 0, 0, 0, 0);
+      });
+    }
+    rd_off += kStageBytes;
+    if (rd_off == S * kStageBytes) rd_off = 0;
+    wr_off += kStageBytes;
+    if (wr_off == S * kStageBytes) wr_off = 0;
+  }
+  // the ring is idle (zero-fill loads of the stages past K included) before the epilogue overlays it
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  float* stage_area = reinterpret_cast<float*>(lds) + wave * epilogue_stage_floats<MT, 1>();
+  if (epilogue_fast_ok(g, batch)) {
+    if (g.sb_mode == MI355Q_GS_PER_COL) epilogue_bf16_fast<MT, 1, true>(g, batch, acc, 0, n0 + wn, stage_area);
+    else epilogue_bf16_fast<MT, 1, false>(g, batch, acc, 0, n0 + wn, stage_area);
+  } else {
+    epilogue<MT, 1>(g, batch, acc, 0, n0 + wn, stage_area);
+  }
+}
+
+template <int BM, bool AK, bool BK_, int FA, int FB>
+void launch_skinny(const GemmArgs& g, int64_t batch, hipStream_t st) {
+  GemmArgs a = g;
+  a.tiles_m = 1;
+  a.tiles_n = (g.N + kSkBN - 1) / kSkBN;
+  dim3 grid((unsigned)a.tiles_n, (unsigned)batch);
+  fp8_gemm_skinny_kernel<BM, AK, BK_, FA, FB><<<grid, kSkThreads, 0, st>>>(a);
+}
+
+// M <= 128.  An MN-major A tile has rows of BM bytes in LDS, for which only
+// 128 has a conflict-free swizzle, so trans_a problems always take BM = 128.
+template <bool AK, bool BK_, int FA, int FB>
+void launch_skinny_by_m(const GemmArgs& g, int64_t batch, hipStream_t st) {
+  if constexpr (AK) {
+    if (g.M <= 32) return launch_skinny<32, AK, BK_, FA, FB>(g, batch, st);
+    if (g.M <= 64) return launch_skinny<64, AK, BK_, FA, FB>(g, batch, st);
+  }
+  launch_skinny<128, AK, BK_, FA, FB>(g, batch, st);
+}
+
+}  // namespace mi355q
