@@ -282,6 +282,77 @@ __global__ __launch_bounds__(kThreads) void rowwise_amax_kernel(const uint8_t* _
   }
 }
 
+// ------------------------------------------------- dynamic per-row quantisation
+//
+// One pass of "per-row amax -> scale = target / amax -> cast with that scale":
+// a workgroup holds one row in registers (VPT 16-byte vectors per thread), so
+// the row is read from HBM once.  Results are bit-identical to the three
+// separate steps (rowwise_amax, an fp32 division, cast_to_fp8 with per-row
+// scales); scale_inv = 1 / scale is what the GEMM takes as A_scale_inv.
+template <bool BF16_IN, int FMT, int VPT>
+__global__ __launch_bounds__(kThreads) void quantize_rows_kernel(
+    const uint8_t* __restrict__ x, uint8_t* __restrict__ y, int64_t vec_per_row, float target,
+    float* __restrict__ scale_out, float* __restrict__ scale_inv_out) {
+  __shared__ uint32_t wave_part[kThreads / 64];
+  constexpr int EPV = BF16_IN ? 8 : 4;  // elements per 16-byte vector
+  const int64_t row = blockIdx.x;
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x) + row * vec_per_row;
+  u32x4 in[VPT];
+  uint32_t am = 0;
+#pragma unroll
+  for (int u = 0; u < VPT; ++u) {
+    const int64_t v = threadIdx.x + (int64_t)u * kThreads;
+    in[u] = u32x4{0u, 0u, 0u, 0u};
+    if (v < vec_per_row) in[u] = __builtin_nontemporal_load(xr + v);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (BF16_IN) {
+        const u16x2 a = __builtin_bit_cast(u16x2, in[u][i] & 0x7fff7fffu);
+        am = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, __builtin_bit_cast(u16x2, am)));
+      } else {
+        const uint32_t a = in[u][i] & 0x7fffffffu;
+        am = am > a ? am : a;
+      }
+    }
+  }
+  if constexpr (BF16_IN) {
+    const uint32_t lo = am & 0xffffu, hi = am >> 16;
+    am = (lo > hi ? lo : hi) << 16;
+  }
+  am = wave_max_u32(am);
+  if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = am;
+  __syncthreads();
+  uint32_t r = wave_part[0];
+#pragma unroll
+  for (int w = 1; w < kThreads / 64; ++w) r = r > wave_part[w] ? r : wave_part[w];
+  const float amax = __uint_as_float(r);
+  const float scale = target / amax;  // correctly rounded fp32 division, as on the host
+  if (threadIdx.x == 0) {
+    if (scale_out) scale_out[row] = scale;
+    if (scale_inv_out) scale_inv_out[row] = 1.0f / scale;
+  }
+  const float s = BF16_IN ? round_to_bf16(scale) : scale;
+#pragma unroll
+  for (int u = 0; u < VPT; ++u) {
+    const int64_t v = threadIdx.x + (int64_t)u * kThreads;
+    if (v >= vec_per_row) continue;
+    if constexpr (BF16_IN) {
+      float p[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[2 * i] = round_to_bf16(__uint_as_float(in[u][i] << 16) * s);
+        p[2 * i + 1] = round_to_bf16(__uint_as_float(in[u][i] & 0xffff0000u) * s);
+      }
+      const u32x2 o = {cvt_fp8x4<FMT>(p[0], p[1], p[2], p[3]), cvt_fp8x4<FMT>(p[4], p[5], p[6], p[7])};
+      __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(y) + row * vec_per_row + v);
+    } else {
+      const uint32_t o = cvt_fp8x4<FMT>(__uint_as_float(in[u][0]) * s, __uint_as_float(in[u][1]) * s,
+                                        __uint_as_float(in[u][2]) * s, __uint_as_float(in[u][3]) * s);
+      __builtin_nontemporal_store(o, reinterpret_cast<uint32_t*>(y) + row * vec_per_row + v);
+    }
+  }
+}
+
 // -------------------------------------------------------------- cast_from_fp8
 //
 // A lane produces one 16-byte store: 8 fp8 bytes in for bf16 output, 4 for
@@ -539,6 +610,18 @@ inline bool scale_args_ok(const float* scale, int mode, int64_t outer, int64_t m
   return true;
 }
 
+template <bool BF16_IN, int FMT>
+int quantize_rows_launch(const uint8_t* x, uint8_t* y, int64_t rows, int64_t vpr, float target,
+                                float* scale_out, float* scale_inv_out, hipStream_t st) {
+  const unsigned grid = (unsigned)rows;
+  if (vpr <= kThreads) quantize_rows_kernel<BF16_IN, FMT, 1><<<grid, kThreads, 0, st>>>(x, y, vpr, target, scale_out, scale_inv_out);
+  else if (vpr <= 2 * kThreads) quantize_rows_kernel<BF16_IN, FMT, 2><<<grid, kThreads, 0, st>>>(x, y, vpr, target, scale_out, scale_inv_out);
+  else if (vpr <= 4 * kThreads) quantize_rows_kernel<BF16_IN, FMT, 4><<<grid, kThreads, 0, st>>>(x, y, vpr, target, scale_out, scale_inv_out);
+  else if (vpr <= 8 * kThreads) quantize_rows_kernel<BF16_IN, FMT, 8><<<grid, kThreads, 0, st>>>(x, y, vpr, target, scale_out, scale_inv_out);
+  else return MI355Q_ERR_UNSUPPORTED;
+  return launch_status();
+}
+
 }  // namespace mi355q
 
 using namespace mi355q;
@@ -589,6 +672,29 @@ int mi355q_rowwise_amax(const void* x, int x_dtype, int64_t rows, int64_t cols, 
   if (x_dtype == MI355Q_BF16) rowwise_amax_kernel<true><<<(unsigned)rows, kThreads, 0, st>>>(xb, cols, vec_ok, amax_out);
   else rowwise_amax_kernel<false><<<(unsigned)rows, kThreads, 0, st>>>(xb, cols, vec_ok, amax_out);
   return launch_status();
+}
+
+int mi355q_quantize_rows(const void* x, int x_dtype, int64_t rows, int64_t cols, void* y, int fp8_fmt,
+                         float target, float* scale_out, float* scale_inv_out, void* stream) {
+  if (rows < 0 || cols < 0) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (fp8_fmt != MI355Q_E4M3FN && fp8_fmt != MI355Q_E5M2) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (x_dtype != MI355Q_F32 && x_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (rows == 0 || cols == 0) return MI355Q_OK;
+  if (x == nullptr || y == nullptr) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (rows > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+  const int epv = x_dtype == MI355Q_BF16 ? 8 : 4;
+  // whole 16-byte vectors only; the row has to fit the registers of one workgroup
+  if (cols % epv != 0 || !aligned(x, 16) || !aligned(y, epv)) return MI355Q_ERR_UNSUPPORTED;
+  const int64_t vpr = cols / epv;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  uint8_t* yb = static_cast<uint8_t*>(y);
+  if (x_dtype == MI355Q_BF16) {
+    if (fp8_fmt == MI355Q_E4M3FN) return quantize_rows_launch<true, MI355Q_E4M3FN>(xb, yb, rows, vpr, target, scale_out, scale_inv_out, st);
+    return quantize_rows_launch<true, MI355Q_E5M2>(xb, yb, rows, vpr, target, scale_out, scale_inv_out, st);
+  }
+  if (fp8_fmt == MI355Q_E4M3FN) return quantize_rows_launch<false, MI355Q_E4M3FN>(xb, yb, rows, vpr, target, scale_out, scale_inv_out, st);
+  return quantize_rows_launch<false, MI355Q_E5M2>(xb, yb, rows, vpr, target, scale_out, scale_inv_out, st);
 }
 
 int mi355q_cast_to_fp8(const void* x, int x_dtype, void* y, int fp8_fmt, const float* scale_dev,

@@ -25,7 +25,6 @@ constexpr int kPpThreads = 256;
 constexpr int kPpWaves = 4;
 constexpr int kPpWavesM = 2, kPpWavesN = 2;
 constexpr int kPpBK = 64;
-constexpr int kPpStages = 3;
 
 template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
 struct PpCore {
@@ -37,7 +36,6 @@ struct PpCore {
   static constexpr int kPartsA = frag_parts<A_KMAJOR>(), kPartsB = frag_parts<B_KMAJOR>();
   static constexpr int kMfmas = MT * NT;
   static constexpr int kDmaOps = LA::kPerWave + LB::kPerWave;
-  static_assert(kDmaOps <= 15, "the per-stage wait counts this many loads in vmcnt");
 
   f32x16 acc[MT][NT];
   i32x8 fa[MT], fb0[NT], fb1[NT];
@@ -114,21 +112,25 @@ struct PpCore {
   }
 };
 
-// s_waitcnt with vmcnt = N (N <= 15), lgkmcnt = 0, expcnt untouched (gfx9 encoding:
+// s_waitcnt with vmcnt = N, lgkmcnt = 0, expcnt untouched (gfx9 encoding:
 // vmcnt low bits [3:0], expcnt [6:4], lgkmcnt [11:8], vmcnt high bits [15:14]).
 template <int N>
 __device__ __forceinline__ void wait_vm_lgkm() {
-  static_assert(N >= 0 && N <= 15, "vmcnt field");
-  __builtin_amdgcn_s_waitcnt(0x0070 | N);
+  static_assert(N >= 0 && N <= 63, "vmcnt field");
+  __builtin_amdgcn_s_waitcnt(0x0070 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
+// S: stages in the ring.  3 lets two workgroups share a CU's LDS; a launch with
+// no more workgroups than CUs takes 6, to keep more bytes in flight per CU.
+template <int BM, int BN, int S, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
 __global__ __launch_bounds__(kPpThreads, 2) void fp8_gemm_pp_kernel(GemmArgs g, int late_from) {
   using Core = PpCore<BM, BN, A_KMAJOR, B_KMAJOR, FMT_A, FMT_B>;
   constexpr int MT = Core::MT, NT = Core::NT;
   constexpr int kStageBytes = Core::kStageBytes;
-  static_assert(kPpWaves * epilogue_stage_floats<MT, NT>() * 4 <= kPpStages * kStageBytes, "epilogue area overlays the ring");
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[kPpStages * kStageBytes];
+  static_assert(kPpWaves * epilogue_stage_floats<MT, NT>() * 4 <= S * kStageBytes, "epilogue area overlays the ring");
+  static_assert(S >= 3 && (S - 2) * Core::kDmaOps <= 63, "per-step wait");
+  constexpr int kRing = S * kStageBytes;
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kRing];
 
   const int nb = gridDim.x, bid = blockIdx.x;
   const int tiles = g.tiles_m * g.tiles_n;
@@ -162,11 +164,10 @@ __global__ __launch_bounds__(kPpThreads, 2) void fp8_gemm_pp_kernel(GemmArgs g, 
     tile_coords(first + idx, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     core.retarget(g, batch, m0, n0);
-    // ring offsets: o_cur holds the stage being computed, o_nxt the next, o_nn the one after
-    int o_cur = 0, o_nxt = kStageBytes, o_nn = 2 * kStageBytes;
-    core.issue_stage(lds + o_cur, 0);
-    core.issue_stage(lds + o_nxt, 1);
-    core.issue_stage(lds + o_nn, 2);   // stages at or beyond K arrive as zeros
+    // stage s lives in buffer s % S; o_cur is the buffer of the stage being computed
+    int o_cur = 0;
+#pragma unroll
+    for (int s = 0; s < S; ++s) core.issue_stage(lds + s * kStageBytes, s);  // stages at or beyond K arrive as zeros
     core.zero_acc();
     // stores of the previous epilogue share the counter: wait for everything once
     __builtin_amdgcn_s_waitcnt(0);
@@ -180,18 +181,21 @@ __global__ __launch_bounds__(kPpThreads, 2) void fp8_gemm_pp_kernel(GemmArgs g, 
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the first fragments are in registers
     // At the top of a step the loads of the next stage are complete (this wave
     // has waited for its own, the barrier covers the others') and every wave has
-    // read the fragments of the current stage, whose buffer the step refills.
-    // After a step the wave's outstanding loads are those of the stage needed
-    // next and, issued after them, those of the step just done: waiting until
-    // only the latter remain is enough.
+    // read the fragments of the current stage, whose buffer the step refills
+    // with the stage S ahead.  After a step the wave's outstanding loads are
+    // those of the stages after the next one, oldest first: the stage needed
+    // next is complete once only (S - 2) stages' worth remain.
+    auto next = [&](int o) { return o + kStageBytes == kRing ? 0 : o + kStageBytes; };
     for (int kt = 0; kt < KT2; kt += 2) {
+      const int o_nxt = next(o_cur);
       __syncthreads();
-      core.step(core.fb0, core.fb1, lds + o_nxt, lds + o_cur, kt + 3);
-      wait_vm_lgkm<Core::kDmaOps>();
+      core.step(core.fb0, core.fb1, lds + o_nxt, lds + o_cur, kt + S);
+      wait_vm_lgkm<(S - 2) * Core::kDmaOps>();
+      const int o_nn = next(o_nxt);
       __syncthreads();
-      core.step(core.fb1, core.fb0, lds + o_nn, lds + o_nxt, kt + 4);
-      wait_vm_lgkm<Core::kDmaOps>();
-      const int t = o_cur; o_cur = o_nn; o_nn = o_nxt; o_nxt = t;
+      core.step(core.fb1, core.fb0, lds + o_nn, lds + o_nxt, kt + S + 1);
+      wait_vm_lgkm<(S - 2) * Core::kDmaOps>();
+      o_cur = o_nn;
     }
     // every wave is done with the ring (its last fragment reads included) before it is overlaid
     __builtin_amdgcn_s_waitcnt(0);
@@ -225,8 +229,12 @@ void launch_pp(const GemmArgs& g, int64_t batch, hipStream_t st) {
   const int cus = compute_units();
   const int64_t wgs = tiles < 2 * cus ? tiles : 2 * cus;
   dim3 grid((unsigned)wgs, (unsigned)batch);
-  // workgroups are placed breadth first: those beyond the CU count are second residents
-  fp8_gemm_pp_kernel<BM, BN, AK, BK_, FA, FB><<<grid, kPpThreads, 0, st>>>(a, cus);
+  if (wgs * batch <= cus) {
+    fp8_gemm_pp_kernel<BM, BN, 6, AK, BK_, FA, FB><<<grid, kPpThreads, 0, st>>>(a, (int)wgs);
+  } else {
+    // workgroups are placed breadth first: those beyond the CU count are second residents
+    fp8_gemm_pp_kernel<BM, BN, 3, AK, BK_, FA, FB><<<grid, kPpThreads, 0, st>>>(a, cus);
+  }
 }
 
 template <bool AK, bool BK_, int FA, int FB>

@@ -604,6 +604,40 @@ Tensor rowwise_amax_op(const Tensor& x) {
   return out;
 }
 
+// Dynamic per-row quantisation: (x8, scale_inv) with scale = fp8_max / rowwise amax.
+// One kernel when the row fits a workgroup's registers, else the three steps it fuses.
+std::tuple<Tensor, Tensor> quantize_rows_op(const Tensor& x, at::ScalarType dtype) {
+  TORCH_CHECK(x.scalar_type() == at::kFloat || x.scalar_type() == at::kBFloat16,
+              "mi355q::quantize_rows input must be float or bfloat16");
+  TORCH_CHECK(dtype == at::kFloat8_e4m3fn || dtype == at::kFloat8_e5m2,
+              "mi355q::quantize_rows dtype must be float8_e4m3fn or float8_e5m2");
+  TORCH_CHECK(x.dim() >= 1, "mi355q::quantize_rows input must have at least 1 dimension");
+  std::vector<int64_t> shp(x.sizes().begin(), x.sizes().end());
+  shp.back() = 1;
+  if (x.is_meta()) return {at::empty(x.sizes(), x.options().dtype(dtype)), at::empty(shp, x.options().dtype(at::kFloat))};
+  DeviceGuard guard(x.device());
+  Tensor c = x.contiguous();
+  Tensor out = at::empty(c.sizes(), c.options().dtype(dtype));
+  Tensor scale_inv = at::empty(shp, c.options().dtype(at::kFloat));
+  const int64_t cols = c.size(-1);
+  const int64_t rows = cols ? c.numel() / cols : 0;
+  const float target = dtype == at::kFloat8_e5m2 ? 57344.0f : 448.0f;
+  const int st = mi355q_quantize_rows(c.data_ptr(), to_mi355q_dtype(c.scalar_type()), rows, cols, out.data_ptr(),
+                                      to_mi355q_dtype(dtype), target, nullptr, scale_inv.data_ptr<float>(),
+                                      current_stream(c));
+  if (st == MI355Q_ERR_UNSUPPORTED) {
+    Tensor amax = rowwise_amax_op(c).reshape(shp);
+    Tensor scale = at::div(at::full_like(amax, target), amax);
+    check_status(mi355q_cast_to_fp8(c.data_ptr(), to_mi355q_dtype(c.scalar_type()), out.data_ptr(),
+                                    to_mi355q_dtype(dtype), scale.data_ptr<float>(), 0.0f, MI355Q_SCALE_MID,
+                                    1, rows, cols, nullptr, current_stream(c)),
+                 "mi355q_cast_to_fp8");
+    return {out, at::reciprocal(scale)};
+  }
+  check_status(st, "mi355q_quantize_rows");
+  return {out, scale_inv};
+}
+
 }  // namespace
 
 TORCH_LIBRARY(hpu, m) {
@@ -624,6 +658,7 @@ TORCH_LIBRARY(hpu, m) {
 TORCH_LIBRARY(mi355q, m) {
   m.def("mi355q::amax(Tensor input) -> Tensor");
   m.def("mi355q::rowwise_amax(Tensor input) -> Tensor");
+  m.def("mi355q::quantize_rows(Tensor input, ScalarType dtype) -> (Tensor, Tensor)");
 }
 
 #define MI355Q_REGISTER_HPU(m)                                                                 \
@@ -645,8 +680,10 @@ TORCH_LIBRARY_IMPL(hpu, Meta, m) { MI355Q_REGISTER_HPU(m) }
 TORCH_LIBRARY_IMPL(mi355q, CUDA, m) {
   m.impl("amax", amax_op);
   m.impl("rowwise_amax", rowwise_amax_op);
+  m.impl("quantize_rows", quantize_rows_op);
 }
 TORCH_LIBRARY_IMPL(mi355q, Meta, m) {
   m.impl("amax", amax_op);
   m.impl("rowwise_amax", rowwise_amax_op);
+  m.impl("quantize_rows", quantize_rows_op);
 }

@@ -91,6 +91,23 @@ int mi355q_rowwise_amax(const void* x, int x_dtype, int64_t rows, int64_t cols,
                         float* amax_out, void* stream);
 
 /*
+ * Dynamic per-row ("per-token") quantisation in one pass over x [rows, cols]:
+ *   amax_r = max|x[r, :]|, scale_r = target / amax_r (fp32 division),
+ *   y[r, :] = cast_to_fp8(x[r, :] * scale_r)   with the rounding rules of mi355q_cast_to_fp8,
+ *   scale_out[r] = scale_r, scale_inv_out[r] = 1 / scale_r   (either may be NULL).
+ * Bit-identical to mi355q_rowwise_amax, the division on the host side and
+ * mi355q_cast_to_fp8 with MI355Q_SCALE_MID, which it replaces when a caller
+ * quantises activations on the fly.  The reference has no such op
+ * (fp8_ops.cpp:170-178: its amax is one scalar and the scale is computed by
+ * the caller).  Rows of up to 2048 16-byte vectors (16384 bf16 / 8192 fp32
+ * elements), x 16-byte aligned, cols a multiple of 8 (bf16) or 4 (fp32);
+ * otherwise MI355Q_ERR_UNSUPPORTED and the caller takes the three-step route.
+ */
+int mi355q_quantize_rows(const void* x, int x_dtype, int64_t rows, int64_t cols,
+                         void* y, int fp8_fmt, float target,
+                         float* scale_out, float* scale_inv_out, void* stream);
+
+/*
  * y = saturating round-to-nearest-even fp8( x * scale ), optional amax of x.
  * Replaces the convert_to_fp8_{f32,bf16} node built by CastToFp8V2::AddNode
  * (hpu_ops/backend/fp8_ops.cpp:192-258; round mode CAST_ROUND_HALF_NE,

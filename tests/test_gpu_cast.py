@@ -241,3 +241,58 @@ def test_c_abi_direct(oracle, pkg, dev):
     assert lib.mi355q_rowwise_amax(xd.data_ptr(), pkg.BF16, 128, 512, ra.data_ptr(), stream) == 0
     torch.cuda.synchronize()
     assert torch.equal(ra.cpu(), x.abs().amax(1).float())
+
+
+@pytest.mark.parametrize("out_dtype", FP8_DTYPES)
+@pytest.mark.parametrize("dtype,shape", [
+    (torch.bfloat16, (16, 8192)),        # decode-shaped activations
+    (torch.bfloat16, (513, 4096)),
+    (torch.bfloat16, (3, 5, 14336)),     # leading dims are rows
+    (torch.bfloat16, (7, 16392)),        # row longer than the one-pass kernel holds: three-step route
+    (torch.bfloat16, (9, 100)),          # not a multiple of 8: three-step route
+    (torch.float32, (64, 1024)),
+    (torch.float32, (5, 8196)),
+])
+def test_quantize_rows(oracle, pkg, dev, dtype, shape, out_dtype):
+    """Dynamic per-row quantisation equals rowwise amax -> target / amax -> cast with per-row scales,
+    bit for bit, both against the separate GPU ops and against the oracle."""
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(*shape, generator=g)
+    x[..., ::97] *= 20
+    x = x.to(dtype)
+    target = 448.0 if out_dtype == E4 else 57344.0
+    y, s_inv = torch.ops.mi355q.quantize_rows(x.to(dev), out_dtype)
+    assert y.shape == x.shape and s_inv.shape == x.shape[:-1] + (1,) and s_inv.dtype == torch.float32
+    amax = x.abs().amax(-1, keepdim=True).float()
+    # tensor / tensor is an IEEE division; torch evaluates scalar / tensor as scalar * (1 / tensor)
+    scale = torch.full_like(amax, target) / amax
+    x2 = x.reshape(-1, shape[-1])
+    ref, _ = oracle.c_cast_to_fp8(x2, scale.reshape(-1), out_dtype, scale_shape=[x2.shape[0], 1])
+    assert_fp8_equal(y.reshape(x2.shape), ref, out_dtype, "vs oracle")
+    assert torch.equal(s_inv.cpu(), torch.ones_like(scale) / scale)
+    amax_d = torch.ops.mi355q.rowwise_amax(x.to(dev)).reshape(-1, 1)
+    y3, _ = ops.cast_to_fp8_v2(x2.to(dev), torch.full_like(amax_d, target) / amax_d, False, False, out_dtype, [x2.shape[0], 1])
+    assert_fp8_equal(y.reshape(x2.shape), y3.cpu(), out_dtype, "vs the three GPU steps")
+
+
+def test_quantize_rows_c_abi(oracle, pkg, dev):
+    lib = pkg.capi()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    x = (torch.randn(33, 2048, generator=torch.Generator().manual_seed(5)) * 3).bfloat16()
+    xd = x.to(dev)
+    y = torch.empty(x.shape, dtype=E4, device=dev)
+    s = torch.empty(33, device=dev)
+    si = torch.empty(33, device=dev)
+    assert lib.mi355q_quantize_rows(xd.data_ptr(), pkg.BF16, 33, 2048, y.data_ptr(), pkg.E4M3FN, 448.0,
+                                    s.data_ptr(), si.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    amax = x.abs().amax(1).float()
+    scale = torch.full_like(amax, 448.0) / amax
+    assert torch.equal(s.cpu(), scale) and torch.equal(si.cpu(), torch.ones_like(scale) / scale)
+    ref, _ = oracle.c_cast_to_fp8(x, scale, E4, scale_shape=[33, 1])
+    assert_fp8_equal(y, ref, E4)
+    # rows that do not fit one workgroup's registers are refused, not mangled
+    assert lib.mi355q_quantize_rows(xd.data_ptr(), pkg.BF16, 1, 33 * 2048, y.data_ptr(), pkg.E4M3FN, 448.0,
+                                    None, None, stream) == 2
+    assert lib.mi355q_quantize_rows(xd.data_ptr(), pkg.BF16, 0, 2048, y.data_ptr(), pkg.E4M3FN, 448.0,
+                                    None, None, stream) == 0

@@ -209,3 +209,17 @@ def test_ops_trace_under_fake_tensors(pkg):
         x8, amax = torch.ops.hpu.cast_to_fp8_v2(x, None, False, True, E4)
         y = torch.ops.hpu.fp8_gemm_v2(x8, False, w, False, None, torch.bfloat16, 0.5, 0.25)
         assert x8.dtype == E4 and amax.shape == () and y.shape == (32, 48) and y.device.type == "cuda"
+
+
+def test_quantize_rows_meta(pkg):
+    """mi355q::quantize_rows: fp8 tensor shaped like the input, fp32 inverse scales [..., 1]."""
+    y, s = torch.ops.mi355q.quantize_rows(meta((3, 16, 64), torch.bfloat16), E4)
+    assert y.shape == (3, 16, 64) and y.dtype == E4
+    assert s.shape == (3, 16, 1) and s.dtype == torch.float32
+    with pytest.raises(RuntimeError, match="float or bfloat16"):
+        torch.ops.mi355q.quantize_rows(meta((4, 8), torch.float16), E4)
+    with pytest.raises(RuntimeError, match="float8"):
+        torch.ops.mi355q.quantize_rows(meta((4, 8), torch.float32), torch.bfloat16)
+    lib = pkg.capi()
+    assert lib.mi355q_quantize_rows(None, pkg.BF16, 4, 8, None, pkg.E4M3FN, 448.0, None, None, None) == 1
+    assert lib.mi355q_quantize_rows(None, pkg.BF16, 0, 8, None, pkg.E4M3FN, 448.0, None, None, None) == 0
