@@ -497,6 +497,53 @@ Tensor fp8_gemm_v2_scalar_list(const Tensor& A, bool trans_A, const Tensor& B, b
                           IValue(B_scale_inv.vec()), bias, accumulate, to_opt_shape(B_scale_shape));
 }
 
+// ------------------------------------------------ v1 ops (caller-allocated outputs)
+//
+// hpu::cast_to_fp8 and hpu::fp8_gemm, the deprecated forms that write into
+// tensors the caller passes (CastToFp8::AddNode, hpu_ops/backend/fp8_ops.cpp:
+// 123-166; Fp8Gemm::AddNode :312-366).  Same arithmetic as the v2 ops.
+
+std::tuple<Tensor&, Tensor&> cast_to_fp8_v1(const Tensor& input, const c10::optional<Tensor>& scale,
+                                            bool stochastic_rounding, Tensor& out, Tensor& amax) {
+  const auto src = input.scalar_type();
+  TORCH_CHECK(src == at::kFloat || src == at::kBFloat16, "CastToFp8 input must be of float or bfloat16 dtype.");
+  TORCH_CHECK(input.sizes() == out.sizes(), "Input and output must have the same shape");
+  TORCH_CHECK(is_fp8(out.scalar_type()), "cast_to_fp8: out must be float8_e4m3fn or float8_e5m2, got ", out.scalar_type());
+  TORCH_CHECK(!stochastic_rounding,
+              "cast_to_fp8: stochastic_rounding=True is not implemented in this build (round-to-nearest-even only)");
+  const bool is_amax = amax.numel() != 0;  // fp8_ops.cpp:138
+  TORCH_CHECK(!is_amax || amax.scalar_type() == at::kFloat, "cast_to_fp8: amax must be a float tensor");
+  if (input.is_meta()) return std::tuple<Tensor&, Tensor&>(out, amax);
+  DeviceGuard guard(input.device());
+  Tensor x = input.contiguous();
+  Tensor y = out.is_contiguous() ? out : at::empty(x.sizes(), x.options().dtype(out.scalar_type()));
+  Tensor am = is_amax ? at::empty({}, x.options().dtype(at::kFloat)) : Tensor();
+  CastScale cs = resolve_cast_scale(opt_tensor_iv(scale), c10::nullopt, x);
+  check_status(mi355q_cast_to_fp8(x.data_ptr(), to_mi355q_dtype(src), y.data_ptr(),
+                                  to_mi355q_dtype(out.scalar_type()), cs.dev, cs.host, cs.mode, cs.outer,
+                                  cs.mid, cs.inner, is_amax ? am.data_ptr<float>() : nullptr,
+                                  current_stream(x)),
+               "mi355q_cast_to_fp8");
+  if (!y.is_same(out)) out.copy_(y);
+  if (is_amax) amax.copy_(am.expand(amax.sizes()));
+  return std::tuple<Tensor&, Tensor&>(out, amax);
+}
+
+Tensor& fp8_gemm_v1(const Tensor& A, bool trans_A, const Tensor& B, bool trans_B, const Tensor& D,
+                    at::ScalarType out_dtype, const c10::optional<Tensor>& A_scale_inv,
+                    const c10::optional<Tensor>& B_scale_inv, const c10::optional<Tensor>& bias,
+                    bool accumulate, Tensor& out) {
+  TORCH_CHECK(out.scalar_type() == out_dtype, "fp8_gemm: out has dtype ", out.scalar_type(),
+              " but out_dtype is ", out_dtype);
+  // D may be the very tensor `out`: the result is complete before it is copied in
+  Tensor r = fp8_gemm_v2_impl(A, trans_A, B, trans_B, c10::optional<Tensor>(D), out_dtype,
+                              opt_tensor_iv(A_scale_inv), opt_tensor_iv(B_scale_inv), bias, accumulate,
+                              c10::nullopt);
+  TORCH_CHECK(r.sizes() == out.sizes(), "fp8_gemm: out has shape ", out.sizes(), ", the product has ", r.sizes());
+  if (!out.is_meta()) out.copy_(r);
+  return out;
+}
+
 // ------------------------------------------------- convert_from_int4 / uint4
 
 Tensor convert_from_int4_common(const char* op_name, bool is_signed, const Tensor& input,
@@ -644,6 +691,8 @@ TORCH_LIBRARY(hpu, m) {
   m.def("hpu::cast_from_fp8(Tensor input, Tensor? scale, ScalarType out_dtype, int[]? scale_shape=None) -> Tensor");
   m.def("hpu::cast_from_fp8.scalar(Tensor input, float scale, ScalarType out_dtype, int[]? scale_shape=None) -> Tensor");
   m.def("hpu::cast_from_fp8.scalar_list(Tensor input, float[] scale, ScalarType out_dtype, int[]? scale_shape=None) -> Tensor");
+  m.def("hpu::cast_to_fp8(Tensor input, Tensor? scale, bool stochastic_rounding, Tensor(a!) out, Tensor(b!) amax) -> (Tensor(a!), Tensor(b!))");
+  m.def("hpu::fp8_gemm(Tensor A, bool trans_A, Tensor B, bool trans_B, Tensor D, ScalarType out_dtype, Tensor? A_scale_inv, Tensor? B_scale_inv, Tensor? bias, bool accumulate, Tensor(a!) out) -> Tensor(a!)");
   m.def("hpu::cast_to_fp8_v2(Tensor input, Tensor? scale=None, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)");
   m.def("hpu::cast_to_fp8_v2.scalar(Tensor input, float scale, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)");
   m.def("hpu::cast_to_fp8_v2.scalar_list(Tensor input, float[] scale, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)");
@@ -672,7 +721,9 @@ TORCH_LIBRARY(mi355q, m) {
   m.impl("fp8_gemm_v2.scalar", fp8_gemm_v2_scalar);                                            \
   m.impl("fp8_gemm_v2.scalar_list", fp8_gemm_v2_scalar_list);                                  \
   m.impl("convert_from_int4", convert_from_int4);                                              \
-  m.impl("convert_from_uint4", convert_from_uint4);
+  m.impl("convert_from_uint4", convert_from_uint4);                                            \
+  m.impl("cast_to_fp8", cast_to_fp8_v1);                                                       \
+  m.impl("fp8_gemm", fp8_gemm_v1);
 
 TORCH_LIBRARY_IMPL(hpu, CUDA, m) { MI355Q_REGISTER_HPU(m) }
 TORCH_LIBRARY_IMPL(hpu, Meta, m) { MI355Q_REGISTER_HPU(m) }
