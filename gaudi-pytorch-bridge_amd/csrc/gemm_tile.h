@@ -206,6 +206,22 @@ struct DmaLoader {
 #pragma unroll
     for (int i = 0; i < kPerWave; ++i) voff[i] += step;
   }
+
+  // Recomputes the per-lane offsets as init() left them plus `stages` advances.
+  // Called after an epilogue: the offsets are then dead while the epilogue
+  // runs, where every register is taken, instead of being spilled around it
+  // (a spill there is a store to memory by every lane for every tile).
+  __device__ __forceinline__ void rebuild_offsets(int64_t ld, int stages) {
+    int lane = threadIdx.x & 63;
+    asm volatile("" : "+v"(lane));
+    const int rin = lane / kCPR, p = lane % kCPR;
+#pragma unroll
+    for (int i = 0; i < kPerWave; ++i) {
+      const int row = (wave * kPerWave + i) * kRowsPerRegion + rin;
+      const int c = p ^ G::swizzle(row);
+      voff[i] = row * (int)ld + c * 16 + stages * step;
+    }
+  }
 };
 
 // A 32-byte MFMA fragment (32 rows of m/n x 32 k for this lane's k-half) is
@@ -785,6 +801,9 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g)
       epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
     }
     if (idx >= count) break;
+    // the loaders stand two stages into the next tile
+    core.la.rebuild_offsets(g.lda, 2);
+    core.lb.rebuild_offsets(g.ldb, 2);
   }
   // drain the (out-of-range) loads issued for the tile that does not exist
   __builtin_amdgcn_s_waitcnt(0);
