@@ -294,7 +294,17 @@ def bench_gemm_c3(ops, oracle, pkg, dev, steps, warmup, cpu):
                      "cores": torch.get_num_threads(), "kind": "port",
                      "sample": f"the full problem ({rows} rows of A), median of up to 5 runs / 10 s: "
                                "((A8.float() @ B8.float()) * sA * sB + bias).bfloat16()"}
-    return {"ms": ms, "tflops": tflops, "flop": flop, "variant": variant, "cpu": cpu_entry}
+    # the vendor library's fp8 GEMM on the same problem, as a calibration point for what this
+    # machine sustains (it wants B column-major, its preferred layout; no bias)
+    lib_tflops = None
+    try:
+        w8_cm = w8.t().contiguous().t()
+        lib_ms = time_gpu(lambda i: torch._scaled_mm(a8, w8_cm, scale_a=sa_inv, scale_b=sw_inv, out_dtype=torch.bfloat16),
+                          steps, warmup)
+        lib_tflops = round(flop / (lib_ms * 1e-3) / 1e12, 1)
+    except Exception:  # noqa: BLE001 - the comparison is optional, the library may refuse the call
+        pass
+    return {"ms": ms, "tflops": tflops, "flop": flop, "variant": variant, "cpu": cpu_entry, "library": lib_tflops}
 
 
 def bench_gemm_decode(ops, oracle, dev, steps, warmup):
@@ -421,7 +431,8 @@ def main():
         g = bench_gemm_c3(ops, oracle, pkg, dev, args.steps, args.warmup, cpu)
         line.update({"value": round(g["tflops"], 1), "unit": "TFLOP/s", "ms_per_step": round(g["ms"], 4),
                      "config": {"workload": "C3 fp8_gemm_v2 M=8192 K=4096 N=14336 e4m3fn, per-tensor scales, bf16 bias",
-                                "kernel_variant": g["variant"]},
+                                "kernel_variant": g["variant"],
+                                "library_gemm_tflops_same_shape": g["library"]},
                      "roofline": {"bound": "mfma", "kernel": "fp8_gemm_tile_kernel", "achieved": round(g["tflops"], 1),
                                   "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(g["tflops"] / FP8_PEAK_TFLOPS, 4),
                                   "algorithmic_flop": g["flop"], "traffic": MEASURED_TRAFFIC.get("fp8_gemm_v2")}})

@@ -180,6 +180,53 @@ __global__ __launch_bounds__(kThreads) void cast_to_fp8_generic(
   if (amax != nullptr) block_amax_commit(am, amax);
 }
 
+// Stochastic-rounding cast: four consecutive elements per thread, any scale
+// broadcast, optional amax.  Not a bandwidth-tuned path (training-side casts of
+// optimizer state use it, the inference path rounds to nearest).
+template <bool BF16_IN, int FMT>
+__global__ __launch_bounds__(kThreads) void cast_to_fp8_sr_kernel(
+    const uint8_t* __restrict__ x, uint8_t* __restrict__ y, const float* __restrict__ scale,
+    float scale_host, int mode, int64_t n, int64_t mid, int64_t inner, uint64_t seed, uint64_t offset,
+    uint32_t* __restrict__ amax) {
+  const int64_t q = (int64_t)blockIdx.x * kThreads + threadIdx.x;  // index of this thread's quad
+  const int64_t i0 = q * 4;
+  uint32_t am = 0;
+  if (i0 < n) {
+    float p[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int64_t i = i0 + e < n ? i0 + e : n - 1;
+      float s = 1.0f;
+      if (mode == MI355Q_SCALE_HOST) s = scale_host;
+      else if (mode == MI355Q_SCALE_DEV) s = scale[0];
+      else if (mode == MI355Q_SCALE_MID) s = scale[(i / inner) % mid];
+      else if (mode == MI355Q_SCALE_FULL) s = scale[i];
+      float v;
+      if constexpr (BF16_IN) {
+        v = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(x)[i]);
+        p[e] = round_to_bf16(v * round_to_bf16(s));
+      } else {
+        v = reinterpret_cast<const float*>(x)[i];
+        p[e] = v * s;
+      }
+      const uint32_t a = __float_as_uint(v) & 0x7fffffffu;
+      am = am > a ? am : a;
+    }
+    const uint64_t ra = counter_random64(seed, offset + 2 * (uint64_t)q);
+    const uint64_t rb = counter_random64(seed, offset + 2 * (uint64_t)q + 1);
+    const uint32_t o = cvt_fp8x4_sr<FMT>(p[0], p[1], p[2], p[3], (uint32_t)ra, (uint32_t)(ra >> 32),
+                                         (uint32_t)rb, (uint32_t)(rb >> 32));
+    if (i0 + 3 < n && (reinterpret_cast<uintptr_t>(y) & 3u) == 0) {
+      reinterpret_cast<uint32_t*>(y)[q] = o;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (i0 + e < n) y[i0 + e] = (uint8_t)(o >> (8 * e));
+    }
+  }
+  if (amax != nullptr) block_amax_commit(am, amax);
+}
+
 // ---------------------------------------------------------------------- amax
 template <bool BF16_IN, int U>
 __global__ __launch_bounds__(kAmaxThreads) void amax_vec(const uint8_t* __restrict__ x, int64_t nvec,
@@ -671,6 +718,33 @@ int mi355q_rowwise_amax(const void* x, int x_dtype, int64_t rows, int64_t cols, 
   const uint8_t* xb = static_cast<const uint8_t*>(x);
   if (x_dtype == MI355Q_BF16) rowwise_amax_kernel<true><<<(unsigned)rows, kThreads, 0, st>>>(xb, cols, vec_ok, amax_out);
   else rowwise_amax_kernel<false><<<(unsigned)rows, kThreads, 0, st>>>(xb, cols, vec_ok, amax_out);
+  return launch_status();
+}
+
+int mi355q_cast_to_fp8_sr(const void* x, int x_dtype, void* y, int fp8_fmt, const float* scale_dev,
+                          float scale_host, int scale_mode, int64_t outer, int64_t mid, int64_t inner,
+                          float* amax_out, uint64_t seed, uint64_t offset, void* stream) {
+  if (fp8_fmt != MI355Q_E4M3FN && fp8_fmt != MI355Q_E5M2) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (x_dtype != MI355Q_F32 && x_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (!scale_args_ok(scale_dev, scale_mode, outer, mid, inner)) return MI355Q_ERR_INVALID_ARGUMENT;
+  const int64_t n = outer * mid * inner;
+  if (n > 0 && (x == nullptr || y == nullptr)) return MI355Q_ERR_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint32_t* am = reinterpret_cast<uint32_t*>(amax_out);
+  if (am) fill_u32_kernel<<<1, 1, 0, st>>>(am, 0u);
+  if (n == 0) return launch_status();
+  const int64_t grid = ((n + 3) / 4 + kThreads - 1) / kThreads;
+  if (grid > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  uint8_t* yb = static_cast<uint8_t*>(y);
+  const unsigned g = (unsigned)grid;
+  if (x_dtype == MI355Q_BF16) {
+    if (fp8_fmt == MI355Q_E4M3FN) cast_to_fp8_sr_kernel<true, MI355Q_E4M3FN><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, am);
+    else cast_to_fp8_sr_kernel<true, MI355Q_E5M2><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, am);
+  } else {
+    if (fp8_fmt == MI355Q_E4M3FN) cast_to_fp8_sr_kernel<false, MI355Q_E4M3FN><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, am);
+    else cast_to_fp8_sr_kernel<false, MI355Q_E5M2><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, am);
+  }
   return launch_status();
 }
 

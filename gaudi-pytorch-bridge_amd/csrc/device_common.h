@@ -58,6 +58,40 @@ __device__ __forceinline__ uint32_t cvt_fp8x4(float a, float b, float c, float d
   return (uint32_t)r;
 }
 
+// Stochastic rounding of four fp32 to fp8 (v_cvt_sr_fp8_f32 / v_cvt_sr_bf8_f32:
+// the 32 random bits are added below the kept mantissa before truncation), after
+// the same saturating clamp as the round-to-nearest path.
+template <int FMT>
+__device__ __forceinline__ uint32_t cvt_fp8x4_sr(float a, float b, float c, float d, uint32_t r0,
+                                                 uint32_t r1, uint32_t r2, uint32_t r3) {
+  a = sat_fp8<FMT>(a);
+  b = sat_fp8<FMT>(b);
+  c = sat_fp8<FMT>(c);
+  d = sat_fp8<FMT>(d);
+  int r = 0;
+  if constexpr (FMT == MI355Q_E5M2) {
+    r = __builtin_amdgcn_cvt_sr_bf8_f32(a, r0, r, 0);
+    r = __builtin_amdgcn_cvt_sr_bf8_f32(b, r1, r, 1);
+    r = __builtin_amdgcn_cvt_sr_bf8_f32(c, r2, r, 2);
+    r = __builtin_amdgcn_cvt_sr_bf8_f32(d, r3, r, 3);
+  } else {
+    r = __builtin_amdgcn_cvt_sr_fp8_f32(a, r0, r, 0);
+    r = __builtin_amdgcn_cvt_sr_fp8_f32(b, r1, r, 1);
+    r = __builtin_amdgcn_cvt_sr_fp8_f32(c, r2, r, 2);
+    r = __builtin_amdgcn_cvt_sr_fp8_f32(d, r3, r, 3);
+  }
+  return (uint32_t)r;
+}
+
+// 64 random bits for counter `idx` of stream `seed` (the splitmix64 finaliser:
+// stateless, so an element's bits depend only on its index and the seed).
+__device__ __forceinline__ uint64_t counter_random64(uint64_t seed, uint64_t idx) {
+  uint64_t z = seed + (idx + 1) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
 // four fp8 bytes of one dword -> four fp32 (exact)
 template <int FMT>
 __device__ __forceinline__ void cvt_f32x4(uint32_t w, float& a, float& b, float& c, float& d) {

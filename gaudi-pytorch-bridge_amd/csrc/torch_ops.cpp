@@ -13,6 +13,7 @@
 // for HIP tensors) and for Meta.  There is no CPU implementation: a CPU tensor
 // fails in the dispatcher.
 #include <ATen/ATen.h>
+#include <ATen/hip/HIPGeneratorImpl.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/library.h>
@@ -175,6 +176,27 @@ CastScale resolve_cast_scale(const IValue& scale, const OptShape& scale_shape, c
   return r;
 }
 
+// (seed, offset) for `numel` stochastically rounded elements, drawn from the
+// device's default generator the way torch's own random kernels do, so that
+// torch.manual_seed makes the cast reproducible and successive casts differ.
+std::pair<uint64_t, uint64_t> reserve_random(const Tensor& t, int64_t numel) {
+  auto gen = at::get_generator_or_default<at::CUDAGeneratorImpl>(
+      c10::nullopt, at::cuda::detail::getDefaultCUDAGenerator(t.device().index()));
+  std::lock_guard<std::mutex> lock(gen->mutex_);
+  return gen->philox_engine_inputs((uint64_t)((numel + 1) / 2));
+}
+
+// One call for both rounding modes.
+int launch_cast_to(const Tensor& x, Tensor& out, const CastScale& cs, float* amax, bool stochastic) {
+  const int xd = to_mi355q_dtype(x.scalar_type()), od = to_mi355q_dtype(out.scalar_type());
+  if (!stochastic)
+    return mi355q_cast_to_fp8(x.data_ptr(), xd, out.data_ptr(), od, cs.dev, cs.host, cs.mode, cs.outer, cs.mid,
+                              cs.inner, amax, current_stream(x));
+  const auto r = reserve_random(x, x.numel());
+  return mi355q_cast_to_fp8_sr(x.data_ptr(), xd, out.data_ptr(), od, cs.dev, cs.host, cs.mode, cs.outer, cs.mid,
+                               cs.inner, amax, r.first, r.second, current_stream(x));
+}
+
 // ------------------------------------------------------------ cast_to_fp8_v2
 
 void check_cast_to_args(const Tensor& input, bool stochastic_rounding, bool is_amax,
@@ -193,9 +215,7 @@ void check_cast_to_args(const Tensor& input, bool stochastic_rounding, bool is_a
                 src, " and ", dst);
   }
   validate_scale_shape(scale, scale_shape);
-  TORCH_CHECK(!stochastic_rounding,
-              "cast_to_fp8_v2: stochastic_rounding=True is not implemented in this build "
-              "(round-to-nearest-even only)");
+  TORCH_CHECK(!(stochastic_rounding && fp8_in), "cast_to_fp8_v2: stochastic rounding needs a float or bfloat16 input");
 }
 
 OptShape shape_from_ivalue(const IValue& v) {
@@ -239,11 +259,7 @@ void cast_to_fp8_v2_boxed(const c10::OperatorHandle& op, c10::DispatchKeySet, to
     } else {
       cs = resolve_cast_scale(scale, scale_shape, x);
     }
-    check_status(mi355q_cast_to_fp8(x.data_ptr(), to_mi355q_dtype(x.scalar_type()), out.data_ptr(),
-                                    to_mi355q_dtype(dst), cs.dev, cs.host, cs.mode, cs.outer, cs.mid,
-                                    cs.inner, is_amax ? amax.data_ptr<float>() : nullptr,
-                                    current_stream(x)),
-                 "mi355q_cast_to_fp8");
+    check_status(launch_cast_to(x, out, cs, is_amax ? amax.data_ptr<float>() : nullptr, sr), "mi355q_cast_to_fp8");
   }
   torch::jit::drop(*stack, 6);
   stack->emplace_back(std::move(out));
@@ -509,8 +525,6 @@ std::tuple<Tensor&, Tensor&> cast_to_fp8_v1(const Tensor& input, const c10::opti
   TORCH_CHECK(src == at::kFloat || src == at::kBFloat16, "CastToFp8 input must be of float or bfloat16 dtype.");
   TORCH_CHECK(input.sizes() == out.sizes(), "Input and output must have the same shape");
   TORCH_CHECK(is_fp8(out.scalar_type()), "cast_to_fp8: out must be float8_e4m3fn or float8_e5m2, got ", out.scalar_type());
-  TORCH_CHECK(!stochastic_rounding,
-              "cast_to_fp8: stochastic_rounding=True is not implemented in this build (round-to-nearest-even only)");
   const bool is_amax = amax.numel() != 0;  // fp8_ops.cpp:138
   TORCH_CHECK(!is_amax || amax.scalar_type() == at::kFloat, "cast_to_fp8: amax must be a float tensor");
   if (input.is_meta()) return std::tuple<Tensor&, Tensor&>(out, amax);
@@ -519,10 +533,7 @@ std::tuple<Tensor&, Tensor&> cast_to_fp8_v1(const Tensor& input, const c10::opti
   Tensor y = out.is_contiguous() ? out : at::empty(x.sizes(), x.options().dtype(out.scalar_type()));
   Tensor am = is_amax ? at::empty({}, x.options().dtype(at::kFloat)) : Tensor();
   CastScale cs = resolve_cast_scale(opt_tensor_iv(scale), c10::nullopt, x);
-  check_status(mi355q_cast_to_fp8(x.data_ptr(), to_mi355q_dtype(src), y.data_ptr(),
-                                  to_mi355q_dtype(out.scalar_type()), cs.dev, cs.host, cs.mode, cs.outer,
-                                  cs.mid, cs.inner, is_amax ? am.data_ptr<float>() : nullptr,
-                                  current_stream(x)),
+  check_status(launch_cast_to(x, y, cs, is_amax ? am.data_ptr<float>() : nullptr, stochastic_rounding),
                "mi355q_cast_to_fp8");
   if (!y.is_same(out)) out.copy_(y);
   if (is_amax) amax.copy_(am.expand(amax.sizes()));

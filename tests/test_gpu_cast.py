@@ -296,3 +296,65 @@ def test_quantize_rows_c_abi(oracle, pkg, dev):
                                     None, None, stream) == 2
     assert lib.mi355q_quantize_rows(xd.data_ptr(), pkg.BF16, 0, 2048, y.data_ptr(), pkg.E4M3FN, 448.0,
                                     None, None, stream) == 0
+
+
+def fp8_grid(dtype):
+    """All finite values of an fp8 format, ascending."""
+    codes = torch.arange(256, dtype=torch.uint8).view(dtype).float()
+    return torch.unique(codes[torch.isfinite(codes)])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("out_dtype", FP8_DTYPES)
+@pytest.mark.parametrize("is_amax", [True, False])
+def test_stochastic_rounding(oracle, dev, dtype, out_dtype, is_amax):
+    """stochastic_rounding=True (test_hpu_fp8_ops_any_mode.py:124-128 and test_hpu_fp8_te.py:89-150):
+    every output is one of the two fp8 neighbours of the exact scaled value, the result differs from
+    round-to-nearest, the mean is preserved, amax is untouched by the rounding mode."""
+    g = torch.Generator().manual_seed(31)
+    pos = torch.rand(256, 333, generator=g).to(dtype) * 30 + 10
+    x = torch.cat((pos, -pos))
+    scale = torch.tensor(1.3)
+    torch.manual_seed(1234)
+    y, amax = ops.cast_to_fp8_v2(x.to(dev), scale.to(dev), True, is_amax, out_dtype)
+    p = (x * scale.to(dtype)).float()            # the value that gets rounded (bf16 product for bf16 input)
+    grid = fp8_grid(out_dtype)
+    hi_i = torch.searchsorted(grid, p.contiguous()).clamp(max=grid.numel() - 1)
+    lo_i = (hi_i - (grid[hi_i] != p).long()).clamp(min=0)
+    yv = y.cpu().float()
+    assert ((yv == grid[lo_i]) | (yv == grid[hi_i])).all()
+    rne, _ = oracle.c_cast_to_fp8(x, scale, out_dtype)
+    assert not torch.equal(yv, rne.float())
+    back = ops.cast_from_fp8(y, scale.reciprocal().to(dev), dtype).cpu()
+    ref_back = oracle.c_cast_from_fp8(rne, scale.reciprocal(), dtype)
+    assert torch.allclose(back, ref_back, rtol=0.26, atol=0.0)      # the reference's own bound
+    if is_amax:
+        assert amax.cpu() == x.abs().max().float() and amax.dim() == 0
+    else:
+        assert amax.numel() == 0
+    # reproducible under the torch seed, and successive calls draw fresh bits
+    torch.manual_seed(1234)
+    y2, _ = ops.cast_to_fp8_v2(x.to(dev), scale.to(dev), True, False, out_dtype)
+    y3, _ = ops.cast_to_fp8_v2(x.to(dev), scale.to(dev), True, False, out_dtype)
+    assert torch.equal(y2.view(torch.uint8), y.view(torch.uint8))
+    assert not torch.equal(y3.view(torch.uint8), y.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("fmt,lo,hi,max_diff", [(E4, 18.0, 20.0, 0.4), (E5, 16.0, 20.0, 0.8)])
+def test_stochastic_rounding_is_unbiased(dev, dtype, fmt, lo, hi, max_diff):
+    """test_hpu_fp8_te.py:105-150: 18.5 rounds to 18 / 20 (e4m3fn) or 16 / 20 (e5m2) with probabilities
+    that keep the mean; here also checked as a rate on 2^18 draws (binomial sigma below 0.001)."""
+    x = torch.full((1 << 18,), 18.5, dtype=dtype, device=dev)
+    torch.manual_seed(7)
+    y = ops.cast_to_fp8_v2(x, None, True, False, fmt)[0].float().cpu()
+    assert set(y.unique().tolist()) == {lo, hi}
+    assert abs(y[:1000].mean().item() - 18.5) < max_diff
+    p_up = (18.5 - lo) / (hi - lo)
+    assert abs((y == hi).float().mean().item() - p_up) < 0.01
+    rne = ops.cast_to_fp8_v2(x, None, False, False, fmt)[0].float().cpu()
+    assert (rne == (18.0 if fmt == E4 else 20.0)).all()
+    # values on the fp8 grid are never moved, saturation still applies
+    z = torch.tensor([448.0, -448.0, 1e6, -1e6, 0.0, 0.5], dtype=dtype, device=dev)
+    zz = ops.cast_to_fp8_v2(z, None, True, False, E4)[0].float().cpu()
+    assert zz.tolist() == [448.0, -448.0, 448.0, -448.0, 0.0, 0.5]

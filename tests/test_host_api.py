@@ -120,8 +120,11 @@ def test_cast_to_fp8_v2_errors(pkg):
         torch.ops.hpu.cast_to_fp8_v2(meta((16, 24, 8), torch.bfloat16), meta((8,), torch.float32), False, False, E4, [24, 1])
     with pytest.raises(RuntimeError, match="dtype must be given"):
         torch.ops.hpu.cast_to_fp8_v2(meta((4,), torch.float32))
-    with pytest.raises(RuntimeError, match="stochastic_rounding=True is not implemented"):
-        torch.ops.hpu.cast_to_fp8_v2(meta((4,), torch.float32), None, True, False, E4)
+    # stochastic rounding changes values, not shapes (GetCastParams, fp8_ops.cpp:105-119)
+    y, a = torch.ops.hpu.cast_to_fp8_v2(meta((4,), torch.float32), None, True, False, E4)
+    assert y.shape == (4,) and y.dtype == E4 and a.shape == (0,)
+    with pytest.raises(RuntimeError, match="stochastic rounding needs a float or bfloat16 input"):
+        torch.ops.hpu.cast_to_fp8_v2(meta((4,), E4), None, True, False, E4)
 
 
 def test_cast_from_fp8_meta_and_errors(pkg):
