@@ -227,6 +227,87 @@ __global__ __launch_bounds__(kThreads) void cast_to_fp8_sr_kernel(
   if (amax != nullptr) block_amax_commit(am, amax);
 }
 
+// ------------------------------------------------------------ cast_to_fp8_hybrid
+//
+// One read of x, two fp8 tensors out (e5m2 with scale_152, e4m3fn with scale_143)
+// and optionally amax.  Stochastic rounding applies to the e5m2 output only; the
+// e4m3fn output always rounds to nearest even.  Scales are per tensor.
+// [first, first + count) elements; VEC = 8 elements per thread per step when the
+// pointers allow 16-byte loads, else 1.
+template <bool BF16_IN, int VEC>
+__global__ __launch_bounds__(kAmaxThreads) void cast_to_fp8_hybrid_kernel(
+    const uint8_t* __restrict__ x, uint8_t* __restrict__ y152, uint8_t* __restrict__ y143,
+    const float* __restrict__ scale152, const float* __restrict__ scale143, int64_t first, int64_t count,
+    int stochastic, uint64_t seed, uint64_t offset, uint32_t* __restrict__ amax) {
+  float s5 = scale152 ? scale152[0] : 1.0f, s4 = scale143 ? scale143[0] : 1.0f;
+  if constexpr (BF16_IN) {
+    s5 = round_to_bf16(s5);
+    s4 = round_to_bf16(s4);
+  }
+  uint32_t am = 0;
+  const int64_t steps = (count + VEC - 1) / VEC;
+  for (int64_t t = (int64_t)blockIdx.x * kAmaxThreads + threadIdx.x; t < steps; t += (int64_t)gridDim.x * kAmaxThreads) {
+    const int64_t i0 = first + t * VEC;
+    float v[VEC];
+    if constexpr (VEC == 8) {
+      if constexpr (BF16_IN) {
+        const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + i0 * 2));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[2 * i] = __uint_as_float(w[i] << 16);
+          v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+      } else {
+        const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + i0 * 4));
+        const f32x4 b = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x + i0 * 4) + 1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[i] = a[i];
+          v[4 + i] = b[i];
+        }
+      }
+    } else {
+      v[0] = BF16_IN ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(x)[i0]) : reinterpret_cast<const float*>(x)[i0];
+    }
+    float p5[VEC], p4[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const uint32_t a = __float_as_uint(v[i]) & 0x7fffffffu;
+      am = am > a ? am : a;
+      p5[i] = BF16_IN ? round_to_bf16(v[i] * s5) : v[i] * s5;
+      p4[i] = BF16_IN ? round_to_bf16(v[i] * s4) : v[i] * s4;
+    }
+    if constexpr (VEC == 8) {
+      u32x2 o5, o4;
+      o4.x = cvt_fp8x4<MI355Q_E4M3FN>(p4[0], p4[1], p4[2], p4[3]);
+      o4.y = cvt_fp8x4<MI355Q_E4M3FN>(p4[4], p4[5], p4[6], p4[7]);
+      if (stochastic) {
+        // element i0 + e draws from counter (i0 + e) / 2, as a scalar step does
+        const uint64_t c = offset + (uint64_t)(i0 >> 1);
+        const uint64_t r0 = counter_random64(seed, c), r1 = counter_random64(seed, c + 1);
+        const uint64_t r2 = counter_random64(seed, c + 2), r3 = counter_random64(seed, c + 3);
+        o5.x = cvt_fp8x4_sr<MI355Q_E5M2>(p5[0], p5[1], p5[2], p5[3], (uint32_t)r0, (uint32_t)(r0 >> 32), (uint32_t)r1, (uint32_t)(r1 >> 32));
+        o5.y = cvt_fp8x4_sr<MI355Q_E5M2>(p5[4], p5[5], p5[6], p5[7], (uint32_t)r2, (uint32_t)(r2 >> 32), (uint32_t)r3, (uint32_t)(r3 >> 32));
+      } else {
+        o5.x = cvt_fp8x4<MI355Q_E5M2>(p5[0], p5[1], p5[2], p5[3]);
+        o5.y = cvt_fp8x4<MI355Q_E5M2>(p5[4], p5[5], p5[6], p5[7]);
+      }
+      __builtin_nontemporal_store(o5, reinterpret_cast<u32x2*>(y152 + i0));
+      __builtin_nontemporal_store(o4, reinterpret_cast<u32x2*>(y143 + i0));
+    } else {
+      y143[i0] = (uint8_t)(cvt_fp8x4<MI355Q_E4M3FN>(p4[0], p4[0], p4[0], p4[0]) & 0xffu);
+      if (stochastic) {
+        const uint64_t r = counter_random64(seed, offset + (uint64_t)(i0 >> 1));
+        const uint32_t rr = (i0 & 1) ? (uint32_t)(r >> 32) : (uint32_t)r;
+        y152[i0] = (uint8_t)(cvt_fp8x4_sr<MI355Q_E5M2>(p5[0], p5[0], p5[0], p5[0], rr, rr, rr, rr) & 0xffu);
+      } else {
+        y152[i0] = (uint8_t)(cvt_fp8x4<MI355Q_E5M2>(p5[0], p5[0], p5[0], p5[0]) & 0xffu);
+      }
+    }
+  }
+  if (amax != nullptr) block_amax_commit(am, amax);
+}
+
 // ---------------------------------------------------------------------- amax
 template <bool BF16_IN, int U>
 __global__ __launch_bounds__(kAmaxThreads) void amax_vec(const uint8_t* __restrict__ x, int64_t nvec,
@@ -744,6 +825,38 @@ int mi355q_cast_to_fp8_sr(const void* x, int x_dtype, void* y, int fp8_fmt, cons
   } else {
     if (fp8_fmt == MI355Q_E4M3FN) cast_to_fp8_sr_kernel<false, MI355Q_E4M3FN><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, am);
     else cast_to_fp8_sr_kernel<false, MI355Q_E5M2><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, am);
+  }
+  return launch_status();
+}
+
+int mi355q_cast_to_fp8_hybrid(const void* x, int x_dtype, int64_t n, void* y_e5m2, void* y_e4m3fn,
+                              const float* scale_e5m2, const float* scale_e4m3fn, int stochastic,
+                              uint64_t seed, uint64_t offset, float* amax_out, void* stream) {
+  if (n < 0 || (x_dtype != MI355Q_F32 && x_dtype != MI355Q_BF16)) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (n > 0 && (x == nullptr || y_e5m2 == nullptr || y_e4m3fn == nullptr)) return MI355Q_ERR_INVALID_ARGUMENT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint32_t* am = reinterpret_cast<uint32_t*>(amax_out);
+  if (am) fill_u32_kernel<<<1, 1, 0, st>>>(am, 0u);
+  if (n == 0) return launch_status();
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  uint8_t* y5 = static_cast<uint8_t*>(y_e5m2);
+  uint8_t* y4 = static_cast<uint8_t*>(y_e4m3fn);
+  const int64_t max_blocks = am ? kAmaxBlocks : 4 * kAmaxBlocks;
+  auto grid_for = [&](int64_t steps) {
+    const int64_t b = (steps + kAmaxThreads - 1) / kAmaxThreads;
+    return (unsigned)(b < max_blocks ? b : max_blocks);
+  };
+  int64_t done = 0;
+  if (aligned(x, 16) && aligned(y5, 8) && aligned(y4, 8) && n >= 8) {
+    const int64_t nv = n / 8;
+    if (x_dtype == MI355Q_BF16) cast_to_fp8_hybrid_kernel<true, 8><<<grid_for(nv), kAmaxThreads, 0, st>>>(xb, y5, y4, scale_e5m2, scale_e4m3fn, 0, nv * 8, stochastic, seed, offset, am);
+    else cast_to_fp8_hybrid_kernel<false, 8><<<grid_for(nv), kAmaxThreads, 0, st>>>(xb, y5, y4, scale_e5m2, scale_e4m3fn, 0, nv * 8, stochastic, seed, offset, am);
+    done = nv * 8;
+  }
+  if (done < n) {
+    const int64_t rest = n - done;
+    if (x_dtype == MI355Q_BF16) cast_to_fp8_hybrid_kernel<true, 1><<<grid_for(rest), kAmaxThreads, 0, st>>>(xb, y5, y4, scale_e5m2, scale_e4m3fn, done, rest, stochastic, seed, offset, am);
+    else cast_to_fp8_hybrid_kernel<false, 1><<<grid_for(rest), kAmaxThreads, 0, st>>>(xb, y5, y4, scale_e5m2, scale_e4m3fn, done, rest, stochastic, seed, offset, am);
   }
   return launch_status();
 }

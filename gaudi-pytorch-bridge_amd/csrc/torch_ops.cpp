@@ -555,6 +555,44 @@ Tensor& fp8_gemm_v1(const Tensor& A, bool trans_A, const Tensor& B, bool trans_B
   return out;
 }
 
+// ------------------------------------------------------- cast_to_fp8_hybrid
+//
+// hpu::cast_to_fp8_hybrid (scripts/hpu_op.yaml:7365-7371; CastToFp8HybridMeta and
+// CastToFp8Hybrid::AddNode, hpu_ops/backend/cast_to_fp8_hybrid_gen.cpp:39-100).
+std::tuple<Tensor, Tensor, Tensor> cast_to_fp8_hybrid(const Tensor& input, const c10::optional<Tensor>& scale_152,
+                                                      const c10::optional<Tensor>& scale_143,
+                                                      bool stochastic_rounding, bool is_amax) {
+  const auto src = input.scalar_type();
+  TORCH_CHECK(src == at::kFloat || src == at::kBFloat16, "CastToFp8Hybrid input must be of float or bfloat16 dtype.");
+  auto scalar_scale = [&](const c10::optional<Tensor>& s, const char* name) -> Tensor {
+    if (!s.has_value() || !s->defined()) return Tensor();
+    TORCH_CHECK(s->numel() == 1, "cast_to_fp8_hybrid: ", name, " must hold one element, got ", s->numel());
+    if (s->is_meta()) return *s;
+    TORCH_CHECK(s->device() == input.device(), "cast_to_fp8_hybrid: ", name, " must be on the device of input");
+    return s->to(at::kFloat).contiguous();
+  };
+  Tensor s5 = scalar_scale(scale_152, "scale_152"), s4 = scalar_scale(scale_143, "scale_143");
+  const std::vector<int64_t> amax_shape = is_amax ? std::vector<int64_t>{} : std::vector<int64_t>{0};
+  if (input.is_meta())
+    return {at::empty(input.sizes(), input.options().dtype(at::kFloat8_e5m2)),
+            at::empty(input.sizes(), input.options().dtype(at::kFloat8_e4m3fn)),
+            at::empty(amax_shape, input.options().dtype(at::kFloat))};
+  DeviceGuard guard(input.device());
+  Tensor x = input.contiguous();
+  Tensor y5 = at::empty(x.sizes(), x.options().dtype(at::kFloat8_e5m2));
+  Tensor y4 = at::empty(x.sizes(), x.options().dtype(at::kFloat8_e4m3fn));
+  Tensor amax = at::empty(amax_shape, x.options().dtype(at::kFloat));
+  std::pair<uint64_t, uint64_t> r{0, 0};
+  if (stochastic_rounding) r = reserve_random(x, x.numel());
+  check_status(mi355q_cast_to_fp8_hybrid(x.data_ptr(), to_mi355q_dtype(src), x.numel(), y5.data_ptr(), y4.data_ptr(),
+                                         s5.defined() ? s5.data_ptr<float>() : nullptr,
+                                         s4.defined() ? s4.data_ptr<float>() : nullptr, stochastic_rounding ? 1 : 0,
+                                         r.first, r.second, is_amax ? amax.data_ptr<float>() : nullptr,
+                                         current_stream(x)),
+               "mi355q_cast_to_fp8_hybrid");
+  return {y5, y4, amax};
+}
+
 // ------------------------------------------------- convert_from_int4 / uint4
 
 Tensor convert_from_int4_common(const char* op_name, bool is_signed, const Tensor& input,
@@ -704,6 +742,7 @@ TORCH_LIBRARY(hpu, m) {
   m.def("hpu::cast_from_fp8.scalar_list(Tensor input, float[] scale, ScalarType out_dtype, int[]? scale_shape=None) -> Tensor");
   m.def("hpu::cast_to_fp8(Tensor input, Tensor? scale, bool stochastic_rounding, Tensor(a!) out, Tensor(b!) amax) -> (Tensor(a!), Tensor(b!))");
   m.def("hpu::fp8_gemm(Tensor A, bool trans_A, Tensor B, bool trans_B, Tensor D, ScalarType out_dtype, Tensor? A_scale_inv, Tensor? B_scale_inv, Tensor? bias, bool accumulate, Tensor(a!) out) -> Tensor(a!)");
+  m.def("hpu::cast_to_fp8_hybrid(Tensor input, Tensor? scale_152=None, Tensor? scale_143=None, bool stochastic_rounding=False, bool is_amax=False) -> (Tensor, Tensor, Tensor)");
   m.def("hpu::cast_to_fp8_v2(Tensor input, Tensor? scale=None, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)");
   m.def("hpu::cast_to_fp8_v2.scalar(Tensor input, float scale, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)");
   m.def("hpu::cast_to_fp8_v2.scalar_list(Tensor input, float[] scale, bool stochastic_rounding=False, bool is_amax=False, ScalarType dtype=None, int[]? scale_shape=None) -> (Tensor, Tensor)");
@@ -734,6 +773,7 @@ TORCH_LIBRARY(mi355q, m) {
   m.impl("convert_from_int4", convert_from_int4);                                              \
   m.impl("convert_from_uint4", convert_from_uint4);                                            \
   m.impl("cast_to_fp8", cast_to_fp8_v1);                                                       \
+  m.impl("cast_to_fp8_hybrid", cast_to_fp8_hybrid);                                            \
   m.impl("fp8_gemm", fp8_gemm_v1);
 
 TORCH_LIBRARY_IMPL(hpu, CUDA, m) { MI355Q_REGISTER_HPU(m) }

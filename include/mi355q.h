@@ -140,6 +140,18 @@ int mi355q_cast_to_fp8_sr(const void* x, int x_dtype, void* y, int fp8_fmt,
                           float* amax_out, uint64_t seed, uint64_t offset, void* stream);
 
 /*
+ * One read of x (fp32 or bf16, n elements), two casts: y_e5m2 = fp8_e5m2(x * scale_e5m2) and
+ * y_e4m3fn = fp8_e4m3fn(x * scale_e4m3fn), plus optionally amax = max|x|.  Replaces the
+ * convert_to_fp8_hybrid node of CastToFp8Hybrid::AddNode
+ * (hpu_ops/backend/cast_to_fp8_hybrid_gen.cpp:66-100).  Scales are one fp32 value in device
+ * memory each, or NULL for 1.  stochastic != 0 rounds the e5m2 output stochastically (random bits
+ * as in mi355q_cast_to_fp8_sr); the e4m3fn output always rounds to nearest even.
+ */
+int mi355q_cast_to_fp8_hybrid(const void* x, int x_dtype, int64_t n, void* y_e5m2, void* y_e4m3fn,
+                              const float* scale_e5m2, const float* scale_e4m3fn, int stochastic,
+                              uint64_t seed, uint64_t offset, float* amax_out, void* stream);
+
+/*
  * y = out_dtype(x_fp8) * scale, computed in out_dtype (fp32 or bf16).
  * Replaces the convert_from_fp8_{f32,bf16} node of CastFromFp8::AddNode
  * (hpu_ops/backend/fp8_ops.cpp:265-308).  Scale arguments as above.

@@ -1,4 +1,4 @@
-"""GPU parity of the deprecated out-variant ops hpu::cast_to_fp8 and hpu::fp8_gemm, written after the
+"""GPU parity of hpu::cast_to_fp8, hpu::fp8_gemm (the deprecated out-variants) and hpu::cast_to_fp8_hybrid, written after the
 reference's own tests of them (tests/pytest_working/eager/test_hpu_fp8_ops.py:34-140)."""
 import pytest
 import torch
@@ -79,3 +79,41 @@ def test_fp8_gemm(oracle, dev, shapeA, shapeB, bias, accumulate, dtype, fp8_dtyp
     if accumulate:
         full = full + out0.float()
     assert (((out.cpu().float() - full) / full) * 100).abs().to(torch.int).max() <= 15
+
+
+@pytest.mark.parametrize("dtype", [torch.float, torch.bfloat16])
+@pytest.mark.parametrize("stochastic", [True, False])
+@pytest.mark.parametrize("is_amax", [True, False])
+@pytest.mark.parametrize("shape,use_152,use_143", [((64, 48), True, True), ((16, 24, 8), True, False),
+                                                   ((16, 24, 8), False, True), ((1031,), False, False)])
+def test_cast_to_fp8_hybrid(oracle, dev, dtype, stochastic, is_amax, shape, use_152, use_143):
+    """test_hpu_fp8_ops_any_mode.py:266-358: one input, an e5m2 and an e4m3fn output with their own scales.
+    The e4m3fn output always rounds to nearest (bit-exact vs the oracle); so does the e5m2 output unless
+    stochastic, where it must be one of the two neighbours and within the reference's rtol of 0.26."""
+    g = torch.Generator().manual_seed(8)
+    pos = torch.rand(shape, generator=g).to(dtype) * 30 + 10
+    x = torch.cat((pos, -pos))
+    s152 = torch.tensor(1.3) if use_152 else None
+    s143 = torch.tensor(0.7) if use_143 else None
+    torch.manual_seed(5)
+    y5, y4, amax = ops.cast_to_fp8_hybrid(x.to(dev), s152.to(dev) if use_152 else None,
+                                          s143.to(dev) if use_143 else None, stochastic, is_amax)
+    ref4, _ = oracle.c_cast_to_fp8(x, s143, torch.float8_e4m3fn)
+    ref5, _ = oracle.c_cast_to_fp8(x, s152, torch.float8_e5m2)
+    assert_fp8_equal(y4, ref4, torch.float8_e4m3fn, "e4m3fn output")
+    if stochastic:
+        p = (x * s152.to(dtype)).float() if use_152 else x.float()
+        codes = torch.arange(256, dtype=torch.uint8).view(torch.float8_e5m2).float()
+        grid = torch.unique(codes[torch.isfinite(codes)])
+        hi = torch.searchsorted(grid, p.contiguous()).clamp(max=grid.numel() - 1)
+        lo = (hi - (grid[hi] != p).long()).clamp(min=0)
+        yv = y5.cpu().float()
+        assert ((yv == grid[lo]) | (yv == grid[hi])).all()
+        assert not torch.equal(yv, ref5.float())
+        assert torch.allclose(yv, ref5.float(), rtol=0.26, atol=0.0)
+    else:
+        assert_fp8_equal(y5, ref5, torch.float8_e5m2, "e5m2 output")
+    if is_amax:
+        assert amax.cpu() == x.abs().max().float() and amax.dim() == 0
+    else:
+        assert amax.numel() == 0
