@@ -49,6 +49,48 @@ def test_exact_small_integers_tiled(dev, fa, fb, ta, tb, M, N, K):
     assert torch.equal(out16.cpu(), expect.bfloat16())
 
 
+# One shape per kernel the dispatcher can pick (256 CUs): the persistent 256 x 256 kernel needs at
+# least 256 tiles, the two-workgroup kernel runs with a 3-stage ring when its 256 x 128 tiles exceed
+# the CU count and with 6 stages otherwise, the strip kernel has three row-tile heights, and
+# 128 x 128 tiles serve N <= 128 < M.  Edges are ragged in M, N and K.
+KERNEL_SHAPES = {
+    "tile256_persistent": (4000, 4112, 208),
+    "two_workgroups_ring3": (1008, 12304, 208),
+    "two_workgroups_ring6": (272, 4112, 400),
+    "strip_32_rows": (16, 1040, 400),
+    "strip_64_rows": (48, 1040, 400),
+    "strip_128_rows": (112, 1040, 400),
+    "tile128": (400, 112, 272),
+}
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("kernel", sorted(KERNEL_SHAPES))
+def test_every_kernel_path(oracle, dev, kernel, ta, tb):
+    """Exact small-integer products through each kernel (fp32 output: general epilogue), then the
+    same operands with per-row x per-column scales, a bias vector and bf16 output (fast epilogue)
+    against the fp32-accumulated CPU reference."""
+    M, N, K = KERNEL_SHAPES[kernel]
+    g = torch.Generator().manual_seed(M + N + K)
+    A = small_int_fp8((K, M) if ta else (M, K), E4, g)
+    B = small_int_fp8((N, K) if tb else (K, N), E5, g)
+    a = A.float().t() if ta else A.float()
+    b = B.float().t() if tb else B.float()
+    expect = a @ b
+    out = ops.fp8_gemm_v2(A.to(dev), ta, B.to(dev), tb, None, torch.float32)
+    assert torch.equal(out.cpu(), expect)
+    sa = torch.rand(M, 1, generator=g) + 0.5
+    sb = torch.rand(N, generator=g) + 0.5
+    bias = torch.randn(N, generator=g).bfloat16()
+    out16 = ops.fp8_gemm_v2(A.to(dev), ta, B.to(dev), tb, None, torch.bfloat16, sa.to(dev), sb.to(dev), bias.to(dev), False, [1, N])
+    ref = oracle.torch_fp8_gemm(A, ta, B, tb, torch.float32, sa, sb.reshape(1, N), bias=bias)
+    check(out16, ref, kernel)
+    # scalar scales fold into one factor in the fast epilogue
+    out_s = ops.fp8_gemm_v2(A.to(dev), ta, B.to(dev), tb, None, torch.bfloat16, 0.5, 0.25, bias.to(dev), False)
+    assert torch.equal(out_s.cpu(), (expect * 0.125 + bias.float()).bfloat16())
+
+
 @pytest.mark.parametrize("shape", [(24, 12, 36), (22, 10, 34), (26, 16, 38), (1, 7, 3), (17, 1, 5), (33, 65, 129)])
 @pytest.mark.parametrize("ta", [False, True])
 @pytest.mark.parametrize("tb", [False, True])
