@@ -61,6 +61,8 @@ inline bool tiled_ok(const void* A, int trans_a, int64_t lda, const void* B, int
   if (!al16(A) || !al16(B) || lda % 16 || ldb % 16 || stride_a % 16 || stride_b % 16) return false;
   if ((trans_a ? M : K) % 16) return false;
   if ((trans_b ? K : N) % 16) return false;
+  // a stage of the tiled kernels spans up to 256 rows of ld bytes, addressed with 31-bit offsets
+  if (lda > (1LL << 22) || ldb > (1LL << 22)) return false;
   return M > 0 && N > 0 && K > 0;
 }
 

@@ -142,33 +142,29 @@ struct DmaLoader {
   static constexpr int kPerWave = kRegions / WAVES;
   static_assert(kRegions % WAVES == 0 && 64 % kCPR == 0, "tile does not split over the waves");
 
-  i32x4 rsrc;  // raw buffer descriptor: base, stride 0, num_records (bytes), dword 3 flags
-  int voff[kPerWave];
-  int kc[kPerWave];  // K-major: byte offset of this lane's chunk inside a stage row
-  int step;          // voffset increment per K stage
+  // Raw buffer descriptor: base, stride 0, num_records (bytes), dword 3 flags.
+  // The base walks along K, one stage per advance(), and num_records shrinks
+  // with it, so the per-lane offsets never change and stay below 2^31 whatever
+  // the size of the matrix (a stage spans at most 256 rows of ld bytes).
+  i32x4 rsrc;
+  int64_t remaining;  // bytes from the base to the end of the addressable part of the matrix
+  int64_t step;       // bytes between K stages
+  int voff[kPerWave]; // this lane's offsets inside a stage
+  int kc[kPerWave];   // K-major: byte offset of this lane's chunk inside a stage row
   int wave;
 
-  // base: first element of this batch's matrix; mn0: first row (K-major) or
-  // column (MN-major) of the tile; extent: matrix extent along m/n.
-  __device__ __forceinline__ void init(const uint8_t* base, int64_t ld, int mn0, int extent, int K) {
-    const int lane = threadIdx.x & 63;
+  static constexpr int64_t kMaxRecords = 0x80000000LL;  // keeps the out-of-range marker out of range
+
+  // Per-lane geometry; depends on the leading dimension only.  The lane number
+  // goes through an empty volatile asm so that these few integer operations
+  // stay where they are written: hoisted out of the tile loop, the results
+  // would have to live through the epilogue, where every register is taken,
+  // and be spilled (a spill there is a store to memory by every lane).
+  __device__ __forceinline__ void set_lane_offsets(int64_t ld) {
+    int lane = threadIdx.x & 63;
+    asm volatile("" : "+v"(lane));
     wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rin = lane / kCPR, p = lane % kCPR;
-    int64_t records;
-    if constexpr (KMAJOR) {
-      base += (int64_t)mn0 * ld;
-      records = (int64_t)(extent - mn0 - 1) * ld + K;
-      step = BK;
-    } else {
-      base += mn0;
-      records = (int64_t)(K - 1) * ld + (extent - mn0);
-      step = BK * (int)ld;
-    }
-    const uint64_t b = reinterpret_cast<uint64_t>(base);
-    rsrc[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
-    rsrc[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((b >> 32) & 0xffffu));
-    rsrc[2] = __builtin_amdgcn_readfirstlane((int)records);
-    rsrc[3] = 0x00020000;
 #pragma unroll
     for (int i = 0; i < kPerWave; ++i) {
       const int row = (wave * kPerWave + i) * kRowsPerRegion + rin;
@@ -178,7 +174,39 @@ struct DmaLoader {
     }
   }
 
-  // Issues load I of this wave's share of the stage that starts at k0.
+  __device__ __forceinline__ void set_records() {
+    const int64_t r = remaining < 0 ? 0 : (remaining > kMaxRecords ? kMaxRecords : remaining);
+    rsrc[2] = __builtin_amdgcn_readfirstlane((int)(uint32_t)r);
+  }
+
+  // Points the descriptor at stage 0 of a tile.  base: first element of this
+  // batch's matrix; mn0: first row (K-major) or column (MN-major) of the tile;
+  // extent: matrix extent along m/n; valid false makes every load fall outside.
+  __device__ __forceinline__ void set_tile(const uint8_t* base, int64_t ld, int mn0, int extent, int K, bool valid = true) {
+    if constexpr (KMAJOR) {
+      base += (int64_t)mn0 * ld;
+      remaining = (int64_t)(extent - mn0 - 1) * ld + K;
+      step = BK;
+    } else {
+      base += mn0;
+      remaining = (int64_t)(K - 1) * ld + (extent - mn0);
+      step = (int64_t)BK * ld;
+    }
+    if (!valid) remaining = 0;
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    rsrc[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    rsrc[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((b >> 32) & 0xffffu));
+    rsrc[3] = 0x00020000;
+    set_records();
+  }
+
+  __device__ __forceinline__ void init(const uint8_t* base, int64_t ld, int mn0, int extent, int K) {
+    set_lane_offsets(ld);
+    set_tile(base, ld, mn0, extent, K);
+  }
+
+  // Issues load I of this wave's share of the stage the descriptor points at,
+  // which starts at k0.
   template <int I>
   __device__ __forceinline__ void issue_one(uint8_t* lds_tile, int k0, int K) const {
     const uint32_t lds_base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)lds_tile;
@@ -202,25 +230,14 @@ struct DmaLoader {
     static_for<kPerWave>([&](auto ic) { issue_one<decltype(ic)::value>(lds_tile, k0, K); });
   }
 
+  // Next K stage: scalar arithmetic on the descriptor only.
   __device__ __forceinline__ void advance() {
-#pragma unroll
-    for (int i = 0; i < kPerWave; ++i) voff[i] += step;
-  }
-
-  // Recomputes the per-lane offsets as init() left them plus `stages` advances.
-  // Called after an epilogue: the offsets are then dead while the epilogue
-  // runs, where every register is taken, instead of being spilled around it
-  // (a spill there is a store to memory by every lane for every tile).
-  __device__ __forceinline__ void rebuild_offsets(int64_t ld, int stages) {
-    int lane = threadIdx.x & 63;
-    asm volatile("" : "+v"(lane));
-    const int rin = lane / kCPR, p = lane % kCPR;
-#pragma unroll
-    for (int i = 0; i < kPerWave; ++i) {
-      const int row = (wave * kPerWave + i) * kRowsPerRegion + rin;
-      const int c = p ^ G::swizzle(row);
-      voff[i] = row * (int)ld + c * 16 + stages * step;
-    }
+    uint64_t b = ((uint64_t)(uint32_t)rsrc[1] << 32) | (uint32_t)rsrc[0];
+    b += (uint64_t)step;
+    rsrc[0] = (int)(uint32_t)b;
+    rsrc[1] = (int)(uint32_t)(b >> 32);
+    remaining -= step;
+    set_records();
   }
 };
 
@@ -612,12 +629,8 @@ struct TileCore {
   // Points the loaders at tile (m0, n0); `valid` false makes every load of the
   // tile fall outside the descriptors (used past the workgroup's last tile).
   __device__ __forceinline__ void retarget(const GemmArgs& g, int64_t batch, int m0, int n0, bool valid) {
-    la.init(g.A + batch * g.stride_a, g.lda, m0, g.M, g.K);
-    lb.init(g.B + batch * g.stride_b, g.ldb, n0, g.N, g.K);
-    if (!valid) {
-      la.rsrc[2] = 0;
-      lb.rsrc[2] = 0;
-    }
+    la.set_tile(g.A + batch * g.stride_a, g.lda, m0, g.M, g.K, valid);
+    lb.set_tile(g.B + batch * g.stride_b, g.ldb, n0, g.N, g.K, valid);
   }
 
   static constexpr int kPartsA = frag_parts<A_KMAJOR>(), kPartsB = frag_parts<B_KMAJOR>();
@@ -777,6 +790,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g)
   if (idx >= count) return;
   int tile_m, tile_n;
   tile_coords(first + idx, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+  core.la.set_lane_offsets(g.lda);
+  core.lb.set_lane_offsets(g.ldb);
   core.retarget(g, batch, tile_m * BM, tile_n * BN, true);
   core.issue_stage(lds0, 0);
   core.issue_stage(lds1, 1);
@@ -801,9 +816,9 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g)
       epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
     }
     if (idx >= count) break;
-    // the loaders stand two stages into the next tile
-    core.la.rebuild_offsets(g.lda, 2);
-    core.lb.rebuild_offsets(g.ldb, 2);
+    // recomputed rather than kept live through the epilogue
+    core.la.set_lane_offsets(g.lda);
+    core.lb.set_lane_offsets(g.ldb);
   }
   // drain the (out-of-range) loads issued for the tile that does not exist
   __builtin_amdgcn_s_waitcnt(0);

@@ -347,3 +347,20 @@ def test_c_abi_direct(oracle, pkg, dev):
     ref = oracle.c_fp8_gemm(A, False, B, True, torch.float32, sa.reshape(M, 1), sb, bias=bias, B_scale_shape=[1, N])
     rel, ok = gemm_errors(C, ref)
     assert rel < 1e-5 and ok, rel
+
+
+@pytest.mark.parametrize("M", [32, 512])
+def test_operand_larger_than_2_gib(dev, M):
+    """B of 16384 x 131200 bytes (2.0 GiB + 2 MiB): the descriptors walk along K, so no offset
+    inside the kernels depends on the size of the matrix.  Exact small-integer products; the
+    columns checked include the last ones, whose high-k rows lie beyond 2 GiB."""
+    K, N = 16384, 131200
+    g = torch.Generator(device=dev).manual_seed(M)
+    B = torch.randint(-4, 5, (K, N), generator=g, device=dev, dtype=torch.int8).to(torch.float16).to(E4)
+    A = torch.randint(-4, 5, (M, K), generator=g, device=dev, dtype=torch.int8).to(torch.float16).to(E4)
+    assert B.numel() > 2 ** 31
+    out = ops.fp8_gemm_v2(A, False, B, False, None, torch.float32)
+    a32 = A.float()
+    for c0 in (0, 65536, N - 256):
+        expect = a32 @ B[:, c0:c0 + 256].float()   # |sum| <= 16 K < 2^24: exact in any order
+        assert torch.equal(out[:, c0:c0 + 256], expect), c0
