@@ -358,3 +358,27 @@ def test_stochastic_rounding_is_unbiased(dev, dtype, fmt, lo, hi, max_diff):
     z = torch.tensor([448.0, -448.0, 1e6, -1e6, 0.0, 0.5], dtype=dtype, device=dev)
     zz = ops.cast_to_fp8_v2(z, None, True, False, E4)[0].float().cpu()
     assert zz.tolist() == [448.0, -448.0, 448.0, -448.0, 0.0, 0.5]
+
+
+def test_cast_more_than_2_31_elements(dev):
+    """2^31 + 4104 bf16 elements in one call: indices are 64-bit throughout.  The whole-tensor
+    result equals the results of two half-size calls, amax equals torch's, and the cast back
+    reproduces the fp8 values."""
+    n = 2 ** 31 + 4104
+    x = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    half = n // 2
+    g = torch.Generator(device=dev).manual_seed(3)
+    x[:half].normal_(generator=g)
+    x[half:].normal_(generator=g)
+    x[-1] = 77.0
+    scale = torch.tensor(3.0, device=dev)
+    y, amax = ops.cast_to_fp8_v2(x, scale, False, True, E4)
+    assert amax.item() == x.abs().max().float().item()
+    y1, _ = ops.cast_to_fp8_v2(x[:half], scale, False, False, E4)
+    y2, _ = ops.cast_to_fp8_v2(x[half:], scale, False, False, E4)
+    assert torch.equal(y[:half].view(torch.uint8), y1.view(torch.uint8))
+    assert torch.equal(y[half:].view(torch.uint8), y2.view(torch.uint8))
+    assert y[-1].float().item() == 224.0  # 77 * 3 = 231 rounds to 224 in e4m3
+    del y1, y2, x
+    back = ops.cast_from_fp8(y, None, torch.bfloat16)
+    assert torch.equal(back[-4096:].float(), y[-4096:].float()) and back.numel() == n
