@@ -16,9 +16,9 @@ __device__ __forceinline__ int nib(uint32_t w, int i) {
   else return (int)__builtin_amdgcn_ubfe(w, 4 * i, 4);
 }
 
-// scale / float zero-point vectors of 8 elements, converted to fp32
+// E consecutive scale / float zero-point values, converted to fp32 (E = 8 bf16 or 4 fp32: 16 bytes)
 template <bool BF16>
-__device__ __forceinline__ void load8(const uint8_t* base, int64_t elem, float* out) {
+__device__ __forceinline__ void load_vals(const uint8_t* base, int64_t elem, float* out) {
   if constexpr (BF16) {
     const u32x4 w = *reinterpret_cast<const u32x4*>(base + elem * 2);
 #pragma unroll
@@ -28,28 +28,33 @@ __device__ __forceinline__ void load8(const uint8_t* base, int64_t elem, float* 
     }
   } else {
     const f32x4 a = *reinterpret_cast<const f32x4*>(base + elem * 4);
-    const f32x4 b = *reinterpret_cast<const f32x4*>(base + elem * 4 + 16);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      out[i] = a[i];
-      out[4 + i] = b[i];
-    }
+    for (int i = 0; i < 4; ++i) out[i] = a[i];
   }
 }
 
 // ZP: 0 none, 1 float, 2 packed.  RPT rows per thread; a thread's rows never
 // straddle a group when HOIST (group % RPT == 0), so scale / zp load once.
+// A lane produces one 16-byte store per row: all 8 nibbles of a packed word for
+// bf16 output, one half of the word (4 nibbles) for fp32 output, so that a
+// wave's store covers whole cache lines in both cases.
 template <bool SIGNED, bool BF16, int ZP, int RPT, bool HOIST>
 __global__ __launch_bounds__(kI4Threads) void dequant_4bit_kernel(
     const uint32_t* __restrict__ packed, const uint8_t* __restrict__ scale,
     const uint8_t* __restrict__ zp, int64_t rows, int64_t pcols, int64_t group,
     uint8_t* __restrict__ out) {
+  constexpr int E = BF16 ? 8 : 4;            // elements per lane per row
+  constexpr int LPW = 8 / E;                 // lanes per packed word
+  const int64_t lanes_per_row = pcols * LPW;
   const int64_t g = (int64_t)blockIdx.x * kI4Threads + threadIdx.x;
-  const int64_t chunk = g / pcols;
-  const int64_t pc = g - chunk * pcols;
+  const int64_t chunk = g / lanes_per_row;
+  const int64_t lc = g - chunk * lanes_per_row;
+  const int64_t pc = lc / LPW;
+  const int nib0 = (int)(lc % LPW) * E;      // first nibble of this lane inside the word
   const int64_t r0 = chunk * RPT;
   if (r0 >= rows) return;
   const int64_t cols = pcols * 8;
+  const int64_t c0 = pc * 8 + nib0;          // first output column of this lane
   const int nr = (int)((rows - r0) < RPT ? (rows - r0) : RPT);
 
   uint32_t w[RPT];
@@ -57,8 +62,8 @@ __global__ __launch_bounds__(kI4Threads) void dequant_4bit_kernel(
   for (int j = 0; j < RPT; ++j)
     if (j < nr) w[j] = __builtin_nontemporal_load(packed + (r0 + j) * pcols + pc);
 
-  float s[8], zf[8];
-  int zi[8];
+  float s[E], zf[E];
+  int zi[E];
   int64_t cur = -1;
 #pragma unroll
   for (int j = 0; j < RPT; ++j) {
@@ -67,18 +72,19 @@ __global__ __launch_bounds__(kI4Threads) void dequant_4bit_kernel(
     const int64_t gi = HOIST ? r0 / group : r / group;
     if ((HOIST && j == 0) || (!HOIST && gi != cur)) {
       cur = gi;
-      load8<BF16>(scale, gi * cols + pc * 8, s);
-      if constexpr (ZP == 1) load8<BF16>(zp, gi * cols + pc * 8, zf);
+      load_vals<BF16>(scale, gi * cols + c0, s);
+      if constexpr (ZP == 1) load_vals<BF16>(zp, gi * cols + c0, zf);
       if constexpr (ZP == 2) {
-        const uint32_t zw = reinterpret_cast<const uint32_t*>(zp)[gi * pcols + pc];
+        const uint32_t zw = reinterpret_cast<const uint32_t*>(zp)[gi * pcols + pc] >> (4 * nib0);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) zi[i] = nib<SIGNED>(zw, i);
+        for (int i = 0; i < E; ++i) zi[i] = nib<SIGNED>(zw, i);
       }
     }
-    float v[8];
+    const uint32_t wj = w[j] >> (4 * nib0);
+    float v[E];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int q = nib<SIGNED>(w[j], i);
+    for (int i = 0; i < E; ++i) {
+      const int q = nib<SIGNED>(wj, i);
       float d;
       if constexpr (ZP == 2) d = (float)(q - zi[i]);
       else if constexpr (ZP == 1) {
@@ -91,12 +97,10 @@ __global__ __launch_bounds__(kI4Threads) void dequant_4bit_kernel(
       u32x4 o;
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
-      __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(out + (r * cols + pc * 8) * 2));
+      __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(out + (r * cols + c0) * 2));
     } else {
-      f32x4 a = {v[0], v[1], v[2], v[3]}, b = {v[4], v[5], v[6], v[7]};
-      f32x4* o = reinterpret_cast<f32x4*>(out + (r * cols + pc * 8) * 4);
-      __builtin_nontemporal_store(a, o);
-      __builtin_nontemporal_store(b, o + 1);
+      const f32x4 o = {v[0], v[1], v[2], v[3]};
+      __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(out + (r * cols + c0) * 4));
     }
   }
 }
@@ -104,7 +108,8 @@ __global__ __launch_bounds__(kI4Threads) void dequant_4bit_kernel(
 template <bool SIGNED, bool BF16, int ZP>
 int dequant_launch(const uint32_t* packed, const uint8_t* scale, const uint8_t* zp, int64_t rows,
                    int64_t pcols, int64_t group, uint8_t* out, hipStream_t st) {
-  auto grid_for = [&](int rpt) { return ((rows + rpt - 1) / rpt * pcols + kI4Threads - 1) / kI4Threads; };
+  const int64_t lanes_per_row = pcols * (BF16 ? 1 : 2);
+  auto grid_for = [&](int rpt) { return ((rows + rpt - 1) / rpt * lanes_per_row + kI4Threads - 1) / kI4Threads; };
   if (group % 16 == 0) {
     const int64_t grid = grid_for(16);
     if (grid > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
