@@ -160,10 +160,12 @@ struct DmaLoader {
   // stay where they are written: hoisted out of the tile loop, the results
   // would have to live through the epilogue, where every register is taken,
   // and be spilled (a spill there is a store to memory by every lane).
-  __device__ __forceinline__ void set_lane_offsets(int64_t ld) {
+  // wave_index: this wave's position among the WAVES waves that share the
+  // loads of this operand (default: its position in the workgroup).
+  __device__ __forceinline__ void set_lane_offsets(int64_t ld, int wave_index = -1) {
     int lane = threadIdx.x & 63;
     asm volatile("" : "+v"(lane));
-    wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    wave = wave_index >= 0 ? wave_index : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rin = lane / kCPR, p = lane % kCPR;
 #pragma unroll
     for (int i = 0; i < kPerWave; ++i) {
