@@ -1,0 +1,50 @@
+"""HIP graph capture of the ops: no entry point allocates, synchronises or records a memset, so a
+captured sequence must replay to the same bits as eager execution, replay after replay, with eager
+work and synchronisation in between."""
+import pytest
+import torch
+
+from helpers import E4
+
+pytestmark = pytest.mark.gpu
+ops = torch.ops.hpu
+
+
+def pipeline(x, w8, sw_inv):
+    x8, sx_inv = torch.ops.mi355q.quantize_rows(x, E4)
+    y = ops.fp8_gemm_v2(x8, False, w8, False, None, torch.bfloat16, sx_inv, sw_inv, None, False, [1, w8.shape[1]])
+    y8, amax = ops.cast_to_fp8_v2(y, None, False, True, E4)          # amax: fill kernel + atomics inside the graph
+    back = ops.cast_from_fp8(y8, None, torch.bfloat16)
+    return y, y8, amax, back
+
+
+def test_graph_replays_match_eager(dev):
+    g = torch.Generator().manual_seed(12)
+    M, K, N = 192, 512, 384
+    w = (torch.randn(K, N, generator=g) * 0.05).bfloat16().to(dev)
+    sw = 448.0 / w.abs().amax(dim=0).float()
+    w8 = ops.cast_to_fp8_v2(w, sw, False, False, E4, [1, N])[0]
+    sw_inv = (1.0 / sw).contiguous()
+    x = torch.randn(M, K, generator=g).bfloat16().to(dev)
+    static_x = x.clone()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):          # warm-up on the capture stream, as torch's graph recipe asks
+        for _ in range(3):
+            pipeline(static_x, w8, sw_inv)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = pipeline(static_x, w8, sw_inv)
+
+    for rep in range(4):
+        xin = torch.randn(M, K, generator=g).bfloat16().to(dev) * (rep + 1)
+        static_x.copy_(xin)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        ref = pipeline(xin, w8, sw_inv)     # eager work between the replays
+        torch.cuda.synchronize()
+        for a, b in zip(got, ref):
+            assert torch.equal(a.view(torch.uint8) if a.dtype == E4 else a, b.view(torch.uint8) if b.dtype == E4 else b), rep
