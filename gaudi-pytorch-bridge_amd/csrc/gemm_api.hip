@@ -1,6 +1,6 @@
 // fp8_gemm_v2 C entry point: argument checks, kernel choice, and the any-shape
 // fallback kernel.  The MFMA tile kernels live in gemm_tile.h.
-#include "gemm_pp.h"
+#include "gemm_dispatch.h"
 
 namespace mi355q {
 
@@ -76,7 +76,7 @@ const char* mi355q_fp8_gemm_variant(int trans_a, int64_t lda, int trans_b, int64
                                     int64_t N, int64_t K) {
   if (lda % 16 || ldb % 16 || (trans_a ? M : K) % 16 || (trans_b ? K : N) % 16) return "simple";
   if (M > 128 && N > 128)
-    return mi355q::use_pp_kernel(M, N, 1) ? "tile256x128x64_two_workgroups_mfma32x32x64" : "tile256x256x128_mfma32x32x64";
+    return mi355q::use_half_width_tiles(M, N, 1) ? "tile256x128x128_mfma32x32x64" : "tile256x256x128_mfma32x32x64";
   if (M <= 128) return "strip_Mx128x128_ring_mfma32x32x64";
   return "tile128x128x128_mfma32x32x64";
 }

@@ -1,0 +1,43 @@
+// Which kernel serves which problem.
+//
+// Large problems take 256 x 256 tiles (least bytes moved from L2 into LDS per
+// flop).  When that tiling leaves compute units without a tile, the same kernel
+// runs with 256 x 128 tiles: twice the tiles at 1.5 times the LDS traffic per
+// flop.  (A 4-wave kernel with two workgroups per CU and 64-byte K stages, meant
+// to hide the epilogue behind the other workgroup's MFMAs, was measured against
+// it: bound by its global->LDS traffic on large problems and no faster on these.)
+// Few rows of A (M <= 128) take the strip kernel, which streams B once through a
+// deep ring.
+#pragma once
+#include "gemm_skinny.h"
+#include "gemm_tile.h"
+
+namespace mi355q {
+
+inline bool use_half_width_tiles(int64_t M, int64_t N, int64_t batch) {
+  const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256) * batch;
+  return tiles256 < compute_units();
+}
+
+template <bool AK, bool BK_, int FA, int FB>
+void launch_by_size(const GemmArgs& g, int64_t batch, hipStream_t st) {
+  if (g.M > 128 && g.N > 128) {
+    if (use_half_width_tiles(g.M, g.N, batch)) launch_tile<256, 128, AK, BK_, FA, FB>(g, batch, st);
+    else launch_tile<256, 256, AK, BK_, FA, FB>(g, batch, st);
+  } else if (g.M <= 128) {
+    launch_skinny_by_m<AK, BK_, FA, FB>(g, batch, st);
+  } else {
+    launch_tile<128, 128, AK, BK_, FA, FB>(g, batch, st);
+  }
+}
+
+// One translation unit per operand layout instantiates this (gemm_inst_*.hip).
+template <bool AK, bool BK_>
+void launch_by_format(const GemmArgs& g, int fmt_a, int fmt_b, int64_t batch, hipStream_t st) {
+  if (fmt_a == MI355Q_E4M3FN && fmt_b == MI355Q_E4M3FN) launch_by_size<AK, BK_, MI355Q_E4M3FN, MI355Q_E4M3FN>(g, batch, st);
+  else if (fmt_a == MI355Q_E4M3FN) launch_by_size<AK, BK_, MI355Q_E4M3FN, MI355Q_E5M2>(g, batch, st);
+  else if (fmt_b == MI355Q_E4M3FN) launch_by_size<AK, BK_, MI355Q_E5M2, MI355Q_E4M3FN>(g, batch, st);
+  else launch_by_size<AK, BK_, MI355Q_E5M2, MI355Q_E5M2>(g, batch, st);
+}
+
+}  // namespace mi355q

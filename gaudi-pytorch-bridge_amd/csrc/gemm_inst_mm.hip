@@ -1,5 +1,5 @@
 // fp8 GEMM tile kernels for one operand layout: A MN-major, B MN-major.
-#include "gemm_pp.h"
+#include "gemm_dispatch.h"
 
 namespace mi355q {
 void launch_gemm_mm(const GemmArgs& g, int fmt_a, int fmt_b, int64_t batch, hipStream_t st) {
