@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME[,NAME...]] [--no-cpu]
 
-A step is one call of the primary workload, BASELINE config 3: fp8_gemm_v2 on
+A step is one call of the primary workload, benchmark configuration 3: fp8_gemm_v2 on
 8192 x 4096 x 14336 (e4m3fn x e4m3fn -> bf16, per-tensor inverse scales, bf16
 bias), with all operands resident in HBM.  The single JSON line printed at the
 end carries that as ``value`` (TFLOP/s) with its MFMA roofline, and under
@@ -135,7 +135,7 @@ def c1_input(gen, rows=4096, cols=4096):
 
 
 def bench_cast(pkg, oracle, dev, steps, warmup, cpu):
-    """BASELINE config 1: amax pass, cast_to_fp8_v2 (scale given), cast_from_fp8.
+    """benchmark configuration 1: amax pass, cast_to_fp8_v2 (scale given), cast_from_fp8.
 
     These kernels run for about ten microseconds, less than the host needs to
     dispatch a torch op, so they are timed through the C ABI (ctypes, outputs
@@ -216,13 +216,13 @@ def bench_cast(pkg, oracle, dev, steps, warmup, cpu):
     ms = time_gpu(lambda i: ok(lib.mi355q_cast_to_fp8(big.data_ptr(), pkg.BF16, big8[i % 2].data_ptr(), pkg.E4M3FN,
                                                       sd.data_ptr(), 0.0, pkg.SCALE_DEV, nb, 1, 1, None, st)),
                   max(steps // 5, 5), 3)
-    out.append(hbm_entry("cast_to_fp8_v2_large", "cast_to_fp8_v2 bf16 [16384,16384] -> e4m3fn (not a BASELINE config)",
+    out.append(hbm_entry("cast_to_fp8_v2_large", "cast_to_fp8_v2 bf16 [16384,16384] -> e4m3fn (not one of the benchmark configurations)",
                          3 * nb, ms, max(steps // 5, 5), "cast_to_fp8_vec8<bf16,e4m3fn,scalar>"))
     return out
 
 
 def bench_int4(pkg, oracle, dev, steps, warmup, cpu):
-    """BASELINE config 2: K = N = 4096, group 128 (timed through the C ABI, see bench_cast)."""
+    """benchmark configuration 2: K = N = 4096, group 128 (timed through the C ABI, see bench_cast)."""
     import ctypes
     lib = pkg.capi()
     out = []
@@ -308,7 +308,7 @@ def bench_gemm_c3(ops, oracle, pkg, dev, steps, warmup, cpu):
 
 
 def bench_gemm_decode(ops, oracle, dev, steps, warmup):
-    """BASELINE config 4: per-token x per-channel scales, K = 8192, N = 28672."""
+    """benchmark configuration 4: per-token x per-channel scales, K = 8192, N = 28672."""
     out = []
     gen = torch.Generator().manual_seed(SEED)
     K, N = 8192, 28672
@@ -338,7 +338,7 @@ def bench_gemm_decode(ops, oracle, dev, steps, warmup):
 
 
 def bench_mlp(ops, dev, steps, warmup):
-    """BASELINE config 5: fp8 decoder MLP block, Llama-3-8B dims, 4096 tokens."""
+    """benchmark configuration 5: fp8 decoder MLP block, Llama-3-8B dims, 4096 tokens."""
     gen = torch.Generator().manual_seed(SEED)
     T, d, ff = 4096, 4096, 14336
 

@@ -194,7 +194,7 @@ def test_amax_ops(oracle, dev, dtype):
 
 
 def test_config1_full_size(oracle, dev):
-    """BASELINE config 1 at full size: amax, scale = 448/amax, cast, cast back.
+    """benchmark configuration 1 at full size: amax, scale = 448/amax, cast, cast back.
     Checked bit-exactly against the PyTorch-CPU twin (multi-threaded; the C
     oracle is pinned to it on smaller inputs) and on a 1/16 slice against C."""
     x = c1_input()

@@ -269,7 +269,7 @@ def quantize_rows(oracle, x, dim):
 
 @pytest.mark.parametrize("M", [16, 64, 256])
 def test_config4_decode_shapes_reduced(oracle, dev, M):
-    """BASELINE config 4 semantics (per-token x per-channel scales, heavy-tail channels) at
+    """benchmark configuration 4 semantics (per-token x per-channel scales, heavy-tail channels) at
     K = 1024, N = 1536 so that the CPU reference finishes in seconds."""
     g = torch.Generator().manual_seed(M)
     K, N = 1024, 1536
@@ -293,7 +293,7 @@ def test_config4_decode_shapes_reduced(oracle, dev, M):
 
 
 def test_config3_shape_properties(oracle, dev):
-    """BASELINE config 3 at full size (8192 x 4096 x 14336, per-tensor scales, bias).
+    """benchmark configuration 3 at full size (8192 x 4096 x 14336, per-tensor scales, bias).
     The CPU reference covers a sampled block of rows and columns; the whole output is
     covered by linearity in the scale and by an exact small-integer run."""
     g = torch.Generator().manual_seed(0xC001A1)

@@ -94,7 +94,7 @@ def test_group_sizes_and_ragged_rows(oracle, dev, group, variant):
 
 
 def test_config2_full_size(oracle, dev):
-    """BASELINE config 2: K = N = 4096, group 128, bf16 scales U(0.001, 0.02), packed uint4
+    """benchmark configuration 2: K = N = 4096, group 128, bf16 scales U(0.001, 0.02), packed uint4
     zero-points; then int4 with signed nibbles and no zero-point.  Bit exact."""
     g = torch.Generator().manual_seed(0xC001A1)
     K = N = 4096
