@@ -50,13 +50,6 @@ __global__ __launch_bounds__(kSkThreads) void fp8_gemm_skinny_kernel(GemmArgs g)
   LB lb;
   la.init(g.A + batch * g.stride_a, g.lda, 0, g.M, g.K);
   lb.init(g.B + batch * g.stride_b, g.ldb, n0, g.N, g.K);
-  auto issue_stage = [&](int off, int kt) {
-    static_for<LA::kPerWave>([&](auto ic) { la.template issue_one<decltype(ic)::value>(lds + off, kt * kBK, g.K); });
-    static_for<LB::kPerWave>([&](auto ic) { lb.template issue_one<decltype(ic)::value>(lds + off + BM * kBK, kt * kBK, g.K); });
-    la.advance();
-    lb.advance();
-  };
-
   f32x16 acc[MT][1];
 #pragma unroll
   for (int i = 0; i < MT; ++i)
@@ -64,8 +57,33 @@ __global__ __launch_bounds__(kSkThreads) void fp8_gemm_skinny_kernel(GemmArgs g)
     for (int e = 0; e < 16; ++e) acc[i][0][e] = 0.0f;
 
   const int KT = (g.K + kBK - 1) / kBK;
-  // stages 0 .. S-2 go out first; stages at or beyond K fall outside the
-  // buffer descriptors and arrive as zeros, so every step issues and waits alike
+  // K is walked from a stage that depends on the strip, wrapping around, when B
+  // is K-major: its rows are K bytes apart, so workgroups that all read the same
+  // k at the same time send their requests, which differ only in high address
+  // bits, to the same few memory channels.  (With B MN-major the strips of one
+  // k row are contiguous in memory and walking in step is the better order.)
+  const int first = B_KMAJOR ? (int)(((int64_t)blockIdx.x * KT) / gridDim.x) : 0;
+  int at = 0;  // the stage the loaders' descriptors point at
+  // Issues the loads of the i-th stage in walking order; beyond the KT-th they
+  // fall outside the descriptors and arrive as zeros, so that every step issues
+  // and waits alike.
+  auto issue_stage = [&](int off, int i) {
+    int stage = first + i;
+    if (stage >= KT) stage -= KT;
+    if (i >= KT) stage = KT;  // out of range
+    if (stage != at) {
+      la.seek(at, stage);
+      lb.seek(at, stage);
+      at = stage;
+    }
+    static_for<LA::kPerWave>([&](auto ic) { la.template issue_one<decltype(ic)::value>(lds + off, stage * kBK, g.K); });
+    static_for<LB::kPerWave>([&](auto ic) { lb.template issue_one<decltype(ic)::value>(lds + off + BM * kBK, stage * kBK, g.K); });
+    la.advance();
+    lb.advance();
+    ++at;
+  };
+
+  // stages 0 .. S-2 (in walking order) go out first
 #pragma unroll
   for (int s = 0; s < S - 1; ++s) issue_stage(s * kStageBytes, s);
 

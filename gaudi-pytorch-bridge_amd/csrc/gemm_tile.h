@@ -232,6 +232,20 @@ struct DmaLoader {
     static_for<kPerWave>([&](auto ic) { issue_one<decltype(ic)::value>(lds_tile, k0, K); });
   }
 
+  // Points the descriptor at K stage `stage` of the tile set_tile() chose, which
+  // has to be the most recent call (it leaves the descriptor at stage 0 and
+  // this walks from wherever advance() has taken it).  Stages at or beyond K
+  // are entirely out of range.
+  __device__ __forceinline__ void seek(int from_stage, int to_stage) {
+    const int64_t d = (int64_t)(to_stage - from_stage) * step;
+    uint64_t b = ((uint64_t)(uint32_t)rsrc[1] << 32) | (uint32_t)rsrc[0];
+    b += (uint64_t)d;
+    rsrc[0] = (int)(uint32_t)b;
+    rsrc[1] = (int)(uint32_t)(b >> 32);
+    remaining -= d;
+    set_records();
+  }
+
   // Next K stage: scalar arithmetic on the descriptor only.
   __device__ __forceinline__ void advance() {
     uint64_t b = ((uint64_t)(uint32_t)rsrc[1] << 32) | (uint32_t)rsrc[0];
