@@ -9,9 +9,11 @@
 // number, which keeps the 128-bit and transposing fragment reads free of bank
 // conflicts; since a DMA load places lane l's chunk at LDS offset 16 l, the
 // swizzle is applied by choosing which global chunk each lane fetches.  Each
-// wave computes its (BM/2) x (BN/2) sub-tile with v_mfma_f32_32x32x64_f8f6f4
+// wave computes its (BM/2) x (BN/4) sub-tile with v_mfma_f32_32x32x64_f8f6f4
 // (fp8/bf8 operands, 64 k per instruction), reading the fragments of the next
-// half-step while the MFMAs of the current one run.
+// half-step while the MFMAs of the current one run.  The buffer descriptors
+// walk along K by scalar arithmetic, so the per-lane offsets are small
+// constants and operands of any size are addressable.
 //
 // Operand layouts.  An operand whose K index is contiguous in memory (A with
 // trans_a == 0, B with trans_b != 0) is "K-major": a lane's 32-byte MFMA
@@ -21,9 +23,10 @@
 // inside each group of 16 lanes on the way into registers.
 //
 // The MFMA is issued with the B fragment as its first operand, so that a lane
-// ends up holding 4 consecutive n for one m: the epilogue stores 8 bytes (bf16)
-// or 16 bytes (fp32) per lane, and per-row / per-column scales, bias and the
-// accumulate input are applied in fp32 before the single final rounding.
+// ends up holding runs of 4 consecutive n for one m.  Per-row / per-column
+// scales, bias and the accumulate input are applied in fp32 before the single
+// final rounding, and the rows pass through LDS once more so that a wave
+// stores whole 128-byte lines.
 #pragma once
 #include <type_traits>
 
