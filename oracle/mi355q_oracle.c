@@ -38,6 +38,11 @@
  *   ora_fp8_gemm                          values pinned to tolerance by test
  *        :361-476,599-704 and by exact small-integer cases; order of scale /
  *        bias / accumulate / rounding in the epilogue is parity unpinned.
+ *   stochastic rounding                   no oracle function: the random bit
+ *        stream is parity unpinned; tests check what the reference's do
+ *        (any_mode/test_hpu_fp8_ops_any_mode.py:124-128, test_hpu_fp8_te.py:
+ *        105-150): each result is one of the two fp8 neighbours of the exact
+ *        value, the mean is preserved, round-to-nearest differs.
  */
 #include <math.h>
 #include <stdint.h>
