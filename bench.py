@@ -49,10 +49,10 @@ MEASURED_TRAFFIC = {
     "cast_to_fp8_v2_large": 805.02e6,
     "convert_from_uint4": 43.37e6,
     "convert_from_int4": 43.12e6,
-    "fp8_gemm_v2": 939.88e6,
+    "fp8_gemm_v2": 939.91e6,
     "fp8_gemm_v2_decode_M16": 237.0e6,
     "fp8_gemm_v2_decode_M64": 243.1e6,
-    "fp8_gemm_v2_decode_M256": 266.7e6,
+    "fp8_gemm_v2_decode_M256": 272.6e6,
 }
 
 
