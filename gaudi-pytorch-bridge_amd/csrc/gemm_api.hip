@@ -119,6 +119,7 @@ int mi355q_fp8_gemm(const void* A, int fmt_a, int trans_a, int64_t lda, const vo
   g.stride_a = stride_a; g.stride_b = stride_b; g.stride_c = stride_c; g.stride_d = stride_d;
   g.stride_bias = stride_bias;
   g.out_bf16 = out_dtype == MI355Q_BF16;
+  g.fast_epi = 0;
   g.tiles_m = g.tiles_n = 0;
 
   const int64_t kMaxBatch = 65535;
@@ -131,6 +132,7 @@ int mi355q_fp8_gemm(const void* A, int fmt_a, int trans_a, int64_t lda, const vo
     gb.C = g.C + b0 * stride_c * es;
     if (g.D) gb.D = g.D + b0 * stride_d * es;
     if (g.bias) gb.bias = g.bias + b0 * stride_bias * es;
+    gb.fast_epi = epilogue_fast_ok(gb, nb);
     if (tiled_ok(gb.A, trans_a, lda, gb.B, trans_b, ldb, M, N, K, stride_a, stride_b)) {
       const bool ak = !trans_a, bk = trans_b != 0;
       if (ak && bk) launch_gemm_kk(gb, fmt_a, fmt_b, nb, st);

@@ -22,12 +22,13 @@ inline bool use_half_width_tiles(int64_t M, int64_t N, int64_t batch) {
 template <bool AK, bool BK_, int FA, int FB>
 void launch_by_size(const GemmArgs& g, int64_t batch, hipStream_t st) {
   if (g.M > 128 && g.N > 128) {
-    if (use_half_width_tiles(g.M, g.N, batch)) launch_tile<256, 128, AK, BK_, FA, FB>(g, batch, st);
-    else launch_tile<256, 256, AK, BK_, FA, FB>(g, batch, st);
+    if (use_half_width_tiles(g.M, g.N, batch)) launch_tile<256, 128, 4, false, AK, BK_, FA, FB>(g, batch, st);
+    else if (g.fast_epi) launch_tile<256, 256, 2, true, AK, BK_, FA, FB>(g, batch, st);
+    else launch_tile<256, 256, 4, false, AK, BK_, FA, FB>(g, batch, st);
   } else if (g.M <= 128) {
     launch_skinny_by_m<AK, BK_, FA, FB>(g, batch, st);
   } else {
-    launch_tile<128, 128, AK, BK_, FA, FB>(g, batch, st);
+    launch_tile<128, 128, 4, false, AK, BK_, FA, FB>(g, batch, st);
   }
 }
 

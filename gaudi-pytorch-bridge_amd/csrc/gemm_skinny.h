@@ -121,9 +121,8 @@ __global__ __launch_bounds__(kSkThreads) void fp8_gemm_skinny_kernel(GemmArgs g)
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   float* stage_area = reinterpret_cast<float*>(lds) + wave * epilogue_stage_floats<MT, 1>();
-  if (epilogue_fast_ok(g, batch)) {
-    if (g.sb_mode == MI355Q_GS_PER_COL) epilogue_bf16_fast<MT, 1, true>(g, batch, acc, 0, n0 + wn, stage_area);
-    else epilogue_bf16_fast<MT, 1, false>(g, batch, acc, 0, n0 + wn, stage_area);
+  if (g.fast_epi) {
+    epilogue_bf16_fast_any<MT, 1>(g, batch, acc, 0, n0 + wn, stage_area);
   } else {
     epilogue<MT, 1>(g, batch, acc, 0, n0 + wn, stage_area);
   }

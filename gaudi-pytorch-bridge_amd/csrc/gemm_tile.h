@@ -43,9 +43,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // Two waves per SIMD: a memory instruction of one wave (LDS fragment read,
 // global->LDS load) holds up that wave's next MFMA for tens of cycles, and only
 // a second resident wave lets the matrix pipe run meanwhile.
-constexpr int kGemmThreads = 512;
-constexpr int kWaves = kGemmThreads / 64;
-constexpr int kWavesM = 2, kWavesN = 4;  // wave grid over the tile
+constexpr int kWavesM = 2;  // the waves of a workgroup form a 2 x WN grid over its tile
 constexpr int kBK = 128;  // bytes (= fp8 elements) of K per LDS stage
 
 // Number of compute units of the current device (workgroups of the persistent kernel).
@@ -77,6 +75,7 @@ struct GemmArgs {
   int64_t ldd;
   int64_t stride_a, stride_b, stride_c, stride_d, stride_bias;
   int out_bf16;
+  int fast_epi;  // epilogue_fast_ok() of this launch
   int tiles_m, tiles_n;
 };
 
@@ -106,6 +105,7 @@ struct TileGeom {
   static constexpr int kChunksPerRow = ROW_BYTES / 16;
   static constexpr int kChunks = ROWS * kChunksPerRow;
   static_assert(KMAJOR ? (ROW_BYTES == 128 || ROW_BYTES == 64) : (ROW_BYTES == 256 || ROW_BYTES == 128), "no swizzle defined");
+  static constexpr int kSwizzlePeriod = KMAJOR ? 16 : 8;  // swizzle(row + kSwizzlePeriod) == swizzle(row)
   __device__ static __forceinline__ int swizzle(int row) {
     if constexpr (KMAJOR && ROW_BYTES == 128) return (row >> 1) & 7;
     else if constexpr (KMAJOR) return (row >> 2) & 3;
@@ -125,6 +125,18 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
+// The lane number, computed on the spot.  Inside the persistent tile loop every
+// value that depends only on the lane number is loop invariant: left alone,
+// the compiler computes it once before the K loop, where no register is free,
+// and spills it (a spill is a memory access by every lane, and the wait for its
+// reload also waits for the next tile's global->LDS loads).  An asm statement is
+// neither hoisted nor merged with another, and it needs no live input.
+__device__ __forceinline__ int lane_id_here() {
+  int lane;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+  return lane;
+}
+
 // Global -> LDS loader for one operand tile, one 16-byte chunk per lane per
 // instruction.  A wave-wide load fills a 1 KiB region of the LDS tile (lane l
 // lands at byte 16 l of the region), i.e. 64 / chunks-per-row consecutive rows;
@@ -136,7 +148,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 //           descriptor; columns past the extent only feed outputs that are
 //           never stored.
 // EXT: tile extent along m/n; BK: bytes of K per stage; WAVES: waves of the workgroup
-template <bool KMAJOR, int EXT, int BK = kBK, int WAVES = kWaves>
+template <bool KMAJOR, int EXT, int BK, int WAVES>
 struct DmaLoader {
   using G = TileGeom<KMAJOR, KMAJOR ? EXT : BK, KMAJOR ? BK : EXT>;
   static constexpr int kCPR = G::kChunksPerRow;
@@ -152,31 +164,34 @@ struct DmaLoader {
   i32x4 rsrc;
   int64_t remaining;  // bytes from the base to the end of the addressable part of the matrix
   int64_t step;       // bytes between K stages
-  int voff[kPerWave]; // this lane's offsets inside a stage
-  int kc[kPerWave];   // K-major: byte offset of this lane's chunk inside a stage row
+  // A wave's regions are consecutive, and regions a swizzle period apart differ
+  // by whole rows only: the offsets of the first kStored regions are kept, the
+  // others are those plus a multiple of region_step (registers are what the K
+  // loop is short of; an addition per load is not).
+  static constexpr int kPeriodRegions = G::kSwizzlePeriod / kRowsPerRegion > 0 ? G::kSwizzlePeriod / kRowsPerRegion : 1;
+  static constexpr int kStored = kPerWave % kPeriodRegions == 0 ? kPeriodRegions : kPerWave;
+  int voff[kStored];  // this lane's offsets inside a stage
+  int kc[kStored];    // K-major: byte offset of this lane's chunk inside a stage row
+  int region_step;    // bytes between regions kStored apart
   int wave;
 
   static constexpr int64_t kMaxRecords = 0x80000000LL;  // keeps the out-of-range marker out of range
 
-  // Per-lane geometry; depends on the leading dimension only.  The lane number
-  // goes through an empty volatile asm so that these few integer operations
-  // stay where they are written: hoisted out of the tile loop, the results
-  // would have to live through the epilogue, where every register is taken,
-  // and be spilled (a spill there is a store to memory by every lane).
+  // Per-lane geometry; depends on the leading dimension only.
   // wave_index: this wave's position among the WAVES waves that share the
   // loads of this operand (default: its position in the workgroup).
   __device__ __forceinline__ void set_lane_offsets(int64_t ld, int wave_index = -1) {
-    int lane = threadIdx.x & 63;
-    asm volatile("" : "+v"(lane));
+    const int lane = lane_id_here();
     wave = wave_index >= 0 ? wave_index : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rin = lane / kCPR, p = lane % kCPR;
 #pragma unroll
-    for (int i = 0; i < kPerWave; ++i) {
+    for (int i = 0; i < kStored; ++i) {
       const int row = (wave * kPerWave + i) * kRowsPerRegion + rin;
       const int c = p ^ G::swizzle(row);
       voff[i] = row * (int)ld + c * 16;
       kc[i] = c * 16;
     }
+    region_step = kStored * kRowsPerRegion * (int)ld;
   }
 
   __device__ __forceinline__ void set_records() {
@@ -217,8 +232,8 @@ struct DmaLoader {
     const uint32_t lds_base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)lds_tile;
     {
       constexpr int i = I;
-      int vo = voff[i];
-      if constexpr (KMAJOR) vo = (k0 + kc[i] < K) ? vo : 0x7fffffff;
+      int vo = voff[i % kStored] + (i / kStored) * region_step;
+      if constexpr (KMAJOR) vo = (k0 + kc[i % kStored] < K) ? vo : 0x7fffffff;
       const uint32_t dst = lds_base + (uint32_t)((wave * kPerWave + i) * 1024);
       // m0 holds the LDS address of the region; lane l's 16 bytes land at m0 + 16 l.
       // Written as asm so that the compiler, which would otherwise make every later
@@ -318,6 +333,71 @@ __device__ __forceinline__ float load_out_as_f32(const uint8_t* p, int64_t idx, 
 // already receive the first stages of the workgroup's next tile.
 constexpr int kEpiRows = 8;
 
+// Fragment reads of one operand with the address registers spelled out.  Every
+// LDS read of the K loop needs its address in a vector register; what can sit in
+// the instruction's 16-bit offset field instead is whatever differs by a
+// compile-time constant.  The XOR swizzle makes some differences depend on the
+// lane, so left to itself the compiler keeps a register per read (about 30 for a
+// 128 x 128 wave tile).  Spelled out, one register per swizzle pattern is enough:
+//   K-major : the pattern depends on (k half, part) - 4 registers; the 32-row
+//             tile index and the stage are constant offsets;
+//   MN-major: the pattern depends on the 32-column tile index - TILES registers;
+//             k half, part and stage are constant offsets.
+// The two stages of an operand are STAGE_BYTES apart (adjacent, so that the
+// offsets stay below 64 KiB).
+template <bool KMAJOR, int EXT, int TILES>
+struct FragReader {
+  using G = TileGeom<KMAJOR, KMAJOR ? EXT : kBK, KMAJOR ? kBK : EXT>;
+  static constexpr int kRowBytes = KMAJOR ? kBK : EXT;
+  static constexpr int kStageBytes = EXT * kBK;
+  static constexpr int kRegs = KMAJOR ? 4 : TILES;
+  static constexpr int kParts = KMAJOR ? 2 : 4;
+  static_assert(kStageBytes + (KMAJOR ? (TILES - 1) * 32 * kRowBytes : (64 + 24) * kRowBytes) < 65536, "offset field");
+  uint32_t addr[kRegs];
+
+  // lds_operand: LDS address of stage 0 of this operand; mn_wave: first row
+  // (column) of the wave's tile inside the workgroup's
+  __device__ __forceinline__ void init(uint32_t lds_operand, int mn_wave) {
+    const int lane = lane_id_here();
+    if constexpr (KMAJOR) {
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int part = 0; part < 2; ++part)
+          addr[ks * 2 + part] = lds_operand + G::lds_offset(mn_wave + (lane & 31), ks * 4 + (lane >> 5) * 2 + part);
+    } else {
+      // Within each group of 16 lanes, lanes 2r and 2r+1 point at the two 8-byte
+      // halves of k-row r; after the transposing read lane i of the group holds
+      // column i for those 8 k-rows.
+      const int blk = lane >> 4, i = lane & 15;
+      const int r = i >> 1, h = i & 1;
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) {
+        const int col = mn_wave + 32 * t + (blk & 1) * 16;  // first column of this 16-lane group
+        addr[t] = lds_operand + G::lds_offset((blk >> 1) * 32 + r, col >> 4) + h * 8;
+      }
+    }
+  }
+
+  // Part PART of the fragment of tile T, k half KS, from stage STAGE.
+  template <int T, int PART, int KS, int STAGE>
+  __device__ __forceinline__ void read(i32x8& f) const {
+    if constexpr (KMAJOR) {
+      constexpr int off = STAGE * kStageBytes + T * 32 * kRowBytes;
+      const u32x4 v = *reinterpret_cast<LDS_AS const u32x4*>(addr[KS * 2 + PART] + off);
+      f[4 * PART + 0] = v[0];
+      f[4 * PART + 1] = v[1];
+      f[4 * PART + 2] = v[2];
+      f[4 * PART + 3] = v[3];
+    } else {
+      constexpr int off = STAGE * kStageBytes + (KS * 64 + PART * 8) * kRowBytes;
+      const i32x2 t = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<LDS_AS i32x2*>(addr[T] + off));
+      f[2 * PART] = t[0];
+      f[2 * PART + 1] = t[1];
+    }
+  }
+};
+
 template <int MT, int NT>
 constexpr int epilogue_stage_floats() {
   constexpr int general = kEpiRows * (32 * NT + 4) + 2 * 32 * MT;  // fp32 rows + row scales
@@ -331,8 +411,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
   constexpr int kRowFloats = 32 * NT + 4;
   constexpr int kLanesPerRow = 8 * NT;           // a lane owns 4 columns
   constexpr int kRowsPerPass = 64 / kLanesPerRow;
-  int lane = threadIdx.x & 63;
-  asm volatile("" : "+v"(lane));  // keeps lane-derived values out of the registers of the K loop
+  const int lane = lane_id_here();
   const int es = g.out_bf16 ? 2 : 4;
   uint8_t* C = g.C + batch * g.stride_c * es;
   const uint8_t* D = g.D ? g.D + batch * g.stride_d * es : nullptr;
@@ -474,35 +553,23 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
   });
 }
 
-// The forms the fast bf16 epilogue serves: bf16 output through 16-byte stores,
-// A scale a scalar or one value per row, B scale a scalar or one value per
-// column, bias none or a row vector, no accumulate input.
-__device__ __forceinline__ bool epilogue_fast_ok(const GemmArgs& g, int64_t batch) {
+// The forms the fast bf16 epilogue serves: bf16 output, rows and row pitch of C
+// multiples of 16 bytes, N a multiple of 8, A scale a scalar or one value per
+// row, B scale a scalar or one 16-byte-aligned value per column, bias none or
+// an 8-byte-aligned row vector, no accumulate input.  The conditions hold for
+// every matrix of a batch or for none, so the host chooses the kernel.
+inline bool epilogue_fast_ok(const GemmArgs& g, int64_t batches) {
   if (!g.out_bf16 || g.D != nullptr || g.bias_mode == MI355Q_BIAS_FULL) return false;
   if (g.sa_mode == MI355Q_GS_PER_COL || g.sb_mode == MI355Q_GS_PER_ROW) return false;
-  const uintptr_t c = reinterpret_cast<uintptr_t>(g.C) + (size_t)(batch * g.stride_c) * 2;
-  return (c & 15u) == 0 && (g.ldc & 7) == 0;
-}
-
-// Four fp32 column values starting at column n (clamped reads past N).
-__device__ __forceinline__ void load_col4_f32(const float* p, int n, int N, float (&out)[4]) {
-  if (n + 3 < N && (reinterpret_cast<uintptr_t>(p + n) & 15u) == 0) {
-    const f32x4 v = *reinterpret_cast<const f32x4*>(p + n);
-    out[0] = v[0]; out[1] = v[1]; out[2] = v[2]; out[3] = v[3];
-  } else {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) out[e] = p[(n + e) < N ? (n + e) : N - 1];
+  if ((reinterpret_cast<uintptr_t>(g.C) & 15u) != 0 || (g.ldc & 7) != 0 || (g.N & 7) != 0) return false;
+  if (g.ldc > (int64_t(1) << 22)) return false;  // byte offsets inside a wave's rows stay below 2^31
+  if (batches > 1 && (g.stride_c & 7) != 0) return false;
+  if (g.sb_mode == MI355Q_GS_PER_COL && (reinterpret_cast<uintptr_t>(g.sb) & 15u) != 0) return false;
+  if (g.bias_mode == MI355Q_BIAS_ROW_VECTOR) {
+    if ((reinterpret_cast<uintptr_t>(g.bias) & 7u) != 0) return false;
+    if (batches > 1 && (g.stride_bias & 3) != 0) return false;
   }
-}
-__device__ __forceinline__ void load_col4_bf16(const uint16_t* p, int n, int N, float (&out)[4]) {
-  if (n + 3 < N && (reinterpret_cast<uintptr_t>(p + n) & 7u) == 0) {
-    const u32x2 v = *reinterpret_cast<const u32x2*>(p + n);
-    out[0] = __uint_as_float(v[0] << 16); out[1] = __uint_as_float(v[0] & 0xffff0000u);
-    out[2] = __uint_as_float(v[1] << 16); out[3] = __uint_as_float(v[1] & 0xffff0000u);
-  } else {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) out[e] = bf16_bits_to_f32(p[(n + e) < N ? (n + e) : N - 1]);
-  }
+  return true;
 }
 
 // bf16 epilogue for the common forms.  Scales and bias are applied in the
@@ -514,26 +581,23 @@ __device__ __forceinline__ void load_col4_bf16(const uint16_t* p, int n, int N, 
 // of a write cycle (32 rows, one logical slot) and the 16 lanes of a read cycle
 // (rows of equal f, consecutive 16-byte chunks) touch distinct banks; an odd f
 // swaps the two halves of a 16-byte chunk, undone after the read.
-template <int MT, int NT, bool PER_COL>
+// The part that consumes the accumulators is one basic block: rows past M and
+// columns past N are dropped by the store's range check instead of by branches
+// (with branches in it the register allocator copies every accumulator out of
+// the accumulation registers at once and spills).
+template <int MT, int NT, bool PER_COL, bool HAS_BIAS>
 __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t batch, f32x16 (&acc)[MT][NT],
                                                    int m_wave, int n_wave, float* stage_f) {
   constexpr int kRowBytes = 64 * NT;
   constexpr int kSlotMask = 8 * NT - 1;
-  constexpr int kFShift = 3 - NT;            // NT == 1: rows r, r+4 share banks; NT == 2: rows r, r+2
-  static_assert(NT == 1 || NT == 2, "swizzle defined for 64- and 128-byte rows");
+  constexpr int kFShift = NT == 1 ? 2 : (NT == 2 ? 1 : 0);
+  static_assert(NT == 1 || NT == 2 || NT == 4, "swizzle defined for 64-, 128- and 256-byte rows");
   constexpr int kLanesPerRow = 4 * NT;       // a lane reads back 16 bytes
   constexpr int kRowsPerPass = 64 / kLanesPerRow;
   constexpr int kPasses = 32 / kRowsPerPass;
   LDS_AS uint8_t* stage = (LDS_AS uint8_t*)stage_f;
-  // The epilogue sits inside the persistent tile loop, and everything below
-  // that depends only on the lane number is invariant in that loop: left
-  // alone, the compiler computes it all once before the K loop, where no
-  // register is free, and spills it to scratch memory.  Routing the lane number through an empty
-  // volatile asm keeps those few integer operations here.
-  int lane = threadIdx.x & 63;
-  asm volatile("" : "+v"(lane));
+  const int lane = lane_id_here();
   const int r = lane & 31, h = lane >> 5;
-  uint16_t* C = reinterpret_cast<uint16_t*>(g.C) + batch * g.stride_c;
 
   float sa_s = 1.0f, sb_s = 1.0f;
   if (g.sa_mode == MI355Q_GS_HOST) sa_s = g.sa_host;
@@ -541,75 +605,117 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
   if (g.sb_mode == MI355Q_GS_HOST) sb_s = g.sb_host;
   else if (g.sb_mode == MI355Q_GS_DEV) sb_s = g.sb[0];
 
-  // Per-column values of the columns this lane holds in the accumulator layout.
+  // Per-column values of the columns this lane holds in the accumulator layout
+  // (columns at or beyond N read the last four: their results are not stored).
   // A scalar B scale is folded into the row factor instead, which leaves one
   // fused multiply-add per element.
-  constexpr bool per_col = PER_COL;
-  float cs[PER_COL ? NT : 1][4][4], cb[NT][4][4];
+  float cs[PER_COL ? NT : 1][4][4], cb[HAS_BIAS ? NT : 1][4][4];
+  const uint16_t* bias = reinterpret_cast<const uint16_t*>(g.bias) + (HAS_BIAS ? batch * g.stride_bias : 0);
 #pragma unroll
   for (int j = 0; j < NT; ++j)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int n = n_wave + 32 * j + 8 * q + 4 * h;
-      if constexpr (per_col) load_col4_f32(g.sb, n, g.N, cs[j][q]);
-      if (g.bias_mode == MI355Q_BIAS_ROW_VECTOR)
-        load_col4_bf16(reinterpret_cast<const uint16_t*>(g.bias) + batch * g.stride_bias, n, g.N, cb[j][q]);
-      else {
+      int n = n_wave + 32 * j + 8 * q + 4 * h;
+      n = n < g.N - 4 ? n : g.N - 4;
+      if constexpr (PER_COL) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(g.sb + n);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) cb[j][q][e] = 0.0f;
+        for (int e = 0; e < 4; ++e) cs[j][q][e] = v[e];
+      }
+      if constexpr (HAS_BIAS) {
+        const u32x2 v = *reinterpret_cast<const u32x2*>(bias + n);
+        cb[j][q][0] = __uint_as_float(v[0] << 16);
+        cb[j][q][1] = __uint_as_float(v[0] & 0xffff0000u);
+        cb[j][q][2] = __uint_as_float(v[1] << 16);
+        cb[j][q][3] = __uint_as_float(v[1] & 0xffff0000u);
       }
     }
   float ra[MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
     const int m = m_wave + 32 * i + r;
-    ra[i] = g.sa_mode == MI355Q_GS_PER_ROW ? g.sa[m < g.M ? m : g.M - 1] : sa_s;
-    if (!per_col) ra[i] *= sb_s;
+    ra[i] = sa_s;
+    if (g.sa_mode == MI355Q_GS_PER_ROW) ra[i] = g.sa[m < g.M ? m : g.M - 1];
+    if (!PER_COL) ra[i] *= sb_s;
   }
+
+  // C as seen by this wave: a buffer that starts at its first row and ends
+  // after its last row inside the matrix.
+  const int rows = g.M - m_wave < 32 * MT ? g.M - m_wave : 32 * MT;
+  uint16_t* cbase = reinterpret_cast<uint16_t*>(g.C) + batch * g.stride_c + (int64_t)m_wave * g.ldc;
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(cbase, 0, rows > 0 ? rows * (int)g.ldc * 2 : 0, 0x00020000);
 
   const int f_w = (r >> kFShift) & kSlotMask;
   // read-back coordinates
   const int row_in_pass = lane / kLanesPerRow, chunk = lane % kLanesPerRow;
   const int n_out = n_wave + 8 * chunk;
-  const bool full = n_out + 7 < g.N;
+  const int pitch = (int)g.ldc * 2;
+  // columns at or beyond N: an offset no descriptor reaches
+  const int voff0 = n_out < g.N ? row_in_pass * pitch + n_out * 2 : 0x7fffffff;
+  const int pass_step = n_out < g.N ? kRowsPerPass * pitch : 0;
 
-  static_for<MT>([&](auto ic) {
+  // scaled, rounded values of the 32 rows of accumulator row i -> staging area
+  auto write_rows = [&](auto ic) {
     constexpr int i = decltype(ic)::value;
 #pragma unroll
     for (int j = 0; j < NT; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         float v[4];
-        if constexpr (per_col) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf(acc[i][j][4 * q + e] * ra[i], cs[j][q][e], cb[j][q][e]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf(acc[i][j][4 * q + e], ra[i], cb[j][q][e]);
+        for (int e = 0; e < 4; ++e) {
+          const float b = HAS_BIAS ? cb[j][q][e] : 0.0f;
+          if constexpr (PER_COL) v[e] = __builtin_fmaf(acc[i][j][4 * q + e] * ra[i], cs[j][q][e], b);
+          else v[e] = __builtin_fmaf(acc[i][j][4 * q + e], ra[i], b);
         }
         const u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
         const int slot = (8 * j + 2 * q + h) ^ f_w;
         *reinterpret_cast<LDS_AS u32x2*>(stage + r * kRowBytes + slot * 8) = o;
       }
+  };
+  // staging area -> registers, a lane holding 8 consecutive columns of a row per pass
+  auto read_rows = [&](u32x4 (&o)[kPasses]) {
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
       const int row = p * kRowsPerPass + row_in_pass;
       const int f = (row >> kFShift) & kSlotMask;
-      u32x4 o = *reinterpret_cast<LDS_AS u32x4*>(stage + row * kRowBytes + ((chunk ^ (f >> 1)) << 4));
-      if (f & 1) o = u32x4{o[2], o[3], o[0], o[1]};
-      const int m = m_wave + 32 * i + row;
-      if (m < g.M) {
-        uint16_t* cp = C + (int64_t)m * g.ldc + n_out;
-        if (full) {
-          __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(cp));  // streamed: keep the operand panels in L2
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (n_out + e < g.N) cp[e] = (uint16_t)(o[e >> 1] >> (16 * (e & 1)));
-        }
-      }
+      o[p] = *reinterpret_cast<LDS_AS u32x4*>(stage + row * kRowBytes + ((chunk ^ (f >> 1)) << 4));
     }
+  };
+  // A wave's LDS instructions execute in the order issued, so the values of row
+  // i + 1 may be written into the one staging area as soon as the reads of row
+  // i have been issued: the arithmetic of row i + 1 runs while those reads are
+  // on their way, and the stores of row i follow without a wait.
+  u32x4 o[kPasses];
+  write_rows(std::integral_constant<int, 0>{});
+  read_rows(o);
+  static_for<MT>([&](auto ic) {
+    constexpr int i = decltype(ic)::value;
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (i + 1 < MT) write_rows(std::integral_constant<int, i + 1>{});
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) {
+      const int f = ((p * kRowsPerPass + row_in_pass) >> kFShift) & kSlotMask;
+      const u32x4 v = (f & 1) ? u32x4{o[p][2], o[p][3], o[p][0], o[p][1]} : o[p];
+      // lanes whose offset lies at or beyond the descriptor's size store nothing;
+      // aux 2 = nt: streamed, keeps the operand panels in L2
+      __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, voff0 + (i * kPasses + p) * pass_step, 0, 2);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (i + 1 < MT) read_rows(o);
   });
+}
+
+template <int MT, int NT>
+__device__ __forceinline__ void epilogue_bf16_fast_any(const GemmArgs& g, int64_t batch, f32x16 (&acc)[MT][NT],
+                                                       int m_wave, int n_wave, float* stage) {
+  const bool per_col = g.sb_mode == MI355Q_GS_PER_COL, bias = g.bias_mode == MI355Q_BIAS_ROW_VECTOR;
+  if (per_col && bias) epilogue_bf16_fast<MT, NT, true, true>(g, batch, acc, m_wave, n_wave, stage);
+  else if (per_col) epilogue_bf16_fast<MT, NT, true, false>(g, batch, acc, m_wave, n_wave, stage);
+  else if (bias) epilogue_bf16_fast<MT, NT, false, true>(g, batch, acc, m_wave, n_wave, stage);
+  else epilogue_bf16_fast<MT, NT, false, false>(g, batch, acc, m_wave, n_wave, stage);
 }
 
 // Per-wave state of the K loop: accumulators, fragments, loaders.
@@ -620,29 +726,41 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
 // the current one is in use), the A fragments are single-buffered and rolled:
 // MFMAs run row by row, A_i is dead after the last MFMA of row i, and the next
 // half-step's A_i is read into the same registers right then.
-template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
+template <int BM, int BN, int WN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
 struct TileCore {
-  static constexpr int TM = BM / kWavesM, TN = BN / kWavesN;
+  static constexpr int TM = BM / kWavesM, TN = BN / WN;
+  using LoaderA = DmaLoader<A_KMAJOR, BM, kBK, kWavesM * WN>;
+  using LoaderB = DmaLoader<B_KMAJOR, BN, kBK, kWavesM * WN>;
   static constexpr int MT = TM / 32, NT = TN / 32;
+  using ReaderA = FragReader<A_KMAJOR, BM, MT>;
+  using ReaderB = FragReader<B_KMAJOR, BN, NT>;
+  // LDS ring: the two stages of A, then the two stages of B
+  static constexpr int kStageA = BM * kBK, kStageB = BN * kBK;
+  static constexpr int kRingBytes = 2 * (kStageA + kStageB);
   f32x16 acc[MT][NT];
   i32x8 fa[MT], fb0[NT], fb1[NT];
-  DmaLoader<A_KMAJOR, BM> la;
-  DmaLoader<B_KMAJOR, BN> lb;
+  LoaderA la;
+  LoaderB lb;
+  ReaderA ra;
+  ReaderB rb;
+  uint8_t* ring;
   int wm, wn, K;
 
-  __device__ __forceinline__ void init(const GemmArgs& g, int wm_, int wn_) {
+  __device__ __forceinline__ void init(const GemmArgs& g, uint8_t* ring_, int wm_, int wn_) {
+    ring = ring_;
     wm = wm_;
     wn = wn_;
     K = g.K;
   }
 
-  __device__ __forceinline__ void zero_acc() {
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  // Per-lane addresses (LDS reads, global->LDS loads); recomputed for every
+  // tile rather than kept live through the epilogue.
+  __device__ __forceinline__ void set_lane_addresses(const GemmArgs& g) {
+    const uint32_t base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)ring;
+    ra.init(base, wm);
+    rb.init(base + 2 * kStageA, wn);
+    la.set_lane_offsets(g.lda);
+    lb.set_lane_offsets(g.ldb);
   }
 
   // Points the loaders at tile (m0, n0); `valid` false makes every load of the
@@ -652,66 +770,61 @@ struct TileCore {
     lb.set_tile(g.B + batch * g.stride_b, g.ldb, n0, g.N, g.K, valid);
   }
 
-  static constexpr int kPartsA = frag_parts<A_KMAJOR>(), kPartsB = frag_parts<B_KMAJOR>();
+  static constexpr int kPartsA = ReaderA::kParts, kPartsB = ReaderB::kParts;
   static constexpr int kMfmas = MT * NT;
-  static constexpr int kDmaOps = DmaLoader<A_KMAJOR, BM>::kPerWave + DmaLoader<B_KMAJOR, BN>::kPerWave;
+  static constexpr int kDmaOps = LoaderA::kPerWave + LoaderB::kPerWave;
 
-  template <int I, int PART>
-  __device__ __forceinline__ void read_a(const uint8_t* stage, int ks) {
-    read_fragment_part<A_KMAJOR, BM, PART>(stage, wm + I * 32, ks, fa[I]);
-  }
-  template <int J, int PART>
-  __device__ __forceinline__ void read_b(const uint8_t* stage, int ks, i32x8 (&fb)[NT]) {
-    read_fragment_part<B_KMAJOR, BN, PART>(stage + BM * kBK, wn + J * 32, ks, fb[J]);
+  template <int OP, int STAGE>
+  __device__ __forceinline__ void dma_op(int kt) {
+    constexpr int na = LoaderA::kPerWave;
+    if constexpr (OP < na) la.template issue_one<OP>(ring + STAGE * kStageA, kt * kBK, K);
+    else lb.template issue_one<OP - na>(ring + 2 * kStageA + STAGE * kStageB, kt * kBK, K);
   }
 
-  template <int OP>
-  __device__ __forceinline__ void dma_op(uint8_t* stage, int kt) {
-    constexpr int na = DmaLoader<A_KMAJOR, BM>::kPerWave;
-    if constexpr (OP < na) la.template issue_one<OP>(stage, kt * kBK, K);
-    else lb.template issue_one<OP - na>(stage + BM * kBK, kt * kBK, K);
-  }
-
-  __device__ __forceinline__ void issue_stage(uint8_t* __restrict__ stage, int kt) {
-    static_for<kDmaOps>([&](auto oc) { dma_op<decltype(oc)::value>(stage, kt); });
+  template <int STAGE>
+  __device__ __forceinline__ void issue_stage(int kt) {
+    static_for<kDmaOps>([&](auto oc) { dma_op<decltype(oc)::value, STAGE>(kt); });
     la.advance();
     lb.advance();
   }
 
   // One MFMA block (every tile of the wave, 64 k) on the fragments (fa, cb),
-  // with the LDS reads of the next block's fragments and, when WITH_DMA, this
-  // wave's global->LDS loads of a later stage dealt out between the MFMAs.
+  // with the LDS reads of the next block's fragments (k half RD_KS of stage
+  // RD_STAGE) and, when DMA_STAGE >= 0, this wave's global->LDS loads of K
+  // stage dma_kt into that stage dealt out between the MFMAs.
   // sched_barrier(0) after each group pins the written order (left alone, the
   // scheduler gathers the reads after the MFMAs).
-  template <bool WITH_DMA>
-  __device__ __forceinline__ void block(const i32x8 (&cb)[NT], i32x8 (&nb)[NT],
-                                        const uint8_t* __restrict__ rd_stage, int rd_ks,
-                                        uint8_t* __restrict__ dma_stage, int dma_kt) {
+  // ZERO_C: the first block of a tile, which starts the sums (no pass over the
+  // accumulators to clear them).
+  template <int RD_STAGE, int RD_KS, int DMA_STAGE, bool ZERO_C>
+  __device__ __forceinline__ void block(const i32x8 (&cb)[NT], i32x8 (&nb)[NT], int dma_kt) {
+    constexpr bool kWithDma = DMA_STAGE >= 0;
     constexpr int kBOps = NT * kPartsB;
     constexpr int kBPerGroup = (kBOps + kMfmas - 1) / kMfmas;
     constexpr int kDmaPerGroup = (kDmaOps + kMfmas - 1) / kMfmas;
     static_for<kMfmas>([&](auto gc) {
       constexpr int gi = decltype(gc)::value;
       constexpr int i = gi / NT, j = gi % NT;
+      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-          cb[j], fa[i], acc[i][j], mfma_code<FMT_B>(), mfma_code<FMT_A>(), 0, 0, 0, 0);
-      if constexpr (WITH_DMA) {
+          cb[j], fa[i], ZERO_C ? zero : acc[i][j], mfma_code<FMT_B>(), mfma_code<FMT_A>(), 0, 0, 0, 0);
+      if constexpr (kWithDma) {
         static_for<kDmaPerGroup>([&](auto dc) {
           constexpr int op = gi * kDmaPerGroup + decltype(dc)::value;
-          if constexpr (op < kDmaOps) dma_op<op>(dma_stage, dma_kt);
+          if constexpr (op < kDmaOps) dma_op<op, kWithDma ? DMA_STAGE : 0>(dma_kt);
         });
       }
       static_for<kBPerGroup>([&](auto rc) {
         constexpr int op = gi * kBPerGroup + decltype(rc)::value;
-        if constexpr (op < kBOps) read_b<op / kPartsB, op % kPartsB>(rd_stage, rd_ks, nb);
+        if constexpr (op < kBOps) rb.template read<op / kPartsB, op % kPartsB, RD_KS, RD_STAGE>(nb[op / kPartsB]);
       });
       if constexpr (j == NT - 1) {
         // row i of MFMAs is done: its A fragment is dead, fetch the next half-step's
-        static_for<kPartsA>([&](auto pc) { read_a<i, decltype(pc)::value>(rd_stage, rd_ks); });
+        static_for<kPartsA>([&](auto pc) { ra.template read<i, decltype(pc)::value, RD_KS, RD_STAGE>(fa[i]); });
       }
       __builtin_amdgcn_sched_barrier(0);
     });
-    if constexpr (WITH_DMA) {
+    if constexpr (kWithDma) {
       la.advance();
       lb.advance();
     }
@@ -726,27 +839,29 @@ struct TileCore {
   }
 
   // First fragments of a tile whose stages 0 and 1 have been issued.
-  __device__ __forceinline__ void first_fragments(uint8_t* __restrict__ s0) {
+  __device__ __forceinline__ void first_fragments() {
     wait_loads_then_barrier();
     static_for<MT>([&](auto ic) {
-      static_for<kPartsA>([&](auto pc) { read_a<decltype(ic)::value, decltype(pc)::value>(s0, 0); });
+      static_for<kPartsA>([&](auto pc) { ra.template read<decltype(ic)::value, decltype(pc)::value, 0, 0>(fa[decltype(ic)::value]); });
     });
     static_for<NT>([&](auto jc) {
-      static_for<kPartsB>([&](auto pc) { read_b<decltype(jc)::value, decltype(pc)::value>(s0, 0, fb0); });
+      static_for<kPartsB>([&](auto pc) { rb.template read<decltype(jc)::value, decltype(pc)::value, 0, 0>(fb0[decltype(jc)::value]); });
     });
   }
 
-  // Two K stages: stage kt sits in s0, stage kt+1 in s1 (or is still landing
-  // there).  After each barrier every wave is done with the stage just
-  // consumed, so the stage two ahead starts to overwrite it while the second
-  // half of the current stage and the whole next stage compute.
-  __device__ __forceinline__ void k_pair(uint8_t* __restrict__ s0, uint8_t* __restrict__ s1, int kt) {
-    block<false>(fb0, fb1, s0, 1, nullptr, 0);
+  // Two K stages: stage kt sits in ring stage 0, stage kt+1 in ring stage 1 (or
+  // is still landing there).  After each barrier every wave is done with the
+  // stage just consumed, so the stage two ahead starts to overwrite it while
+  // the second half of the current stage and the whole next stage compute.
+  // FIRST: the first two stages of a tile.
+  template <bool FIRST>
+  __device__ __forceinline__ void k_pair(int kt) {
+    block<0, 1, -1, FIRST>(fb0, fb1, 0);
     wait_loads_then_barrier();
-    block<true>(fb1, fb0, s1, 0, s0, kt + 2);
-    block<false>(fb0, fb1, s1, 1, nullptr, 0);
+    block<1, 0, 0, false>(fb1, fb0, kt + 2);
+    block<1, 1, -1, false>(fb0, fb1, 0);
     wait_loads_then_barrier();
-    block<true>(fb1, fb0, s0, 0, s1, kt + 3);
+    block<0, 0, 1, false>(fb1, fb0, kt + 3);
   }
 };
 
@@ -768,15 +883,15 @@ __device__ __forceinline__ void tile_coords(int logical, int tiles_m, int tiles_
 // a contiguous range of the tile order, and in round r its workgroups take the
 // next gridDim.x / 8 tiles of that range, so that the tiles in flight on one
 // XCD form a compact patch that shares A and B panels in its L2.
-template <int BM, int BN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
-__global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g) {
-  constexpr int TM = BM / kWavesM, TN = BN / kWavesN;   // per-wave tile
+template <int BM, int BN, int WN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B, bool FAST_ONLY>
+__global__ __launch_bounds__(kWavesM * WN * 64) void fp8_gemm_tile_kernel(GemmArgs g) {
+  constexpr int kWaves = kWavesM * WN;
+  constexpr int TM = BM / kWavesM, TN = BN / WN;   // per-wave tile
   constexpr int MT = TM / 32, NT = TN / 32;             // MFMA tiles per wave
   constexpr int kStageBytes = (BM + BN) * kBK;
-  // Two stages as two separate arrays, so that loads into one and reads from
-  // the other are provably disjoint; the epilogue has its own staging area.
-  __shared__ __attribute__((aligned(1024))) uint8_t lds0[kStageBytes];
-  __shared__ __attribute__((aligned(1024))) uint8_t lds1[kStageBytes];
+  using Core = TileCore<BM, BN, WN, A_KMAJOR, B_KMAJOR, FMT_A, FMT_B>;
+  // two stages of each operand; the epilogue has its own staging area
+  __shared__ __attribute__((aligned(1024))) uint8_t lds_ring[Core::kRingBytes];
   __shared__ __attribute__((aligned(16))) float lds_epi[kWaves * epilogue_stage_floats<MT, NT>()];
 
   const int nb = gridDim.x, bid = blockIdx.x;
@@ -788,14 +903,12 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g)
   const int count = per + (xcd < rem ? 1 : 0);        // tiles of this XCD
 
   const int64_t batch = blockIdx.y;
-  const int wave = threadIdx.x >> 6;
-  const int wm = (wave / kWavesN) * TM, wn = (wave % kWavesN) * TN;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = (wave / WN) * TM, wn = (wave % WN) * TN;
   float* stage = lds_epi + wave * epilogue_stage_floats<MT, NT>();
 
-  const bool fast_epilogue = epilogue_fast_ok(g, batch);
-
-  TileCore<BM, BN, A_KMAJOR, B_KMAJOR, FMT_A, FMT_B> core;
-  core.init(g, wm, wn);
+  Core core;
+  core.init(g, lds_ring, wm, wn);
   const int KT = (g.K + kBK - 1) / kBK;
   const int KT2 = (KT + 1) & ~1;
 
@@ -809,16 +922,16 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g)
   if (idx >= count) return;
   int tile_m, tile_n;
   tile_coords(first + idx, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-  core.la.set_lane_offsets(g.lda);
-  core.lb.set_lane_offsets(g.ldb);
+  core.set_lane_addresses(g);
   core.retarget(g, batch, tile_m * BM, tile_n * BN, true);
-  core.issue_stage(lds0, 0);
-  core.issue_stage(lds1, 1);
+  core.template issue_stage<0>(0);
+  core.template issue_stage<1>(1);
   for (;;) {
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    core.zero_acc();
-    core.first_fragments(lds0);
-    for (int kt = 0; kt < KT2; kt += 2) {
+    core.first_fragments();
+    // Two stages per step; the step that issues the last loads of this tile's
+    // stages (the last one) first points the loaders at the next tile.
+    auto k_step = [&](auto first_c, int kt) {
       if (kt + 2 == KT2) {
         idx += slots;
         const bool more = idx < count;
@@ -826,24 +939,25 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_tile_kernel(GemmArgs g)
         core.retarget(g, batch, tile_m * BM, tile_n * BN, more);
       }
       // stage numbers restart at 0 for the next tile
-      core.k_pair(lds0, lds1, kt + 2 == KT2 ? -2 : kt);
-    }
-    if (fast_epilogue) {
-      if (g.sb_mode == MI355Q_GS_PER_COL) epilogue_bf16_fast<MT, NT, true>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
-      else epilogue_bf16_fast<MT, NT, false>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
+      core.template k_pair<decltype(first_c)::value>(kt + 2 == KT2 ? -2 : kt);
+    };
+    k_step(std::true_type{}, 0);
+    for (int kt = 2; kt < KT2; kt += 2) k_step(std::false_type{}, kt);
+    if (FAST_ONLY || g.fast_epi) {
+      epilogue_bf16_fast_any<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
     } else {
       epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
     }
     if (idx >= count) break;
-    // recomputed rather than kept live through the epilogue
-    core.la.set_lane_offsets(g.lda);
-    core.lb.set_lane_offsets(g.ldb);
+    core.set_lane_addresses(g);
   }
   // drain the (out-of-range) loads issued for the tile that does not exist
   __builtin_amdgcn_s_waitcnt(0);
 }
 
-template <int BM, int BN, bool AK, bool BK_, int FA, int FB>
+// WN: waves along n (the workgroup has 2 x WN); FAST_ONLY: the kernel carries
+// the fast bf16 epilogue alone and the launch must satisfy epilogue_fast_ok().
+template <int BM, int BN, int WN, bool FAST_ONLY, bool AK, bool BK_, int FA, int FB>
 void launch_tile(const GemmArgs& g, int64_t batch, hipStream_t st) {
   GemmArgs a = g;
   a.tiles_m = (g.M + BM - 1) / BM;
@@ -851,7 +965,7 @@ void launch_tile(const GemmArgs& g, int64_t batch, hipStream_t st) {
   const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
   const int cus = compute_units();
   dim3 grid((unsigned)(tiles < cus ? tiles : cus), (unsigned)batch);
-  fp8_gemm_tile_kernel<BM, BN, AK, BK_, FA, FB><<<grid, kGemmThreads, 0, st>>>(a);
+  fp8_gemm_tile_kernel<BM, BN, WN, AK, BK_, FA, FB, FAST_ONLY><<<grid, kWavesM * WN * 64, 0, st>>>(a);
 }
 
 // A K-major / B K-major etc.; defined in gemm_inst_*.hip
