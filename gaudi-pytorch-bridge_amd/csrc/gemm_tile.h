@@ -398,6 +398,22 @@ struct FragReader {
   }
 };
 
+// The scalar (per-tensor) scales of a launch.
+struct ScalarScales {
+  float sa, sb;
+};
+__device__ __forceinline__ ScalarScales load_scalar_scales(const GemmArgs& g) {
+  ScalarScales s = {1.0f, 1.0f};
+  if (g.sa_mode == MI355Q_GS_HOST) s.sa = g.sa_host;
+  else if (g.sa_mode == MI355Q_GS_DEV) s.sa = g.sa[0];
+  if (g.sb_mode == MI355Q_GS_HOST) s.sb = g.sb_host;
+  else if (g.sb_mode == MI355Q_GS_DEV) s.sb = g.sb[0];
+  // consumed here, so the wait for the loads is here as well
+  s.sa = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s.sa)));
+  s.sb = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s.sb)));
+  return s;
+}
+
 template <int MT, int NT>
 constexpr int epilogue_stage_floats() {
   constexpr int general = kEpiRows * (32 * NT + 4) + 2 * 32 * MT;  // fp32 rows + row scales
@@ -416,11 +432,8 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
   uint8_t* C = g.C + batch * g.stride_c * es;
   const uint8_t* D = g.D ? g.D + batch * g.stride_d * es : nullptr;
   const uint8_t* bias = g.bias ? g.bias + batch * g.stride_bias * es : nullptr;
-  float sa_s = 1.0f, sb_s = 1.0f;
-  if (g.sa_mode == MI355Q_GS_HOST) sa_s = g.sa_host;
-  else if (g.sa_mode == MI355Q_GS_DEV) sa_s = g.sa[0];
-  if (g.sb_mode == MI355Q_GS_HOST) sb_s = g.sb_host;
-  else if (g.sb_mode == MI355Q_GS_DEV) sb_s = g.sb[0];
+  const ScalarScales scalars = load_scalar_scales(g);
+  const float sa_s = scalars.sa, sb_s = scalars.sb;
 
   // the 4 columns this lane owns in the read-back layout, and what depends on them only
   const int r_in = lane / kLanesPerRow;
@@ -572,6 +585,10 @@ inline bool epilogue_fast_ok(const GemmArgs& g, int64_t batches) {
   return true;
 }
 
+// Stores a wave issues in epilogue_bf16_fast, all of them after its loads.
+template <int MT, int NT>
+constexpr int fast_epilogue_stores() { return MT * 2 * NT; }
+
 // bf16 epilogue for the common forms.  Scales and bias are applied in the
 // accumulator layout (a lane holds one row m and runs of 4 columns), the
 // rounded bf16 values of 32 rows pass through a per-wave LDS area of 32 rows x
@@ -585,9 +602,21 @@ inline bool epilogue_fast_ok(const GemmArgs& g, int64_t batches) {
 // columns past N are dropped by the store's range check instead of by branches
 // (with branches in it the register allocator copies every accumulator out of
 // the accumulation registers at once and spills).
-template <int MT, int NT, bool PER_COL, bool HAS_BIAS>
+// STAGED: the scale and bias values of the wave's rows and columns already sit
+// in its staging area (ScaleStager, below) and the scalar scales come as
+// arguments, so that the epilogue loads nothing from global memory: a wait for
+// such a load would also wait for every global->LDS load issued before it,
+// that is for the next tile's first stages.
+// Layout of the staged values in a wave's staging area (bytes): B scales of its
+// 32 NT columns (fp32), bias of the same columns (bf16), A scales of its 32 MT
+// rows (fp32).  Values of a kind the problem does not have are zeros.
+constexpr int kStagedColScale = 0, kStagedBias = 512, kStagedRowScale = 768, kStagedBytes = 1280;
+
+template <int MT, int NT, bool PER_COL, bool HAS_BIAS, bool STAGED = false>
 __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t batch, f32x16 (&acc)[MT][NT],
-                                                   int m_wave, int n_wave, float* stage_f) {
+                                                   int m_wave, int n_wave, float* stage_f,
+                                                   ScalarScales scalars = ScalarScales{1.0f, 1.0f}) {
+  static_assert(MT <= 4 && NT <= 4, "staged layout");
   constexpr int kRowBytes = 64 * NT;
   constexpr int kSlotMask = 8 * NT - 1;
   constexpr int kFShift = NT == 1 ? 2 : (NT == 2 ? 1 : 0);
@@ -599,11 +628,8 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
   const int lane = lane_id_here();
   const int r = lane & 31, h = lane >> 5;
 
-  float sa_s = 1.0f, sb_s = 1.0f;
-  if (g.sa_mode == MI355Q_GS_HOST) sa_s = g.sa_host;
-  else if (g.sa_mode == MI355Q_GS_DEV) sa_s = g.sa[0];
-  if (g.sb_mode == MI355Q_GS_HOST) sb_s = g.sb_host;
-  else if (g.sb_mode == MI355Q_GS_DEV) sb_s = g.sb[0];
+  if constexpr (!STAGED) scalars = load_scalar_scales(g);
+  const float sa_s = scalars.sa, sb_s = scalars.sb;
 
   // Per-column values of the columns this lane holds in the accumulator layout
   // (columns at or beyond N read the last four: their results are not stored).
@@ -615,15 +641,18 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
   for (int j = 0; j < NT; ++j)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      int n = n_wave + 32 * j + 8 * q + 4 * h;
+      const int col = 32 * j + 8 * q + 4 * h;  // inside the wave's tile
+      int n = n_wave + col;
       n = n < g.N - 4 ? n : g.N - 4;
       if constexpr (PER_COL) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(g.sb + n);
+        const f32x4 v = STAGED ? *reinterpret_cast<LDS_AS const f32x4*>(stage + kStagedColScale + col * 4)
+                               : *reinterpret_cast<const f32x4*>(g.sb + n);
 #pragma unroll
         for (int e = 0; e < 4; ++e) cs[j][q][e] = v[e];
       }
       if constexpr (HAS_BIAS) {
-        const u32x2 v = *reinterpret_cast<const u32x2*>(bias + n);
+        const u32x2 v = STAGED ? *reinterpret_cast<LDS_AS const u32x2*>(stage + kStagedBias + col * 2)
+                               : *reinterpret_cast<const u32x2*>(bias + n);
         cb[j][q][0] = __uint_as_float(v[0] << 16);
         cb[j][q][1] = __uint_as_float(v[0] & 0xffff0000u);
         cb[j][q][2] = __uint_as_float(v[1] << 16);
@@ -634,8 +663,13 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
     const int m = m_wave + 32 * i + r;
-    ra[i] = sa_s;
-    if (g.sa_mode == MI355Q_GS_PER_ROW) ra[i] = g.sa[m < g.M ? m : g.M - 1];
+    if constexpr (STAGED) {
+      const float staged = *reinterpret_cast<LDS_AS const float*>(stage + kStagedRowScale + (32 * i + r) * 4);
+      ra[i] = g.sa_mode == MI355Q_GS_PER_ROW ? staged : sa_s;
+    } else {
+      ra[i] = sa_s;
+      if (g.sa_mode == MI355Q_GS_PER_ROW) ra[i] = g.sa[m < g.M ? m : g.M - 1];
+    }
     if (!PER_COL) ra[i] *= sb_s;
   }
 
@@ -687,6 +721,7 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
   // i + 1 may be written into the one staging area as soon as the reads of row
   // i have been issued: the arithmetic of row i + 1 runs while those reads are
   // on their way, and the stores of row i follow without a wait.
+  static_assert(MT * kPasses == fast_epilogue_stores<MT, NT>(), "the K loop counts these stores");
   u32x4 o[kPasses];
   write_rows(std::integral_constant<int, 0>{});
   read_rows(o);
@@ -708,15 +743,59 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
   });
 }
 
-template <int MT, int NT>
+template <int MT, int NT, bool STAGED = false>
 __device__ __forceinline__ void epilogue_bf16_fast_any(const GemmArgs& g, int64_t batch, f32x16 (&acc)[MT][NT],
-                                                       int m_wave, int n_wave, float* stage) {
+                                                       int m_wave, int n_wave, float* stage,
+                                                       ScalarScales scalars = ScalarScales{1.0f, 1.0f}) {
   const bool per_col = g.sb_mode == MI355Q_GS_PER_COL, bias = g.bias_mode == MI355Q_BIAS_ROW_VECTOR;
-  if (per_col && bias) epilogue_bf16_fast<MT, NT, true, true>(g, batch, acc, m_wave, n_wave, stage);
-  else if (per_col) epilogue_bf16_fast<MT, NT, true, false>(g, batch, acc, m_wave, n_wave, stage);
-  else if (bias) epilogue_bf16_fast<MT, NT, false, true>(g, batch, acc, m_wave, n_wave, stage);
-  else epilogue_bf16_fast<MT, NT, false, false>(g, batch, acc, m_wave, n_wave, stage);
+  if (per_col && bias) epilogue_bf16_fast<MT, NT, true, true, STAGED>(g, batch, acc, m_wave, n_wave, stage, scalars);
+  else if (per_col) epilogue_bf16_fast<MT, NT, true, false, STAGED>(g, batch, acc, m_wave, n_wave, stage, scalars);
+  else if (bias) epilogue_bf16_fast<MT, NT, false, true, STAGED>(g, batch, acc, m_wave, n_wave, stage, scalars);
+  else epilogue_bf16_fast<MT, NT, false, false, STAGED>(g, batch, acc, m_wave, n_wave, stage, scalars);
 }
+
+// Brings the scale and bias values the fast epilogue of one wave tile needs
+// into the wave's staging area with global->LDS loads, which join the K loop's
+// stream of such loads (and its waits).  Ranges past N or M read as zeros.
+struct ScaleStager {
+  // 64 lanes x 4 bytes from `base` + 256 `part` (at most `bytes` valid from base) to lds_dst + 256 part
+  __device__ __forceinline__ static void load_256(const void* base, int64_t bytes, int part, uint32_t lds_dst) {
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    const int64_t rec = bytes < 0 ? 0 : (bytes > 0x40000000 ? 0x40000000 : bytes);
+    i32x4 rsrc;
+    rsrc[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    rsrc[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((b >> 32) & 0xffffu));
+    rsrc[2] = __builtin_amdgcn_readfirstlane((int)rec);
+    rsrc[3] = 0x00020000;
+    const int vo = lane_id_here() * 4 + part * 256;
+    const uint32_t dst = lds_dst + part * 256;
+    // m0 holds the LDS address; lane l's 4 bytes land at m0 + 4 l.  The s_nop
+    // covers a descriptor word that reaches its scalar register through
+    // v_readfirstlane (five wait states before a memory instruction reads it).
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dword %1, %2, 0 offen lds"
+                 :
+                 : "s"(dst), "v"(vo), "s"(rsrc)
+                 : "memory", "m0");
+  }
+
+  template <int MT, int NT>
+  __device__ __forceinline__ static void issue(const GemmArgs& g, int64_t batch, int m_wave, int n_wave, float* stage_f) {
+    const uint32_t lds = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)stage_f;
+    const bool per_col = g.sb_mode == MI355Q_GS_PER_COL, per_row = g.sa_mode == MI355Q_GS_PER_ROW;
+    const bool has_bias = g.bias_mode == MI355Q_BIAS_ROW_VECTOR;
+    constexpr int kColParts = (32 * NT * 4 + 255) / 256, kRowParts = (32 * MT * 4 + 255) / 256;
+    static_for<kColParts>([&](auto pc) {
+      load_256(g.sb + n_wave, per_col ? (int64_t)(g.N - n_wave) * 4 : 0, decltype(pc)::value, lds + kStagedColScale);
+    });
+    load_256(reinterpret_cast<const uint16_t*>(g.bias) + batch * g.stride_bias + n_wave,
+             has_bias ? (int64_t)(g.N - n_wave) * 2 : 0, 0, lds + kStagedBias);
+    static_for<kRowParts>([&](auto pc) {
+      load_256(g.sa + m_wave, per_row ? (int64_t)(g.M - m_wave) * 4 : 0, decltype(pc)::value, lds + kStagedRowScale);
+    });
+  }
+  template <int MT, int NT>
+  static constexpr int ops() { return (32 * NT * 4 + 255) / 256 + 1 + (32 * MT * 4 + 255) / 256; }
+};
 
 // Per-wave state of the K loop: accumulators, fragments, loaders.
 //
@@ -744,10 +823,11 @@ struct TileCore {
   ReaderA ra;
   ReaderB rb;
   uint8_t* ring;
-  int wm, wn, K;
+  int wave, wm, wn, K;  // wave: index in the workgroup (uniform)
 
-  __device__ __forceinline__ void init(const GemmArgs& g, uint8_t* ring_, int wm_, int wn_) {
+  __device__ __forceinline__ void init(const GemmArgs& g, uint8_t* ring_, int wave_, int wm_, int wn_) {
     ring = ring_;
+    wave = wave_;
     wm = wm_;
     wn = wn_;
     K = g.K;
@@ -759,8 +839,8 @@ struct TileCore {
     const uint32_t base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)ring;
     ra.init(base, wm);
     rb.init(base + 2 * kStageA, wn);
-    la.set_lane_offsets(g.lda);
-    lb.set_lane_offsets(g.ldb);
+    la.set_lane_offsets(g.lda, wave);
+    lb.set_lane_offsets(g.ldb, wave);
   }
 
   // Points the loaders at tile (m0, n0); `valid` false makes every load of the
@@ -831,16 +911,25 @@ struct TileCore {
   }
 
   // A workgroup barrier orders LDS traffic but does not wait for this wave's
-  // outstanding global->LDS loads: drain them first (vmcnt(0)), so that after
-  // the barrier every wave sees every wave's share of the stage.
-  __device__ __forceinline__ static void wait_loads_then_barrier() {
-    __builtin_amdgcn_s_waitcnt(0);
+  // outstanding global->LDS loads: drain them first, so that after the barrier
+  // every wave sees every wave's share of the stage.
+  // The counter of outstanding vector memory operations retires in issue order.
+  // The first two stages of a tile are issued before the previous tile's
+  // epilogue, whose kEpilogueStores stores are therefore younger: when those are
+  // pending (younger_stores), waiting until only that many operations are
+  // outstanding waits for the loads and not for the stores, which take a few
+  // microseconds to be acknowledged when every workgroup stores at once.
+  static constexpr int kEpilogueStores = fast_epilogue_stores<MT, NT>();
+  static_assert(kEpilogueStores < 64, "vmcnt holds 6 bits");
+  __device__ __forceinline__ static void wait_loads_then_barrier(bool younger_stores = false) {
+    if (younger_stores) __builtin_amdgcn_s_waitcnt((kEpilogueStores & 15) | ((kEpilogueStores >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
   }
 
   // First fragments of a tile whose stages 0 and 1 have been issued.
-  __device__ __forceinline__ void first_fragments() {
-    wait_loads_then_barrier();
+  __device__ __forceinline__ void first_fragments(bool younger_stores) {
+    wait_loads_then_barrier(younger_stores);
     static_for<MT>([&](auto ic) {
       static_for<kPartsA>([&](auto pc) { ra.template read<decltype(ic)::value, decltype(pc)::value, 0, 0>(fa[decltype(ic)::value]); });
     });
@@ -854,11 +943,14 @@ struct TileCore {
   // stage just consumed, so the stage two ahead starts to overwrite it while
   // the second half of the current stage and the whole next stage compute.
   // FIRST: the first two stages of a tile.
-  template <bool FIRST>
-  __device__ __forceinline__ void k_pair(int kt) {
+  // after_first_loads: called once the first pair has issued its loads (the
+  // place for other loads that the tile's later waits should cover).
+  template <bool FIRST, typename F>
+  __device__ __forceinline__ void k_pair(int kt, bool younger_stores, F&& after_first_loads) {
     block<0, 1, -1, FIRST>(fb0, fb1, 0);
-    wait_loads_then_barrier();
+    wait_loads_then_barrier(FIRST && younger_stores);  // stage 1 of a tile is as old as stage 0
     block<1, 0, 0, false>(fb1, fb0, kt + 2);
+    if constexpr (FIRST) after_first_loads();
     block<1, 1, -1, false>(fb0, fb1, 0);
     wait_loads_then_barrier();
     block<0, 0, 1, false>(fb1, fb0, kt + 3);
@@ -908,7 +1000,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void fp8_gemm_tile_kernel(GemmAr
   float* stage = lds_epi + wave * epilogue_stage_floats<MT, NT>();
 
   Core core;
-  core.init(g, lds_ring, wm, wn);
+  core.init(g, lds_ring, wave, wm, wn);
   const int KT = (g.K + kBK - 1) / kBK;
   const int KT2 = (KT + 1) & ~1;
 
@@ -926,9 +1018,11 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void fp8_gemm_tile_kernel(GemmAr
   core.retarget(g, batch, tile_m * BM, tile_n * BN, true);
   core.template issue_stage<0>(0);
   core.template issue_stage<1>(1);
+  const ScalarScales scalars = load_scalar_scales(g);
+  bool stores_pending = false;  // the fast epilogue's stores of the previous tile
   for (;;) {
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    core.first_fragments();
+    core.first_fragments(stores_pending);
     // Two stages per step; the step that issues the last loads of this tile's
     // stages (the last one) first points the loaders at the next tile.
     auto k_step = [&](auto first_c, int kt) {
@@ -939,12 +1033,15 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void fp8_gemm_tile_kernel(GemmAr
         core.retarget(g, batch, tile_m * BM, tile_n * BN, more);
       }
       // stage numbers restart at 0 for the next tile
-      core.template k_pair<decltype(first_c)::value>(kt + 2 == KT2 ? -2 : kt);
+      core.template k_pair<decltype(first_c)::value>(kt + 2 == KT2 ? -2 : kt, stores_pending, [&] {
+        if (FAST_ONLY || g.fast_epi) ScaleStager::issue<MT, NT>(g, batch, m0 + wm, n0 + wn, stage);
+      });
     };
     k_step(std::true_type{}, 0);
     for (int kt = 2; kt < KT2; kt += 2) k_step(std::false_type{}, kt);
     if (FAST_ONLY || g.fast_epi) {
-      epilogue_bf16_fast_any<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
+      epilogue_bf16_fast_any<MT, NT, true>(g, batch, core.acc, m0 + wm, n0 + wn, stage, scalars);
+      stores_pending = true;
     } else {
       epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
     }
