@@ -1,11 +1,14 @@
 // Which kernel serves which problem.
 //
 // Large problems take 256 x 256 tiles (least bytes moved from L2 into LDS per
-// flop).  When that tiling leaves compute units without a tile, the same kernel
-// runs with 256 x 128 tiles: twice the tiles at 1.5 times the LDS traffic per
-// flop.  (A 4-wave kernel with two workgroups per CU and 64-byte K stages, meant
-// to hide the epilogue behind the other workgroup's MFMAs, was measured against
-// it: bound by its global->LDS traffic on large problems and no faster on these.)
+// flop): with four waves of 128 x 128 when the fast bf16 epilogue applies (see
+// gemm_tile.h), otherwise with eight waves of 128 x 64 and the general
+// epilogue.  When that tiling leaves compute units without a tile, the
+// eight-wave kernel runs with 256 x 128 tiles: twice the tiles at 1.5 times the
+// LDS traffic per flop.  (A 4-wave kernel with two workgroups per CU and
+// 64-byte K stages, meant to hide the epilogue behind the other workgroup's
+// MFMAs, was measured against it: bound by its global->LDS traffic on large
+// problems and no faster on these.)
 // Few rows of A (M <= 128) take the strip kernel, which streams B once through a
 // deep ring.
 #pragma once

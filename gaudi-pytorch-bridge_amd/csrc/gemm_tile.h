@@ -1,19 +1,27 @@
 // fp8 x fp8 -> fp32-accumulate -> bf16/fp32 GEMM for gfx950 (fp8_gemm_v2).
 //
-// Tiled kernel: a 512-thread workgroup (8 waves, 2 x 4, two per SIMD) owns a BM x BN tile of C
-// and walks K in steps of 128 bytes.  Operand tiles travel from global memory
-// straight into LDS (buffer_load_dwordx4 ... lds: no staging registers, and the
-// buffer descriptor's bounds check zero-fills rows past the matrix edge) into
-// one of two LDS stages, so the loads of step k+2 fly while step k computes.
-// Inside a stage, the 16-byte chunks of a row are XOR-swizzled with the row
-// number, which keeps the 128-bit and transposing fragment reads free of bank
+// Tiled kernel: a workgroup of 2 x WN waves owns a BM x BN tile of C and walks K
+// in steps of 128 bytes.  Operand tiles travel from global memory straight into
+// LDS (buffer_load_dwordx4 ... lds: no staging registers, and the buffer
+// descriptor's bounds check zero-fills rows past the matrix edge) into one of
+// two LDS stages, so the loads of step k+2 fly while step k computes.  Inside a
+// stage, the 16-byte chunks of a row are XOR-swizzled with the row number,
+// which keeps the 128-bit and transposing fragment reads free of bank
 // conflicts; since a DMA load places lane l's chunk at LDS offset 16 l, the
 // swizzle is applied by choosing which global chunk each lane fetches.  Each
-// wave computes its (BM/2) x (BN/4) sub-tile with v_mfma_f32_32x32x64_f8f6f4
+// wave computes its (BM/2) x (BN/WN) sub-tile with v_mfma_f32_32x32x64_f8f6f4
 // (fp8/bf8 operands, 64 k per instruction), reading the fragments of the next
 // half-step while the MFMAs of the current one run.  The buffer descriptors
 // walk along K by scalar arithmetic, so the per-lane offsets are small
 // constants and operands of any size are addressable.
+//
+// Two wave grids are built.  2 x 4 (eight waves, two per SIMD, 128 x 64 wave
+// tiles at BM = BN = 256): while one wave of a SIMD sits in its epilogue or
+// waits for a fragment, the other keeps the matrix pipe busy; this grid carries
+// both epilogues.  2 x 2 (four waves, one per SIMD, 128 x 128 wave tiles, all
+// 256 accumulation registers): a third fewer LDS fragment bytes per MFMA, which
+// is what matters once the chip runs at its power limit; its epilogue is not
+// hidden by a second wave, so it exists with the fast bf16 epilogue only.
 //
 // Operand layouts.  An operand whose K index is contiguous in memory (A with
 // trans_a == 0, B with trans_b != 0) is "K-major": a lane's 32-byte MFMA
@@ -27,6 +35,14 @@
 // scales, bias and the accumulate input are applied in fp32 before the single
 // final rounding, and the rows pass through LDS once more so that a wave
 // stores whole 128-byte lines.
+//
+// One counter tracks a wave's outstanding vector memory operations, and it
+// retires them in issue order.  Everything in the persistent tile loop is
+// arranged around that: the fast epilogue loads nothing from global memory
+// (its scales and bias arrive in LDS through the K loop's own load stream), so
+// that no wait of its own also waits for the next tile's first stages, which
+// are already in flight; and the wait for those stages at the start of a tile
+// lets the previous tile's stores stay outstanding.
 #pragma once
 #include <type_traits>
 
@@ -40,9 +56,6 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define LDS_AS __attribute__((address_space(3)))
 
-// Two waves per SIMD: a memory instruction of one wave (LDS fragment read,
-// global->LDS load) holds up that wave's next MFMA for tens of cycles, and only
-// a second resident wave lets the matrix pipe run meanwhile.
 constexpr int kWavesM = 2;  // the waves of a workgroup form a 2 x WN grid over its tile
 constexpr int kBK = 128;  // bytes (= fp8 elements) of K per LDS stage
 
@@ -799,12 +812,14 @@ struct ScaleStager {
 
 // Per-wave state of the K loop: accumulators, fragments, loaders.
 //
-// Register budget.  Two waves per SIMD leave 256 registers per lane: 128 hold
-// the accumulators of the (BM/2) x (BN/4) wave tile, so the fragments get 64:
-// the B fragments are double-buffered (the next half-step's set is read while
-// the current one is in use), the A fragments are single-buffered and rolled:
-// MFMAs run row by row, A_i is dead after the last MFMA of row i, and the next
-// half-step's A_i is read into the same registers right then.
+// Register budget.  Two waves per SIMD (WN = 4) leave 256 registers per lane:
+// 128 hold the accumulators of the 128 x 64 wave tile, so the fragments get 64.
+// One wave per SIMD (WN = 2) has 512: 256 accumulators of the 128 x 128 wave
+// tile, 96 for fragments.  In both the B fragments are double-buffered (the
+// next half-step's set is read while the current one is in use), the A
+// fragments are single-buffered and rolled: MFMAs run row by row, A_i is dead
+// after the last MFMA of row i, and the next half-step's A_i is read into the
+// same registers right then.
 template <int BM, int BN, int WN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
 struct TileCore {
   static constexpr int TM = BM / kWavesM, TN = BN / WN;

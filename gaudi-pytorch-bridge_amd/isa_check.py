@@ -1,0 +1,120 @@
+"""Checks the generated gfx950 assembly for hazards the compiler does not cover.
+
+The GEMM kernels issue their global->LDS loads from asm statements (the compiler has no
+way to express "do not wait for this load before the next LDS read").  The compiler
+inserts the wait states the hardware needs between dependent instructions it generates
+itself, but it does not look inside an asm statement.  Two requirements of gfx9-family
+hardware are therefore checked on the compiler's output:
+
+* a vector instruction that writes a scalar register (v_readfirstlane_b32, v_readlane_b32,
+  a compare that writes a scalar pair) must be followed by at least five wait states before
+  a vector memory instruction reads that register (here: as part of its buffer descriptor);
+* a write of M0 must be followed by at least one wait state before a memory instruction
+  that uses M0 as its LDS address.
+
+``scan(text)`` returns a list of human-readable findings (empty when clean);
+``compile_to_isa(source)`` produces the text to scan.
+"""
+import os
+import re
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+_SGPR = re.compile(r"\bs(\d+)\b|\bs\[(\d+):(\d+)\]")
+_MEM = re.compile(r"^\s*(buffer_|global_|flat_|scratch_)")
+
+
+def _sgprs(text):
+    regs = set()
+    for m in _SGPR.finditer(text):
+        if m.group(1) is not None:
+            regs.add(int(m.group(1)))
+        else:
+            regs.update(range(int(m.group(2)), int(m.group(3)) + 1))
+    return regs
+
+
+def _is_instruction(line):
+    s = line.strip()
+    return bool(s) and not s.startswith((";", ".", "//")) and not s.endswith(":")
+
+
+def _wait_states(line):
+    m = re.match(r"\s*s_nop\s+(\d+)", line)
+    return int(m.group(1)) + 1 if m else 1
+
+
+def _valu_scalar_dest(line):
+    """Scalar registers written by a vector instruction, or an empty set."""
+    s = line.strip()
+    if not s.startswith("v_"):
+        return set()
+    ops = s.split(None, 1)
+    if len(ops) < 2:
+        return set()
+    dest = ops[1].split(",")[0]
+    if s.startswith(("v_readfirstlane_b32", "v_readlane_b32")) or re.match(r"v_cmp\w*_e64", s) or "_e64" in ops[0]:
+        return _sgprs(dest)
+    return set()
+
+
+def scan(text):
+    lines = text.splitlines()
+    findings = []
+    i = 0
+    while i < len(lines):
+        if "#ASMSTART" not in lines[i]:
+            i += 1
+            continue
+        start = i
+        j = i + 1
+        while j < len(lines) and "#ASMEND" not in lines[j]:
+            j += 1
+        block = [l for l in lines[start + 1:j] if _is_instruction(l)]
+        i = j + 1
+        # wait states inside the block before its first memory instruction, M0 rule on the way
+        waited = 0
+        m0_age = None
+        for l in block:
+            if _MEM.match(l):
+                used = _sgprs(l)
+                if " lds" in l and m0_age is not None and m0_age < 1:
+                    findings.append(f"line {start + 1}: M0 written {m0_age} wait states before '{l.strip()}'")
+                # look back over the compiler's instructions
+                need = 5 - waited
+                k = start - 1
+                seen = 0
+                while k >= 0 and seen < need:
+                    if _is_instruction(lines[k]) and "#ASM" not in lines[k]:
+                        hit = _valu_scalar_dest(lines[k]) & used
+                        if hit:
+                            findings.append(
+                                f"line {k + 1}: '{lines[k].strip()}' writes s{sorted(hit)} {seen + waited} wait states "
+                                f"before '{l.strip()}' (line {start + 1}) reads it; 5 are required")
+                        seen += _wait_states(lines[k])
+                    k -= 1
+                break
+            if re.match(r"\s*s_mov_b32\s+m0\b", l):
+                m0_age = 0
+            else:
+                if m0_age is not None:
+                    m0_age += _wait_states(l)
+            waited += _wait_states(l)
+    return findings
+
+
+def compile_to_isa(source, extra_flags=()):
+    """Device-only assembly of one HIP source of csrc/ with the build's flags."""
+    import importlib.util  # noqa: PLC0415
+    spec = importlib.util.spec_from_file_location("_mi355q_build_flags", os.path.join(HERE, "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    HIPCC_FLAGS, CSRC = build.HIPCC_FLAGS, build.CSRC
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc] + [f for f in HIPCC_FLAGS if f != "-fPIC"] + list(extra_flags) + \
+          ["--cuda-device-only", "-S", "-x", "hip", os.path.join(CSRC, source), "-o", "-"]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed: " + r.stderr[-2000:])
+    return r.stdout

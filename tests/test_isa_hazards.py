@@ -1,0 +1,87 @@
+"""The generated gfx950 assembly of the GEMM kernels is free of the wait-state hazards that the
+compiler does not check inside asm statements (see isa_check.py).  CPU only: hipcc cross-compiles."""
+import importlib.util
+import os
+from concurrent.futures import ThreadPoolExecutor
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_spec = importlib.util.spec_from_file_location(
+    "mi355q_isa_check", os.path.join(ROOT, "gaudi-pytorch-bridge_amd", "isa_check.py"))
+isa_check = importlib.util.module_from_spec(_spec)
+_spec.loader.exec_module(isa_check)
+
+
+def test_scanner_flags_scalar_register_written_too_late():
+    text = """
+	v_readfirstlane_b32 s30, v68
+	v_lshl_add_u32 v68, v189, 3, v172
+	;;#ASMSTART
+	s_mov_b32 m0, s5
+	s_nop 0
+	buffer_load_dwordx4 v1, s[28:31], 0 offen lds
+	;;#ASMEND
+"""
+    found = isa_check.scan(text)
+    assert len(found) == 1 and "s[30]" in found[0]
+
+
+def test_scanner_accepts_enough_wait_states():
+    late_enough = """
+	v_readfirstlane_b32 s30, v68
+	v_add_u32_e32 v1, v2, v3
+	v_add_u32_e32 v1, v2, v3
+	v_add_u32_e32 v1, v2, v3
+	;;#ASMSTART
+	s_mov_b32 m0, s5
+	s_nop 0
+	buffer_load_dwordx4 v1, s[28:31], 0 offen lds
+	;;#ASMEND
+"""
+    nop_inside = """
+	v_readfirstlane_b32 s30, v68
+	;;#ASMSTART
+	s_mov_b32 m0, s5
+	s_nop 4
+	buffer_load_dword v1, s[28:31], 0 offen lds
+	;;#ASMEND
+"""
+    other_register = """
+	v_readfirstlane_b32 s40, v68
+	;;#ASMSTART
+	s_mov_b32 m0, s5
+	s_nop 0
+	buffer_load_dwordx4 v1, s[28:31], 0 offen lds
+	;;#ASMEND
+"""
+    scalar_write = """
+	s_add_u32 s28, s28, s2
+	;;#ASMSTART
+	s_mov_b32 m0, s5
+	s_nop 0
+	buffer_load_dwordx4 v1, s[28:31], 0 offen lds
+	;;#ASMEND
+"""
+    for text in (late_enough, nop_inside, other_register, scalar_write):
+        assert isa_check.scan(text) == []
+
+
+def test_scanner_flags_m0_used_at_once():
+    text = """
+	;;#ASMSTART
+	s_mov_b32 m0, s5
+	buffer_load_dwordx4 v1, s[28:31], 0 offen lds
+	;;#ASMEND
+"""
+    assert any("M0" in f for f in isa_check.scan(text))
+
+
+@pytest.mark.timeout(900)
+def test_gemm_kernels_have_no_uncovered_hazard():
+    sources = ["gemm_inst_kk.hip", "gemm_inst_km.hip", "gemm_inst_mk.hip", "gemm_inst_mm.hip"]
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        texts = list(ex.map(isa_check.compile_to_isa, sources))
+    for src, text in zip(sources, texts):
+        assert text.count("#ASMSTART") > 100, f"{src}: the asm statements are gone?"
+        assert isa_check.scan(text) == [], src
