@@ -75,8 +75,13 @@ extern "C" {
 const char* mi355q_fp8_gemm_variant(int trans_a, int64_t lda, int trans_b, int64_t ldb, int64_t M,
                                     int64_t N, int64_t K) {
   if (lda % 16 || ldb % 16 || (trans_a ? M : K) % 16 || (trans_b ? K : N) % 16) return "simple";
-  if (M > 128 && N > 128)
-    return mi355q::use_half_width_tiles(M, N, 1) ? "tile256x128x128_mfma32x32x64" : "tile256x256x128_mfma32x32x64";
+  if (M > 128 && N > 128) {
+    switch (mi355q::choose_tiles(M, N, 1)) {
+      case mi355q::TileChoice::k256x256: return "tile256x256x128_mfma32x32x64";
+      case mi355q::TileChoice::k256x128: return "tile256x128x128_mfma32x32x64";
+      case mi355q::TileChoice::k128x128: return "tile128x128x128_mfma32x32x64";
+    }
+  }
   if (M <= 128) return "strip_Mx128x128_ring_mfma32x32x64";
   return "tile128x128x128_mfma32x32x64";
 }

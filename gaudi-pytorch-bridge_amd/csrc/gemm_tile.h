@@ -1069,13 +1069,15 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void fp8_gemm_tile_kernel(GemmAr
 
 // WN: waves along n (the workgroup has 2 x WN); FAST_ONLY: the kernel carries
 // the fast bf16 epilogue alone and the launch must satisfy epilogue_fast_ok().
-template <int BM, int BN, int WN, bool FAST_ONLY, bool AK, bool BK_, int FA, int FB>
+// WGS_PER_CU: workgroups of the persistent grid per compute unit (2 where the
+// kernel's LDS and registers let two be resident).
+template <int BM, int BN, int WN, bool FAST_ONLY, bool AK, bool BK_, int FA, int FB, int WGS_PER_CU = 1>
 void launch_tile(const GemmArgs& g, int64_t batch, hipStream_t st) {
   GemmArgs a = g;
   a.tiles_m = (g.M + BM - 1) / BM;
   a.tiles_n = (g.N + BN - 1) / BN;
   const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
-  const int cus = compute_units();
+  const int cus = compute_units() * WGS_PER_CU;
   dim3 grid((unsigned)(tiles < cus ? tiles : cus), (unsigned)batch);
   fp8_gemm_tile_kernel<BM, BN, WN, AK, BK_, FA, FB, FAST_ONLY><<<grid, kWavesM * WN * 64, 0, st>>>(a);
 }

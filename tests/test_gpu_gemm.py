@@ -49,17 +49,21 @@ def test_exact_small_integers_tiled(dev, fa, fb, ta, tb, M, N, K):
     assert torch.equal(out16.cpu(), expect.bfloat16())
 
 
-# One shape per kernel the dispatcher can pick (256 CUs): 256 x 256 tiles need at least 256 of them,
-# below that the kernel runs with 256 x 128 tiles (more, or fewer, than one per CU), the strip kernel
-# has three row-tile heights, and 128 x 128 tiles serve N <= 128 < M.  Edges are ragged in M, N and K.
+# One shape per kernel the dispatcher can pick (256 CUs): 256 x 256 tiles need at least 256 of them;
+# below that the eight-wave kernel runs with 256 x 128 tiles while those fill more than half the CUs
+# (more, or fewer, tiles than CUs), else with 128 x 128 tiles, two workgroups per CU; the strip kernel
+# has three row-tile heights, and 128 x 128 tiles also serve N <= 128 < M (fewer, or more, tiles than
+# the 512 workgroup slots).  Edges are ragged in M, N and K.
 KERNEL_SHAPES = {
     "tile256_persistent": (4000, 4112, 208),
     "tile256x128_more_tiles_than_cus": (1008, 12304, 208),
-    "tile256x128_fewer_tiles_than_cus": (272, 4112, 400),
+    "tile256x128_fewer_tiles_than_cus": (272, 10256, 272),
+    "tile128_underfilled": (272, 4112, 400),
     "strip_32_rows": (16, 1040, 400),
     "strip_64_rows": (48, 1040, 400),
     "strip_128_rows": (112, 1040, 400),
     "tile128": (400, 112, 272),
+    "tile128_more_tiles_than_slots": (66576, 112, 144),
 }
 
 
