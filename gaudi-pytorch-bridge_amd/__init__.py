@@ -90,3 +90,29 @@ EXPORTED_SYMBOLS = (
 _load()
 
 hpu = torch.ops.hpu
+
+_aten_override = None
+
+
+def use_for_aten_scaled_mm(enable=True):
+    """Route ``torch._scaled_mm`` on HIP tensors to this package's fp8 GEMM (``mi355q::scaled_mm``).
+
+    The reference serves ``aten::_scaled_mm`` with the same node as ``hpu::fp8_gemm_v2``
+    (hpu_ops/backend/scaled_mm_gen.cpp:66-141).  On PyTorch-ROCm the operator already has a
+    kernel (the vendor library), so the replacement is opt-in and reversible:
+    ``use_for_aten_scaled_mm(False)`` restores what was registered before.
+    """
+    global _aten_override
+    if not enable:
+        if _aten_override is not None:
+            _aten_override._destroy()
+            _aten_override = None
+        return
+    if _aten_override is not None:
+        return
+    import warnings
+    lib = torch.library.Library("aten", "IMPL")
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")  # "Overriding a previously registered kernel": intended
+        lib.impl("_scaled_mm", torch.ops.mi355q.scaled_mm.default, "CUDA")
+    _aten_override = lib

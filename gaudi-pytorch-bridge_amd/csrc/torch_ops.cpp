@@ -734,6 +734,72 @@ std::tuple<Tensor, Tensor> quantize_rows_op(const Tensor& x, at::ScalarType dtyp
   return {out, scale_inv};
 }
 
+// ------------------------------------------------------------- _scaled_mm
+//
+// aten::_scaled_mm on the fp8 GEMM kernel: the reference lowers it to the same
+// fp8_gemm node as hpu::fp8_gemm_v2, with scale_result as a further input
+// (ScaledMm::AddNode, hpu_ops/backend/scaled_mm_gen.cpp:66-141; checks and their
+// messages :78-107; the default out_dtype is mat1's, :72-75).
+//   out = to_out_dtype( (mat1 @ mat2) * scale_a * scale_b * scale_result + bias )
+// (the form the reference's test checks against: any_mode/test_hpu_scaled_mm.py:
+// 177).  scale_a / scale_b hold one value, or one per row of mat1 ([M, 1]) / per
+// column of mat2 ([1, N]).  An fp8 out_dtype is produced by the saturating
+// round-to-nearest cast of the fp32 result (one rounding).  Registered as
+// mi355q::scaled_mm with aten::_scaled_mm's signature; the package can also put
+// it behind torch._scaled_mm for HIP tensors (use_for_aten_scaled_mm()).
+// use_fast_accum is accepted and has no effect: accumulation is fp32 throughout.
+Tensor scaled_mm(const Tensor& mat1, const Tensor& mat2, const Tensor& scale_a, const Tensor& scale_b,
+                 const c10::optional<Tensor>& bias, const c10::optional<Tensor>& scale_result,
+                 c10::optional<at::ScalarType> out_dtype, bool /*use_fast_accum*/) {
+  TORCH_CHECK(mat1.dim() == 2, "mat1 must be a matrix");
+  TORCH_CHECK(mat2.dim() == 2, "mat2 must be a matrix");
+  TORCH_CHECK(mat1.size(1) == mat2.size(0), "mat1 and mat2 shapes cannot be multiplied (", mat1.size(0), "x",
+              mat1.size(1), " and ", mat2.size(0), "x", mat2.size(1), ")");
+  const int64_t M = mat1.size(0), N = mat2.size(1);
+  const bool has_bias = bias.has_value() && bias->defined();
+  TORCH_CHECK(!has_bias || bias->numel() == N, "Bias must be size ", N, " but got ", has_bias ? bias->numel() : 0);
+  TORCH_CHECK(is_fp8(mat1.scalar_type()), "Expected mat1 to be Float8_e5m2 or Float8_e4m3fn matrix got ",
+              mat1.scalar_type());
+  TORCH_CHECK(is_fp8(mat2.scalar_type()), "Expected mat2 to be Float8_e5m2 or Float8_e4m3fn matrix got ",
+              mat2.scalar_type());
+  const at::ScalarType out_t = out_dtype.value_or(mat1.scalar_type());
+  TORCH_CHECK(out_t == at::kFloat || out_t == at::kBFloat16 || is_fp8(out_t),
+              "_scaled_mm out_dtype must be float, bfloat16, float8_e5m2 or float8_e4m3fn, got ", out_t);
+  auto scale_ok = [&](const Tensor& s, int64_t rows, int64_t cols) {
+    return s.numel() == 1 || (s.dim() == 2 && s.size(0) == rows && s.size(1) == cols);
+  };
+  TORCH_CHECK(scale_ok(scale_a, M, 1), "scale_a must hold one value or have shape [", M, ", 1], got ", scale_a.sizes());
+  TORCH_CHECK(scale_ok(scale_b, 1, N), "scale_b must hold one value or have shape [1, ", N, "], got ", scale_b.sizes());
+  const bool has_sr = scale_result.has_value() && scale_result->defined();
+  TORCH_CHECK(!has_sr || scale_result->numel() == 1, "scale_result must hold one value");
+  if (mat1.is_meta()) return at::empty({M, N}, mat1.options().dtype(out_t));
+
+  // a transposed view of a contiguous matrix is multiplied in place (no copy)
+  Tensor a = mat1, b = mat2;
+  bool ta = false, tb = false;
+  if (!a.is_contiguous() && a.t().is_contiguous()) {
+    a = a.t();
+    ta = true;
+  }
+  if (!b.is_contiguous() && b.t().is_contiguous()) {
+    b = b.t();
+    tb = true;
+  }
+  Tensor sa = scale_a.to(at::kFloat);
+  if (has_sr) sa = sa * scale_result->to(at::kFloat).reshape({});
+  const at::ScalarType gemm_t = is_fp8(out_t) ? at::kFloat : out_t;
+  OptShape sb_shape;
+  if (scale_b.numel() > 1) sb_shape = std::vector<int64_t>{1, N};
+  Tensor r = fp8_gemm_v2_impl(a, ta, b, tb, c10::nullopt, gemm_t, IValue(sa), IValue(scale_b),
+                              has_bias ? c10::optional<Tensor>(bias->reshape({N})) : c10::nullopt, false, sb_shape);
+  if (!is_fp8(out_t)) return r;
+  Tensor out = at::empty({M, N}, r.options().dtype(out_t));
+  if (out.numel() == 0) return out;
+  DeviceGuard guard(r.device());
+  check_status(launch_cast_to(r, out, resolve_cast_scale(IValue(), c10::nullopt, r), nullptr, false), "mi355q_cast_to_fp8");
+  return out;
+}
+
 }  // namespace
 
 TORCH_LIBRARY(hpu, m) {
@@ -758,6 +824,7 @@ TORCH_LIBRARY(mi355q, m) {
   m.def("mi355q::amax(Tensor input) -> Tensor");
   m.def("mi355q::rowwise_amax(Tensor input) -> Tensor");
   m.def("mi355q::quantize_rows(Tensor input, ScalarType dtype) -> (Tensor, Tensor)");
+  m.def("mi355q::scaled_mm(Tensor self, Tensor mat2, Tensor scale_a, Tensor scale_b, Tensor? bias=None, Tensor? scale_result=None, ScalarType? out_dtype=None, bool use_fast_accum=False) -> Tensor");
 }
 
 #define MI355Q_REGISTER_HPU(m)                                                                 \
@@ -783,9 +850,11 @@ TORCH_LIBRARY_IMPL(mi355q, CUDA, m) {
   m.impl("amax", amax_op);
   m.impl("rowwise_amax", rowwise_amax_op);
   m.impl("quantize_rows", quantize_rows_op);
+  m.impl("scaled_mm", scaled_mm);
 }
 TORCH_LIBRARY_IMPL(mi355q, Meta, m) {
   m.impl("amax", amax_op);
   m.impl("rowwise_amax", rowwise_amax_op);
   m.impl("quantize_rows", quantize_rows_op);
+  m.impl("scaled_mm", scaled_mm);
 }

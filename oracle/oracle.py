@@ -301,6 +301,25 @@ def torch_fp8_gemm(A, trans_A, B, trans_B, out_dtype, A_scale_inv=None, B_scale_
     return v.to(out_dtype)
 
 
+def torch_scaled_mm(mat1, mat2, scale_a, scale_b, bias=None, scale_result=None, out_dtype=None):
+    """aten::_scaled_mm as the reference's test states it (any_mode/test_hpu_scaled_mm.py:177):
+    (mat1 @ mat2) * scale_a * scale_b * scale_result + bias, accumulated and scaled in fp32,
+    one rounding to out_dtype (default: mat1's dtype, scaled_mm_gen.cpp:72-75); an fp8
+    out_dtype saturates."""
+    v = torch.matmul(mat1.detach().cpu().float(), mat2.detach().cpu().float())
+    sa = scale_a.detach().cpu().float()
+    if scale_result is not None:
+        sa = sa * scale_result.detach().cpu().float().reshape(())
+    v = v * sa * scale_b.detach().cpu().float()
+    if bias is not None:
+        v = v + bias.detach().cpu().float()
+    out_dtype = out_dtype or mat1.dtype
+    if out_dtype in FP8_MAX:
+        mx = FP8_MAX[out_dtype]
+        return v.clamp(-mx, mx).to(out_dtype)
+    return v.to(out_dtype)
+
+
 def pack_nibbles(q):
     """int tensor [..., 8P] with values in -8..15 -> packed int32 [..., P]."""
     q = q.detach().cpu().to(torch.int64) & 0xF

@@ -241,3 +241,26 @@ def test_cast_to_fp8_hybrid_meta(pkg, is_amax):
     assert amax.dtype == torch.float32 and amax.shape == (() if is_amax else (0,))
     with pytest.raises(RuntimeError, match="CastToFp8Hybrid input must be of float or bfloat16 dtype."):
         torch.ops.hpu.cast_to_fp8_hybrid(meta((4,), torch.float16))
+
+
+def test_scaled_mm_meta_shapes_and_errors(pkg):
+    """mi355q::scaled_mm carries aten::_scaled_mm's signature, the reference's checks
+    (scaled_mm_gen.cpp:78-107) and its default out_dtype (:72-75)."""
+    import re
+    schema = str(torch.ops.mi355q.scaled_mm.default._schema)
+    aten = str(torch.ops.aten._scaled_mm.default._schema)
+    assert re.sub(r"^mi355q::scaled_mm", "", schema) == re.sub(r"^aten::_scaled_mm", "", aten)
+    a = torch.empty(12, 16, dtype=torch.float8_e5m2, device="meta")
+    b = torch.empty(16, 24, dtype=torch.float8_e4m3fn, device="meta")
+    s = torch.empty((), device="meta")
+    out = torch.ops.mi355q.scaled_mm(a, b, s, s)
+    assert out.shape == (12, 24) and out.dtype == torch.float8_e5m2
+    assert torch.ops.mi355q.scaled_mm(a, b, s, s, None, None, torch.bfloat16).dtype == torch.bfloat16
+    with pytest.raises(RuntimeError, match="mat2 must be a matrix"):
+        torch.ops.mi355q.scaled_mm(a, b[0], s, s)
+    with pytest.raises(RuntimeError, match=r"mat1 and mat2 shapes cannot be multiplied \(12x16 and 24x16\)"):
+        torch.ops.mi355q.scaled_mm(a, b.t(), s, s)
+    with pytest.raises(RuntimeError, match="Expected mat2 to be Float8_e5m2 or Float8_e4m3fn matrix got"):
+        torch.ops.mi355q.scaled_mm(a, b.to(torch.bfloat16), s, s)
+    with pytest.raises(RuntimeError, match="scale_a must hold one value or have shape"):
+        torch.ops.mi355q.scaled_mm(a, b, torch.empty(3, device="meta"), s)

@@ -82,3 +82,31 @@ def test_nan_and_inf_codes_propagate(oracle):
     A.view(torch.uint8)[2, 5] = 0x7F  # nan
     out = oracle.c_fp8_gemm(A, False, B, False, torch.float32)
     assert torch.isinf(out[1]).all() and torch.isnan(out[2]).all() and (out[0] == 16).all()
+
+
+def test_scaled_mm_oracle_known_answers(oracle):
+    """torch_scaled_mm against hand-computed values, the reference test's own formula
+    (any_mode/test_hpu_scaled_mm.py:177, evaluated in bf16 as there) and the fp8_gemm oracle."""
+    E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+    a = torch.tensor([[1.0, 2.0]]).to(E4)
+    b = torch.tensor([[3.0], [4.0]]).to(E4)
+    out = oracle.torch_scaled_mm(a, b, torch.tensor(2.5), torch.tensor(0.5), torch.tensor([1.0]), torch.tensor(2.0), torch.float32)
+    assert out.item() == 11 * 2.5 * 0.5 * 2.0 + 1.0
+    # default out dtype is mat1's, and an fp8 result saturates instead of overflowing
+    big = oracle.torch_scaled_mm(torch.full((2, 8), 16.0).to(E5), torch.full((8, 2), 16.0).to(E4),
+                                 torch.tensor(4.0), torch.tensor(8.0))
+    assert big.dtype == E5 and torch.equal(big.float(), torch.full((2, 2), 57344.0))
+    g = torch.Generator().manual_seed(11)
+    a = (torch.rand(12, 16, generator=g) * 5.0).to(E5)
+    b = (torch.rand(16, 24, generator=g) * 10.0).to(E4)
+    sa, sb = torch.tensor(2.71), torch.tensor(3.14)
+    bias = (torch.randn(24, generator=g) * 50.0).bfloat16()
+    mine = oracle.torch_scaled_mm(a, b, sa, sb, bias, None, torch.bfloat16)
+    theirs = torch.mm(a.bfloat16(), b.bfloat16()) * (sa * sb).bfloat16() * torch.tensor(1.0).bfloat16() + bias
+    torch.testing.assert_close(mine, theirs, atol=1e-3, rtol=0.015)
+    same = oracle.torch_fp8_gemm(a, False, b, False, torch.bfloat16, sa, sb, bias=bias)
+    assert torch.equal(mine, same)
+    # row-wise scales broadcast as [M,1] x [1,N]
+    ra, rb = torch.rand(12, 1, generator=g) + 0.5, torch.rand(1, 24, generator=g) + 0.5
+    rw = oracle.torch_scaled_mm(a, b, ra, rb, None, None, torch.float32)
+    assert torch.allclose(rw, (a.float() @ b.float()) * ra * rb, rtol=1e-6)
