@@ -32,14 +32,65 @@ inline TileChoice choose_tiles(int64_t M, int64_t N, int64_t batch) {
   return 2 * tiles_half > cus ? TileChoice::k256x128 : TileChoice::k128x128;
 }
 
+// Tile columns to split off a 256 x 256 tiling whose last round of tiles would
+// leave at least three quarters of the compute units idle (320 tiles on 256
+// CUs: one full round and one of 64).  Those last columns then run as a second
+// launch with 256 x 128 tiles, twice as many for about 0.6 of the time each
+// (2048 x 10240 x 8192: 0.156 -> 0.145 ms).  With a last round that is half
+// full the second launch costs what it saves (4096 x 14336 x 4096: 0.177 ms
+// either way), so those are left alone.  0: no split.
+inline int64_t tail_tile_columns(int64_t M, int64_t N, int64_t batch) {
+  const int64_t cus = compute_units();
+  const int64_t tm = (M + 255) / 256, tn = (N + 255) / 256;
+  const int64_t tiles = tm * tn;
+  if (batch != 1 || tiles < cus) return 0;
+  const int64_t tail = tiles % cus;
+  if (tail == 0 || 4 * tail > cus) return 0;
+  const int64_t c = (tail + tm - 1) / tm;  // whole tile columns that hold the tail
+  // the rest must still be whole rounds, and the split-off part must fit one round of half tiles
+  if (c >= tn || 2 * c * tm > cus + cus / 4) return 0;
+  return c;
+}
+
+// The same problem restricted to columns [n_off, N) of B and C.
+template <bool B_KMAJOR>
+GemmArgs columns_from(const GemmArgs& g, int64_t n_off, int64_t batch) {
+  GemmArgs t = g;
+  const int es = g.out_bf16 ? 2 : 4;
+  t.N = g.N - (int)n_off;
+  t.B = g.B + (B_KMAJOR ? n_off * g.ldb : n_off);
+  t.C = g.C + n_off * es;
+  if (g.sb_mode == MI355Q_GS_PER_COL) t.sb = g.sb + n_off;
+  if (g.bias_mode != MI355Q_BIAS_NONE) t.bias = g.bias + n_off * es;
+  if (g.D) t.D = g.D + n_off * es;
+  t.fast_epi = epilogue_fast_ok(t, batch);
+  return t;
+}
+
+template <bool AK, bool BK_, int FA, int FB>
+void launch_256x256(const GemmArgs& g, int64_t batch, hipStream_t st) {
+  if (g.fast_epi) launch_tile<256, 256, 2, true, AK, BK_, FA, FB>(g, batch, st);
+  else launch_tile<256, 256, 4, false, AK, BK_, FA, FB>(g, batch, st);
+}
+
 template <bool AK, bool BK_, int FA, int FB>
 void launch_by_size(const GemmArgs& g, int64_t batch, hipStream_t st) {
   if (g.M > 128 && g.N > 128) {
     switch (choose_tiles(g.M, g.N, batch)) {
-      case TileChoice::k256x256:
-        if (g.fast_epi) launch_tile<256, 256, 2, true, AK, BK_, FA, FB>(g, batch, st);
-        else launch_tile<256, 256, 4, false, AK, BK_, FA, FB>(g, batch, st);
+      case TileChoice::k256x256: {
+        const int64_t c = tail_tile_columns(g.M, g.N, batch);
+        if (c == 0) {
+          launch_256x256<AK, BK_, FA, FB>(g, batch, st);
+        } else {
+          const int64_t n_main = ((g.N + 255) / 256 - c) * 256;
+          GemmArgs head = g;
+          head.N = (int)n_main;
+          head.fast_epi = epilogue_fast_ok(head, batch);
+          launch_256x256<AK, BK_, FA, FB>(head, batch, st);
+          launch_tile<256, 128, 4, false, AK, BK_, FA, FB>(columns_from<BK_>(g, n_main, batch), batch, st);
+        }
         break;
+      }
       case TileChoice::k256x128: launch_tile<256, 128, 4, false, AK, BK_, FA, FB>(g, batch, st); break;
       case TileChoice::k128x128: launch_tile<128, 128, 4, false, AK, BK_, FA, FB, 2>(g, batch, st); break;
     }
