@@ -57,6 +57,7 @@ def capi():
     L.mi355q_amax.argtypes = [vp, i32, i64, vp, vp]
     L.mi355q_rowwise_amax.argtypes = [vp, i32, i64, i64, vp, vp]
     L.mi355q_quantize_rows.argtypes = [vp, i32, i64, i64, vp, i32, f32, vp, vp, vp]
+    L.mi355q_silu_mul_quantize_rows.argtypes = [vp, i64, vp, i64, i64, i64, vp, i32, f32, vp, vp, vp, vp]
     L.mi355q_cast_to_fp8.argtypes = [vp, i32, vp, i32, vp, f32, i32, i64, i64, i64, vp, vp]
     L.mi355q_cast_to_fp8_sr.argtypes = [vp, i32, vp, i32, vp, f32, i32, i64, i64, i64, vp, c.c_uint64, c.c_uint64, vp]
     L.mi355q_cast_to_fp8_hybrid.argtypes = [vp, i32, i64, vp, vp, vp, vp, i32, c.c_uint64, c.c_uint64, vp, vp]
@@ -67,7 +68,7 @@ def capi():
                                   vp, i32, i64, vp, i64, i64, i64, i64, i64, i64, i64, vp]
     L.mi355q_fp8_gemm_variant.argtypes = [i32, i64, i32, i64, i64, i64, i64]
     L.mi355q_fp8_gemm_variant.restype = c.c_char_p
-    for name in ("mi355q_amax", "mi355q_rowwise_amax", "mi355q_quantize_rows", "mi355q_cast_to_fp8", "mi355q_cast_to_fp8_sr", "mi355q_cast_to_fp8_hybrid", "mi355q_cast_from_fp8",
+    for name in ("mi355q_amax", "mi355q_rowwise_amax", "mi355q_quantize_rows", "mi355q_silu_mul_quantize_rows", "mi355q_cast_to_fp8", "mi355q_cast_to_fp8_sr", "mi355q_cast_to_fp8_hybrid", "mi355q_cast_from_fp8",
                  "mi355q_dequant_4bit", "mi355q_fp8_gemm"):
         getattr(L, name).restype = i32
     L._typed = True
@@ -83,7 +84,7 @@ ZP_NONE, ZP_FLOAT, ZP_PACKED = 0, 1, 2
 
 EXPORTED_SYMBOLS = (
     "mi355q_abi_version", "mi355q_status_string", "mi355q_amax", "mi355q_rowwise_amax",
-    "mi355q_quantize_rows", "mi355q_cast_to_fp8", "mi355q_cast_to_fp8_sr", "mi355q_cast_to_fp8_hybrid", "mi355q_cast_from_fp8", "mi355q_dequant_4bit", "mi355q_fp8_gemm",
+    "mi355q_quantize_rows", "mi355q_silu_mul_quantize_rows", "mi355q_cast_to_fp8", "mi355q_cast_to_fp8_sr", "mi355q_cast_to_fp8_hybrid", "mi355q_cast_from_fp8", "mi355q_dequant_4bit", "mi355q_fp8_gemm",
     "mi355q_fp8_gemm_variant",
 )
 

@@ -481,6 +481,73 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(
   }
 }
 
+// SiLU(gate) * up in bf16 followed by the dynamic per-row quantisation above,
+// in one pass: bf16(bf16(silu(gate)) * up), row amax of that, scale = target /
+// amax, cast.  The glue between the gate / up projections and the down
+// projection of a decoder MLP block; gate and up may be column ranges of one
+// wider matrix (row pitches ld_gate, ld_up in elements).  h_out, when given,
+// receives the bf16 products.
+template <int FMT, int VPT>
+__global__ __launch_bounds__(kThreads) void silu_mul_quantize_rows_kernel(
+    const uint16_t* __restrict__ gate, int64_t ld_gate, const uint16_t* __restrict__ up, int64_t ld_up,
+    uint8_t* __restrict__ y, uint16_t* __restrict__ h_out, int64_t vec_per_row, float target,
+    float* __restrict__ scale_out, float* __restrict__ scale_inv_out) {
+  __shared__ uint32_t wave_part[kThreads / 64];
+  const int64_t row = blockIdx.x;
+  const u32x4* gr = reinterpret_cast<const u32x4*>(gate + row * ld_gate);
+  const u32x4* ur = reinterpret_cast<const u32x4*>(up + row * ld_up);
+  u32x4 h[VPT];
+  uint32_t am = 0;
+#pragma unroll
+  for (int u = 0; u < VPT; ++u) {
+    const int64_t v = threadIdx.x + (int64_t)u * kThreads;
+    u32x4 gv = {0u, 0u, 0u, 0u}, uv = {0u, 0u, 0u, 0u};
+    if (v < vec_per_row) {
+      gv = __builtin_nontemporal_load(gr + v);
+      uv = __builtin_nontemporal_load(ur + v);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float s0 = round_to_bf16(silu_f32(__uint_as_float(gv[i] << 16)));
+      const float s1 = round_to_bf16(silu_f32(__uint_as_float(gv[i] & 0xffff0000u)));
+      h[u][i] = pack_bf16x2(s0 * __uint_as_float(uv[i] << 16), s1 * __uint_as_float(uv[i] & 0xffff0000u));
+      const u16x2 a = __builtin_bit_cast(u16x2, h[u][i] & 0x7fff7fffu);
+      am = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, __builtin_bit_cast(u16x2, am)));
+    }
+    if (h_out && v < vec_per_row) reinterpret_cast<u32x4*>(h_out)[row * vec_per_row + v] = h[u];
+  }
+  {
+    const uint32_t lo = am & 0xffffu, hi = am >> 16;
+    am = (lo > hi ? lo : hi) << 16;
+  }
+  am = wave_max_u32(am);
+  if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = am;
+  __syncthreads();
+  uint32_t r = wave_part[0];
+#pragma unroll
+  for (int w = 1; w < kThreads / 64; ++w) r = r > wave_part[w] ? r : wave_part[w];
+  const float amax = __uint_as_float(r);
+  const float scale = target / amax;
+  if (threadIdx.x == 0) {
+    if (scale_out) scale_out[row] = scale;
+    if (scale_inv_out) scale_inv_out[row] = 1.0f / scale;
+  }
+  const float s = round_to_bf16(scale);
+#pragma unroll
+  for (int u = 0; u < VPT; ++u) {
+    const int64_t v = threadIdx.x + (int64_t)u * kThreads;
+    if (v >= vec_per_row) continue;
+    float p[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[2 * i] = round_to_bf16(__uint_as_float(h[u][i] << 16) * s);
+      p[2 * i + 1] = round_to_bf16(__uint_as_float(h[u][i] & 0xffff0000u) * s);
+    }
+    const u32x2 o = {cvt_fp8x4<FMT>(p[0], p[1], p[2], p[3]), cvt_fp8x4<FMT>(p[4], p[5], p[6], p[7])};
+    __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(y) + row * vec_per_row + v);
+  }
+}
+
 // -------------------------------------------------------------- cast_from_fp8
 //
 // A lane produces one 16-byte store: 8 fp8 bytes in for bf16 output, 4 for
@@ -750,6 +817,19 @@ int quantize_rows_launch(const uint8_t* x, uint8_t* y, int64_t rows, int64_t vpr
   return launch_status();
 }
 
+template <int FMT>
+int silu_mul_quantize_rows_launch(const uint16_t* gate, int64_t ld_gate, const uint16_t* up, int64_t ld_up,
+                                  uint8_t* y, uint16_t* h_out, int64_t rows, int64_t vpr, float target,
+                                  float* scale_out, float* scale_inv_out, hipStream_t st) {
+  const unsigned grid = (unsigned)rows;
+  if (vpr <= kThreads) silu_mul_quantize_rows_kernel<FMT, 1><<<grid, kThreads, 0, st>>>(gate, ld_gate, up, ld_up, y, h_out, vpr, target, scale_out, scale_inv_out);
+  else if (vpr <= 2 * kThreads) silu_mul_quantize_rows_kernel<FMT, 2><<<grid, kThreads, 0, st>>>(gate, ld_gate, up, ld_up, y, h_out, vpr, target, scale_out, scale_inv_out);
+  else if (vpr <= 4 * kThreads) silu_mul_quantize_rows_kernel<FMT, 4><<<grid, kThreads, 0, st>>>(gate, ld_gate, up, ld_up, y, h_out, vpr, target, scale_out, scale_inv_out);
+  else if (vpr <= 8 * kThreads) silu_mul_quantize_rows_kernel<FMT, 8><<<grid, kThreads, 0, st>>>(gate, ld_gate, up, ld_up, y, h_out, vpr, target, scale_out, scale_inv_out);
+  else return MI355Q_ERR_UNSUPPORTED;
+  return launch_status();
+}
+
 }  // namespace mi355q
 
 using namespace mi355q;
@@ -882,6 +962,28 @@ int mi355q_quantize_rows(const void* x, int x_dtype, int64_t rows, int64_t cols,
   }
   if (fp8_fmt == MI355Q_E4M3FN) return quantize_rows_launch<false, MI355Q_E4M3FN>(xb, yb, rows, vpr, target, scale_out, scale_inv_out, st);
   return quantize_rows_launch<false, MI355Q_E5M2>(xb, yb, rows, vpr, target, scale_out, scale_inv_out, st);
+}
+
+int mi355q_silu_mul_quantize_rows(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                                  int64_t rows, int64_t cols, void* y, int fp8_fmt, float target,
+                                  void* h_out, float* scale_out, float* scale_inv_out, void* stream) {
+  if (rows < 0 || cols < 0 || ld_gate < cols || ld_up < cols) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (fp8_fmt != MI355Q_E4M3FN && fp8_fmt != MI355Q_E5M2) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (rows == 0 || cols == 0) return MI355Q_OK;
+  if (gate == nullptr || up == nullptr || y == nullptr) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (rows > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+  // whole 16-byte vectors only; the row has to fit the registers of one workgroup
+  if (cols % 8 != 0 || ld_gate % 8 != 0 || ld_up % 8 != 0 || !aligned(gate, 16) || !aligned(up, 16) ||
+      !aligned(y, 8) || (h_out && !aligned(h_out, 16)))
+    return MI355Q_ERR_UNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint16_t* g = static_cast<const uint16_t*>(gate);
+  const uint16_t* u = static_cast<const uint16_t*>(up);
+  uint8_t* yb = static_cast<uint8_t*>(y);
+  uint16_t* hb = static_cast<uint16_t*>(h_out);
+  if (fp8_fmt == MI355Q_E4M3FN)
+    return silu_mul_quantize_rows_launch<MI355Q_E4M3FN>(g, ld_gate, u, ld_up, yb, hb, rows, cols / 8, target, scale_out, scale_inv_out, st);
+  return silu_mul_quantize_rows_launch<MI355Q_E5M2>(g, ld_gate, u, ld_up, yb, hb, rows, cols / 8, target, scale_out, scale_inv_out, st);
 }
 
 int mi355q_cast_to_fp8(const void* x, int x_dtype, void* y, int fp8_fmt, const float* scale_dev,

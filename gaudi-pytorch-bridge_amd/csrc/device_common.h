@@ -31,6 +31,37 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, r);
 }
 
+// exp(t) for -87 <= t <= 88 as a fixed sequence of IEEE operations (Cody-Waite
+// reduction by ln 2 in two parts, the degree-5 polynomial of Cephes' expf,
+// scaling by two powers of two): the CPU oracle runs the same sequence and gets
+// the same bits, which a library or hardware exp would not guarantee.
+__device__ __forceinline__ float exp_spelled_out(float t) {
+  const float n = __builtin_rintf(t * 1.44269504088896341f);
+  float r = __builtin_fmaf(n, -0.693145751953125f, t);
+  r = __builtin_fmaf(n, -1.42860682030941723212e-6f, r);
+  float q = 1.9875691500e-4f;
+  q = __builtin_fmaf(q, r, 1.3981999507e-3f);
+  q = __builtin_fmaf(q, r, 8.3334519073e-3f);
+  q = __builtin_fmaf(q, r, 4.1665795894e-2f);
+  q = __builtin_fmaf(q, r, 1.6666665459e-1f);
+  q = __builtin_fmaf(q, r, 5.0000001201e-1f);
+  float y = __builtin_fmaf(q, r * r, r);
+  y = y + 1.0f;
+  const int k = (int)n, k1 = k / 2, k2 = k - k1;
+  return y * __uint_as_float((uint32_t)(k1 + 127) << 23) * __uint_as_float((uint32_t)(k2 + 127) << 23);
+}
+
+// x / (1 + exp(-x)) in fp32; results smaller than 3.3e-37 in magnitude (x <= -88.5) are -0.
+__device__ __forceinline__ float silu_f32(float x) {
+  if (x != x) return x;
+  const float t = -x;
+  float e;
+  if (t > 88.0f) e = __builtin_inff();
+  else if (t < -87.0f) e = 0.0f;
+  else e = exp_spelled_out(t);
+  return x / (1.0f + e);
+}
+
 // Clamp to the finite fp8 range.  minimum/maximum propagate NaN, so a NaN
 // input still converts to an fp8 NaN; +-Inf saturates like any overflow.
 template <int FMT>

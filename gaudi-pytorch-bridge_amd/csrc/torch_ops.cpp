@@ -734,6 +734,39 @@ std::tuple<Tensor, Tensor> quantize_rows_op(const Tensor& x, at::ScalarType dtyp
   return {out, scale_inv};
 }
 
+// SiLU(gate) * up in bf16 and the dynamic per-row quantisation of the product in
+// one kernel: (h8, scale_inv), bit-identical to quantize_rows of
+// bf16(bf16(silu(gate)) * up) with the oracle's silu.  gate and up are 2-D bf16
+// with unit column stride (they may be the two halves of one GEMM output).
+// Shapes the kernel does not take go through aten's silu and mul, whose exp may
+// differ from the oracle's in the last place.
+std::tuple<Tensor, Tensor> silu_mul_quantize_rows_op(const Tensor& gate, const Tensor& up, at::ScalarType dtype) {
+  TORCH_CHECK(gate.scalar_type() == at::kBFloat16 && up.scalar_type() == at::kBFloat16,
+              "mi355q::silu_mul_quantize_rows inputs must be bfloat16");
+  TORCH_CHECK(dtype == at::kFloat8_e4m3fn || dtype == at::kFloat8_e5m2,
+              "mi355q::silu_mul_quantize_rows dtype must be float8_e4m3fn or float8_e5m2");
+  TORCH_CHECK(gate.dim() == 2 && gate.sizes() == up.sizes(),
+              "mi355q::silu_mul_quantize_rows takes two matrices of the same shape, got ", gate.sizes(), " and ", up.sizes());
+  const int64_t rows = gate.size(0), cols = gate.size(1);
+  if (gate.is_meta())
+    return {at::empty({rows, cols}, gate.options().dtype(dtype)), at::empty({rows, 1}, gate.options().dtype(at::kFloat))};
+  TORCH_CHECK(gate.device() == up.device(), "mi355q::silu_mul_quantize_rows inputs must be on the same device");
+  DeviceGuard guard(gate.device());
+  Tensor g = gate.stride(1) == 1 || cols <= 1 ? gate : gate.contiguous();
+  Tensor u = up.stride(1) == 1 || cols <= 1 ? up : up.contiguous();
+  Tensor out = at::empty({rows, cols}, g.options().dtype(dtype));
+  Tensor scale_inv = at::empty({rows, 1}, g.options().dtype(at::kFloat));
+  if (out.numel() == 0) return {out, scale_inv};
+  const float target = dtype == at::kFloat8_e5m2 ? 57344.0f : 448.0f;
+  const int st = mi355q_silu_mul_quantize_rows(g.data_ptr(), rows > 1 ? g.stride(0) : cols, u.data_ptr(),
+                                               rows > 1 ? u.stride(0) : cols, rows, cols, out.data_ptr(),
+                                               to_mi355q_dtype(dtype), target, nullptr, nullptr,
+                                               scale_inv.data_ptr<float>(), current_stream(g));
+  if (st == MI355Q_ERR_UNSUPPORTED) return quantize_rows_op(at::mul(at::silu(gate), up), dtype);
+  check_status(st, "mi355q_silu_mul_quantize_rows");
+  return {out, scale_inv};
+}
+
 // ------------------------------------------------------------- _scaled_mm
 //
 // aten::_scaled_mm on the fp8 GEMM kernel: the reference lowers it to the same
@@ -824,6 +857,7 @@ TORCH_LIBRARY(mi355q, m) {
   m.def("mi355q::amax(Tensor input) -> Tensor");
   m.def("mi355q::rowwise_amax(Tensor input) -> Tensor");
   m.def("mi355q::quantize_rows(Tensor input, ScalarType dtype) -> (Tensor, Tensor)");
+  m.def("mi355q::silu_mul_quantize_rows(Tensor gate, Tensor up, ScalarType dtype) -> (Tensor, Tensor)");
   m.def("mi355q::scaled_mm(Tensor self, Tensor mat2, Tensor scale_a, Tensor scale_b, Tensor? bias=None, Tensor? scale_result=None, ScalarType? out_dtype=None, bool use_fast_accum=False) -> Tensor");
 }
 
@@ -851,10 +885,12 @@ TORCH_LIBRARY_IMPL(mi355q, CUDA, m) {
   m.impl("rowwise_amax", rowwise_amax_op);
   m.impl("quantize_rows", quantize_rows_op);
   m.impl("scaled_mm", scaled_mm);
+  m.impl("silu_mul_quantize_rows", silu_mul_quantize_rows_op);
 }
 TORCH_LIBRARY_IMPL(mi355q, Meta, m) {
   m.impl("amax", amax_op);
   m.impl("rowwise_amax", rowwise_amax_op);
   m.impl("quantize_rows", quantize_rows_op);
   m.impl("scaled_mm", scaled_mm);
+  m.impl("silu_mul_quantize_rows", silu_mul_quantize_rows_op);
 }

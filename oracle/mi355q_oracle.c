@@ -78,6 +78,49 @@ uint16_t ora_f32_to_bf16(float f) {
   return (uint16_t)keep;
 }
 
+/* ---- SiLU(gate) * up in bf16 (the glue between the gate / up and the down
+ * projections of the decoder MLP block; not an op of the reference, which
+ * leaves it to aten) -----------------------------------------------------
+ * silu(x) = x / (1 + exp(-x)) evaluated in fp32 with a spelled-out exp
+ * (Cody-Waite reduction by ln 2 in two parts, the degree-5 polynomial of
+ * Cephes' expf, scaling by two powers of two), rounded to bf16; the product
+ * with `up` (exact in fp32) is rounded to bf16 again.  Every operation is an
+ * IEEE add, multiply, divide or fused multiply-add, written out one by one, so
+ * that the GPU kernel, which uses the same sequence, gets the same bits.
+ */
+static float exp_spelled_out(float t) { /* -87 <= t <= 88 */
+  const float n = rintf(t * 1.44269504088896341f);
+  float r = fmaf(n, -0.693145751953125f, t);
+  r = fmaf(n, -1.42860682030941723212e-6f, r);
+  float q = 1.9875691500e-4f;
+  q = fmaf(q, r, 1.3981999507e-3f);
+  q = fmaf(q, r, 8.3334519073e-3f);
+  q = fmaf(q, r, 4.1665795894e-2f);
+  q = fmaf(q, r, 1.6666665459e-1f);
+  q = fmaf(q, r, 5.0000001201e-1f);
+  float y = fmaf(q, r * r, r);
+  y = y + 1.0f;
+  const int k = (int)n, k1 = k / 2, k2 = k - k1;
+  return y * u2f((uint32_t)(k1 + 127) << 23) * u2f((uint32_t)(k2 + 127) << 23);
+}
+
+float ora_silu_f32(float x) {
+  if (x != x) return x;
+  const float t = -x;
+  float e;
+  if (t > 88.0f) e = INFINITY;
+  else if (t < -87.0f) e = 0.0f;
+  else e = exp_spelled_out(t);
+  return x / (1.0f + e);
+}
+
+void ora_silu_mul_bf16(const uint16_t* gate, const uint16_t* up, uint16_t* h, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) {
+    const float s = ora_bf16_to_f32(ora_f32_to_bf16(ora_silu_f32(ora_bf16_to_f32(gate[i]))));
+    h[i] = ora_f32_to_bf16(s * ora_bf16_to_f32(up[i]));
+  }
+}
+
 /* ---- fp32 -> fp8 -------------------------------------------------------
  * Round to nearest even onto the fp8 grid with gradual underflow, then
  * saturate to the largest finite value (e4m3fn 448 = 0x7E, e5m2 57344 = 0x7B):

@@ -301,6 +301,31 @@ def torch_fp8_gemm(A, trans_A, B, trans_B, out_dtype, A_scale_inv=None, B_scale_
     return v.to(out_dtype)
 
 
+def c_silu_mul_bf16(gate, up):
+    """bf16(bf16(silu(gate)) * up) with the oracle's spelled-out exp (ora_silu_mul_bf16)."""
+    g = gate.detach().cpu().contiguous()
+    u = up.detach().cpu().contiguous()
+    assert g.dtype == torch.bfloat16 and u.dtype == torch.bfloat16 and g.shape == u.shape
+    h = torch.empty_like(g)
+    L = lib()
+    L.ora_silu_mul_bf16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+    L.ora_silu_mul_bf16.restype = None
+    L.ora_silu_mul_bf16(_ptr(g), _ptr(u), _ptr(h), g.numel())
+    return h
+
+
+def quantize_rows(x, out_dtype):
+    """Dynamic per-row quantisation as mi355q::quantize_rows states it: (x8, 1 / scale) with
+    scale = fp8_max / rowwise amax (fp32 division) and cast_to_fp8_v2's rounding."""
+    x = x.detach().cpu()
+    x2 = x.reshape(-1, x.shape[-1])
+    amax = x2.abs().amax(dim=-1, keepdim=True).float()
+    # tensor / tensor is an IEEE division; torch evaluates scalar / tensor as scalar * (1 / tensor)
+    scale = torch.full_like(amax, FP8_MAX[out_dtype]) / amax
+    y, _ = c_cast_to_fp8(x2, scale.reshape(-1), out_dtype, scale_shape=[x2.shape[0], 1])
+    return y.reshape(x.shape), (torch.ones_like(scale) / scale).reshape(x.shape[:-1] + (1,))
+
+
 def torch_scaled_mm(mat1, mat2, scale_a, scale_b, bias=None, scale_result=None, out_dtype=None):
     """aten::_scaled_mm as the reference's test states it (any_mode/test_hpu_scaled_mm.py:177):
     (mat1 @ mat2) * scale_a * scale_b * scale_result + bias, accumulated and scaled in fp32,

@@ -1,0 +1,82 @@
+"""GPU parity of mi355q::silu_mul_quantize_rows (SiLU(gate) * up in bf16 fused with the dynamic
+per-row quantisation) against the CPU oracle: bit-exact, the fp8 codes and the inverse scales."""
+import ctypes
+
+import pytest
+import torch
+
+from helpers import E4, E5, FP8_DTYPES
+
+pytestmark = pytest.mark.gpu
+
+ALL = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+
+
+def same_codes(a, b):
+    return torch.equal(a.cpu().view(torch.uint8), b.cpu().view(torch.uint8))
+
+
+def test_silu_bits_on_every_bf16_value(oracle, pkg, dev):
+    """h_out of the C entry point for all 65536 gate values (up = 1 and up = an odd constant)."""
+    lib = pkg.capi()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for upv in (1.0, -0.337890625):
+        g = ALL.reshape(32, 2048)
+        u = torch.full_like(g, upv)
+        gd, ud = g.to(dev), u.to(dev)
+        y = torch.empty(g.shape, dtype=E4, device=dev)
+        h = torch.empty(g.shape, dtype=torch.bfloat16, device=dev)
+        assert lib.mi355q_silu_mul_quantize_rows(gd.data_ptr(), 2048, ud.data_ptr(), 2048, 32, 2048, y.data_ptr(),
+                                                 pkg.E4M3FN, 448.0, h.data_ptr(), None, None, stream) == 0
+        torch.cuda.synchronize()
+        ref = oracle.c_silu_mul_bf16(g, u)
+        nan = torch.isnan(ref.float())
+        assert torch.equal(torch.isnan(h.cpu().float()), nan)
+        assert torch.equal(h.cpu().view(torch.int16)[~nan], ref.view(torch.int16)[~nan])
+
+
+@pytest.mark.parametrize("out_dtype", FP8_DTYPES)
+@pytest.mark.parametrize("shape", [(64, 1024), (33, 2048), (5, 14336), (3, 8), (16, 16384)])
+def test_against_oracle(oracle, dev, shape, out_dtype):
+    gen = torch.Generator().manual_seed(shape[0] * 131 + shape[1])
+    g = (torch.randn(*shape, generator=gen) * 3).bfloat16()
+    u = torch.randn(*shape, generator=gen).bfloat16()
+    g[:, ::97] *= 10
+    y, s_inv = torch.ops.mi355q.silu_mul_quantize_rows(g.to(dev), u.to(dev), out_dtype)
+    assert y.shape == g.shape and y.dtype == out_dtype and s_inv.shape == (shape[0], 1)
+    ref_y, ref_s = oracle.quantize_rows(oracle.c_silu_mul_bf16(g, u), out_dtype)
+    assert same_codes(y, ref_y)
+    assert torch.equal(s_inv.cpu(), ref_s)
+
+
+def test_halves_of_one_wide_matrix(oracle, dev):
+    """gate and up as column ranges of one [T, 2 ff] GEMM output (row pitch 2 ff)."""
+    gen = torch.Generator().manual_seed(9)
+    gu = (torch.randn(48, 2 * 1536, generator=gen) * 2).bfloat16()
+    d = gu.to(dev)
+    y, s_inv = torch.ops.mi355q.silu_mul_quantize_rows(d[:, :1536], d[:, 1536:], E4)
+    ref_y, ref_s = oracle.quantize_rows(oracle.c_silu_mul_bf16(gu[:, :1536].contiguous(), gu[:, 1536:].contiguous()), E4)
+    assert same_codes(y, ref_y) and torch.equal(s_inv.cpu(), ref_s)
+    # equals the unfused route on the device, where aten's silu agrees with the oracle's
+    h = torch.nn.functional.silu(d[:, :1536]) * d[:, 1536:]
+    y2, s2 = torch.ops.mi355q.quantize_rows(h, E4)
+    assert (y.view(torch.uint8) != y2.view(torch.uint8)).float().mean().item() < 1e-3
+
+
+def test_shapes_the_kernel_refuses_take_the_aten_route(dev):
+    g = torch.randn(4, 20, device=dev).bfloat16()        # 20 columns: not whole 16-byte vectors
+    u = torch.randn(4, 20, device=dev).bfloat16()
+    y, s_inv = torch.ops.mi355q.silu_mul_quantize_rows(g, u, E5)
+    y2, s2 = torch.ops.mi355q.quantize_rows(torch.nn.functional.silu(g) * u, E5)
+    assert same_codes(y, y2) and torch.equal(s_inv, s2)
+
+
+def test_argument_checks(dev):
+    g = torch.randn(4, 16, device=dev)
+    with pytest.raises(RuntimeError, match="inputs must be bfloat16"):
+        torch.ops.mi355q.silu_mul_quantize_rows(g, g, E4)
+    b = g.bfloat16()
+    with pytest.raises(RuntimeError, match="two matrices of the same shape"):
+        torch.ops.mi355q.silu_mul_quantize_rows(b, b[:, :8], E4)
+    with pytest.raises(RuntimeError, match="dtype must be float8_e4m3fn or float8_e5m2"):
+        torch.ops.mi355q.silu_mul_quantize_rows(b, b, torch.bfloat16)
