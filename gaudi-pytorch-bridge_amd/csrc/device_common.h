@@ -32,10 +32,12 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 }
 
 // exp(t) for -87 <= t <= 88 as a fixed sequence of IEEE operations (Cody-Waite
-// reduction by ln 2 in two parts, the degree-5 polynomial of Cephes' expf,
-// scaling by two powers of two): the CPU oracle runs the same sequence and gets
-// the same bits, which a library or hardware exp would not guarantee.
+// reduction by ln 2 in two parts, the degree-5 polynomial of Cephes' expf, an
+// exact scaling by a power of two): the CPU oracle runs the same sequence and
+// gets the same bits, which a library or hardware exp would not guarantee.
+// Contraction is off so that no multiply and add merge that the oracle keeps apart.
 __device__ __forceinline__ float exp_spelled_out(float t) {
+#pragma clang fp contract(off)
   const float n = __builtin_rintf(t * 1.44269504088896341f);
   float r = __builtin_fmaf(n, -0.693145751953125f, t);
   r = __builtin_fmaf(n, -1.42860682030941723212e-6f, r);
@@ -47,18 +49,18 @@ __device__ __forceinline__ float exp_spelled_out(float t) {
   q = __builtin_fmaf(q, r, 5.0000001201e-1f);
   float y = __builtin_fmaf(q, r * r, r);
   y = y + 1.0f;
-  const int k = (int)n, k1 = k / 2, k2 = k - k1;
-  return y * __uint_as_float((uint32_t)(k1 + 127) << 23) * __uint_as_float((uint32_t)(k2 + 127) << 23);
+  return __builtin_ldexpf(y, (int)n);
 }
 
-// x / (1 + exp(-x)) in fp32; results smaller than 3.3e-37 in magnitude (x <= -88.5) are -0.
+// x / (1 + exp(-x)) in fp32, branch-free; results smaller than 3.3e-37 in
+// magnitude (x <= -88.5) are -0, NaN stays NaN.
 __device__ __forceinline__ float silu_f32(float x) {
-  if (x != x) return x;
+#pragma clang fp contract(off)
   const float t = -x;
-  float e;
-  if (t > 88.0f) e = __builtin_inff();
-  else if (t < -87.0f) e = 0.0f;
-  else e = exp_spelled_out(t);
+  // fmin / fmax return the other operand for a NaN, so the exp below never sees one
+  float e = exp_spelled_out(__builtin_fminf(__builtin_fmaxf(t, -87.0f), 88.0f));
+  e = t > 88.0f ? __builtin_inff() : e;
+  e = t < -87.0f ? 0.0f : e;
   return x / (1.0f + e);
 }
 

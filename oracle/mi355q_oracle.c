@@ -83,7 +83,7 @@ uint16_t ora_f32_to_bf16(float f) {
  * leaves it to aten) -----------------------------------------------------
  * silu(x) = x / (1 + exp(-x)) evaluated in fp32 with a spelled-out exp
  * (Cody-Waite reduction by ln 2 in two parts, the degree-5 polynomial of
- * Cephes' expf, scaling by two powers of two), rounded to bf16; the product
+ * Cephes' expf, an exact scaling by a power of two), rounded to bf16; the product
  * with `up` (exact in fp32) is rounded to bf16 again.  Every operation is an
  * IEEE add, multiply, divide or fused multiply-add, written out one by one, so
  * that the GPU kernel, which uses the same sequence, gets the same bits.
@@ -100,17 +100,15 @@ static float exp_spelled_out(float t) { /* -87 <= t <= 88 */
   q = fmaf(q, r, 5.0000001201e-1f);
   float y = fmaf(q, r * r, r);
   y = y + 1.0f;
-  const int k = (int)n, k1 = k / 2, k2 = k - k1;
-  return y * u2f((uint32_t)(k1 + 127) << 23) * u2f((uint32_t)(k2 + 127) << 23);
+  return ldexpf(y, (int)n);
 }
 
 float ora_silu_f32(float x) {
-  if (x != x) return x;
   const float t = -x;
-  float e;
+  /* fminf / fmaxf return the other operand for a NaN, so the exp never sees one */
+  float e = exp_spelled_out(fminf(fmaxf(t, -87.0f), 88.0f));
   if (t > 88.0f) e = INFINITY;
-  else if (t < -87.0f) e = 0.0f;
-  else e = exp_spelled_out(t);
+  if (t < -87.0f) e = 0.0f;
   return x / (1.0f + e);
 }
 
