@@ -32,11 +32,11 @@ inline TileChoice choose_tiles(int64_t M, int64_t N, int64_t batch) {
   return 2 * tiles_half > cus ? TileChoice::k256x128 : TileChoice::k128x128;
 }
 
-// Tile columns to split off a 256 x 256 tiling whose last round of tiles would
+// Tile columns to split off a 256 x 256 tiling whose last pass over the tiles would
 // leave at least three quarters of the compute units idle (320 tiles on 256
-// CUs: one full round and one of 64).  Those last columns then run as a second
+// CUs: one full pass and one of 64 tiles).  Those last columns then run as a second
 // launch with 256 x 128 tiles, twice as many for about 0.6 of the time each
-// (2048 x 10240 x 8192: 0.156 -> 0.145 ms).  With a last round that is half
+// (2048 x 10240 x 8192: 0.156 -> 0.145 ms).  With a last pass that is half
 // full the second launch costs what it saves (4096 x 14336 x 4096: 0.177 ms
 // either way), so those are left alone.  0: no split.
 inline int64_t tail_tile_columns(int64_t M, int64_t N, int64_t batch) {
@@ -47,7 +47,7 @@ inline int64_t tail_tile_columns(int64_t M, int64_t N, int64_t batch) {
   const int64_t tail = tiles % cus;
   if (tail == 0 || 4 * tail > cus) return 0;
   const int64_t c = (tail + tm - 1) / tm;  // whole tile columns that hold the tail
-  // the rest must still be whole rounds, and the split-off part must fit one round of half tiles
+  // the rest must still be whole passes, and the split-off part must fit one pass of half tiles
   if (c >= tn || 2 * c * tm > cus + cus / 4) return 0;
   return c;
 }

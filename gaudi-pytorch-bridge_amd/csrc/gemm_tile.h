@@ -987,7 +987,7 @@ __device__ __forceinline__ void tile_coords(int logical, int tiles_m, int tiles_
 
 // Persistent kernel: gridDim.x workgroups (at most one per CU) each walk a list
 // of tiles.  Workgroups are dealt to the 8 XCDs round-robin by id; each XCD owns
-// a contiguous range of the tile order, and in round r its workgroups take the
+// a contiguous range of the tile order, and in pass r its workgroups take the
 // next gridDim.x / 8 tiles of that range, so that the tiles in flight on one
 // XCD form a compact patch that shares A and B panels in its L2.
 template <int BM, int BN, int WN, bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B, bool FAST_ONLY>

@@ -50,16 +50,16 @@ def test_exact_small_integers_tiled(dev, fa, fb, ta, tb, M, N, K):
 
 
 # One shape per kernel the dispatcher can pick (256 CUs): 256 x 256 tiles need at least 256 of them
-# (a last round that fills at most a quarter of the CUs is split off as columns of 256 x 128 tiles:
+# (a last pass that fills at most a quarter of the CUs is split off as columns of 256 x 128 tiles:
 # 272 and 528 tiles do that, 464 do not);
 # below that the eight-wave kernel runs with 256 x 128 tiles while those fill more than half the CUs
 # (more, or fewer, tiles than CUs), else with 128 x 128 tiles, two workgroups per CU; the strip kernel
 # has three row-tile heights, and 128 x 128 tiles also serve N <= 128 < M (fewer, or more, tiles than
 # the 512 workgroup slots).  Edges are ragged in M, N and K.
 KERNEL_SHAPES = {
-    "tile256_one_round_and_tail_columns": (4000, 4112, 208),
-    "tile256_two_rounds_and_tail_columns": (4000, 8208, 208),
-    "tile256_two_rounds_no_split": (4000, 7184, 144),
+    "tile256_one_pass_and_tail_columns": (4000, 4112, 208),
+    "tile256_two_passes_and_tail_columns": (4000, 8208, 208),
+    "tile256_two_passes_no_split": (4000, 7184, 144),
     "tile256x128_more_tiles_than_cus": (1008, 12304, 208),
     "tile256x128_fewer_tiles_than_cus": (272, 10256, 272),
     "tile128_underfilled": (272, 4112, 400),
