@@ -422,7 +422,6 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(
     const uint8_t* __restrict__ x, uint8_t* __restrict__ y, int64_t vec_per_row, float target,
     float* __restrict__ scale_out, float* __restrict__ scale_inv_out) {
   __shared__ uint32_t wave_part[kThreads / 64];
-  constexpr int EPV = BF16_IN ? 8 : 4;  // elements per 16-byte vector
   const int64_t row = blockIdx.x;
   const u32x4* xr = reinterpret_cast<const u32x4*>(x) + row * vec_per_row;
   u32x4 in[VPT];

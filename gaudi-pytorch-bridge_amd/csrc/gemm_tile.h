@@ -521,7 +521,8 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
       if (!general && !row_scales) {
         // scales and bias depend on the column only: two VALU ops per element
 #pragma unroll
-        for (int r = r_in; r < kEpiRows; r += kRowsPerPass) {
+        for (int it = 0; it < kEpiRows / kRowsPerPass; ++it) {
+          const int r = r_in + it * kRowsPerPass;
           const f32x4 a = *reinterpret_cast<const f32x4*>(stage + r * kRowFloats + (lane % kLanesPerRow) * 4);
           const int m = m_wave + row0 + r;
           if (m < g.M && n < g.N) {
@@ -537,7 +538,8 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
         }
       } else if (!general) {
 #pragma unroll
-        for (int r = r_in; r < kEpiRows; r += kRowsPerPass) {
+        for (int it = 0; it < kEpiRows / kRowsPerPass; ++it) {
+          const int r = r_in + it * kRowsPerPass;
           const f32x4 a = *reinterpret_cast<const f32x4*>(stage + r * kRowFloats + (lane % kLanesPerRow) * 4);
           const float ra = row_sa[row0 + r], rb = row_sb[row0 + r];
           const int m = m_wave + row0 + r;
@@ -995,7 +997,6 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void fp8_gemm_tile_kernel(GemmAr
   constexpr int kWaves = kWavesM * WN;
   constexpr int TM = BM / kWavesM, TN = BN / WN;   // per-wave tile
   constexpr int MT = TM / 32, NT = TN / 32;             // MFMA tiles per wave
-  constexpr int kStageBytes = (BM + BN) * kBK;
   using Core = TileCore<BM, BN, WN, A_KMAJOR, B_KMAJOR, FMT_A, FMT_B>;
   // two stages of each operand; the epilogue has its own staging area
   __shared__ __attribute__((aligned(1024))) uint8_t lds_ring[Core::kRingBytes];
