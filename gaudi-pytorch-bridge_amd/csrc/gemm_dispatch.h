@@ -69,7 +69,7 @@ GemmArgs columns_from(const GemmArgs& g, int64_t n_off, int64_t batch) {
 
 template <bool AK, bool BK_, int FA, int FB>
 void launch_256x256(const GemmArgs& g, int64_t batch, hipStream_t st) {
-  if (g.fast_epi) launch_tile<256, 256, 2, true, AK, BK_, FA, FB>(g, batch, st);
+  if (g.fast_epi && g.D == nullptr) launch_tile<256, 256, 2, true, AK, BK_, FA, FB>(g, batch, st);
   else launch_tile<256, 256, 4, false, AK, BK_, FA, FB>(g, batch, st);
 }
 

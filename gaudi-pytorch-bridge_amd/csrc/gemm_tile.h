@@ -584,10 +584,14 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, int64_t batch, f32x1
 // The forms the fast bf16 epilogue serves: bf16 output, rows and row pitch of C
 // multiples of 16 bytes, N a multiple of 8, A scale a scalar or one value per
 // row, B scale a scalar or one 16-byte-aligned value per column, bias none or
-// an 8-byte-aligned row vector, no accumulate input.  The conditions hold for
+// an 8-byte-aligned row vector, accumulate input none or 8-byte-aligned rows.  The conditions hold for
 // every matrix of a batch or for none, so the host chooses the kernel.
 inline bool epilogue_fast_ok(const GemmArgs& g, int64_t batches) {
-  if (!g.out_bf16 || g.D != nullptr || g.bias_mode == MI355Q_BIAS_FULL) return false;
+  if (!g.out_bf16 || g.bias_mode == MI355Q_BIAS_FULL) return false;
+  if (g.D != nullptr) {  // read in 8-byte pieces
+    if ((reinterpret_cast<uintptr_t>(g.D) & 7u) != 0 || (g.ldd & 3) != 0 || g.ldd > (int64_t(1) << 22)) return false;
+    if (batches > 1 && (g.stride_d & 3) != 0) return false;
+  }
   if (g.sa_mode == MI355Q_GS_PER_COL || g.sb_mode == MI355Q_GS_PER_ROW) return false;
   if ((reinterpret_cast<uintptr_t>(g.C) & 15u) != 0 || (g.ldc & 7) != 0 || (g.N & 7) != 0) return false;
   if (g.ldc > (int64_t(1) << 22)) return false;  // byte offsets inside a wave's rows stay below 2^31
@@ -627,7 +631,7 @@ constexpr int fast_epilogue_stores() { return MT * 2 * NT; }
 // rows (fp32).  Values of a kind the problem does not have are zeros.
 constexpr int kStagedColScale = 0, kStagedBias = 512, kStagedRowScale = 768, kStagedBytes = 1280;
 
-template <int MT, int NT, bool PER_COL, bool HAS_BIAS, bool STAGED = false>
+template <int MT, int NT, bool PER_COL, bool HAS_BIAS, bool STAGED = false, bool HAS_D = false>
 __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t batch, f32x16 (&acc)[MT][NT],
                                                    int m_wave, int n_wave, float* stage_f,
                                                    ScalarScales scalars = ScalarScales{1.0f, 1.0f}) {
@@ -704,9 +708,29 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
   const int voff0 = n_out < g.N ? row_in_pass * pitch + n_out * 2 : 0x7fffffff;
   const int pass_step = n_out < g.N ? kRowsPerPass * pitch : 0;
 
+  // The accumulate input, read in the accumulator layout (4 bf16 per lane and
+  // column group): rows past M fall outside the descriptor and read as zero.
+  __amdgpu_buffer_rsrc_t rsrc_d = rsrc;
+  int d_off0 = 0, d_pitch = 0;
+  if constexpr (HAS_D) {
+    const uint16_t* dbase = reinterpret_cast<const uint16_t*>(g.D) + batch * g.stride_d + (int64_t)m_wave * g.ldd;
+    rsrc_d = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(dbase), 0, rows > 0 ? rows * (int)g.ldd * 2 : 0, 0x00020000);
+    d_pitch = (int)g.ldd * 2;
+    d_off0 = r * d_pitch + (n_wave + 4 * h) * 2;
+  }
+
   // scaled, rounded values of the 32 rows of accumulator row i -> staging area
   auto write_rows = [&](auto ic) {
     constexpr int i = decltype(ic)::value;
+    u32x2 dv[HAS_D ? NT : 1][4];
+    if constexpr (HAS_D) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          dv[j][q] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(
+              rsrc_d, d_off0 + 32 * i * d_pitch + (32 * j + 8 * q) * 2, 0, 0));
+    }
 #pragma unroll
     for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -717,6 +741,12 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
           const float b = HAS_BIAS ? cb[j][q][e] : 0.0f;
           if constexpr (PER_COL) v[e] = __builtin_fmaf(acc[i][j][4 * q + e] * ra[i], cs[j][q][e], b);
           else v[e] = __builtin_fmaf(acc[i][j][4 * q + e], ra[i], b);
+        }
+        if constexpr (HAS_D) {
+          v[0] += __uint_as_float(dv[j][q][0] << 16);
+          v[1] += __uint_as_float(dv[j][q][0] & 0xffff0000u);
+          v[2] += __uint_as_float(dv[j][q][1] << 16);
+          v[3] += __uint_as_float(dv[j][q][1] & 0xffff0000u);
         }
         const u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
         const int slot = (8 * j + 2 * q + h) ^ f_w;
@@ -758,11 +788,21 @@ __device__ __forceinline__ void epilogue_bf16_fast(const GemmArgs& g, int64_t ba
   });
 }
 
-template <int MT, int NT, bool STAGED = false>
+// ALLOW_D false: the caller guarantees there is no accumulate input (the
+// kernel with 256 accumulator registers per lane keeps its epilogue to four
+// variants; with more, the compiler copies accumulators to scratch memory).
+template <int MT, int NT, bool STAGED = false, bool ALLOW_D = true>
 __device__ __forceinline__ void epilogue_bf16_fast_any(const GemmArgs& g, int64_t batch, f32x16 (&acc)[MT][NT],
                                                        int m_wave, int n_wave, float* stage,
                                                        ScalarScales scalars = ScalarScales{1.0f, 1.0f}) {
   const bool per_col = g.sb_mode == MI355Q_GS_PER_COL, bias = g.bias_mode == MI355Q_BIAS_ROW_VECTOR;
+  if (ALLOW_D && g.D != nullptr) {
+    if (per_col && bias) epilogue_bf16_fast<MT, NT, true, true, STAGED, true>(g, batch, acc, m_wave, n_wave, stage, scalars);
+    else if (per_col) epilogue_bf16_fast<MT, NT, true, false, STAGED, true>(g, batch, acc, m_wave, n_wave, stage, scalars);
+    else if (bias) epilogue_bf16_fast<MT, NT, false, true, STAGED, true>(g, batch, acc, m_wave, n_wave, stage, scalars);
+    else epilogue_bf16_fast<MT, NT, false, false, STAGED, true>(g, batch, acc, m_wave, n_wave, stage, scalars);
+    return;
+  }
   if (per_col && bias) epilogue_bf16_fast<MT, NT, true, true, STAGED>(g, batch, acc, m_wave, n_wave, stage, scalars);
   else if (per_col) epilogue_bf16_fast<MT, NT, true, false, STAGED>(g, batch, acc, m_wave, n_wave, stage, scalars);
   else if (bias) epilogue_bf16_fast<MT, NT, false, true, STAGED>(g, batch, acc, m_wave, n_wave, stage, scalars);
@@ -1056,7 +1096,7 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void fp8_gemm_tile_kernel(GemmAr
     k_step(std::true_type{}, 0);
     for (int kt = 2; kt < KT2; kt += 2) k_step(std::false_type{}, kt);
     if (FAST_ONLY || g.fast_epi) {
-      epilogue_bf16_fast_any<MT, NT, true>(g, batch, core.acc, m0 + wm, n0 + wn, stage, scalars);
+      epilogue_bf16_fast_any<MT, NT, true, !FAST_ONLY>(g, batch, core.acc, m0 + wm, n0 + wn, stage, scalars);
       stores_pending = true;
     } else {
       epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
@@ -1069,7 +1109,8 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void fp8_gemm_tile_kernel(GemmAr
 }
 
 // WN: waves along n (the workgroup has 2 x WN); FAST_ONLY: the kernel carries
-// the fast bf16 epilogue alone and the launch must satisfy epilogue_fast_ok().
+// the fast bf16 epilogue alone, without an accumulate input: the launch must
+// satisfy epilogue_fast_ok() and have no D.
 // WGS_PER_CU: workgroups of the persistent grid per compute unit (2 where the
 // kernel's LDS and registers let two be resident).
 template <int BM, int BN, int WN, bool FAST_ONLY, bool AK, bool BK_, int FA, int FB, int WGS_PER_CU = 1>

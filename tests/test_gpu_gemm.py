@@ -77,7 +77,7 @@ KERNEL_SHAPES = {
 def test_every_kernel_path(oracle, dev, kernel, ta, tb):
     """Exact small-integer products through each kernel (fp32 output: general epilogue), then the
     same operands with per-row x per-column scales, a bias vector and bf16 output (fast epilogue)
-    against the fp32-accumulated CPU reference."""
+    against the fp32-accumulated CPU reference, with and without an accumulate input."""
     M, N, K = KERNEL_SHAPES[kernel]
     g = torch.Generator().manual_seed(M + N + K)
     A = small_int_fp8((K, M) if ta else (M, K), E4, g)
@@ -96,6 +96,12 @@ def test_every_kernel_path(oracle, dev, kernel, ta, tb):
     # scalar scales fold into one factor in the fast epilogue
     out_s = ops.fp8_gemm_v2(A.to(dev), ta, B.to(dev), tb, None, torch.bfloat16, 0.5, 0.25, bias.to(dev), False)
     assert torch.equal(out_s.cpu(), (expect * 0.125 + bias.float()).bfloat16())
+    # accumulate input in the fast epilogue: added after the bias, in fp32
+    D = torch.randint(-64, 65, (M, N), generator=g).bfloat16()
+    out_d = ops.fp8_gemm_v2(A.to(dev), ta, B.to(dev), tb, D.to(dev), torch.bfloat16, 0.5, 0.25, bias.to(dev), True)
+    assert torch.equal(out_d.cpu(), (expect * 0.125 + bias.float() + D.float()).bfloat16())
+    out_d = ops.fp8_gemm_v2(A.to(dev), ta, B.to(dev), tb, D.to(dev), torch.bfloat16, sa.to(dev), sb.to(dev), None, True, [1, N])
+    check(out_d, oracle.torch_fp8_gemm(A, ta, B, tb, torch.float32, sa, sb.reshape(1, N), D=D), kernel + " accumulate")
 
 
 @pytest.mark.parametrize("shape", [(24, 12, 36), (22, 10, 34), (26, 16, 38), (1, 7, 3), (17, 1, 5), (33, 65, 129)])
