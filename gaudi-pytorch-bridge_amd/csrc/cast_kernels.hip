@@ -5,6 +5,8 @@
 // loads in flight.  Rounding and saturation use the CDNA4 conversion
 // instructions (v_cvt_pk_{fp8,bf8}_f32, v_cvt_pk_f32_{fp8,bf8},
 // v_cvt_pk_bf16_f32); see device_common.h.
+#include <type_traits>
+
 #include "device_common.h"
 
 namespace mi355q {
@@ -52,94 +54,101 @@ __device__ __forceinline__ void block_amax_commit(uint32_t m, uint32_t* amax) {
 //   SK_ROW     scale[row % mid]
 //   SK_COL     scale[column]
 //   SK_FULL    scale[element]
+//
+// The body has no divergent branch: loads and stores go through buffer
+// descriptors that cover exactly the block's vectors, so a lane past the end
+// of the row loads zeros and its store is dropped.  (With a branch around each
+// load the compiler cannot tell that the previous iteration's load into the
+// same registers was consumed, and makes every load wait for all earlier ones.)
 template <bool BF16_IN, int FMT, int SK, bool AMAX, int U>
 __global__ __launch_bounds__(AMAX ? kAmaxThreads : kThreads) void cast_to_fp8_vec8(
     const uint8_t* __restrict__ x, uint8_t* __restrict__ y, const float* __restrict__ scale,
     float scale_host, int scale_is_dev, int64_t vec_per_row, int64_t blocks_per_row,
     int64_t total_blocks, int64_t mid, uint32_t* __restrict__ amax) {
   constexpr int THREADS = AMAX ? kAmaxThreads : kThreads;
+  constexpr int IN_BYTES = BF16_IN ? 16 : 32;
+  constexpr int kNt = 2;  // non-temporal
   uint32_t am = 0;
   // a logical block is THREADS * U consecutive vectors of one row; without amax
   // the grid holds one workgroup per logical block and this loop runs once
   for (int64_t lb = blockIdx.x; lb < total_blocks; lb += gridDim.x) {
-  const int64_t row = lb / blocks_per_row;
-  const int64_t bir = lb - row * blocks_per_row;
-  const int64_t v0 = bir * (int64_t)(THREADS * U) + threadIdx.x;
-  const int64_t row_base = row * vec_per_row;
+    const int64_t row = lb / blocks_per_row;
+    const int64_t vec0 = (lb - row * blocks_per_row) * (int64_t)(THREADS * U);  // first vector, within the row
+    const int64_t left = vec_per_row - vec0;
+    const int nvec = (int)(left < THREADS * U ? left : THREADS * U);
+    const int64_t first = row * vec_per_row + vec0;                             // first vector, within the tensor
+    const __amdgpu_buffer_rsrc_t rin =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(x) + first * IN_BYTES, 0, nvec * IN_BYTES, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(y + first * 8, 0, nvec * 8, 0x00020000);
 
-  float s = 1.0f;
-  if constexpr (SK == SK_SCALAR) s = scale_is_dev ? scale[0] : scale_host;
-  if constexpr (SK == SK_ROW) s = scale[row % mid];
-  if constexpr (BF16_IN) s = round_to_bf16(s);
+    float s = 1.0f;
+    if constexpr (SK == SK_SCALAR) s = scale_is_dev ? scale[0] : scale_host;
+    if constexpr (SK == SK_ROW) s = scale[row % mid];
+    if constexpr (BF16_IN) s = round_to_bf16(s);
 
-  constexpr int IN_BYTES = BF16_IN ? 16 : 32;
-  u32x4 in[U][BF16_IN ? 1 : 2];
-  bool ok[U];
+    u32x4 in[U][BF16_IN ? 1 : 2];
 #pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int64_t vr = v0 + (int64_t)u * THREADS;
-    ok[u] = vr < vec_per_row;
-    if (ok[u]) {
-      const u32x4* p = reinterpret_cast<const u32x4*>(x + (row_base + vr) * IN_BYTES);
-      in[u][0] = __builtin_nontemporal_load(p);
-      if constexpr (!BF16_IN) in[u][1] = __builtin_nontemporal_load(p + 1);
+    for (int u = 0; u < U; ++u) {
+      const int off = ((int)threadIdx.x + u * THREADS) * IN_BYTES;
+      in[u][0] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rin, off, 0, kNt));
+      if constexpr (!BF16_IN) in[u][1] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rin, off + 16, 0, kNt));
     }
-  }
+    // per-column / per-element scales: 8 floats per vector, out-of-range lanes read zeros
+    u32x4 sc[(SK == SK_COL || SK == SK_FULL) ? U : 1][2];
+    if constexpr (SK == SK_COL || SK == SK_FULL) {
+      const float* sbase = scale + (SK == SK_COL ? vec0 : first) * 8;
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sbase), 0, nvec * 32, 0x00020000);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int off = ((int)threadIdx.x + u * THREADS) * 32;
+        sc[u][0] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0));
+        sc[u][1] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, off + 16, 0, 0));
+      }
+    }
 
 #pragma unroll
-  for (int u = 0; u < U; ++u) {
-    if (!ok[u]) continue;
-    const int64_t vr = v0 + (int64_t)u * THREADS;
-    float v[8];
-    if constexpr (BF16_IN) {
+    for (int u = 0; u < U; ++u) {
+      float v[8];
+      if constexpr (BF16_IN) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t w = in[u][0][i];
-        v[2 * i] = __uint_as_float(w << 16);
-        v[2 * i + 1] = __uint_as_float(w & 0xffff0000u);
-        if constexpr (AMAX) {
-          // packed 16-bit max over the two abs bit patterns of this dword
-          const u16x2 a = __builtin_bit_cast(u16x2, w & 0x7fff7fffu);
-          const u16x2 m = __builtin_elementwise_max(a, __builtin_bit_cast(u16x2, am));
-          am = __builtin_bit_cast(uint32_t, m);
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t w = in[u][0][i];
+          v[2 * i] = __uint_as_float(w << 16);
+          v[2 * i + 1] = __uint_as_float(w & 0xffff0000u);
+          if constexpr (AMAX) {
+            // packed 16-bit max over the two abs bit patterns of this dword
+            const u16x2 a = __builtin_bit_cast(u16x2, w & 0x7fff7fffu);
+            const u16x2 m = __builtin_elementwise_max(a, __builtin_bit_cast(u16x2, am));
+            am = __builtin_bit_cast(uint32_t, m);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const uint32_t w = in[u][i >> 2][i & 3];
+          v[i] = __uint_as_float(w);
+          if constexpr (AMAX) {
+            const uint32_t a = w & 0x7fffffffu;
+            am = am > a ? am : a;
+          }
         }
       }
-    } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const uint32_t w = in[u][i >> 2][i & 3];
-        v[i] = __uint_as_float(w);
-        if constexpr (AMAX) {
-          const uint32_t a = w & 0x7fffffffu;
-          am = am > a ? am : a;
+        float sv = s;
+        if constexpr (SK == SK_COL || SK == SK_FULL) {
+          sv = __uint_as_float(sc[u][i >> 2][i & 3]);
+          if constexpr (BF16_IN) sv = round_to_bf16(sv);
         }
+        float p = v[i] * sv;
+        if constexpr (BF16_IN) p = round_to_bf16(p);
+        v[i] = p;
       }
+      u32x2 out;
+      out.x = cvt_fp8x4<FMT>(v[0], v[1], v[2], v[3]);
+      out.y = cvt_fp8x4<FMT>(v[4], v[5], v[6], v[7]);
+      __builtin_amdgcn_raw_buffer_store_b64(out, rout, ((int)threadIdx.x + u * THREADS) * 8, 0, kNt);
     }
-    float sv[8];
-    if constexpr (SK == SK_COL || SK == SK_FULL) {
-      const int64_t si = (SK == SK_COL ? vr : row_base + vr) * 8;
-      const f32x4 s0 = *reinterpret_cast<const f32x4*>(scale + si);
-      const f32x4 s1 = *reinterpret_cast<const f32x4*>(scale + si + 4);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        sv[i] = BF16_IN ? round_to_bf16(s0[i]) : s0[i];
-        sv[4 + i] = BF16_IN ? round_to_bf16(s1[i]) : s1[i];
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) sv[i] = s;
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float p = v[i] * sv[i];
-      if constexpr (BF16_IN) p = round_to_bf16(p);
-      v[i] = p;
-    }
-    u32x2 out;
-    out.x = cvt_fp8x4<FMT>(v[0], v[1], v[2], v[3]);
-    out.y = cvt_fp8x4<FMT>(v[4], v[5], v[6], v[7]);
-    __builtin_nontemporal_store(out, reinterpret_cast<u32x2*>(y + (row_base + vr) * 8));
-  }
   }
 
   if constexpr (AMAX) {
@@ -423,14 +432,21 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(
     float* __restrict__ scale_out, float* __restrict__ scale_inv_out) {
   __shared__ uint32_t wave_part[kThreads / 64];
   const int64_t row = blockIdx.x;
-  const u32x4* xr = reinterpret_cast<const u32x4*>(x) + row * vec_per_row;
+  // Descriptors over the row: a lane past its end loads zeros and its store is
+  // dropped, so the body has no divergent branch and all loads are in flight
+  // before the first is used.
+  constexpr int OUT_BYTES = BF16_IN ? 8 : 4;  // per 16-byte input vector
+  const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(x) + row * vec_per_row * 16, 0, (int)vec_per_row * 16, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rout =
+      __builtin_amdgcn_make_buffer_rsrc(y + row * vec_per_row * OUT_BYTES, 0, (int)vec_per_row * OUT_BYTES, 0x00020000);
   u32x4 in[VPT];
   uint32_t am = 0;
 #pragma unroll
+  for (int u = 0; u < VPT; ++u)
+    in[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rin, ((int)threadIdx.x + u * kThreads) * 16, 0, 2));
+#pragma unroll
   for (int u = 0; u < VPT; ++u) {
-    const int64_t v = threadIdx.x + (int64_t)u * kThreads;
-    in[u] = u32x4{0u, 0u, 0u, 0u};
-    if (v < vec_per_row) in[u] = __builtin_nontemporal_load(xr + v);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if constexpr (BF16_IN) {
@@ -461,8 +477,7 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(
   const float s = BF16_IN ? round_to_bf16(scale) : scale;
 #pragma unroll
   for (int u = 0; u < VPT; ++u) {
-    const int64_t v = threadIdx.x + (int64_t)u * kThreads;
-    if (v >= vec_per_row) continue;
+    const int off = ((int)threadIdx.x + u * kThreads) * OUT_BYTES;
     if constexpr (BF16_IN) {
       float p[8];
 #pragma unroll
@@ -471,11 +486,11 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(
         p[2 * i + 1] = round_to_bf16(__uint_as_float(in[u][i] & 0xffff0000u) * s);
       }
       const u32x2 o = {cvt_fp8x4<FMT>(p[0], p[1], p[2], p[3]), cvt_fp8x4<FMT>(p[4], p[5], p[6], p[7])};
-      __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(y) + row * vec_per_row + v);
+      __builtin_amdgcn_raw_buffer_store_b64(o, rout, off, 0, 2);
     } else {
       const uint32_t o = cvt_fp8x4<FMT>(__uint_as_float(in[u][0]) * s, __uint_as_float(in[u][1]) * s,
                                         __uint_as_float(in[u][2]) * s, __uint_as_float(in[u][3]) * s);
-      __builtin_nontemporal_store(o, reinterpret_cast<uint32_t*>(y) + row * vec_per_row + v);
+      __builtin_amdgcn_raw_buffer_store_b32(o, rout, off, 0, 2);
     }
   }
 }
@@ -493,27 +508,34 @@ __global__ __launch_bounds__(kThreads) void silu_mul_quantize_rows_kernel(
     float* __restrict__ scale_out, float* __restrict__ scale_inv_out) {
   __shared__ uint32_t wave_part[kThreads / 64];
   const int64_t row = blockIdx.x;
-  const u32x4* gr = reinterpret_cast<const u32x4*>(gate + row * ld_gate);
-  const u32x4* ur = reinterpret_cast<const u32x4*>(up + row * ld_up);
-  u32x4 h[VPT];
+  // Descriptors over the row (zeros past its end, stores dropped there): no
+  // divergent branch, and every load is in flight before the first is used.
+  const int row_bytes = (int)vec_per_row * 16;
+  const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(gate) + row * ld_gate, 0, row_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ru = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(up) + row * ld_up, 0, row_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(
+      h_out ? h_out + row * vec_per_row * 8 : nullptr, 0, h_out ? row_bytes : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(y + row * vec_per_row * 8, 0, (int)vec_per_row * 8, 0x00020000);
+  u32x4 gv[VPT], h[VPT];
   uint32_t am = 0;
 #pragma unroll
   for (int u = 0; u < VPT; ++u) {
-    const int64_t v = threadIdx.x + (int64_t)u * kThreads;
-    u32x4 gv = {0u, 0u, 0u, 0u}, uv = {0u, 0u, 0u, 0u};
-    if (v < vec_per_row) {
-      gv = __builtin_nontemporal_load(gr + v);
-      uv = __builtin_nontemporal_load(ur + v);
-    }
+    const int off = ((int)threadIdx.x + u * kThreads) * 16;
+    gv[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rg, off, 0, 2));
+    h[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ru, off, 0, 2));
+  }
+#pragma unroll
+  for (int u = 0; u < VPT; ++u) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float s0 = round_to_bf16(silu_f32(__uint_as_float(gv[i] << 16)));
-      const float s1 = round_to_bf16(silu_f32(__uint_as_float(gv[i] & 0xffff0000u)));
-      h[u][i] = pack_bf16x2(s0 * __uint_as_float(uv[i] << 16), s1 * __uint_as_float(uv[i] & 0xffff0000u));
+      const float s0 = round_to_bf16(silu_f32(__uint_as_float(gv[u][i] << 16)));
+      const float s1 = round_to_bf16(silu_f32(__uint_as_float(gv[u][i] & 0xffff0000u)));
+      h[u][i] = pack_bf16x2(s0 * __uint_as_float(h[u][i] << 16), s1 * __uint_as_float(h[u][i] & 0xffff0000u));
       const u16x2 a = __builtin_bit_cast(u16x2, h[u][i] & 0x7fff7fffu);
       am = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, __builtin_bit_cast(u16x2, am)));
     }
-    if (h_out && v < vec_per_row) reinterpret_cast<u32x4*>(h_out)[row * vec_per_row + v] = h[u];
+    // without h_out the descriptor is empty and the store goes nowhere
+    __builtin_amdgcn_raw_buffer_store_b128(h[u], rh, ((int)threadIdx.x + u * kThreads) * 16, 0, 0);
   }
   {
     const uint32_t lo = am & 0xffffu, hi = am >> 16;
@@ -534,8 +556,6 @@ __global__ __launch_bounds__(kThreads) void silu_mul_quantize_rows_kernel(
   const float s = round_to_bf16(scale);
 #pragma unroll
   for (int u = 0; u < VPT; ++u) {
-    const int64_t v = threadIdx.x + (int64_t)u * kThreads;
-    if (v >= vec_per_row) continue;
     float p[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -543,7 +563,7 @@ __global__ __launch_bounds__(kThreads) void silu_mul_quantize_rows_kernel(
       p[2 * i + 1] = round_to_bf16(__uint_as_float(h[u][i] & 0xffff0000u) * s);
     }
     const u32x2 o = {cvt_fp8x4<FMT>(p[0], p[1], p[2], p[3]), cvt_fp8x4<FMT>(p[4], p[5], p[6], p[7])};
-    __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(y) + row * vec_per_row + v);
+    __builtin_amdgcn_raw_buffer_store_b64(o, rout, ((int)threadIdx.x + u * kThreads) * 8, 0, 2);
   }
 }
 
@@ -556,69 +576,84 @@ __global__ __launch_bounds__(kThreads) void silu_mul_quantize_rows_kernel(
 template <bool BF16_OUT>
 constexpr int from_vec() { return BF16_OUT ? 8 : 4; }
 
-template <int FMT, bool BF16_OUT, int SK, int U>
+// WINDOW: stores a wave may still have outstanding when it issues the next one
+// (-1: no limit).  Measured for bf16 output, which writes twice the bytes it
+// reads: with 2 the kernel is 3-8 % faster than unlimited from 64 MiB of output
+// up (6.2 TB/s at 512 MiB), with 0 it is 9 % faster at 32 MiB; other sizes do
+// not care.  fp32 output and cast_to_fp8 (more reads than writes) lose with any limit.
+template <int FMT, bool BF16_OUT, int SK, int U, int WINDOW>
 __global__ __launch_bounds__(kThreads) void cast_from_fp8_vec(
     const uint8_t* __restrict__ x, uint8_t* __restrict__ y, const float* __restrict__ scale,
     float scale_host, int scale_is_dev, int has_scale, int64_t vec_per_row,
     int64_t blocks_per_row, int64_t mid) {
   constexpr int V = from_vec<BF16_OUT>();
+  constexpr int kNt = 2;  // non-temporal
   const int64_t row = blockIdx.x / blocks_per_row;
-  const int64_t bir = blockIdx.x - row * blocks_per_row;
-  const int64_t v0 = bir * (int64_t)(kThreads * U) + threadIdx.x;
-  const int64_t row_base = row * vec_per_row;
+  const int64_t vec0 = (blockIdx.x - row * blocks_per_row) * (int64_t)(kThreads * U);  // first vector, within the row
+  const int64_t left = vec_per_row - vec0;
+  const int nvec = (int)(left < kThreads * U ? left : kThreads * U);
+  const int64_t first = row * vec_per_row + vec0;                                    // first vector, within the tensor
+  // Branch-free like cast_to_fp8_vec8: descriptors that cover the block's
+  // vectors make a lane past the end load zeros and drop its store.
+  const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(x) + first * V, 0, nvec * V, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(y + first * 16, 0, nvec * 16, 0x00020000);
 
   float s = 1.0f;
   if constexpr (SK == SK_SCALAR) s = scale_is_dev ? scale[0] : scale_host;
   if constexpr (SK == SK_ROW) s = scale[row % mid];
   if constexpr (BF16_OUT) s = round_to_bf16(s);
+  if (!has_scale) s = 1.0f;  // x * 1 == x bit for bit (NaN payloads aside, and fp8 NaNs have one)
 
   uint32_t in[U][V / 4];
-  bool ok[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    const int64_t vr = v0 + (int64_t)u * kThreads;
-    ok[u] = vr < vec_per_row;
-    if (ok[u]) {
-      if constexpr (V == 8) {
-        const u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(x) + row_base + vr);
-        in[u][0] = t[0];
-        in[u][1] = t[1];
-      } else {
-        in[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(x) + row_base + vr);
-      }
+    const int off = ((int)threadIdx.x + u * kThreads) * V;
+    if constexpr (V == 8) {
+      const u32x2 t = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rin, off, 0, kNt));
+      in[u][0] = t[0];
+      in[u][1] = t[1];
+    } else {
+      in[u][0] = __builtin_amdgcn_raw_buffer_load_b32(rin, off, 0, kNt);
     }
+  }
+  constexpr bool kVecScale = SK == SK_COL || SK == SK_FULL;
+  u32x4 sc[kVecScale ? U : 1][V / 4];
+  if constexpr (kVecScale) {  // the launcher picks these kinds only for a scale tensor
+    const float* sbase = scale + (SK == SK_COL ? vec0 : first) * V;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sbase), 0, nvec * V * 4, 0x00020000);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q)
+        sc[u][q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, ((int)threadIdx.x + u * kThreads) * V * 4 + 16 * q, 0, 0));
   }
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    if (!ok[u]) continue;
-    const int64_t vr = v0 + (int64_t)u * kThreads;
     float v[V];
 #pragma unroll
     for (int i = 0; i < V / 4; ++i)
       cvt_f32x4<FMT>(in[u][i], v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
-    if (has_scale) {
-      if constexpr (SK == SK_COL || SK == SK_FULL) {
-        const int64_t si = (SK == SK_COL ? vr : row_base + vr) * V;
 #pragma unroll
-        for (int q = 0; q < V / 4; ++q) {
-          const f32x4 sq = *reinterpret_cast<const f32x4*>(scale + si + 4 * q);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) v[4 * q + i] *= BF16_OUT ? round_to_bf16(sq[i]) : sq[i];
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < V; ++i) v[i] *= s;
+    for (int i = 0; i < V; ++i) {
+      float sv = s;
+      if constexpr (kVecScale) {
+        sv = __uint_as_float(sc[u][i >> 2][i & 3]);
+        if constexpr (BF16_OUT) sv = round_to_bf16(sv);
       }
+      v[i] *= sv;
     }
-    u32x4* o = reinterpret_cast<u32x4*>(y) + row_base + vr;
+    u32x4 t;
     if constexpr (BF16_OUT) {
-      u32x4 t;
 #pragma unroll
       for (int i = 0; i < 4; ++i) t[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
-      __builtin_nontemporal_store(t, o);
     } else {
-      u32x4 t = {__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])};
-      __builtin_nontemporal_store(t, o);
+      t = u32x4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])};
+    }
+    __builtin_amdgcn_raw_buffer_store_b128(t, rout, ((int)threadIdx.x + u * kThreads) * 16, 0, kNt);
+    if constexpr (WINDOW >= 0) {
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(0x0F70 | WINDOW);  // vmcnt(WINDOW), other counters unlimited
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 }
@@ -649,10 +684,24 @@ __global__ __launch_bounds__(kThreads) void copy_bytes_kernel(const uint8_t* __r
   if (i < n) y[i] = x[i];
 }
 
-__global__ __launch_bounds__(kThreads) void copy_vec16_kernel(const u32x4* __restrict__ x,
-                                                              u32x4* __restrict__ y, int64_t nvec) {
-  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-  if (i < nvec) __builtin_nontemporal_store(__builtin_nontemporal_load(x + i), y + i);
+constexpr int kCopyU = 4;  // 16-byte vectors per thread
+
+// A block copies kThreads * kCopyU vectors through descriptors that end with
+// the tensor: all loads of a lane are issued before its first store.
+__global__ __launch_bounds__(kThreads) void copy_vec16_kernel(const uint8_t* __restrict__ x,
+                                                              uint8_t* __restrict__ y, int64_t nvec) {
+  const int64_t v0 = (int64_t)blockIdx.x * (kThreads * kCopyU);
+  const int64_t left = nvec - v0;
+  const int bytes = (int)(left < kThreads * kCopyU ? left : kThreads * kCopyU) * 16;
+  const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(x) + v0 * 16, 0, bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(y + v0 * 16, 0, bytes, 0x00020000);
+  u32x4 t[kCopyU];
+#pragma unroll
+  for (int u = 0; u < kCopyU; ++u)
+    t[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rin, ((int)threadIdx.x + u * kThreads) * 16, 0, 2));
+#pragma unroll
+  for (int u = 0; u < kCopyU; ++u)
+    __builtin_amdgcn_raw_buffer_store_b128(t[u], rout, ((int)threadIdx.x + u * kThreads) * 16, 0, 2);
 }
 
 // --------------------------------------------------------------- host helpers
@@ -771,19 +820,28 @@ int cast_from_dispatch(const uint8_t* x, uint8_t* y, const float* scale, float s
       const unsigned grid = (unsigned)grid64;
       const int is_dev = mode == MI355Q_SCALE_DEV;
       const int has_scale = mode != MI355Q_SCALE_NONE;
-      switch (p.sk) {
-        case SK_SCALAR:
-          cast_from_fp8_vec<FMT, BF16_OUT, SK_SCALAR, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
-          break;
-        case SK_ROW:
-          cast_from_fp8_vec<FMT, BF16_OUT, SK_ROW, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
-          break;
-        case SK_COL:
-          cast_from_fp8_vec<FMT, BF16_OUT, SK_COL, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
-          break;
-        default:
-          cast_from_fp8_vec<FMT, BF16_OUT, SK_FULL, U><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
-          break;
+      auto launch = [&](auto window) {
+        constexpr int W = decltype(window)::value;
+        switch (p.sk) {
+          case SK_SCALAR:
+            cast_from_fp8_vec<FMT, BF16_OUT, SK_SCALAR, U, W><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+            break;
+          case SK_ROW:
+            cast_from_fp8_vec<FMT, BF16_OUT, SK_ROW, U, W><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+            break;
+          case SK_COL:
+            cast_from_fp8_vec<FMT, BF16_OUT, SK_COL, U, W><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+            break;
+          default:
+            cast_from_fp8_vec<FMT, BF16_OUT, SK_FULL, U, W><<<grid, kThreads, 0, st>>>(x, y, scale, sh, is_dev, has_scale, vpr, bpr, p.mid);
+            break;
+        }
+      };
+      if constexpr (BF16_OUT) {
+        if (n * 2 <= (int64_t(48) << 20)) launch(std::integral_constant<int, 0>{});
+        else launch(std::integral_constant<int, 2>{});
+      } else {
+        launch(std::integral_constant<int, -1>{});
       }
       done = p.rows == 1 ? vpr * V : n;
     }
@@ -1003,8 +1061,8 @@ int mi355q_cast_to_fp8(const void* x, int x_dtype, void* y, int fp8_fmt, const f
     int64_t done = 0;
     if (aligned(x, 16) && aligned(y, 16) && n >= 16) {
       const int64_t nvec = n / 16;
-      copy_vec16_kernel<<<blocks_for(nvec, kThreads), kThreads, 0, st>>>(
-          reinterpret_cast<const u32x4*>(xb), reinterpret_cast<u32x4*>(yb), nvec);
+      if ((nvec + kThreads * kCopyU - 1) / (kThreads * kCopyU) > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+      copy_vec16_kernel<<<blocks_for(nvec, kThreads * kCopyU), kThreads, 0, st>>>(xb, yb, nvec);
       done = nvec * 16;
     }
     if (done < n)

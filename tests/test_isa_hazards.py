@@ -1,5 +1,6 @@
 """The generated gfx950 assembly of the GEMM kernels is free of the wait-state hazards that the
-compiler does not check inside asm statements (see isa_check.py).  CPU only: hipcc cross-compiles."""
+compiler does not check inside asm statements, and the streaming kernels issue their loads back to
+back (see isa_check.py).  CPU only: hipcc cross-compiles."""
 import importlib.util
 import os
 from concurrent.futures import ThreadPoolExecutor
@@ -85,3 +86,36 @@ def test_gemm_kernels_have_no_uncovered_hazard():
     for src, text in zip(sources, texts):
         assert text.count("#ASMSTART") > 100, f"{src}: the asm statements are gone?"
         assert isa_check.scan(text) == [], src
+
+
+def test_memory_order_reads_a_kernel():
+    text = """
+_Z3foov:                                ; @_Z3foov
+	global_load_dwordx4 v[2:5], v[0:1], off
+	s_waitcnt vmcnt(0)
+	global_load_dwordx4 v[6:9], v[0:1], off offset:16
+	s_waitcnt vmcnt(1) lgkmcnt(0)
+	buffer_store_dwordx2 v[2:3], v10, s[4:7], 0 offen
+	s_endpgm
+.Lfunc_end0:
+"""
+    assert isa_check.memory_order(text) == {"_Z3foov": "LWLwS"}
+
+
+@pytest.mark.timeout(600)
+def test_streaming_kernels_issue_their_loads_back_to_back():
+    """Every bandwidth-tuned streaming kernel issues all its independent loads before its first
+    full wait (a full wait before each load is what a divergent branch around it produces)."""
+    order = isa_check.memory_order(isa_check.compile_to_isa("cast_kernels.hip"))
+    seen = 0
+    for name, seq in order.items():
+        if "cast_to_fp8_vec8" in name or "cast_from_fp8_vec" in name:
+            loads = 4                                   # U
+        elif "quantize_rows_kernel" in name:            # VPT is the last template argument
+            loads = int(name.split("ELi")[-1].split("E")[0]) * (2 if "silu_mul" in name else 1)
+        else:
+            continue
+        seen += 1
+        first_full_wait = seq.find("W") if "W" in seq else len(seq)
+        assert seq[:first_full_wait].count("L") >= loads, (name, seq)
+    assert seen >= 60
