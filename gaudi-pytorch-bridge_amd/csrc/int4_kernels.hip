@@ -110,10 +110,11 @@ int dequant_launch(const uint32_t* packed, const uint8_t* scale, const uint8_t* 
                    int64_t pcols, int64_t group, uint8_t* out, hipStream_t st) {
   const int64_t lanes_per_row = pcols * (BF16 ? 1 : 2);
   auto grid_for = [&](int rpt) { return ((rows + rpt - 1) / rpt * lanes_per_row + kI4Threads - 1) / kI4Threads; };
-  if (group % 16 == 0) {
-    const int64_t grid = grid_for(16);
+  // 8 rows per thread measured best (K = N = 4096: 4 rows 9.0 us, 8 rows 7.3, 16 rows 7.7, 32 rows 7.9)
+  if (group % 8 == 0) {
+    const int64_t grid = grid_for(8);
     if (grid > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
-    dequant_4bit_kernel<SIGNED, BF16, ZP, 16, true><<<(unsigned)grid, kI4Threads, 0, st>>>(packed, scale, zp, rows, pcols, group, out);
+    dequant_4bit_kernel<SIGNED, BF16, ZP, 8, true><<<(unsigned)grid, kI4Threads, 0, st>>>(packed, scale, zp, rows, pcols, group, out);
   } else if (group == 1) {
     const int64_t grid = grid_for(1);
     if (grid > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
