@@ -133,6 +133,10 @@ def test_cast_to_fp8_v2_out_of_range(dev, dtype, big_tensor):
     ((33, 40), (1, 40)),          # per column, generic kernel
     ((3, 5, 64), (3, 1, 64)),     # two separate runs -> expanded to full
     ((6, 50), (6, 50)),           # elementwise
+    ((3, 40984), (3, 1)),         # rows of 5123 vectors: several blocks per row, the last one ragged
+    ((3, 40984), (1, 40984)),     # the same, per column
+    ((3, 40984), (3, 40984)),     # the same, elementwise
+    ((3, 40984), None),           # the same, one scale
     ((1031,), None),              # ragged flat tail
     ((0, 8), None),               # empty
 ])
