@@ -263,6 +263,43 @@ def bench_int4(pkg, oracle, dev, steps, warmup, cpu):
     return out
 
 
+def bench_reductions(pkg, oracle, dev, steps, warmup, cpu):
+    """softmax_fp8 and sum_fp8 (not BASELINE configurations; the next rows of the op family): attention-sized
+    probabilities, bf16 scores [4, 32, 2048, 2048] -> e4m3fn, and sums of an e4m3fn [8192, 8192] over either
+    dimension to fp32.  Timed through the torch ops (each call runs for 0.05 - 0.3 ms)."""
+    out = []
+    ops = torch.ops.hpu
+    gen = torch.Generator().manual_seed(SEED)
+    cores = torch.get_num_threads()
+    shape = (4, 32, 2048, 2048)
+    n = 4 * 32 * 2048 * 2048
+    base = (torch.randn(2048, 2048, generator=gen) * 2).bfloat16().to(dev)
+    xs = [(base.roll(i, 0)[None, None] + torch.zeros(shape[:2] + (1, 1), dtype=torch.bfloat16, device=dev)).contiguous() for i in range(2)]
+    ms = time_gpu(lambda i: ops.softmax_fp8(xs[i % 2], -1, 0.125, 256.0, None), steps, warmup)
+    c = None
+    if cpu:
+        sample = xs[0][0, :2].cpu()
+        t = time_cpu(lambda: oracle.torch_softmax_fp8(sample, -1, 0.125, 256.0), max_runs=3)
+        c = {"value": round(3 * sample.numel() / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+             "sample": "2 of the 128 [2048, 2048] score matrices, torch.softmax in fp32, bf16 rounding, scaled e4m3fn cast"}
+    out.append(hbm_entry("softmax_fp8", "softmax_fp8 bf16 [4,32,2048,2048] -> e4m3fn, scalar scales", 3 * n, ms, steps,
+                         "softmax_rows_kernel<bf16,e4m3fn,1 wave per row,4 vectors per lane>", c))
+    del xs
+    m = 8192
+    x8 = [torch.randint(-8, 9, (m, m), generator=gen).float().to(E4).to(dev) for _ in range(n_sets(m * m))]
+    for dim, what, kernel in ((1, "rows", "sum_rows_kernel<e4m3fn,16>"), (0, "columns", "sum_columns_kernel<e4m3fn,16> + sum_finish_kernel")):
+        ms = time_gpu(lambda i: ops.sum_fp8(x8[i % len(x8)], [dim], False, torch.float), max(steps, 50), max(warmup, 10))
+        c = None
+        if cpu and dim == 1:
+            xc = x8[0].cpu()
+            t = time_cpu(lambda: oracle.torch_sum_fp8(xc, [1], False, torch.float), max_runs=3)
+            c = {"value": round(m * m / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                 "sample": "the full [8192, 8192] tensor, torch.sum in float64"}
+        out.append(hbm_entry(f"sum_fp8_{what}", f"sum_fp8 e4m3fn [8192,8192] over dim {dim} -> fp32", m * m + 4 * m, ms,
+                             max(steps, 50), kernel, c))
+    return out
+
+
 def quant_per_tensor(ops, x_dev):
     amax = torch.ops.mi355q.amax(x_dev)
     s = 448.0 / amax
@@ -406,7 +443,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,cast,int4,decode,mlp")
+    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,cast,int4,decode,mlp,reduce")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -423,7 +460,7 @@ def main():
     ops = torch.ops.hpu
     dev = torch.device("cuda:0")
     torch.set_num_threads(min(os.cpu_count() or 1, 16))
-    which = set(args.only.split(",")) if args.only else {"gemm", "cast", "int4", "decode", "mlp"}
+    which = set(args.only.split(",")) if args.only else {"gemm", "cast", "int4", "decode", "mlp", "reduce"}
     cpu = not args.no_cpu
     k_stream = max(args.steps, 50)      # the microsecond-scale kernels need more calls for a stable mean
     w_stream = max(args.warmup, 10)
@@ -437,6 +474,8 @@ def main():
         ops_out += bench_gemm_decode(ops, oracle, dev, args.steps, args.warmup)
     if "mlp" in which:
         ops_out.append(bench_mlp(ops, dev, max(args.steps // 2, 5), args.warmup))
+    if "reduce" in which:
+        ops_out += bench_reductions(pkg, oracle, dev, args.steps, args.warmup, cpu)
 
     line = {"metric": "cast/dequant GB/s (% HBM peak); fp8_gemm_v2 TFLOP/s (% fp8 MFMA peak)",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,

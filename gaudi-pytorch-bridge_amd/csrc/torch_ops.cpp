@@ -668,6 +668,169 @@ Tensor convert_from_uint4(const Tensor& input, const Tensor& scale,
   return convert_from_int4_common("convert_from_uint4", false, input, scale, zero_point, out_dtype);
 }
 
+// ------------------------------------------------------------------ sum_fp8
+
+// hpu::sum_fp8 (hpu_ops/backend/fp8_ops_gen.cpp:20-49): sum of an fp8 tensor over `dim`
+// (all dimensions when absent), as out_dtype (the input's dtype when absent).
+Tensor sum_fp8(const Tensor& self, at::OptionalIntArrayRef dim, bool keepdim, c10::optional<at::ScalarType> out_dtype) {
+  TORCH_CHECK(is_fp8(self.scalar_type()), "sum_fp8 input must be float8_e4m3fn or float8_e5m2, got ", self.scalar_type());
+  const at::ScalarType odt = out_dtype.value_or(self.scalar_type());
+  TORCH_CHECK(odt == at::kFloat || odt == at::kBFloat16 || is_fp8(odt), "sum_fp8 out_dtype must be float, bfloat16 or an fp8 dtype, got ", odt);
+  const int64_t nd = self.dim();
+  std::vector<bool> reduced(std::max<int64_t>(nd, 1), false);
+  if (!dim.has_value() || dim->empty()) {
+    std::fill(reduced.begin(), reduced.end(), true);
+  } else {
+    for (int64_t d : *dim) {
+      const int64_t w = at::maybe_wrap_dim(d, nd);
+      TORCH_CHECK(!reduced[w], "dim ", w, " appears multiple times in the list of dims");
+      reduced[w] = true;
+    }
+  }
+  std::vector<int64_t> out_shape;
+  for (int64_t d = 0; d < nd; ++d) {
+    if (!reduced[d]) out_shape.push_back(self.size(d));
+    else if (keepdim) out_shape.push_back(1);
+  }
+  if (self.is_meta()) return at::empty(out_shape, self.options().dtype(odt));
+  DeviceGuard guard(self.device());
+  // reduced dimensions that are adjacent: [outer, reduce, inner] of the contiguous tensor;
+  // else they are moved to the end first (a copy)
+  int64_t first = -1, last = -1, count = 0;
+  for (int64_t d = 0; d < nd; ++d)
+    if (reduced[d]) { if (first < 0) first = d; last = d; ++count; }
+  Tensor c;
+  int64_t outer = 1, red = 1, inner = 1;
+  if (nd == 0 || count == 0) {
+    c = self.contiguous();
+    red = (nd == 0) ? 1 : 1;
+    outer = c.numel();
+  } else if (last - first + 1 == count) {
+    c = self.contiguous();
+    for (int64_t d = 0; d < first; ++d) outer *= c.size(d);
+    for (int64_t d = first; d <= last; ++d) red *= c.size(d);
+    for (int64_t d = last + 1; d < nd; ++d) inner *= c.size(d);
+  } else {
+    std::vector<int64_t> perm;
+    for (int64_t d = 0; d < nd; ++d) if (!reduced[d]) { perm.push_back(d); outer *= self.size(d); }
+    for (int64_t d = 0; d < nd; ++d) if (reduced[d]) { perm.push_back(d); red *= self.size(d); }
+    c = self.permute(perm).contiguous();
+  }
+  Tensor out = at::empty(out_shape, self.options().dtype(odt));
+  MI355Q_OP_INFO("sum_fp8 : input=" << self.sizes() << " as [" << outer << ", " << red << ", " << inner << "] -> " << odt);
+  if (out.numel() == 0) return out;
+  const size_t ws_bytes = mi355q_sum_fp8_workspace_bytes(outer, red, inner);
+  Tensor ws;
+  if (ws_bytes) ws = at::empty({(int64_t)ws_bytes}, self.options().dtype(at::kByte));
+  check_status(mi355q_sum_fp8(c.data_ptr(), to_mi355q_dtype(c.scalar_type()), outer, red, inner, out.data_ptr(),
+                              to_mi355q_dtype(odt), ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, current_stream(c)),
+               "mi355q_sum_fp8");
+  return out;
+}
+
+// -------------------------------------------------------------- softmax_fp8
+
+struct SoftmaxScale {
+  const float* dev = nullptr;
+  float host = 1.0f;
+  bool given = false;
+};
+
+SoftmaxScale softmax_scale(const c10::optional<Tensor>& t, const Tensor& input, const char* name) {
+  SoftmaxScale s;
+  if (!t.has_value() || !t->defined()) return s;
+  // addOptionalTensor, softmax_fp8_gen.cpp:25-40
+  TORCH_CHECK(t->scalar_type() == at::kFloat, "Input ", name, " must be of dtype: ", at::kFloat);
+  TORCH_CHECK(t->numel() == 1, "softmax_fp8 ", name, " must have one element, got ", t->sizes());
+  s.given = true;
+  if (!input.is_meta()) {
+    TORCH_CHECK(t->device() == input.device(), "softmax_fp8 ", name, " must be on the same device as input");
+    s.dev = t->data_ptr<float>();
+  }
+  return s;
+}
+SoftmaxScale softmax_scale(double v) {
+  SoftmaxScale s;
+  s.host = (float)v;
+  s.given = true;
+  return s;
+}
+
+// SoftmaxFp8::AddNode, hpu_ops/backend/softmax_fp8_gen.cpp:73-158 (checks and messages :88-119)
+Tensor softmax_fp8_common(const Tensor& input, int64_t dim, const SoftmaxScale& in_scale, const SoftmaxScale& out_scale,
+                          const SoftmaxScale& inv_heads, const c10::optional<Tensor>& fused_add) {
+  const int64_t rank = input.dim();
+  dim = at::maybe_wrap_dim(dim, rank, /*wrap_scalar=*/true);
+  const at::ScalarType dt = input.scalar_type();
+  TORCH_CHECK(dt == at::kBFloat16 || dt == at::kFloat8_e4m3fn,
+              "Input tensor must be of torch.bfloat16 or torch.float8_e4m3fn dtype.");
+  TORCH_CHECK(in_scale.given == out_scale.given, "Output and input scales must be both given or None");
+  TORCH_CHECK(dt != at::kFloat8_e4m3fn || in_scale.given,
+              "If Input is of torch.float8_e4m3fn dtype then input scale must be given.");
+  const bool has_add = fused_add.has_value() && fused_add->defined();
+  if (has_add) {
+    TORCH_CHECK(in_scale.given, "FusedAdd available only for Float8 output, but input scale is not given.");
+    TORCH_CHECK(rank == fused_add->dim(), "FusedAdd tensor must have the same rank as the input tensor");
+    TORCH_CHECK(rank >= 1 && input.size(0) == fused_add->size(0) && input.size(rank - 1) == fused_add->size(rank - 1),
+                "FusedAdd tensor must have the same first and last dim as the input tensor");
+    for (int64_t d = 1; d < rank - 1; ++d)
+      TORCH_CHECK(fused_add->size(d) == 1 || fused_add->size(d) == input.size(d),
+                  "FusedAdd tensor's dim other than first and last should be equal to 1 or the same as the input tensor");
+    TORCH_CHECK(fused_add->scalar_type() == at::kBFloat16, "Input fused_add must be of dtype: ", at::kBFloat16);
+    TORCH_CHECK(dim == rank - 1, "softmax_fp8 with fused_add is over the last dimension");
+    TORCH_CHECK(rank <= 7, "softmax_fp8 with fused_add takes at most 7 dimensions");
+  }
+  const at::ScalarType odt = in_scale.given ? at::kFloat8_e4m3fn : at::kBFloat16;   // SoftmaxFp8Meta, :65-71
+  if (input.is_meta()) return at::empty(input.sizes(), input.options().dtype(odt));
+  DeviceGuard guard(input.device());
+  if (rank == 0) {  // one element: its softmax is 1
+    return softmax_fp8_common(input.reshape({1}), 0, in_scale, out_scale, inv_heads, c10::nullopt).reshape({});
+  }
+  if (dim != rank - 1) {
+    Tensor moved = input.movedim(dim, -1).contiguous();
+    return softmax_fp8_common(moved, -1, in_scale, out_scale, inv_heads, c10::nullopt).movedim(-1, dim).contiguous();
+  }
+  Tensor c = input.contiguous();
+  Tensor out = at::empty(c.sizes(), c.options().dtype(odt));
+  MI355Q_OP_INFO("softmax_fp8 : input=" << input.sizes() << " " << dt << " -> " << odt << (has_add ? " +fused_add" : ""));
+  if (out.numel() == 0) return out;
+  const int64_t cols = c.size(-1);
+  const int64_t rows = c.numel() / cols;
+  Tensor fa;
+  std::vector<int64_t> row_sizes, fa_strides;
+  if (has_add) {
+    TORCH_CHECK(fused_add->device() == c.device(), "softmax_fp8 fused_add must be on the same device as input");
+    fa = fused_add->contiguous();
+    for (int64_t d = rank - 2; d >= 0; --d) {
+      row_sizes.push_back(c.size(d));
+      fa_strides.push_back(fa.size(d) == 1 ? 0 : fa.stride(d));
+    }
+  }
+  check_status(mi355q_softmax_fp8(c.data_ptr(), to_mi355q_dtype(dt), rows, cols, in_scale.dev, in_scale.host, out_scale.dev,
+                                  out_scale.host, inv_heads.dev, inv_heads.host, has_add ? fa.data_ptr() : nullptr,
+                                  (int)row_sizes.size(), row_sizes.data(), fa_strides.data(), out.data_ptr(),
+                                  to_mi355q_dtype(odt), current_stream(c)),
+               "mi355q_softmax_fp8");
+  return out;
+}
+
+Tensor softmax_fp8(const Tensor& input, int64_t dim, const c10::optional<Tensor>& input_scale,
+                   const c10::optional<Tensor>& output_scale, const c10::optional<Tensor>& inv_attn_heads,
+                   const c10::optional<Tensor>& fused_add) {
+  return softmax_fp8_common(input, dim, softmax_scale(input_scale, input, "scale"), softmax_scale(output_scale, input, "scale"),
+                            softmax_scale(inv_attn_heads, input, "scale"), fused_add);
+}
+Tensor softmax_fp8_scalar_scales(const Tensor& input, int64_t dim, double input_scale, double output_scale,
+                                 const c10::optional<Tensor>& inv_attn_heads, const c10::optional<Tensor>& fused_add) {
+  return softmax_fp8_common(input, dim, softmax_scale(input_scale), softmax_scale(output_scale),
+                            softmax_scale(inv_attn_heads, input, "scale"), fused_add);
+}
+Tensor softmax_fp8_scalar(const Tensor& input, int64_t dim, double input_scale, double output_scale, double inv_attn_heads,
+                          const c10::optional<Tensor>& fused_add) {
+  return softmax_fp8_common(input, dim, softmax_scale(input_scale), softmax_scale(output_scale), softmax_scale(inv_attn_heads),
+                            fused_add);
+}
+
 // ------------------------------------------------------------- amax helpers
 
 Tensor amax_op(const Tensor& x) {
@@ -850,6 +1013,10 @@ TORCH_LIBRARY(hpu, m) {
   m.def("hpu::fp8_gemm_v2(Tensor A, bool trans_A, Tensor B, bool trans_B, Tensor? D, ScalarType out_dtype, Tensor? A_scale_inv=None, Tensor? B_scale_inv=None, Tensor? bias=None, bool accumulate=False, int[]? B_scale_shape=None) -> Tensor");
   m.def("hpu::fp8_gemm_v2.scalar(Tensor A, bool trans_A, Tensor B, bool trans_B, Tensor? D, ScalarType out_dtype, float A_scale_inv, float B_scale_inv, Tensor? bias=None, bool accumulate=False, int[]? B_scale_shape=None) -> Tensor");
   m.def("hpu::fp8_gemm_v2.scalar_list(Tensor A, bool trans_A, Tensor B, bool trans_B, Tensor? D, ScalarType out_dtype, float[] A_scale_inv, float[] B_scale_inv, Tensor? bias=None, bool accumulate=False, int[]? B_scale_shape=None) -> Tensor");
+  m.def("hpu::softmax_fp8(Tensor input, int dim, Tensor? input_scale=None, Tensor? output_scale=None, Tensor? inv_attn_heads=None, Tensor? fused_add=None) -> Tensor");
+  m.def("hpu::softmax_fp8.Scalar_scales(Tensor input, int dim, float input_scale, float output_scale, Tensor? inv_attn_heads=None, Tensor? fused_add=None) -> Tensor");
+  m.def("hpu::softmax_fp8.Scalar(Tensor input, int dim, float input_scale, float output_scale, float inv_attn_heads, Tensor? fused_add=None) -> Tensor");
+  m.def("hpu::sum_fp8(Tensor self, int[1]? dim=None, bool keepdim=False, ScalarType? out_dtype=None) -> Tensor");
 }
 
 // Helpers the reference has no op for: amax alone and per-row amax.
@@ -875,7 +1042,11 @@ TORCH_LIBRARY(mi355q, m) {
   m.impl("convert_from_uint4", convert_from_uint4);                                            \
   m.impl("cast_to_fp8", cast_to_fp8_v1);                                                       \
   m.impl("cast_to_fp8_hybrid", cast_to_fp8_hybrid);                                            \
-  m.impl("fp8_gemm", fp8_gemm_v1);
+  m.impl("fp8_gemm", fp8_gemm_v1);                                                             \
+  m.impl("softmax_fp8", softmax_fp8);                                                          \
+  m.impl("softmax_fp8.Scalar_scales", softmax_fp8_scalar_scales);                              \
+  m.impl("softmax_fp8.Scalar", softmax_fp8_scalar);                                            \
+  m.impl("sum_fp8", sum_fp8);
 
 TORCH_LIBRARY_IMPL(hpu, CUDA, m) { MI355Q_REGISTER_HPU(m) }
 TORCH_LIBRARY_IMPL(hpu, Meta, m) { MI355Q_REGISTER_HPU(m) }

@@ -223,6 +223,40 @@ int mi355q_fp8_gemm(const void* A, int fmt_a, int trans_a, int64_t lda,
                     int64_t stride_c, int64_t stride_d, int64_t stride_bias,
                     void* stream);
 
+/*
+ * Sum over the middle dimension of an fp8 tensor viewed as [outer, reduce, inner]
+ * (a sum over adjacent dimensions of a contiguous tensor), accumulated in fp32 in a
+ * fixed order and written as out_dtype (fp32, bf16, or fp8 with the saturating
+ * round-to-nearest cast of mi355q_cast_to_fp8) [outer, inner].  Replaces the
+ * reduce_sum_multi_dim_fwd node of hpu::sum_fp8 (hpu_ops/backend/fp8_ops_gen.cpp:20-49,
+ * schema scripts/hpu_op.yaml:7448-7453).  When the launch splits the reduction it
+ * needs mi355q_sum_fp8_workspace_bytes(...) bytes of device memory for partial sums
+ * (0 when it does not); nothing is allocated here.
+ */
+size_t mi355q_sum_fp8_workspace_bytes(int64_t outer, int64_t reduce, int64_t inner);
+int mi355q_sum_fp8(const void* x, int fp8_fmt, int64_t outer, int64_t reduce, int64_t inner,
+                   void* out, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Softmax over the rows of x [rows, cols] (bf16 or e4m3fn):
+ *   v = (x * inv_attn_heads) * input_scale + fused_add,   each term optional,
+ *   p = bf16( exp(v - max v) / sum exp(v - max v) ),
+ *   y = p                              when y_dtype is bf16,
+ *   y = e4m3fn( p * output_scale )     when y_dtype is e4m3fn (saturating round to nearest),
+ * in fp32 up to the rounding to bf16.  Replaces the softmax_fwd_hf8 node of
+ * SoftmaxFp8::AddNode (hpu_ops/backend/softmax_fp8_gen.cpp:73-158).  A scale is a
+ * device scalar (pointer not NULL) or the host value (1 = absent).  fused_add is bf16
+ * or NULL; its rows are found by decomposing the row index over row_sizes[0 .. row_dims)
+ * (innermost first, product = rows) and adding digit * fused_add_row_strides[d] elements
+ * (0 where fused_add is broadcast), row_dims <= 6.
+ */
+int mi355q_softmax_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols,
+                       const float* input_scale_dev, float input_scale_host,
+                       const float* output_scale_dev, float output_scale_host,
+                       const float* inv_attn_heads_dev, float inv_attn_heads_host,
+                       const void* fused_add, int row_dims, const int64_t* row_sizes,
+                       const int64_t* fused_add_row_strides, void* y, int y_dtype, void* stream);
+
 /* Name of the kernel variant mi355q_fp8_gemm would pick for a problem
  * (for logs and profiles; static string). */
 const char* mi355q_fp8_gemm_variant(int trans_a, int64_t lda, int trans_b, int64_t ldb,

@@ -345,6 +345,42 @@ def torch_scaled_mm(mat1, mat2, scale_a, scale_b, bias=None, scale_result=None, 
     return v.to(out_dtype)
 
 
+def torch_sum_fp8(x, dim=None, keepdim=False, out_dtype=None):
+    """hpu::sum_fp8 as the reference's test states it (any_mode/test_hpu_sum_fp8.py:36-47): torch.sum of
+    the fp8 values; here accumulated in float64, so that the result is the exactly rounded sum whatever
+    the order (for inputs whose fp32 partial sums are all exact, as the test's are, any fp32 order gives
+    the same).  An fp8 out_dtype (the default, the input's) is the saturating round-to-nearest cast of
+    the sum: the reference compares that case with its own device result only -- parity unpinned."""
+    out_dtype = out_dtype or x.dtype
+    dims = list(range(x.dim())) if dim is None or (isinstance(dim, (list, tuple)) and len(dim) == 0) else dim
+    v = torch.sum(x.detach().cpu().to(torch.float64), dims, keepdim) if x.dim() else x.detach().cpu().to(torch.float64)
+    v = v.to(torch.float32)
+    if out_dtype in FP8_MAX:
+        mx = FP8_MAX[out_dtype]
+        return v.clamp(-mx, mx).to(out_dtype)
+    return v.to(out_dtype)
+
+
+def torch_softmax_fp8(x, dim=-1, input_scale=None, output_scale=None, inv_attn_heads=None, fused_add=None):
+    """hpu::softmax_fp8 (hpu_ops/backend/softmax_fp8_gen.cpp:73-158; semantics from
+    any_mode/test_hpu_fp8_ops_any_mode.py:1030-1045): softmax((x * inv_attn_heads) * input_scale + fused_add),
+    rounded to bf16; with scales the bf16 value times output_scale, cast to e4m3fn (saturating).  fp32
+    arithmetic up to the rounding to bf16 (the test rounds every step to bf16 and allows rtol 0.1251,
+    one e4m3 step; the device's internal precision is not stated) -- parity pinned to that tolerance only."""
+    v = x.detach().cpu().float()
+    if inv_attn_heads is not None:
+        v = v * float(inv_attn_heads)
+    if input_scale is not None:
+        v = v * torch.tensor(float(input_scale), dtype=torch.float32)
+        if fused_add is not None:
+            v = v + fused_add.detach().cpu().float()
+    p = torch.softmax(v, dim).to(torch.bfloat16)
+    if input_scale is None:
+        return p
+    q = p.float() * torch.tensor(float(output_scale), dtype=torch.float32)
+    return q.clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+
+
 def pack_nibbles(q):
     """int tensor [..., 8P] with values in -8..15 -> packed int32 [..., P]."""
     q = q.detach().cpu().to(torch.int64) & 0xF

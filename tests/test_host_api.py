@@ -40,7 +40,7 @@ def meta(shape, dtype):
 
 def test_library_exports_every_declared_symbol(pkg):
     header = open(os.path.join(ROOT, "include", "mi355q.h")).read()
-    declared = set(re.findall(r"^(?:int|const char\*)\s+(mi355q_[a-z0-9_]+)\s*\(", header, flags=re.M))
+    declared = set(re.findall(r"^(?:int|size_t|const char\*)\s+(mi355q_[a-z0-9_]+)\s*\(", header, flags=re.M))
     assert declared == set(pkg.EXPORTED_SYMBOLS)
     lib = pkg.capi()
     for name in declared:
