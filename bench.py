@@ -53,6 +53,9 @@ MEASURED_TRAFFIC = {
     "fp8_gemm_v2_decode_M16": 236.93e6,
     "fp8_gemm_v2_decode_M64": 242.94e6,
     "fp8_gemm_v2_decode_M256": 273.84e6,
+    "softmax_fp8": 1609.31e6,
+    "sum_fp8_rows": 67.32e6,
+    "sum_fp8_columns": 79.75e6,   # sum_columns_kernel 71.30 + sum_finish_kernel 8.45
 }
 
 
@@ -264,7 +267,7 @@ def bench_int4(pkg, oracle, dev, steps, warmup, cpu):
 
 
 def bench_reductions(pkg, oracle, dev, steps, warmup, cpu):
-    """softmax_fp8 and sum_fp8 (not BASELINE configurations; the next rows of the op family): attention-sized
+    """softmax_fp8 and sum_fp8 (no published configuration names sizes for them): attention-sized
     probabilities, bf16 scores [4, 32, 2048, 2048] -> e4m3fn, and sums of an e4m3fn [8192, 8192] over either
     dimension to fp32.  Timed through the torch ops (each call runs for 0.05 - 0.3 ms)."""
     out = []
