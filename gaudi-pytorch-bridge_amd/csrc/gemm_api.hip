@@ -137,6 +137,15 @@ int mi355q_fp8_gemm(const void* A, int fmt_a, int trans_a, int64_t lda, const vo
     gb.C = g.C + b0 * stride_c * es;
     if (g.D) gb.D = g.D + b0 * stride_d * es;
     if (g.bias) gb.bias = g.bias + b0 * stride_bias * es;
+    // A full [M, N] bias and an accumulate input are the same kind of addend (out_dtype, added in
+    // fp32 after the scales): alone, the bias takes D's place, which the fast epilogue knows.
+    if (gb.bias_mode == MI355Q_BIAS_FULL && gb.D == nullptr) {
+      gb.D = gb.bias;
+      gb.ldd = gb.ldbias;
+      gb.stride_d = gb.stride_bias;
+      gb.bias = nullptr;
+      gb.bias_mode = MI355Q_BIAS_NONE;
+    }
     gb.fast_epi = epilogue_fast_ok(gb, nb);
     if (tiled_ok(gb.A, trans_a, lda, gb.B, trans_b, ldb, M, N, K, stride_a, stride_b)) {
       const bool ak = !trans_a, bk = trans_b != 0;
