@@ -42,15 +42,17 @@ __device__ __forceinline__ void store_sum(void* out, int out_dtype, int64_t i, f
 // every fourth row of the slice (so 16 row segments of 64 * VEC bytes are in flight per
 // workgroup) and their sums are added through LDS, in wave order.
 template <int FMT, int VEC>
-__global__ __launch_bounds__(kRedThreads) void sum_columns_kernel(const uint8_t* __restrict__ x, int64_t R, int64_t inner,
-                                                                  int64_t per, int splits, void* __restrict__ out,
-                                                                  int out_dtype, float* __restrict__ partial) {
+__global__ __launch_bounds__(kRedThreads) void sum_columns_kernel(const uint8_t* __restrict__ x, int64_t outer, int64_t R,
+                                                                  int64_t inner, int64_t per, int splits, int col_blocks,
+                                                                  void* __restrict__ out, int out_dtype,
+                                                                  float* __restrict__ partial) {
   constexpr int WAVES = kRedThreads / 64;
   __shared__ float part[WAVES - 1][64][VEC];
-  const int64_t o = blockIdx.y;
-  const int s = blockIdx.z;
+  // blockIdx.x = outer index * col_blocks + column block (outer can exceed the 65535 of grid.y)
+  const int64_t o = blockIdx.x / col_blocks;
+  const int s = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t c0 = ((int64_t)blockIdx.x * 64 + lane) * VEC;
+  const int64_t c0 = ((int64_t)(blockIdx.x - o * col_blocks) * 64 + lane) * VEC;
   const int64_t r0 = s * per;
   const int64_t r1 = (r0 + per) < R ? (r0 + per) : R;
   const bool inside = c0 < inner;
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(kRedThreads) void sum_columns_kernel(const uint8_t*
 #pragma unroll
       for (int w = 0; w < WAVES - 1; ++w) v += part[w][lane][e];
       if (splits == 1) store_sum(out, out_dtype, o * inner + c0 + e, v);
-      else partial[((int64_t)s * gridDim.y + o) * inner + c0 + e] = v;
+      else partial[((int64_t)s * outer + o) * inner + c0 + e] = v;
     }
   }
 }
@@ -242,11 +244,12 @@ int sum_fp8_launch(const uint8_t* x, int64_t outer, int64_t R, int64_t inner, vo
   if (outer > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
   if (inner > 1) {
     const int64_t bx = (inner / p.vec + 63) / 64;
-    if (bx > 0x7fffffffLL || outer > 65535) return MI355Q_ERR_UNSUPPORTED;
-    dim3 grid((unsigned)bx, (unsigned)outer, (unsigned)p.splits);
-    if (p.vec == 16) sum_columns_kernel<FMT, 16><<<grid, kRedThreads, 0, st>>>(x, R, inner, p.per, p.splits, out, out_dtype, ws);
-    else if (p.vec == 4) sum_columns_kernel<FMT, 4><<<grid, kRedThreads, 0, st>>>(x, R, inner, p.per, p.splits, out, out_dtype, ws);
-    else sum_columns_kernel<FMT, 1><<<grid, kRedThreads, 0, st>>>(x, R, inner, p.per, p.splits, out, out_dtype, ws);
+    if (bx * outer > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+    dim3 grid((unsigned)(bx * outer), (unsigned)p.splits);
+    const int cb = (int)bx;
+    if (p.vec == 16) sum_columns_kernel<FMT, 16><<<grid, kRedThreads, 0, st>>>(x, outer, R, inner, p.per, p.splits, cb, out, out_dtype, ws);
+    else if (p.vec == 4) sum_columns_kernel<FMT, 4><<<grid, kRedThreads, 0, st>>>(x, outer, R, inner, p.per, p.splits, cb, out, out_dtype, ws);
+    else sum_columns_kernel<FMT, 1><<<grid, kRedThreads, 0, st>>>(x, outer, R, inner, p.per, p.splits, cb, out, out_dtype, ws);
   } else {
     dim3 grid((unsigned)outer, (unsigned)p.splits);
     if (p.vec == 16) sum_rows_kernel<FMT, 16><<<grid, kRedThreads, 0, st>>>(x, R, p.per, p.splits, out, out_dtype, ws);

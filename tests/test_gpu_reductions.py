@@ -35,6 +35,7 @@ def test_sum_fp8(oracle, dev, dim, keep_dim, dtype, out_dtype):
     ((8, 1000, 256), [1]),        # columns, 16 per thread
     ((2, 5000, 20), [1]),         # columns, 4 per thread, split
     ((3, 700, 30), [1]),          # columns, 1 per thread
+    ((70000, 3, 8), [1]),         # more outer positions than one grid dimension holds
     ((6, 7, 8, 9), [0, 2]),       # dimensions that are not adjacent
     ((6, 7, 8, 9), [1, 2]),       # adjacent, in the middle
     ((4, 0, 5), [1]),             # empty reduction: zeros
