@@ -50,6 +50,40 @@ def test_graph_replays_match_eager(dev):
             assert torch.equal(a.view(torch.uint8) if a.dtype == E4 else a, b.view(torch.uint8) if b.dtype == E4 else b), rep
 
 
+def attention_like(q8, k8, sq, sk):
+    """scores = q k^T in fp8, probabilities through softmax_fp8, their row sums through sum_fp8 (split: workspace)."""
+    scores = ops.fp8_gemm_v2(q8, False, k8, True, None, torch.bfloat16, sq, sk, None, False)
+    p8 = ops.softmax_fp8(scores, -1, 0.125, 256.0, None)
+    return scores, p8, ops.sum_fp8(p8, [0, 1], False, torch.float), ops.sum_fp8(p8, [2], False, torch.bfloat16)
+
+
+def test_graph_replays_of_the_reductions(dev):
+    g = torch.Generator().manual_seed(13)
+    B, L, D = 4, 256, 128
+    k8 = torch.randn(B, L, D, generator=g).to(E4).to(dev)
+    sq, sk = torch.tensor(0.5, device=dev), torch.tensor(0.25, device=dev)
+    static_q = torch.randn(B, L, D, generator=g).to(E4).to(dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            attention_like(static_q, k8, sq, sk)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = attention_like(static_q, k8, sq, sk)
+    for rep in range(4):
+        q = (torch.randn(B, L, D, generator=g) * (rep + 1)).to(E4).to(dev)
+        static_q.copy_(q)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        ref = attention_like(q, k8, sq, sk)
+        torch.cuda.synchronize()
+        for a, b in zip(got, ref):
+            assert torch.equal(a.view(torch.uint8) if a.dtype == E4 else a, b.view(torch.uint8) if b.dtype == E4 else b), rep
+
+
 def test_ops_follow_the_current_stream(oracle, dev):
     """Work is enqueued on torch's current stream (as the reference uses the current HPUStream,
     habana_eager/eager_exec.cpp:341), not on the default one: results are right when the inputs were
