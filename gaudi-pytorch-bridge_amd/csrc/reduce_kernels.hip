@@ -297,103 +297,112 @@ __device__ __forceinline__ int64_t add_row_offset(const SoftmaxArgs& a, int64_t 
   return off;
 }
 
-// WPR waves share a row (1: four rows per workgroup; 4: one row); a lane holds VPT vectors of 8.
-template <bool IN_FP8, bool OUT_FP8, int WPR, int VPT>
+// WPR waves share a row (1 or 4); a lane holds VPT vectors of 8 of each of its RPW rows (RPW > 1
+// only with WPR == 1: a wave then owns RPW consecutive short rows, so that a lane still has four
+// loads in flight).  A workgroup covers 4 / WPR * RPW rows.
+template <bool IN_FP8, bool OUT_FP8, int WPR, int VPT, int RPW>
 __global__ __launch_bounds__(kRedThreads) void softmax_rows_kernel(SoftmaxArgs a) {
+  static_assert(WPR == 1 || RPW == 1, "several rows per wave only when a wave owns whole rows");
   constexpr int LANES = 64 * WPR;
-  constexpr int IN_VEC_BYTES = IN_FP8 ? 8 : 16;
-  constexpr int OUT_VEC_BYTES = OUT_FP8 ? 8 : 16;
+  constexpr int IN_ELEM = IN_FP8 ? 1 : 2, OUT_ELEM = OUT_FP8 ? 1 : 2;
   __shared__ float xchg[2][kRedThreads / 64];
   const int wave = threadIdx.x >> 6;
   const int lane = WPR == 1 ? (threadIdx.x & 63) : threadIdx.x;
-  const int64_t row = WPR == 1 ? (int64_t)blockIdx.x * 4 + wave : (int64_t)blockIdx.x;
-  const bool live = row < a.rows;                       // uniform per wave
-  const int64_t rrow = live ? row : 0;
+  const int64_t row0 = WPR == 1 ? ((int64_t)blockIdx.x * 4 + wave) * RPW : (int64_t)blockIdx.x;
   const int cols = (int)a.cols;
-  const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint8_t*>(a.x) + rrow * cols * (IN_FP8 ? 1 : 2), 0, live ? cols * (IN_FP8 ? 1 : 2) : 0, kRsrcFlags);
-  const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(
-      a.y + rrow * cols * (OUT_FP8 ? 1 : 2), 0, live ? cols * (OUT_FP8 ? 1 : 2) : 0, kRsrcFlags);
   const bool has_add = a.add != nullptr;
-  const __amdgpu_buffer_rsrc_t radd = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint16_t*>(a.add) + (has_add ? add_row_offset(a, rrow) : 0), 0, (live && has_add) ? cols * 2 : 0, kRsrcFlags);
-
   const float s_in = a.in_scale ? a.in_scale[0] : a.in_scale_host;
   const float s_out = a.out_scale ? a.out_scale[0] : a.out_scale_host;
   const float s_inv = a.inv_heads ? a.inv_heads[0] : a.inv_heads_host;
 
-  u32x4 raw[VPT];   // IN_FP8 uses the first two words
-  u32x4 addv[VPT];
+  u32x4 raw[RPW][VPT];   // IN_FP8 uses the first two words
+  u32x4 addv[RPW][VPT];
 #pragma unroll
-  for (int u = 0; u < VPT; ++u) {
-    const int v = lane + u * LANES;
-    if constexpr (IN_FP8) {
-      const u32x2 t = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rin, v * IN_VEC_BYTES, 0, 2));
-      raw[u] = u32x4{t[0], t[1], 0u, 0u};
-    } else {
-      raw[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rin, v * IN_VEC_BYTES, 0, 2));
+  for (int rr = 0; rr < RPW; ++rr) {
+    const bool live = row0 + rr < a.rows;                 // uniform per wave
+    const int64_t row = live ? row0 + rr : 0;
+    const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(a.x) + row * cols * IN_ELEM, 0, live ? cols * IN_ELEM : 0, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t radd = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(a.add) + (has_add ? add_row_offset(a, row) : 0), 0, (live && has_add) ? cols * 2 : 0, kRsrcFlags);
+#pragma unroll
+    for (int u = 0; u < VPT; ++u) {
+      const int v = lane + u * LANES;
+      if constexpr (IN_FP8) {
+        const u32x2 t = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rin, v * 8, 0, 2));
+        raw[rr][u] = u32x4{t[0], t[1], 0u, 0u};
+      } else {
+        raw[rr][u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rin, v * 16, 0, 2));
+      }
+      addv[rr][u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(radd, v * 16, 0, 0));  // zeros without fused_add
     }
-    addv[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(radd, v * 16, 0, 0));  // zeros without fused_add
   }
-  float val[VPT][8];
-  float m = -__builtin_inff();
 #pragma unroll
-  for (int u = 0; u < VPT; ++u) {
-    if constexpr (IN_FP8) {
-      cvt_f32x4<MI355Q_E4M3FN>(raw[u][0], val[u][0], val[u][1], val[u][2], val[u][3]);
-      cvt_f32x4<MI355Q_E4M3FN>(raw[u][1], val[u][4], val[u][5], val[u][6], val[u][7]);
-    } else {
+  for (int rr = 0; rr < RPW; ++rr) {
+    const bool live = row0 + rr < a.rows;
+    const int64_t row = live ? row0 + rr : 0;
+    const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(
+        a.y + row * cols * OUT_ELEM, 0, live ? cols * OUT_ELEM : 0, kRsrcFlags);
+    float val[VPT][8];
+    float m = -__builtin_inff();
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        val[u][2 * i] = __uint_as_float(raw[u][i] << 16);
-        val[u][2 * i + 1] = __uint_as_float(raw[u][i] & 0xffff0000u);
+    for (int u = 0; u < VPT; ++u) {
+      if constexpr (IN_FP8) {
+        cvt_f32x4<MI355Q_E4M3FN>(raw[rr][u][0], val[u][0], val[u][1], val[u][2], val[u][3]);
+        cvt_f32x4<MI355Q_E4M3FN>(raw[rr][u][1], val[u][4], val[u][5], val[u][6], val[u][7]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          val[u][2 * i] = __uint_as_float(raw[rr][u][i] << 16);
+          val[u][2 * i + 1] = __uint_as_float(raw[rr][u][i] & 0xffff0000u);
+        }
+      }
+      const bool inside = (lane + u * LANES) * 8 < cols;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float ad = __uint_as_float((i & 1) ? (addv[rr][u][i >> 1] & 0xffff0000u) : (addv[rr][u][i >> 1] << 16));
+        const float t = (val[u][i] * s_inv) * s_in + ad;
+        val[u][i] = inside ? t : -__builtin_inff();
+        m = __builtin_fmaxf(m, val[u][i]);
       }
     }
-    const bool inside = (lane + u * LANES) * 8 < cols;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float ad = __uint_as_float((i & 1) ? (addv[u][i >> 1] & 0xffff0000u) : (addv[u][i >> 1] << 16));
-      const float t = (val[u][i] * s_inv) * s_in + ad;
-      val[u][i] = inside ? t : -__builtin_inff();
-      m = __builtin_fmaxf(m, val[u][i]);
+    m = wave_max_f32(m);
+    if constexpr (WPR > 1) {
+      if ((threadIdx.x & 63) == 0) xchg[0][wave] = m;
+      __syncthreads();
+      m = __builtin_fmaxf(__builtin_fmaxf(xchg[0][0], xchg[0][1]), __builtin_fmaxf(xchg[0][2], xchg[0][3]));
     }
-  }
-  m = wave_max_f32(m);
-  if constexpr (WPR > 1) {
-    if ((threadIdx.x & 63) == 0) xchg[0][wave] = m;
-    __syncthreads();
-    m = __builtin_fmaxf(__builtin_fmaxf(xchg[0][0], xchg[0][1]), __builtin_fmaxf(xchg[0][2], xchg[0][3]));
-  }
-  // a row of -inf only (or NaN) gives NaN, as torch.softmax does
-  float sum = 0.0f;
+    // a row of -inf only (or NaN) gives NaN, as torch.softmax does
+    float sum = 0.0f;
 #pragma unroll
-  for (int u = 0; u < VPT; ++u)
+    for (int u = 0; u < VPT; ++u)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      val[u][i] = __expf(val[u][i] - m);
-      sum += val[u][i];
+      for (int i = 0; i < 8; ++i) {
+        val[u][i] = __expf(val[u][i] - m);
+        sum += val[u][i];
+      }
+    sum = wave_sum_f32(sum);
+    if constexpr (WPR > 1) {
+      if ((threadIdx.x & 63) == 0) xchg[1][wave] = sum;
+      __syncthreads();
+      sum = (xchg[1][0] + xchg[1][1]) + (xchg[1][2] + xchg[1][3]);
     }
-  sum = wave_sum_f32(sum);
-  if constexpr (WPR > 1) {
-    if ((threadIdx.x & 63) == 0) xchg[1][wave] = sum;
-    __syncthreads();
-    sum = (xchg[1][0] + xchg[1][1]) + (xchg[1][2] + xchg[1][3]);
-  }
-  const float inv = 1.0f / sum;
+    const float inv = 1.0f / sum;
 #pragma unroll
-  for (int u = 0; u < VPT; ++u) {
-    const int v = lane + u * LANES;
-    float p[8];
+    for (int u = 0; u < VPT; ++u) {
+      const int v = lane + u * LANES;
+      float p[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) p[i] = val[u][i] * inv;
-    if constexpr (OUT_FP8) {
+      for (int i = 0; i < 8; ++i) p[i] = val[u][i] * inv;
+      if constexpr (OUT_FP8) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) p[i] = round_to_bf16(p[i]) * s_out;
-      const u32x2 o = {cvt_fp8x4<MI355Q_E4M3FN>(p[0], p[1], p[2], p[3]), cvt_fp8x4<MI355Q_E4M3FN>(p[4], p[5], p[6], p[7])};
-      __builtin_amdgcn_raw_buffer_store_b64(o, rout, v * OUT_VEC_BYTES, 0, 2);
-    } else {
-      const u32x4 o = {pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7])};
-      __builtin_amdgcn_raw_buffer_store_b128(o, rout, v * OUT_VEC_BYTES, 0, 2);
+        for (int i = 0; i < 8; ++i) p[i] = round_to_bf16(p[i]) * s_out;
+        const u32x2 o = {cvt_fp8x4<MI355Q_E4M3FN>(p[0], p[1], p[2], p[3]), cvt_fp8x4<MI355Q_E4M3FN>(p[4], p[5], p[6], p[7])};
+        __builtin_amdgcn_raw_buffer_store_b64(o, rout, v * 8, 0, 2);
+      } else {
+        const u32x4 o = {pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7])};
+        __builtin_amdgcn_raw_buffer_store_b128(o, rout, v * 16, 0, 2);
+      }
     }
   }
 }
@@ -461,18 +470,21 @@ int softmax_launch(const SoftmaxArgs& a, hipStream_t st) {
   const bool one_wave = nv <= 64 * 8;
   const int64_t lanes = one_wave ? 64 : 256;
   const int64_t need = (nv + lanes - 1) / lanes;
-  const int64_t blocks = one_wave ? (a.rows + 3) / 4 : a.rows;
+  // short rows: a wave takes 4 (one vector per lane and row) or 2 (two vectors) rows
+  const int rpw = !one_wave ? 1 : need <= 1 ? 4 : need <= 2 ? 2 : 1;
+  const int64_t rows_per_block = one_wave ? 4 * rpw : 1;
+  const int64_t blocks = (a.rows + rows_per_block - 1) / rows_per_block;
   if (blocks > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
   const unsigned g = (unsigned)blocks;
-#define MI355Q_SOFTMAX(WPR, VPT) softmax_rows_kernel<IN_FP8, OUT_FP8, WPR, VPT><<<g, kRedThreads, 0, st>>>(a)
+#define MI355Q_SOFTMAX(WPR, VPT, RPW) softmax_rows_kernel<IN_FP8, OUT_FP8, WPR, VPT, RPW><<<g, kRedThreads, 0, st>>>(a)
   if (one_wave) {
-    if (need <= 1) MI355Q_SOFTMAX(1, 1);
-    else if (need <= 2) MI355Q_SOFTMAX(1, 2);
-    else if (need <= 4) MI355Q_SOFTMAX(1, 4);
-    else MI355Q_SOFTMAX(1, 8);
+    if (need <= 1) MI355Q_SOFTMAX(1, 1, 4);
+    else if (need <= 2) MI355Q_SOFTMAX(1, 2, 2);
+    else if (need <= 4) MI355Q_SOFTMAX(1, 4, 1);
+    else MI355Q_SOFTMAX(1, 8, 1);
   } else {
-    if (need <= 4) MI355Q_SOFTMAX(4, 4);
-    else MI355Q_SOFTMAX(4, 8);
+    if (need <= 4) MI355Q_SOFTMAX(4, 4, 1);
+    else MI355Q_SOFTMAX(4, 8, 1);
   }
 #undef MI355Q_SOFTMAX
   return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
