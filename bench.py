@@ -53,9 +53,9 @@ MEASURED_TRAFFIC = {
     "fp8_gemm_v2_decode_M16": 236.93e6,
     "fp8_gemm_v2_decode_M64": 242.94e6,
     "fp8_gemm_v2_decode_M256": 273.84e6,
-    "softmax_fp8": 1609.31e6,
+    "softmax_fp8": 1609.30e6,
     "sum_fp8_rows": 67.32e6,
-    "sum_fp8_columns": 79.75e6,   # sum_columns_kernel 71.30 + sum_finish_kernel 8.45
+    "sum_fp8_columns": 73.45e6,   # sum_columns_kernel 69.20 + sum_finish_kernel 4.25
 }
 
 
@@ -286,7 +286,7 @@ def bench_reductions(pkg, oracle, dev, steps, warmup, cpu):
         c = {"value": round(3 * sample.numel() / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
              "sample": "2 of the 128 [2048, 2048] score matrices, torch.softmax in fp32, bf16 rounding, scaled e4m3fn cast"}
     out.append(hbm_entry("softmax_fp8", "softmax_fp8 bf16 [4,32,2048,2048] -> e4m3fn, scalar scales", 3 * n, ms, steps,
-                         "softmax_rows_kernel<bf16,e4m3fn,1 wave per row,4 vectors per lane>", c))
+                         "softmax_rows_kernel<bf16,e4m3fn,1 wave per row,4 vectors per lane,1 row per wave>", c))
     del xs
     m = 8192
     x8 = [torch.randint(-8, 9, (m, m), generator=gen).float().to(E4).to(dev) for _ in range(n_sets(m * m))]
