@@ -360,6 +360,11 @@ def bench_gemm_decode(ops, oracle, dev, steps, warmup):
     del w
     # two copies of the weights exceed the Infinity Cache: alternate between them
     w8s = [w8, w8.clone()]
+    # the vendor library's row-wise scaled fp8 GEMM as a calibration point (it wants B column-major)
+    try:
+        w8_cm = [t.t().contiguous().t() for t in w8s]
+    except Exception:  # noqa: BLE001 - optional
+        w8_cm = None
     cols = torch.randperm(K, generator=gen)[:82]
     for M in (16, 64, 256):
         x = torch.randn(M, K, generator=gen)
@@ -370,10 +375,18 @@ def bench_gemm_decode(ops, oracle, dev, steps, warmup):
                                                 None, False, [1, N]), steps, warmup)
         nbytes = K * N + M * K + 2 * M * N + 4 * (M + N)
         flop = 2.0 * M * N * K
+        lib_ms = None
+        if w8_cm is not None:
+            try:
+                sa2, sb2 = sx_inv.reshape(M, 1).contiguous(), sw_inv.reshape(1, N).contiguous()
+                lib_ms = round(time_gpu(lambda i: torch._scaled_mm(x8, w8_cm[i % 2], scale_a=sa2, scale_b=sb2,
+                                                                   out_dtype=torch.bfloat16), steps, warmup), 5)
+            except Exception:  # noqa: BLE001 - the library may refuse the call
+                lib_ms = None
         out.append(hbm_entry(f"fp8_gemm_v2_decode_M{M}",
                              f"C4 fp8_gemm_v2 M={M} K=8192 N=28672 per-token x per-channel scales -> bf16",
-                             nbytes, ms, steps, "fp8_gemm_tile_kernel",
-                             extra={"tflops": round(flop / (ms * 1e-3) / 1e12, 2)}))
+                             nbytes, ms, steps, "fp8_gemm_skinny_kernel" if M <= 128 else "fp8_gemm_tile_kernel<256,128>",
+                             extra={"tflops": round(flop / (ms * 1e-3) / 1e12, 2), "library_gemm_ms_same_shape": lib_ms}))
     return out
 
 
