@@ -4,11 +4,15 @@
 // flop): with four waves of 128 x 128 when the fast bf16 epilogue applies (see
 // gemm_tile.h), otherwise with eight waves of 128 x 64 and the general
 // epilogue.  When that tiling leaves compute units without a tile, smaller
-// tiles run on the eight-wave kernel: 256 x 128 (twice the tiles at 1.5 times
-// the LDS traffic per flop) while those fill more than half the compute units,
-// else 128 x 128, of which two workgroups fit a compute unit (80 KB of LDS and
-// at most 128 registers each) and cover each other's waits: 6 to 27 % faster
-// than 256 x 128 on shapes such as 1024 x 4096 x 4096 or 1536 x 1536 x 8192.
+// tiles run: 256 x 128 (twice the tiles at 1.5 times the global->LDS traffic
+// per flop) while those fill more than half the compute units, with four waves
+// of 128 x 64 (1.5 KB of LDS fragments read per MFMA; as eight waves of
+// 128 x 32 it read 2.5 KB and was 3 to 8 % slower at 256 x 8192 x 28672);
+// else 128 x 128 with eight waves, of which two workgroups fit a compute unit
+// (80 KB of LDS and at most 128 registers each) and cover each other's waits:
+// 6 to 27 % faster than 256 x 128 on shapes such as 1024 x 4096 x 4096 or
+// 1536 x 1536 x 8192 (four waves there gained nothing with a bf16 output and
+// lost 4 to 6 % with an fp32 one).
 // (A 4-wave kernel with two workgroups per CU and 64-byte K stages, meant to
 // hide the epilogue behind the other workgroup's MFMAs, was measured against
 // the 256 x 128 tiles: bound by its global->LDS traffic on large problems and
@@ -87,11 +91,11 @@ void launch_by_size(const GemmArgs& g, int64_t batch, hipStream_t st) {
           head.N = (int)n_main;
           head.fast_epi = epilogue_fast_ok(head, batch);
           launch_256x256<AK, BK_, FA, FB>(head, batch, st);
-          launch_tile<256, 128, 4, false, AK, BK_, FA, FB>(columns_from<BK_>(g, n_main, batch), batch, st);
+          launch_tile<256, 128, 2, false, AK, BK_, FA, FB>(columns_from<BK_>(g, n_main, batch), batch, st);
         }
         break;
       }
-      case TileChoice::k256x128: launch_tile<256, 128, 4, false, AK, BK_, FA, FB>(g, batch, st); break;
+      case TileChoice::k256x128: launch_tile<256, 128, 2, false, AK, BK_, FA, FB>(g, batch, st); break;
       case TileChoice::k128x128: launch_tile<128, 128, 4, false, AK, BK_, FA, FB, 2>(g, batch, st); break;
     }
   } else if (g.M <= 128) {
