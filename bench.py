@@ -52,7 +52,7 @@ MEASURED_TRAFFIC = {
     "fp8_gemm_v2": 939.86e6,
     "fp8_gemm_v2_decode_M16": 236.93e6,
     "fp8_gemm_v2_decode_M64": 242.94e6,
-    "fp8_gemm_v2_decode_M256": 273.84e6,
+    "fp8_gemm_v2_decode_M256": 266.46e6,
     "softmax_fp8": 1609.30e6,
     "sum_fp8_rows": 67.32e6,
     "sum_fp8_columns": 73.45e6,   # sum_columns_kernel 69.20 + sum_finish_kernel 4.25
