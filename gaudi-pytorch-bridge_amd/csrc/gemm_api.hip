@@ -52,15 +52,20 @@ __global__ __launch_bounds__(256) void fp8_gemm_simple_kernel(GemmArgs g, int64_
 
 inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// The tiled kernel moves 16-byte chunks: the contiguous dimension of each
-// operand, its leading dimension, batch stride and base address must all be
-// multiples of 16 bytes.
+// The tiled kernels move 16-byte chunks: each operand's leading dimension,
+// batch stride and base address must be multiples of 16 bytes, and so must K
+// where K is an operand's contiguous dimension (a chunk is either all inside K
+// or all outside).  Where m or n is contiguous, the chunk that straddles the
+// extent brings in bytes of the row's padding (ld >= extent rounded up): those
+// columns only feed outputs that are never stored.
+inline bool k_chunks_ok(int trans_a, int trans_b, int64_t K) {
+  return K % 16 == 0 || (trans_a && !trans_b);
+}
 inline bool tiled_ok(const void* A, int trans_a, int64_t lda, const void* B, int trans_b,
                      int64_t ldb, int64_t M, int64_t N, int64_t K, int64_t stride_a,
                      int64_t stride_b) {
   if (!al16(A) || !al16(B) || lda % 16 || ldb % 16 || stride_a % 16 || stride_b % 16) return false;
-  if ((trans_a ? M : K) % 16) return false;
-  if ((trans_b ? K : N) % 16) return false;
+  if (!k_chunks_ok(trans_a, trans_b, K)) return false;
   // a stage of the tiled kernels spans up to 256 rows of ld bytes, addressed with 31-bit offsets
   if (lda > (1LL << 22) || ldb > (1LL << 22)) return false;
   return M > 0 && N > 0 && K > 0;
@@ -74,7 +79,7 @@ extern "C" {
 
 const char* mi355q_fp8_gemm_variant(int trans_a, int64_t lda, int trans_b, int64_t ldb, int64_t M,
                                     int64_t N, int64_t K) {
-  if (lda % 16 || ldb % 16 || (trans_a ? M : K) % 16 || (trans_b ? K : N) % 16) return "simple";
+  if (lda % 16 || ldb % 16 || !mi355q::k_chunks_ok(trans_a, trans_b, K)) return "simple";
   if (M > 128 && N > 128) {
     switch (mi355q::choose_tiles(M, N, 1)) {
       case mi355q::TileChoice::k256x256: return "tile256x256x128_mfma32x32x64";

@@ -222,7 +222,9 @@ struct DmaLoader {
       step = BK;
     } else {
       base += mn0;
-      remaining = (int64_t)(K - 1) * ld + (extent - mn0);
+      // up to the end of the 16-byte chunk that holds the last column (ld is a multiple of 16 and
+      // at least the extent): a chunk that straddles the descriptor's end would read as zero whole
+      remaining = (int64_t)(K - 1) * ld + (((extent + 15) & ~15) - mn0);
       step = (int64_t)BK * ld;
     }
     if (!valid) remaining = 0;

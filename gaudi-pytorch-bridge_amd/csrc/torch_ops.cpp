@@ -446,6 +446,34 @@ Tensor fp8_gemm_v2_impl(const Tensor& A, bool trans_A, const Tensor& B, bool tra
   Tensor out = at::empty(out_shape, A.options().dtype(out_dtype));
   if (out.numel() == 0) return out;
 
+  // The MFMA kernels move 16-byte chunks: they need 16-byte aligned operands and pitches and, where
+  // K is an operand's contiguous dimension, K % 16 == 0; anything else runs on a simple kernel at a
+  // few TFLOP/s.  When the product is large enough for that to cost more than two copies, such
+  // operands go into zero-filled buffers with every extent rounded up to 16 (zeros along K add
+  // nothing to any sum; padding along m or n is never read into a stored output).
+  int64_t lda = ac, ldb = bc, k_call = K;
+  auto misaligned = [](const Tensor& t) { return (reinterpret_cast<uintptr_t>(t.data_ptr()) & 15u) != 0; };
+  const bool k_ragged = K % 16 != 0 && !(ta && !tb);
+  if ((ac % 16 || bc % 16 || k_ragged || misaligned(ac_t) || misaligned(bc_t)) &&
+      (double)M * (double)N * (double)K >= (double)(1 << 26)) {
+    const int64_t kp = (ta && !tb) ? K : (K + 15) / 16 * 16;  // K is contiguous in neither operand: any K
+    auto pad = [&](Tensor& t, int64_t rows, int64_t cols, bool k_is_rows, int64_t* ld, int64_t* stride) {
+      const int64_t rp = k_is_rows ? kp : rows, cp = k_is_rows ? (cols + 15) / 16 * 16 : kp;
+      if (rp == rows && cp == cols && !misaligned(t)) return;
+      std::vector<int64_t> shape = t.sizes().vec();
+      shape[shape.size() - 2] = rp;
+      shape[shape.size() - 1] = cp;
+      Tensor padded = at::zeros(shape, t.options());
+      padded.narrow(-2, 0, rows).narrow(-1, 0, cols).copy_(t);
+      t = padded;
+      *ld = cp;
+      if (*stride != 0) *stride = rp * cp;
+    };
+    pad(ac_t, ar, ac, ta, &lda, &stride_a);    // A is stored [K, M] when transposed
+    pad(bc_t, br, bc, !tb, &ldb, &stride_b);   // B is stored [K, N] unless transposed
+    k_call = kp;
+  }
+
   GemmScale sa = resolve_gemm_scale(A_scale_inv, c10::nullopt, M, N, A, "A_scale_inv");
   GemmScale sb = resolve_gemm_scale(B_scale_inv, B_scale_shape, M, N, A, "B_scale_inv");
 
@@ -475,9 +503,9 @@ Tensor fp8_gemm_v2_impl(const Tensor& A, bool trans_A, const Tensor& B, bool tra
   }
 
   check_status(
-      mi355q_fp8_gemm(ac_t.data_ptr(), to_mi355q_dtype(A.scalar_type()), ta ? 1 : 0, ac,
-                      bc_t.data_ptr(), to_mi355q_dtype(B.scalar_type()), tb ? 1 : 0, bc,
-                      out.data_ptr(), to_mi355q_dtype(out_dtype), N, M, N, K, sa.dev, sa.host, sa.mode,
+      mi355q_fp8_gemm(ac_t.data_ptr(), to_mi355q_dtype(A.scalar_type()), ta ? 1 : 0, lda,
+                      bc_t.data_ptr(), to_mi355q_dtype(B.scalar_type()), tb ? 1 : 0, ldb,
+                      out.data_ptr(), to_mi355q_dtype(out_dtype), N, M, N, k_call, sa.dev, sa.host, sa.mode,
                       sb.dev, sb.host, sb.mode, bias_mode != MI355Q_BIAS_NONE ? bias_t.data_ptr() : nullptr,
                       bias_mode, ldbias, accumulate ? d_t.data_ptr() : nullptr, N, batch, stride_a,
                       stride_b, M * N, stride_d, stride_bias, current_stream(A)),

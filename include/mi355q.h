@@ -209,7 +209,10 @@ int mi355q_dequant_4bit(const int32_t* packed, const void* scale, const void* zp
  *   bias   out_dtype, per mi355q_bias_mode; D: out_dtype [M, N] stride ldd or NULL
  *   batch  number of problems; stride_* are element strides between them
  *          (0 broadcasts an operand)
- * Leading dimensions and batch strides are in elements.
+ * Leading dimensions and batch strides are in elements.  As in BLAS, an
+ * operand is an array of whole rows: where lda (ldb) is a multiple of 16, the
+ * bytes of a row up to the next multiple of 16 past its last element are
+ * read, the last row's included (they never reach a stored output).
  */
 int mi355q_fp8_gemm(const void* A, int fmt_a, int trans_a, int64_t lda,
                     const void* B, int fmt_b, int trans_b, int64_t ldb,

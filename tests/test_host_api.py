@@ -74,6 +74,10 @@ def test_variant_names(pkg):
     lib = pkg.capi()
     assert b"256x256" in lib.mi355q_fp8_gemm_variant(0, 4096, 0, 14336, 8192, 14336, 4096)
     assert lib.mi355q_fp8_gemm_variant(0, 24, 0, 36, 12, 36, 24) == b"simple"
+    # where m or n is the contiguous dimension only the pitch has to be a multiple of 16
+    assert b"simple" not in lib.mi355q_fp8_gemm_variant(0, 1024, 0, 1008, 515, 1001, 1024)
+    assert b"simple" not in lib.mi355q_fp8_gemm_variant(1, 528, 0, 1008, 515, 1001, 1030)   # K contiguous in neither operand
+    assert lib.mi355q_fp8_gemm_variant(0, 1040, 0, 1008, 515, 1001, 1030) == b"simple"       # K contiguous and ragged
 
 
 @pytest.mark.parametrize("key", sorted(REFERENCE_SCHEMAS))
