@@ -50,6 +50,35 @@ def test_graph_replays_match_eager(dev):
             assert torch.equal(a.view(torch.uint8) if a.dtype == E4 else a, b.view(torch.uint8) if b.dtype == E4 else b), rep
 
 
+def test_graph_replays_of_a_ragged_product(dev):
+    """A large product with ragged extents: the operator's zero-padded operand copies (torch's
+    allocator, a fill kernel and a copy kernel) are part of the captured sequence."""
+    g = torch.Generator().manual_seed(3)
+    M, K, N = 333, 1001, 515
+    w8 = torch.randint(-4, 5, (K, N), generator=g).float().to(E4).to(dev)
+    static_a = torch.zeros(M, K, dtype=E4, device=dev)
+    run = lambda a: ops.fp8_gemm_v2(a, False, w8, False, None, torch.float32)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            run(static_a)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = run(static_a)
+    for rep in range(4):
+        a = torch.randint(-4, 5, (M, K), generator=g).float()
+        static_a.copy_(a.to(E4))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        eager = run(a.to(E4).to(dev))       # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager) and torch.equal(got.cpu(), a @ w8.cpu().float()), rep
+
+
 def attention_like(q8, k8, sq, sk):
     """scores = q k^T in fp8, probabilities through softmax_fp8, their row sums through sum_fp8 (split: workspace)."""
     scores = ops.fp8_gemm_v2(q8, False, k8, True, None, torch.bfloat16, sq, sk, None, False)
