@@ -469,7 +469,7 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_kernel(
 #pragma unroll
   for (int w = 1; w < kThreads / 64; ++w) r = r > wave_part[w] ? r : wave_part[w];
   const float amax = __uint_as_float(r);
-  const float scale = target / amax;  // correctly rounded fp32 division, as on the host
+  const float scale = row_scale(target, amax);
   if (threadIdx.x == 0) {
     if (scale_out) scale_out[row] = scale;
     if (scale_inv_out) scale_inv_out[row] = 1.0f / scale;
@@ -548,7 +548,7 @@ __global__ __launch_bounds__(kThreads) void silu_mul_quantize_rows_kernel(
 #pragma unroll
   for (int w = 1; w < kThreads / 64; ++w) r = r > wave_part[w] ? r : wave_part[w];
   const float amax = __uint_as_float(r);
-  const float scale = target / amax;
+  const float scale = row_scale(target, amax);
   if (threadIdx.x == 0) {
     if (scale_out) scale_out[row] = scale;
     if (scale_inv_out) scale_inv_out[row] = 1.0f / scale;

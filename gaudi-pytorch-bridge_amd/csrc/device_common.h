@@ -17,6 +17,19 @@ typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 
 constexpr float kFp8Max[2] = {448.0f, 57344.0f};  // e4m3fn, e5m2
 
+// Dynamic per-row quantisation computes scale = target / amax.  A row of zeros
+// (amax 0) or of values so small that the quotient overflows would give an
+// infinite scale, and 0 * inf = NaN would turn every zero of the row into an
+// fp8 NaN.  The scale is therefore capped at the largest finite bf16 value
+// (0x7f7f0000; finite in fp32 and after the rounding to bf16 that a bf16 input
+// applies to it): a zero row then gives zero codes and a finite 1 / scale.  A
+// NaN amax (a NaN in the row) compares false and stays NaN.
+constexpr float kRowScaleCap = 3.3895313892515355e38f;
+__device__ __forceinline__ float row_scale(float target, float amax) {
+  const float s = target / amax;  // correctly rounded fp32 division, as on the host
+  return s > kRowScaleCap ? kRowScaleCap : s;
+}
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
 // fp32 -> bf16 round-to-nearest-even (v_cvt_pk_bf16_f32), returned as fp32.

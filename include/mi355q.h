@@ -92,7 +92,10 @@ int mi355q_rowwise_amax(const void* x, int x_dtype, int64_t rows, int64_t cols,
 
 /*
  * Dynamic per-row ("per-token") quantisation in one pass over x [rows, cols]:
- *   amax_r = max|x[r, :]|, scale_r = target / amax_r (fp32 division),
+ *   amax_r = max|x[r, :]|, scale_r = min(target / amax_r, 0x1.fep127f) (fp32 division; the cap,
+ *   the largest finite bf16 value, only acts on a row of zeros or of values below
+ *   target / 3.4e38: such a row gets zero (or saturated) codes and a finite 1 / scale_r
+ *   instead of the NaN codes that 0 * inf would give; a NaN in the row makes scale_r NaN),
  *   y[r, :] = cast_to_fp8(x[r, :] * scale_r)   with the rounding rules of mi355q_cast_to_fp8,
  *   scale_out[r] = scale_r, scale_inv_out[r] = 1 / scale_r   (either may be NULL).
  * Bit-identical to mi355q_rowwise_amax, the division on the host side and

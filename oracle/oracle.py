@@ -29,6 +29,7 @@ SCALE_NONE, SCALE_HOST, SCALE_DEV, SCALE_MID, SCALE_FULL = 0, 1, 2, 3, 4
 _DT = {torch.float32: F32, torch.bfloat16: BF16,
        torch.float8_e4m3fn: E4M3FN, torch.float8_e5m2: E5M2}
 FP8_MAX = {torch.float8_e4m3fn: 448.0, torch.float8_e5m2: 57344.0}
+ROW_SCALE_CAP = 3.3895313892515355e38   # 0x7f7f0000, the largest finite bf16
 
 
 def build(force=False):
@@ -322,6 +323,9 @@ def quantize_rows(x, out_dtype):
     amax = x2.abs().amax(dim=-1, keepdim=True).float()
     # tensor / tensor is an IEEE division; torch evaluates scalar / tensor as scalar * (1 / tensor)
     scale = torch.full_like(amax, FP8_MAX[out_dtype]) / amax
+    # capped at the largest finite bf16 value: a row of zeros (amax 0, quotient inf) would otherwise turn
+    # into NaN codes through 0 * inf; a NaN amax stays NaN (the comparison is false)
+    scale = torch.where(scale > ROW_SCALE_CAP, torch.full_like(scale, ROW_SCALE_CAP), scale)
     y, _ = c_cast_to_fp8(x2, scale.reshape(-1), out_dtype, scale_shape=[x2.shape[0], 1])
     return y.reshape(x.shape), (torch.ones_like(scale) / scale).reshape(x.shape[:-1] + (1,))
 

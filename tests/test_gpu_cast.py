@@ -279,6 +279,40 @@ def test_quantize_rows(oracle, pkg, dev, dtype, shape, out_dtype):
     assert_fp8_equal(y.reshape(x2.shape), y3.cpu(), out_dtype, "vs the three GPU steps")
 
 
+@pytest.mark.parametrize("out_dtype", FP8_DTYPES)
+@pytest.mark.parametrize("dtype,cols", [
+    (torch.bfloat16, 4096),    # the one-pass kernel
+    (torch.bfloat16, 100),     # not whole vectors: rowwise_amax, the division and cast_to_fp8 with per-row scales
+    (torch.float32, 1024),
+    (torch.float32, 1022),
+])
+def test_quantize_rows_zero_and_tiny_rows(oracle, dev, dtype, cols, out_dtype):
+    """Rows of zeros (padding tokens) among ordinary rows: zero codes and a finite 1 / scale, never the
+    NaN codes of 0 * inf; a row whose amax makes fp8_max / amax overflow is quantised with the capped
+    scale; both on the fused kernel and on the three-step route, bit for bit as the oracle."""
+    g = torch.Generator().manual_seed(cols)
+    x = torch.randn(12, cols, generator=g) * 2
+    x[0] = 0
+    x[5] = 0
+    x[5, 3] = -0.0
+    x[7] = 0
+    x[7, 1] = 1e-38
+    x[7, 9] = -3e-39
+    x[11] = 0
+    x = x.to(dtype)
+    y, s_inv = torch.ops.mi355q.quantize_rows(x.to(dev), out_dtype)
+    ref, s_ref = oracle.quantize_rows(x, out_dtype)
+    assert_fp8_equal(y, ref, out_dtype)
+    assert torch.equal(s_inv.cpu(), s_ref)
+    assert torch.isfinite(s_inv).all() and not torch.isnan(y.float()).any()
+    assert (y.cpu().view(torch.uint8)[[0, 5, 11]] & 0x7F).eq(0).all()
+    # a GEMM fed with the zero rows gives zeros there, not NaN
+    w = torch.randint(-3, 4, (cols // 16 * 16, 32), generator=g).float().to(E4)
+    if cols % 16 == 0:
+        out = ops.fp8_gemm_v2(y, False, w.to(dev), False, None, torch.bfloat16, s_inv)
+        assert torch.isfinite(out.float()).all() and out[[0, 5, 11]].float().abs().max().item() == 0.0
+
+
 def test_quantize_rows_c_abi(oracle, pkg, dev):
     lib = pkg.capi()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)

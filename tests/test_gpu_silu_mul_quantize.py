@@ -49,6 +49,23 @@ def test_against_oracle(oracle, dev, shape, out_dtype):
     assert torch.equal(s_inv.cpu(), ref_s)
 
 
+def test_zero_rows(oracle, dev):
+    """SiLU(gate) * up rows that are all zero (up = 0, or gate = 0) among ordinary rows: zero codes
+    and a finite 1 / scale as the oracle gives them, no NaN."""
+    gen = torch.Generator().manual_seed(4)
+    g = (torch.randn(9, 2048, generator=gen) * 3).bfloat16()
+    u = torch.randn(9, 2048, generator=gen).bfloat16()
+    u[0] = 0
+    g[4] = 0
+    u[8] = 0
+    for out_dtype in FP8_DTYPES:
+        y, s_inv = torch.ops.mi355q.silu_mul_quantize_rows(g.to(dev), u.to(dev), out_dtype)
+        ref_y, ref_s = oracle.quantize_rows(oracle.c_silu_mul_bf16(g, u), out_dtype)
+        assert same_codes(y, ref_y) and torch.equal(s_inv.cpu(), ref_s)
+        assert torch.isfinite(s_inv).all() and not torch.isnan(y.float()).any()
+        assert (y.cpu().view(torch.uint8)[[0, 4, 8]] & 0x7F).eq(0).all()
+
+
 def test_halves_of_one_wide_matrix(oracle, dev):
     """gate and up as column ranges of one [T, 2 ff] GEMM output (row pitch 2 ff)."""
     gen = torch.Generator().manual_seed(9)

@@ -204,3 +204,38 @@ def test_scale_forms_agree(oracle, out_dtype, axis):
     assert_bits_equal(back, expect * vals.reciprocal().unsqueeze(axis).to(torch.bfloat16), "per-channel round trip")
     with pytest.raises(ValueError, match="is not equal to number of scale_shape elements"):
         oracle.c_cast_to_fp8(x, vals, out_dtype, scale_shape=[3, 1])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("out_dtype", FP8_DTYPES)
+def test_quantize_rows_of_zero_and_tiny_rows(oracle, dtype, out_dtype):
+    """Dynamic per-row quantisation caps scale = fp8_max / amax at the largest finite bf16 value:
+    a row of zeros gives zero codes (not the NaN of 0 * inf) and a finite, non-zero 1 / scale, a row
+    whose amax is so small that the quotient overflows is quantised with the cap, every other row is
+    untouched by the cap, and a row holding a NaN keeps a NaN scale."""
+    x = torch.zeros(6, 64, dtype=dtype)
+    x[1] = torch.linspace(-3, 3, 64).to(dtype)
+    x[2, 5] = 1e-38            # 448 / 1e-38 overflows fp32
+    x[2, 6] = -5e-39
+    x[3, ::2] = 2.5
+    x[4, 7] = float("nan")
+    x[5, 0] = -0.0
+    y, s_inv = oracle.quantize_rows(x, out_dtype)
+    codes = y.view(torch.uint8)
+    assert torch.equal(codes[0], torch.zeros(64, dtype=torch.uint8))
+    assert (codes[5] & 0x7F).eq(0).all()
+    cap = oracle.ROW_SCALE_CAP
+    assert cap == torch.tensor([0x7F7F0000], dtype=torch.int32).view(torch.float32).item()
+    assert torch.isfinite(s_inv[[0, 2, 5]]).all() and (s_inv[[0, 2, 5]] > 0).all()
+    assert s_inv[0, 0].item() == (torch.ones(()) / torch.tensor(cap)).item()
+    # the capped row: x * cap, saturating, with cast_to_fp8_v2's rounding
+    ref2, _ = oracle.c_cast_to_fp8(x[2:3], torch.tensor(cap), out_dtype)
+    assert_fp8_equal(y[2:3], ref2, out_dtype)
+    assert not torch.isnan(y[2].float()).any() and y[2].float().abs().max() > 0
+    # ordinary rows: exactly fp8_max / amax
+    mx = oracle.FP8_MAX[out_dtype]
+    for r in (1, 3):
+        amax = x[r].abs().max().float()
+        assert s_inv[r, 0].item() == (torch.ones(()) / (torch.tensor(mx) / amax)).item()
+        assert y[r].float().abs().max().item() == mx
+    assert torch.isnan(s_inv[4]).all()
