@@ -474,8 +474,36 @@ Tensor fp8_gemm_v2_impl(const Tensor& A, bool trans_A, const Tensor& B, bool tra
     k_call = kp;
   }
 
-  GemmScale sa = resolve_gemm_scale(A_scale_inv, c10::nullopt, M, N, A, "A_scale_inv");
+  // A [..., M, K] times one matrix B is one product over all batch * M rows: B is streamed once
+  // and the rows fill the kernels' tiles, where batch separate problems would each re-read B with
+  // M rows only (a [64, 1, K] decode activation against [K, N] weights would be 64 one-row products).
+  const bool can_flatten = batch > 1 && stride_b == 0 && stride_a != 0 && !ta;
+  // Per-row scales that cover the batch as well ([..., M, 1], what quantize_rows returns for a
+  // batched activation) are per-row scales of the flattened product.
+  auto batched_rows = [&](const IValue& sc) {
+    if (!can_flatten || !sc.isTensor()) return false;
+    const Tensor& t = sc.toTensor();
+    if (t.numel() != batch * M || t.numel() == 1 || t.dim() != (int64_t)batch_shape.size() + 2) return false;
+    for (size_t i = 0; i < batch_shape.size(); ++i)
+      if (t.size(i) != batch_shape[i]) return false;
+    return t.size(-2) == M && t.size(-1) == 1;
+  };
+  const bool sa_batched = batched_rows(A_scale_inv);
+  GemmScale sa = sa_batched ? resolve_gemm_scale(A_scale_inv, std::vector<int64_t>{batch * M, 1}, batch * M, N, A, "A_scale_inv")
+                            : resolve_gemm_scale(A_scale_inv, c10::nullopt, M, N, A, "A_scale_inv");
   GemmScale sb = resolve_gemm_scale(B_scale_inv, B_scale_shape, M, N, A, "B_scale_inv");
+  int64_t m_call = M, batch_call = batch;
+  if (can_flatten) {
+    // [M] scales shared by every batch element are repeated per batch element
+    auto repeat_rows = [&](GemmScale& g) {
+      g.holder = g.holder.reshape({1, M}).expand({batch, M}).contiguous();
+      g.dev = g.holder.data_ptr<float>();
+    };
+    if (sa.mode == MI355Q_GS_PER_ROW && !sa_batched) repeat_rows(sa);
+    if (sb.mode == MI355Q_GS_PER_ROW) repeat_rows(sb);
+    m_call = batch * M;
+    batch_call = 1;
+  }
 
   std::vector<int64_t> full_out = batch_shape;
   full_out.push_back(M);
@@ -505,9 +533,9 @@ Tensor fp8_gemm_v2_impl(const Tensor& A, bool trans_A, const Tensor& B, bool tra
   check_status(
       mi355q_fp8_gemm(ac_t.data_ptr(), to_mi355q_dtype(A.scalar_type()), ta ? 1 : 0, lda,
                       bc_t.data_ptr(), to_mi355q_dtype(B.scalar_type()), tb ? 1 : 0, ldb,
-                      out.data_ptr(), to_mi355q_dtype(out_dtype), N, M, N, k_call, sa.dev, sa.host, sa.mode,
+                      out.data_ptr(), to_mi355q_dtype(out_dtype), N, m_call, N, k_call, sa.dev, sa.host, sa.mode,
                       sb.dev, sb.host, sb.mode, bias_mode != MI355Q_BIAS_NONE ? bias_t.data_ptr() : nullptr,
-                      bias_mode, ldbias, accumulate ? d_t.data_ptr() : nullptr, N, batch, stride_a,
+                      bias_mode, ldbias, accumulate ? d_t.data_ptr() : nullptr, N, batch_call, stride_a,
                       stride_b, M * N, stride_d, stride_bias, current_stream(A)),
       "mi355q_fp8_gemm");
   return out;
@@ -914,7 +942,8 @@ std::tuple<Tensor, Tensor> quantize_rows_op(const Tensor& x, at::ScalarType dtyp
                                       current_stream(c));
   if (st == MI355Q_ERR_UNSUPPORTED) {
     Tensor amax = rowwise_amax_op(c).reshape(shp);
-    Tensor scale = at::div(at::full_like(amax, target), amax);
+    // capped like the kernel's row_scale (largest finite bf16): a zero row gets zero codes, not NaN
+    Tensor scale = at::clamp_max(at::div(at::full_like(amax, target), amax), 3.3895313892515355e38);
     check_status(mi355q_cast_to_fp8(c.data_ptr(), to_mi355q_dtype(c.scalar_type()), out.data_ptr(),
                                     to_mi355q_dtype(dtype), scale.data_ptr<float>(), 0.0f, MI355Q_SCALE_MID,
                                     1, rows, cols, nullptr, current_stream(c)),
