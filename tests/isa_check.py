@@ -142,7 +142,7 @@ def memory_order(text):
 def compile_to_isa(source, extra_flags=()):
     """Device-only assembly of one HIP source of csrc/ with the build's flags."""
     import importlib.util  # noqa: PLC0415
-    spec = importlib.util.spec_from_file_location("_mi355q_build_flags", os.path.join(HERE, "build.py"))
+    spec = importlib.util.spec_from_file_location("_mi355q_build_flags", os.path.join(os.path.dirname(HERE), "gaudi-pytorch-bridge_amd", "build.py"))
     build = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(build)
     HIPCC_FLAGS, CSRC = build.HIPCC_FLAGS, build.CSRC

@@ -9,7 +9,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 _spec = importlib.util.spec_from_file_location(
-    "mi355q_isa_check", os.path.join(ROOT, "gaudi-pytorch-bridge_amd", "isa_check.py"))
+    "mi355q_isa_check", os.path.join(ROOT, "tests", "isa_check.py"))
 isa_check = importlib.util.module_from_spec(_spec)
 _spec.loader.exec_module(isa_check)
 
