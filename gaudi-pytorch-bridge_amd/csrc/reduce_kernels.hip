@@ -4,6 +4,8 @@
 // through buffer descriptors that end with the row or block they cover, so the
 // bodies have no divergent branch around a load and every lane's loads are in
 // flight before the first is used (see cast_kernels.hip).
+#include <mutex>
+
 #include "device_common.h"
 
 namespace mi355q {
@@ -490,6 +492,36 @@ int softmax_launch(const SoftmaxArgs& a, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
 }
 
+// ------------------------------------------- sum_fp8 without a caller's workspace
+//
+// The partial sums of a split reduction live in this file-scope device array instead of
+// a workspace the caller allocates.  Every GPU the library runs on holds its own copy
+// until the process ends.  In host code the array's name is only a handle: the device
+// address is asked for once per device (hipGetSymbolAddress) and that pointer is what the
+// kernels get, exactly as they get a caller's workspace.
+static __device__ __align__(256) unsigned char sum_scratch[MI355Q_SUM_FP8_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static std::mutex sum_scratch_mutex;
+static void* sum_scratch_ptr[kMaxDevices];  // device address of sum_scratch, per device
+
+// Address of the current device's copy of sum_scratch (looked up on the first call per device).
+inline int sum_scratch_of_current_device(float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MI355Q_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(sum_scratch_mutex);
+  if (sum_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(sum_scratch)) != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      return MI355Q_ERR_LAUNCH;
+    }
+    sum_scratch_ptr[dev] = p;
+  }
+  *out = static_cast<float*>(sum_scratch_ptr[dev]);
+  return MI355Q_OK;
+}
+
 }  // namespace mi355q
 
 using namespace mi355q;
@@ -520,6 +552,27 @@ int mi355q_sum_fp8(const void* x, int fp8_fmt, int64_t outer, int64_t reduce, in
   // an empty reduction gives zeros: the kernels' loops do not run and store 0
   if (fp8_fmt == MI355Q_E4M3FN) return sum_fp8_launch<MI355Q_E4M3FN>(xb, outer, reduce, inner, out, out_dtype, ws, workspace_bytes, st);
   return sum_fp8_launch<MI355Q_E5M2>(xb, outer, reduce, inner, out, out_dtype, ws, workspace_bytes, st);
+}
+
+int mi355q_sum_fp8_static(const void* x, int fp8_fmt, int64_t outer, int64_t reduce, int64_t inner, void* out,
+                          int out_dtype, void* stream) {
+  if (fp8_fmt != MI355Q_E4M3FN && fp8_fmt != MI355Q_E5M2) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (out_dtype < MI355Q_F32 || out_dtype > MI355Q_E5M2) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (outer < 0 || reduce < 0 || inner < 0) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (outer == 0 || inner == 0) return MI355Q_OK;
+  if (out == nullptr || (reduce > 0 && x == nullptr)) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (mi355q_sum_fp8_workspace_bytes(outer, reduce, inner) > (size_t)MI355Q_SUM_FP8_STATIC_SCRATCH_BYTES)
+    return MI355Q_ERR_TOO_LARGE;
+  float* ws = nullptr;
+  const int got = sum_scratch_of_current_device(&ws);
+  if (got != MI355Q_OK) return got;
+  // Nothing has to be cleared between calls: every slice writes its partial sum of every
+  // output before sum_finish_kernel, ordered behind it on the stream, reads them.
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint8_t* xb = static_cast<const uint8_t*>(x);
+  if (fp8_fmt == MI355Q_E4M3FN)
+    return sum_fp8_launch<MI355Q_E4M3FN>(xb, outer, reduce, inner, out, out_dtype, ws, MI355Q_SUM_FP8_STATIC_SCRATCH_BYTES, st);
+  return sum_fp8_launch<MI355Q_E5M2>(xb, outer, reduce, inner, out, out_dtype, ws, MI355Q_SUM_FP8_STATIC_SCRATCH_BYTES, st);
 }
 
 int mi355q_softmax_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols, const float* input_scale_dev,

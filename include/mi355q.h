@@ -26,7 +26,9 @@ typedef enum {
   MI355Q_ERR_INVALID_ARGUMENT = 1, /* null pointer, bad enum, negative size */
   MI355Q_ERR_UNSUPPORTED = 2,      /* valid request this build has no kernel for */
   MI355Q_ERR_LAUNCH = 3,           /* hipLaunchKernel reported an error */
-  MI355Q_ERR_WORKSPACE = 4         /* workspace missing or too small */
+  MI355Q_ERR_WORKSPACE = 4,        /* workspace missing or too small */
+  MI355Q_ERR_TOO_LARGE = 5         /* problem needs more than the fixed scratch buffer of an
+                                      allocation-free entry point */
 } mi355q_status;
 
 typedef enum {
@@ -242,6 +244,23 @@ int mi355q_fp8_gemm(const void* A, int fmt_a, int trans_a, int64_t lda,
 size_t mi355q_sum_fp8_workspace_bytes(int64_t outer, int64_t reduce, int64_t inner);
 int mi355q_sum_fp8(const void* x, int fp8_fmt, int64_t outer, int64_t reduce, int64_t inner,
                    void* out, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * mi355q_sum_fp8 for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same arguments without the
+ * workspace, same kernels, same results bit for bit.  It has no counterpart in the reference.
+ * The partial sums of a split reduction go to a fixed buffer of
+ * MI355Q_SUM_FP8_STATIC_SCRATCH_BYTES inside the library's device image (one copy per GPU,
+ * held until the process ends); a problem whose mi355q_sum_fp8_workspace_bytes(...) exceeds
+ * that returns MI355Q_ERR_TOO_LARGE and launches nothing.  The call allocates and frees
+ * nothing.  The stream's device must be the current device.  All calls on one GPU share the
+ * buffer: calls that may overlap on one GPU (different streams) race; calls on one stream,
+ * or ordered by events, do not.  The first call on a device looks the buffer's address up
+ * (hipGetSymbolAddress, once per device): make it before a graph capture starts.
+ */
+#define MI355Q_SUM_FP8_STATIC_SCRATCH_BYTES (2u << 20)
+int mi355q_sum_fp8_static(const void* x, int fp8_fmt, int64_t outer, int64_t reduce, int64_t inner,
+                          void* out, int out_dtype, void* stream);
 
 /*
  * Softmax over the rows of x [rows, cols] (bf16 or e4m3fn):
