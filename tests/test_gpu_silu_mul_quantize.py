@@ -35,8 +35,44 @@ def test_silu_bits_on_every_bf16_value(oracle, pkg, dev):
         assert torch.equal(h.cpu().view(torch.int16)[~nan], ref.view(torch.int16)[~nan])
 
 
+@pytest.mark.parametrize("cols", [2048, 8192])
+def test_table_kernel_on_every_bf16_value(oracle, pkg, dev, cols):
+    """From 2048 rows on, bf16(silu(gate)) comes from a table in LDS with range fix-ups outside it:
+    every one of the 65536 gate values, in every lane position, against the oracle (h_out, codes and
+    scales); rows of zeros and a ragged last workgroup share included."""
+    lib = pkg.capi()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rows = 2048 + 7
+    gen = torch.Generator().manual_seed(cols)
+    g = ALL[torch.randperm(65536, generator=gen)].repeat(-(-rows * cols // 65536))[: rows * cols].reshape(rows, cols).clone()
+    # NaN, -inf and gates whose product overflows make a row's scale NaN: keep them to the first 64 rows
+    bad = torch.isnan(g.float()) | torch.isinf(g.float()) | (g.float().abs() > 1e30)
+    bad[:64] = False
+    g[bad] = 0.75
+    u = torch.randn(rows, cols, generator=gen).bfloat16()
+    u[5] = 0
+    u[:, ::3] = 1.0
+    gd, ud = g.to(dev), u.to(dev)
+    y = torch.empty(g.shape, dtype=E4, device=dev)
+    h = torch.empty(g.shape, dtype=torch.bfloat16, device=dev)
+    si = torch.empty(rows, device=dev)
+    assert lib.mi355q_silu_mul_quantize_rows(gd.data_ptr(), cols, ud.data_ptr(), cols, rows, cols, y.data_ptr(),
+                                             pkg.E4M3FN, 448.0, h.data_ptr(), None, si.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    ref = oracle.c_silu_mul_bf16(g, u)
+    nan = torch.isnan(ref.float())
+    assert torch.equal(torch.isnan(h.cpu().float()), nan)
+    assert torch.equal(h.cpu().view(torch.int16)[~nan], ref.view(torch.int16)[~nan])
+    # rows without a NaN: codes and scales as the oracle's
+    clean = ~nan.any(dim=1)
+    assert clean.sum() > 100
+    ref_y, ref_s = oracle.quantize_rows(ref[clean], E4)
+    assert same_codes(y.cpu()[clean], ref_y)
+    assert torch.equal(si.cpu()[clean], ref_s.reshape(-1))
+
+
 @pytest.mark.parametrize("out_dtype", FP8_DTYPES)
-@pytest.mark.parametrize("shape", [(64, 1024), (33, 2048), (5, 14336), (3, 8), (16, 16384)])
+@pytest.mark.parametrize("shape", [(64, 1024), (33, 2048), (5, 14336), (3, 8), (16, 16384), (2050, 1032), (2048, 14336)])
 def test_against_oracle(oracle, dev, shape, out_dtype):
     gen = torch.Generator().manual_seed(shape[0] * 131 + shape[1])
     g = (torch.randn(*shape, generator=gen) * 3).bfloat16()
