@@ -50,6 +50,9 @@ __global__ __launch_bounds__(kSkThreads) void fp8_gemm_skinny_kernel(GemmArgs g)
   LB lb;
   la.init(g.A + batch * g.stride_a, g.lda, 0, g.M, g.K);
   lb.init(g.B + batch * g.stride_b, g.ldb, n0, g.N, g.K);
+  // rows of the tiles past M or N: loads that go to memory (see DmaLoader::clamp_rows)
+  if constexpr (A_KMAJOR) la.clamp_rows(g.lda, g.M);
+  if constexpr (B_KMAJOR) lb.clamp_rows(g.ldb, g.N - n0);
   f32x16 acc[MT][1];
 #pragma unroll
   for (int i = 0; i < MT; ++i)
@@ -62,7 +65,9 @@ __global__ __launch_bounds__(kSkThreads) void fp8_gemm_skinny_kernel(GemmArgs g)
   // k at the same time send their requests, which differ only in high address
   // bits, to the same few memory channels.  (With B MN-major the strips of one
   // k row are contiguous in memory and walking in step is the better order.)
-  const int first = B_KMAJOR ? (int)(((int64_t)blockIdx.x * KT) / gridDim.x) : 0;
+  // (Not with an MN-major A and a ragged K: the stage that holds the K tail then has loads that
+  // fall outside A's descriptor altogether, and the counted waits below need it to be the last.)
+  const int first = (B_KMAJOR && (A_KMAJOR || g.K % kBK == 0)) ? (int)(((int64_t)blockIdx.x * KT) / gridDim.x) : 0;
   int at = 0;  // the stage the loaders' descriptors point at
   // Issues the loads of the i-th stage in walking order; beyond the KT-th they
   // fall outside the descriptors and arrive as zeros, so that every step issues
@@ -76,11 +81,21 @@ __global__ __launch_bounds__(kSkThreads) void fp8_gemm_skinny_kernel(GemmArgs g)
       lb.seek(at, stage);
       at = stage;
     }
-    static_for<LA::kPerWave>([&](auto ic) { la.template issue_one<decltype(ic)::value>(lds + off, stage * kBK, g.K); });
-    static_for<LB::kPerWave>([&](auto ic) { lb.template issue_one<decltype(ic)::value>(lds + off + BM * kBK, stage * kBK, g.K); });
+    static_for<LA::kPerWave>([&](auto ic) { la.template issue_one<decltype(ic)::value, A_KMAJOR>(lds + off, stage * kBK, g.K); });
+    static_for<LB::kPerWave>([&](auto ic) { lb.template issue_one<decltype(ic)::value, B_KMAJOR>(lds + off + BM * kBK, stage * kBK, g.K); });
     la.advance();
     lb.advance();
     ++at;
+  };
+
+  // waits until at most min(later, S - 2) stages' loads of this wave are outstanding
+  auto wait_for_stage = [&](int later) {
+    static_for<S - 1>([&](auto sc) {
+      constexpr int n = decltype(sc)::value;  // 0 .. S - 2
+      constexpr int cnt = n * kOps;
+      if (later == n || (n == S - 2 && later > n) || (n == 0 && later < 0))
+        __builtin_amdgcn_s_waitcnt((cnt & 15) | ((cnt >> 4) << 14) | 0x0070);
+    });
   };
 
   // stages 0 .. S-2 (in walking order) go out first
@@ -90,8 +105,12 @@ __global__ __launch_bounds__(kSkThreads) void fp8_gemm_skinny_kernel(GemmArgs g)
   int rd_off = 0;                        // buffer of stage kt
   int wr_off = (S - 1) * kStageBytes;    // buffer of stage kt + S - 1 (the one stage kt - 1 used)
   for (int kt = 0; kt < KT; ++kt) {
-    // this wave's part of stage kt has landed once only the later stages' loads are outstanding
-    __builtin_amdgcn_s_waitcnt((kInFlight & 15) | ((kInFlight >> 4) << 14) | 0x0070);
+    // This wave's part of stage kt has landed once only the loads of the later stages are
+    // outstanding: the counter retires loads that go to memory in issue order.  A load whose
+    // lanes are all out of range completes at once, ahead of older ones, so it must not be
+    // counted.  Such loads are those of the stages past K and, in the last stage, of k rows
+    // (MN-major) past K: towards the end only the stages up to KT - 2 are counted.
+    wait_for_stage(KT - 2 - kt);
     __syncthreads();  // everyone's part has; and everyone is done with the buffer of stage kt - 1
     issue_stage(wr_off, kt + S - 1);
     const uint8_t* st = lds + rd_off;

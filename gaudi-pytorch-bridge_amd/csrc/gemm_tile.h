@@ -207,6 +207,20 @@ struct DmaLoader {
     region_step = kStored * kRowsPerRegion * (int)ld;
   }
 
+  // For kernels that count their outstanding loads (K-major operands): tile rows from
+  // rows_valid on are fetched from the last valid row instead of falling outside the
+  // descriptor.  Their products are never stored, so what they hold does not matter; but a
+  // load whose lanes are all out of range completes at once, ahead of older loads, while one
+  // that goes to memory retires in issue order, which is what a counted wait relies on.
+  int last_row_off = 0, first_row = 0, rows_valid = 0x7fffffff;
+  __device__ __forceinline__ void clamp_rows(int64_t ld, int valid) {
+    static_assert(KMAJOR, "rows of an MN-major tile are K");
+    const int lane = lane_id_here();
+    first_row = wave * kPerWave * kRowsPerRegion + lane / kCPR;
+    rows_valid = valid;
+    last_row_off = (valid - 1) * (int)ld;
+  }
+
   __device__ __forceinline__ void set_records() {
     const int64_t r = remaining < 0 ? 0 : (remaining > kMaxRecords ? kMaxRecords : remaining);
     rsrc[2] = __builtin_amdgcn_readfirstlane((int)(uint32_t)r);
@@ -242,12 +256,13 @@ struct DmaLoader {
 
   // Issues load I of this wave's share of the stage the descriptor points at,
   // which starts at k0.
-  template <int I>
+  template <int I, bool CLAMP_ROWS = false>
   __device__ __forceinline__ void issue_one(uint8_t* lds_tile, int k0, int K) const {
     const uint32_t lds_base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)lds_tile;
     {
       constexpr int i = I;
       int vo = voff[i % kStored] + (i / kStored) * region_step;
+      if constexpr (CLAMP_ROWS) vo = (first_row + i * kRowsPerRegion < rows_valid) ? vo : last_row_off + kc[i % kStored];
       if constexpr (KMAJOR) vo = (k0 + kc[i % kStored] < K) ? vo : 0x7fffffff;
       const uint32_t dst = lds_base + (uint32_t)((wave * kPerWave + i) * 1024);
       // m0 holds the LDS address of the region; lane l's 16 bytes land at m0 + 16 l.
@@ -1099,7 +1114,9 @@ __global__ __launch_bounds__(kWavesM * WN * 64) void fp8_gemm_tile_kernel(GemmAr
     for (int kt = 2; kt < KT2; kt += 2) k_step(std::false_type{}, kt);
     if (FAST_ONLY || g.fast_epi) {
       epilogue_bf16_fast_any<MT, NT, true, !FAST_ONLY>(g, batch, core.acc, m0 + wm, n0 + wn, stage, scalars);
-      stores_pending = true;
+      // A store whose lanes are all past M or N completes at once and must not be counted as
+      // outstanding: after a tile on the matrix edge the next tile waits for everything.
+      stores_pending = m0 + BM <= g.M && n0 + BN <= g.N;
     } else {
       epilogue<MT, NT>(g, batch, core.acc, m0 + wm, n0 + wn, stage);
     }
