@@ -66,6 +66,8 @@ def capi():
     L.mi355q_fp8_gemm.argtypes = [vp, i32, i32, i64, vp, i32, i32, i64, vp, i32, i64,
                                   i64, i64, i64, vp, f32, i32, vp, f32, i32,
                                   vp, i32, i64, vp, i64, i64, i64, i64, i64, i64, i64, vp]
+    L.mi355q_w4a8_gemm.argtypes = [vp, i32, i64, vp, i64, vp, i32, vp, i32, i64, vp, i32, i64, i64, i64, i64,
+                                   vp, f32, i32, vp, vp]
     L.mi355q_fp8_gemm_variant.argtypes = [i32, i64, i32, i64, i64, i64, i64]
     L.mi355q_sum_fp8_workspace_bytes.argtypes = [i64, i64, i64]
     L.mi355q_sum_fp8_workspace_bytes.restype = c.c_size_t
@@ -74,7 +76,7 @@ def capi():
     L.mi355q_softmax_fp8.argtypes = [vp, i32, i64, i64, vp, f32, vp, f32, vp, f32, vp, i32, vp, vp, vp, i32, vp]
     L.mi355q_fp8_gemm_variant.restype = c.c_char_p
     for name in ("mi355q_amax", "mi355q_rowwise_amax", "mi355q_quantize_rows", "mi355q_silu_mul_quantize_rows", "mi355q_cast_to_fp8", "mi355q_cast_to_fp8_sr", "mi355q_cast_to_fp8_hybrid", "mi355q_cast_from_fp8",
-                 "mi355q_dequant_4bit", "mi355q_fp8_gemm", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8"):
+                 "mi355q_dequant_4bit", "mi355q_fp8_gemm", "mi355q_w4a8_gemm", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8"):
         getattr(L, name).restype = i32
     L._typed = True
     return L
@@ -90,7 +92,7 @@ ZP_NONE, ZP_FLOAT, ZP_PACKED = 0, 1, 2
 EXPORTED_SYMBOLS = (
     "mi355q_abi_version", "mi355q_status_string", "mi355q_amax", "mi355q_rowwise_amax",
     "mi355q_quantize_rows", "mi355q_silu_mul_quantize_rows", "mi355q_cast_to_fp8", "mi355q_cast_to_fp8_sr", "mi355q_cast_to_fp8_hybrid", "mi355q_cast_from_fp8", "mi355q_dequant_4bit", "mi355q_fp8_gemm",
-    "mi355q_fp8_gemm_variant", "mi355q_sum_fp8_workspace_bytes", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8",
+    "mi355q_w4a8_gemm", "mi355q_fp8_gemm_variant", "mi355q_sum_fp8_workspace_bytes", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8",
 )
 
 _load()

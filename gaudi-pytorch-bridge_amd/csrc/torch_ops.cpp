@@ -724,6 +724,71 @@ Tensor convert_from_uint4(const Tensor& input, const Tensor& scale,
   return convert_from_int4_common("convert_from_uint4", false, input, scale, zero_point, out_dtype);
 }
 
+// ---------------------------------------------------------------- w4a8_gemm
+//
+// Fused int4-dequant GEMM: fp8 activations [..., K] times the packed 4-bit weights that
+// hpu::convert_from_int4 / convert_from_uint4 take (int4_ops.cpp:40-56), without the bf16 [K, N]
+// matrix in between.  out = out_dtype((A @ ((q - z) * s)) * A_scale_inv + bias).  The reference has no
+// fused op; shapes the kernel does not take raise (there is no second route to the same bits).
+Tensor w4a8_gemm(const Tensor& A, const Tensor& packed, const Tensor& scale, const c10::optional<Tensor>& zero_point,
+                 bool is_signed, at::ScalarType out_dtype, const c10::optional<Tensor>& A_scale_inv,
+                 const c10::optional<Tensor>& bias) {
+  TORCH_CHECK(is_fp8(A.scalar_type()), "mi355q::w4a8_gemm A must be float8_e4m3fn or float8_e5m2, got ", A.scalar_type());
+  TORCH_CHECK(packed.scalar_type() == at::kInt && packed.dim() == 2,
+              "mi355q::w4a8_gemm packed weights must be a 2-D int32 tensor [K, N / 8], got ", packed.scalar_type(), " ", packed.sizes());
+  TORCH_CHECK(out_dtype == at::kFloat || out_dtype == at::kBFloat16, "mi355q::w4a8_gemm out_dtype must be float or bfloat16, got ", out_dtype);
+  TORCH_CHECK(A.dim() >= 1, "mi355q::w4a8_gemm A must have at least 1 dimension");
+  const int64_t K = packed.size(0), N = packed.size(1) * 8;
+  TORCH_CHECK(A.size(-1) == K, "Common dimension sizes of matmul inputs should be the same. Got ", A.size(-1), " and ", K);
+  TORCH_CHECK(scale.dim() == 2 && scale.size(1) == N && scale.size(0) > 0 && K % scale.size(0) == 0,
+              "mi355q::w4a8_gemm scale must be [K / group, N] = [*, ", N, "], got ", scale.sizes());
+  const int64_t groups = scale.size(0), group = K / groups;
+  const bool has_zp = zero_point.has_value() && zero_point->defined();
+  if (has_zp)
+    TORCH_CHECK(zero_point->scalar_type() == at::kInt && zero_point->dim() == 2 && zero_point->size(0) == groups &&
+                    zero_point->size(1) == N / 8,
+                "mi355q::w4a8_gemm zero_point must be packed int32 [K / group, N / 8], got ", zero_point->scalar_type(), " ",
+                zero_point->sizes());
+  std::vector<int64_t> out_shape(A.sizes().begin(), A.sizes().end());
+  out_shape.back() = N;
+  if (A.is_meta()) return at::empty(out_shape, A.options().dtype(out_dtype));
+  TORCH_CHECK(A.device() == packed.device() && A.device() == scale.device(), "mi355q::w4a8_gemm operands must be on the same device");
+  DeviceGuard guard(A.device());
+  Tensor a = A.contiguous();
+  const int64_t M = K ? a.numel() / K : 0;
+  Tensor out = at::empty(out_shape, A.options().dtype(out_dtype));
+  if (out.numel() == 0) return out;
+  Tensor w = packed.contiguous();
+  Tensor s = (scale.scalar_type() == at::kBFloat16 ? scale : scale.to(at::kFloat)).contiguous();
+  Tensor z;
+  if (has_zp) z = zero_point->contiguous();
+  Tensor sa_t;
+  const float* sa_dev = nullptr;
+  int sa_mode = MI355Q_GS_NONE;
+  if (A_scale_inv.has_value() && A_scale_inv->defined()) {
+    sa_t = A_scale_inv->to(at::kFloat).contiguous();
+    TORCH_CHECK(sa_t.device() == A.device(), "A_scale_inv must be on the same device as A");
+    TORCH_CHECK(sa_t.numel() == 1 || sa_t.numel() == M, "A_scale_inv must hold one value or one per row of A (", M, "), got ", sa_t.sizes());
+    sa_dev = sa_t.data_ptr<float>();
+    sa_mode = (sa_t.numel() == 1 && M != 1) ? MI355Q_GS_DEV : (sa_t.numel() == 1 ? MI355Q_GS_DEV : MI355Q_GS_PER_ROW);
+  }
+  Tensor b;
+  if (bias.has_value() && bias->defined()) {
+    TORCH_CHECK(bias->numel() == N, "Bias must be size ", N, " but got ", bias->numel());
+    b = bias->to(out_dtype).contiguous();
+  }
+  MI355Q_OP_INFO("w4a8_gemm : A=" << A.sizes() << " packed=" << packed.sizes() << " group=" << group << " signed=" << is_signed);
+  const int st = mi355q_w4a8_gemm(a.data_ptr(), to_mi355q_dtype(a.scalar_type()), K, w.data_ptr<int32_t>(), N / 8, s.data_ptr(),
+                                  to_mi355q_dtype(s.scalar_type()), has_zp ? z.data_ptr<int32_t>() : nullptr, is_signed ? 1 : 0,
+                                  group, out.data_ptr(), to_mi355q_dtype(out_dtype), N, M, N, K, sa_dev, 1.0f, sa_mode,
+                                  b.defined() ? b.data_ptr() : nullptr, current_stream(a));
+  TORCH_CHECK(st != MI355Q_ERR_UNSUPPORTED,
+              "mi355q::w4a8_gemm takes groups that are multiples of 128, N a multiple of 32 and K a multiple of 16 (got group ",
+              group, ", N ", N, ", K ", K, "); expand the weights with hpu::convert_from_", is_signed ? "int4" : "uint4", " for other shapes");
+  check_status(st, "mi355q_w4a8_gemm");
+  return out;
+}
+
 // ------------------------------------------------------------------ sum_fp8
 
 // hpu::sum_fp8 (hpu_ops/backend/fp8_ops_gen.cpp:20-49): sum of an fp8 tensor over `dim`
@@ -1082,6 +1147,7 @@ TORCH_LIBRARY(mi355q, m) {
   m.def("mi355q::rowwise_amax(Tensor input) -> Tensor");
   m.def("mi355q::quantize_rows(Tensor input, ScalarType dtype) -> (Tensor, Tensor)");
   m.def("mi355q::silu_mul_quantize_rows(Tensor gate, Tensor up, ScalarType dtype) -> (Tensor, Tensor)");
+  m.def("mi355q::w4a8_gemm(Tensor A, Tensor packed, Tensor scale, Tensor? zero_point, bool is_signed, ScalarType out_dtype, Tensor? A_scale_inv=None, Tensor? bias=None) -> Tensor");
   m.def("mi355q::scaled_mm(Tensor self, Tensor mat2, Tensor scale_a, Tensor scale_b, Tensor? bias=None, Tensor? scale_result=None, ScalarType? out_dtype=None, bool use_fast_accum=False) -> Tensor");
 }
 
@@ -1114,6 +1180,7 @@ TORCH_LIBRARY_IMPL(mi355q, CUDA, m) {
   m.impl("quantize_rows", quantize_rows_op);
   m.impl("scaled_mm", scaled_mm);
   m.impl("silu_mul_quantize_rows", silu_mul_quantize_rows_op);
+  m.impl("w4a8_gemm", w4a8_gemm);
 }
 TORCH_LIBRARY_IMPL(mi355q, Meta, m) {
   m.impl("amax", amax_op);
@@ -1121,4 +1188,5 @@ TORCH_LIBRARY_IMPL(mi355q, Meta, m) {
   m.impl("quantize_rows", quantize_rows_op);
   m.impl("scaled_mm", scaled_mm);
   m.impl("silu_mul_quantize_rows", silu_mul_quantize_rows_op);
+  m.impl("w4a8_gemm", w4a8_gemm);
 }

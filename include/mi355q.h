@@ -232,6 +232,30 @@ int mi355q_fp8_gemm(const void* A, int fmt_a, int trans_a, int64_t lda,
                     void* stream);
 
 /*
+ * Fused int4-dequant GEMM, fp8 activations times 4-bit weights (W4A8):
+ *   C = out_dtype( (A @ W) * sa + bias ),   W[k, n] = (q[k, n] - z[k / group, n]) * s[k / group, n],
+ * with the weights as convert_from_int4 / convert_from_uint4 take them and mi355q_dequant_4bit
+ * would expand them (Int4BaseOp::AddNode, hpu_ops/backend/int4_ops.cpp:40-56: packed int32
+ * [K, N / 8], nibble i of word p is column 8 p + i, is_signed selects int4 over uint4), multiplied as
+ * Fp8GemmV2::AddNode multiplies (hpu_ops/backend/fp8_ops.cpp:403-496) without the bf16 [K, N]
+ * matrix in between: the packed words are what travels from HBM, (q - z) enters the fp8 MFMA exactly,
+ * each K group is accumulated in fp32 and multiplied by its scales as it joins the total.  The
+ * reference has no fused op; it is the composition of those two.
+ *   A           fp8 (fmt_a) [M, K], row pitch lda
+ *   packed      int32 [K, N / 8], row pitch ld_packed (in words)
+ *   scale       bf16 or fp32 (scale_dtype) [K / group, N], dense
+ *   zero_point  packed int32 [K / group, N / 8] (same nibble order and signedness) or NULL
+ *   sa          none, host scalar, device scalar or per row (mi355q_gemm_scale_mode); bias: out_dtype [N] or NULL
+ * group must be a multiple of 128 that divides K; N a multiple of 32; K, lda multiples of 16; all
+ * pointers 16-byte aligned; otherwise MI355Q_ERR_UNSUPPORTED, and the caller expands the weights
+ * with mi355q_dequant_4bit.
+ */
+int mi355q_w4a8_gemm(const void* A, int fmt_a, int64_t lda, const int32_t* packed, int64_t ld_packed,
+                     const void* scale, int scale_dtype, const int32_t* zero_point, int is_signed,
+                     int64_t group, void* C, int out_dtype, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                     const float* sa_dev, float sa_host, int sa_mode, const void* bias, void* stream);
+
+/*
  * Sum over the middle dimension of an fp8 tensor viewed as [outer, reduce, inner]
  * (a sum over adjacent dimensions of a contiguous tensor), accumulated in fp32 in a
  * fixed order and written as out_dtype (fp32, bf16, or fp8 with the saturating

@@ -1,0 +1,126 @@
+"""GPU parity of mi355q::w4a8_gemm (fp8 activations times packed 4-bit weights, dequantisation fused into
+the GEMM) against the oracle: bit-exact where the arithmetic is exact (small-integer activations,
+power-of-two scales), max|out - ref| / max|ref| <= 1e-2 against the float64-accumulated reference otherwise,
+and against the unfused route convert_from_[u]int4 -> fp32 weights on the CPU."""
+import ctypes
+
+import pytest
+import torch
+
+from helpers import E4, E5, gemm_errors
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def weights(oracle, gen, K, N, group, signed, zp, scale_dtype=torch.bfloat16, pow2=False):
+    lo, hi = (-8, 8) if signed else (0, 16)
+    q = torch.randint(lo, hi, (K, N), generator=gen)
+    z = torch.randint(lo, hi, (K // group, N), generator=gen) if zp else None
+    if pow2:
+        s = torch.exp2(torch.randint(-3, 3, (K // group, N), generator=gen).float()).to(scale_dtype)
+    else:
+        s = (torch.rand(K // group, N, generator=gen) * 0.019 + 0.001).to(scale_dtype)
+    return q, z, s, oracle.pack_nibbles(q), (oracle.pack_nibbles(z) if zp else None)
+
+
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("zp", [False, True])
+@pytest.mark.parametrize("M,K,N,group", [
+    (16, 512, 256, 128),      # 32-row strip
+    (5, 1024, 160, 256),      # ragged M, a strip with 32 columns, groups of two stages
+    (48, 640, 4096, 128),     # 64-row strip, K not a multiple of the ring
+    (100, 384, 1056, 384),    # 128-row strip, one group
+    (300, 256, 288, 128),     # three row blocks
+    (64, 4096, 128, 4096),    # per-channel scales, a ring walked several times
+])
+def test_exact(oracle, dev, M, K, N, group, signed, zp):
+    gen = torch.Generator().manual_seed(M * 3 + K + N + signed * 7 + zp)
+    q, z, s, pk, pz = weights(oracle, gen, K, N, group, signed, zp, pow2=True)
+    a = torch.randint(-4, 5, (M, K), generator=gen).float()
+    sa = torch.exp2(torch.randint(-2, 3, (M, 1), generator=gen).float())
+    bias = torch.randint(-8, 9, (N,), generator=gen).float()
+    w = (q - (z.repeat_interleave(group, 0) if zp else 0)).double() * s.double().repeat_interleave(group, 0)
+    expect = ((a.double() @ w) * sa.double() + bias.double())                    # integers times powers of two: exact
+    assert expect.abs().max() < 2 ** 24
+    for fmt in (E4, E5):
+        out = torch.ops.mi355q.w4a8_gemm(a.to(fmt).to(dev), pk.to(dev), s.to(dev), pz.to(dev) if zp else None, signed,
+                                         torch.float32, sa.to(dev), bias.to(dev))
+        assert out.shape == (M, N) and torch.equal(out.cpu().double(), expect), fmt
+    out16 = torch.ops.mi355q.w4a8_gemm(a.to(E4).to(dev), pk.to(dev), s.to(dev), pz.to(dev) if zp else None, signed,
+                                       torch.bfloat16, sa.to(dev), bias.bfloat16().to(dev))
+    assert torch.equal(out16.cpu(), expect.float().bfloat16())
+
+
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("scale_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M", [16, 64, 256])
+def test_against_oracle_config2_weights(oracle, dev, M, signed, scale_dtype):
+    """Benchmark configuration 2's weights (K = N = 4096, group 128, scales U(0.001, 0.02), zero-points for
+    uint4) with configuration 4's activations (per-token e4m3fn of N(0, 1) with heavy-tail channels)."""
+    gen = torch.Generator().manual_seed(0xC001A1 + M)
+    K = N = 4096
+    q, z, s, pk, pz = weights(oracle, gen, K, N, 128, signed, not signed, scale_dtype)
+    x = torch.randn(M, K, generator=gen)
+    x[:, torch.randperm(K, generator=gen)[:41]] *= 20
+    x8, sx = oracle.quantize_rows(x.bfloat16(), E4)
+    bias = (torch.randn(N, generator=gen) * 0.01).bfloat16()
+    out = torch.ops.mi355q.w4a8_gemm(x8.to(dev), pk.to(dev), s.to(dev), pz.to(dev) if pz is not None else None, signed,
+                                     torch.bfloat16, sx.to(dev), bias.to(dev))
+    ref = oracle.torch_w4a8_gemm(x8, pk, s, pz, signed, torch.float32, sx, bias)
+    rel, ok = gemm_errors(out, ref)
+    assert rel <= TOL and ok, rel
+    # the unfused route: convert_from_[u]int4 to fp32 on the GPU (bit-exact op), product on the CPU
+    conv = torch.ops.hpu.convert_from_int4 if signed else torch.ops.hpu.convert_from_uint4
+    w32 = conv(pk.to(dev), s.float().to(dev), pz.to(dev) if pz is not None else None, torch.float32).cpu()
+    ref2 = (x8.float() @ w32) * sx + bias.float()
+    rel, ok = gemm_errors(out, ref2)
+    assert rel <= TOL and ok, rel
+
+
+def test_batched_activations_scalar_scale_and_c_abi(oracle, pkg, dev):
+    gen = torch.Generator().manual_seed(3)
+    K, N, group = 256, 320, 128
+    q, z, s, pk, pz = weights(oracle, gen, K, N, group, False, True)
+    a8 = (torch.randn(2, 3, 7, K, generator=gen) * 2).to(E4)
+    sa = torch.tensor(0.37)
+    out = torch.ops.mi355q.w4a8_gemm(a8.to(dev), pk.to(dev), s.to(dev), pz.to(dev), False, torch.float32, sa.to(dev), None)
+    assert out.shape == (2, 3, 7, N)
+    ref = oracle.torch_w4a8_gemm(a8.reshape(-1, K), pk, s, pz, False, torch.float32, sa).reshape(2, 3, 7, N)
+    rel, ok = gemm_errors(out, ref)
+    assert rel < 1e-5 and ok, rel
+    # the C entry point with a host scalar, wider row pitches of A and C
+    lib = pkg.capi()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    M = 40
+    A = torch.zeros(M, K + 64, dtype=torch.uint8)
+    A[:, :K] = (torch.randn(M, K, generator=gen)).to(E4).view(torch.uint8)
+    Ad, pkd, sd, pzd = A.to(dev), pk.to(dev), s.to(dev), pz.to(dev)
+    C = torch.full((M, N + 32), -5.0, device=dev)
+    st = lib.mi355q_w4a8_gemm(Ad.data_ptr(), pkg.E4M3FN, K + 64, pkd.data_ptr(), N // 8, sd.data_ptr(), pkg.BF16, pzd.data_ptr(), 0,
+                              group, C.data_ptr(), pkg.F32, N + 32, M, N, K, None, 0.5, pkg.GS_HOST, None, stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    ref = oracle.torch_w4a8_gemm(A[:, :K].view(E4), pk, s, pz, False, torch.float32, 0.5)
+    rel, ok = gemm_errors(C[:, :N], ref)
+    assert rel < 1e-5 and ok, rel
+    assert (C[:, N:] == -5.0).all()
+    # refused shapes launch nothing: a group of 64, N not a multiple of 32
+    assert lib.mi355q_w4a8_gemm(Ad.data_ptr(), pkg.E4M3FN, K + 64, pkd.data_ptr(), N // 8, sd.data_ptr(), pkg.BF16, None, 0,
+                                64, C.data_ptr(), pkg.F32, N + 32, M, N, K, None, 1.0, pkg.GS_NONE, None, stream) == 2
+    assert lib.mi355q_w4a8_gemm(Ad.data_ptr(), pkg.E4M3FN, K + 64, pkd.data_ptr(), N // 8, sd.data_ptr(), pkg.BF16, None, 0,
+                                128, C.data_ptr(), pkg.F32, N + 32, M, N - 8, K, None, 1.0, pkg.GS_NONE, None, stream) == 2
+    with pytest.raises(RuntimeError, match="multiples of 128"):
+        torch.ops.mi355q.w4a8_gemm(a8.to(dev), pk.to(dev), s.repeat(2, 1).to(dev), None, False, torch.float32, None, None)
+
+
+def test_meta_and_checks(dev):
+    a = torch.empty(4, 256, device="meta", dtype=E4)
+    pk = torch.empty(256, 16, device="meta", dtype=torch.int32)
+    s = torch.empty(2, 128, device="meta", dtype=torch.bfloat16)
+    out = torch.ops.mi355q.w4a8_gemm(a, pk, s, None, True, torch.bfloat16, None, None)
+    assert out.shape == (4, 128) and out.dtype == torch.bfloat16
+    with pytest.raises(RuntimeError, match="Common dimension"):
+        torch.ops.mi355q.w4a8_gemm(torch.empty(4, 128, device="meta", dtype=E4), pk, s, None, True, torch.bfloat16, None, None)
+    with pytest.raises(RuntimeError, match="scale must be"):
+        torch.ops.mi355q.w4a8_gemm(a, pk, torch.empty(3, 128, device="meta"), None, True, torch.bfloat16, None, None)

@@ -80,8 +80,8 @@ def test_scanner_flags_m0_used_at_once():
 
 @pytest.mark.timeout(900)
 def test_gemm_kernels_have_no_uncovered_hazard():
-    sources = ["gemm_inst_kk.hip", "gemm_inst_km.hip", "gemm_inst_mk.hip", "gemm_inst_mm.hip"]
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    sources = ["gemm_inst_kk.hip", "gemm_inst_km.hip", "gemm_inst_mk.hip", "gemm_inst_mm.hip", "w4_gemm.hip"]
+    with ThreadPoolExecutor(max_workers=5) as ex:
         texts = list(ex.map(isa_check.compile_to_isa, sources))
     for src, text in zip(sources, texts):
         assert text.count("#ASMSTART") > 100, f"{src}: the asm statements are gone?"
