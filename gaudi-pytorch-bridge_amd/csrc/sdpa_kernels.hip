@@ -1,0 +1,483 @@
+// fp8 scaled-dot-product attention (inference forward) for gfx950 and its C entry point.
+//
+// out = softmax(q k^T * scale + mask) v with q, k, v in fp8, an online softmax over blocks of 64
+// keys, the probabilities quantised to fp8 before the second product, fp32 accumulation.
+//
+// Work split.  A workgroup of four waves owns 128 query rows of one (batch, head); a wave owns 32
+// of them for the whole key loop.  Both products run on v_mfma_f32_32x32x64_f8f6f4 and both are
+// issued transposed, keys (then columns of v) as the first operand and queries as the second:
+//     S^T [64 keys, 32 queries]  = K_blk  Q^T        (two 32-key tiles, head_dim_qk / 64 steps)
+//     O^T [dv,      32 queries] += V_blk^T P^T       (dv / 32 tiles, one step over the 64 keys)
+// The MFMA leaves a lane with one query (lane % 32) and, per 32-row tile, the rows 8 j + 4 (lane /
+// 32) + i of the first operand in register 4 j + i.  A query's row statistics are therefore
+// per-lane values (one exchange between the two half-waves), rescaling O is a per-lane multiply,
+// and the 32 probabilities a lane holds after S^T are, converted to fp8 and packed in register
+// order, exactly the 32 k-slots of the second MFMA's second operand for that lane: P never passes
+// through LDS.  The k-slot s = 16 t + 4 j + i of half-wave h then stands for key 32 t + 8 j + 4 h + i,
+// and the V^T fragment is gathered from LDS in the same key order by the transposing reads
+// (ds_read_b64_tr_b8 takes each of its 8 k-rows from its own address).
+//
+// K and V blocks go global -> registers -> LDS, double buffered, one barrier per block: the loads
+// of block i + 1 are issued before the arithmetic of block i and written to the other buffer after
+// it.  Rows are XOR-swizzled so that the fragment reads are bank-conflict free.
+#include "device_common.h"
+
+namespace mi355q {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+#define SDPA_LDS_AS __attribute__((address_space(3)))
+
+constexpr int kSdpaThreads = 256;
+constexpr int kSdpaBM = 128;  // query rows per workgroup
+constexpr int kSdpaBN = 64;   // keys per block
+constexpr int kVRow = 256;    // bytes of an LDS row of V, whatever head_dim_v is
+constexpr float kLog2e = 1.44269504088896341f;
+
+enum { kMaskNone = MI355Q_SDPA_MASK_NONE, kMaskBool = MI355Q_SDPA_MASK_BOOL, kMaskBf16 = MI355Q_SDPA_MASK_BF16, kMaskF32 = MI355Q_SDPA_MASK_F32 };
+
+struct SdpaArgs {
+  const uint8_t* q;
+  const uint8_t* k;
+  const uint8_t* v;
+  const uint8_t* mask;
+  uint8_t* out;
+  int64_t bdim[3];
+  int64_t q_bs[3], k_bs[3], v_bs[3], m_bs[3], o_bs[3];
+  int64_t ldq, ldk, ldv, ldm, ldo;
+  int L, S, Dk, Dv;
+  int mask_kind, causal, out_fp8;
+  int vec_q, vec_k, vec_v, vec_o;  // 16-byte (q, k, v) / 4-element (out) accesses are possible
+  int nqb;                         // query blocks per (batch, head)
+  float scale;
+  const float* sc_dev[6];  // d_scale_q, d_scale_k, d_scale_v, q_scale_s, q_scale_o, d_scale_s
+  float sc_host[6];        // used where sc_dev is null; 0 = absent
+  float* amax_s;
+  float* amax_o;
+};
+
+__device__ __forceinline__ float sdpa_scale(const SdpaArgs& a, int i, float absent) {
+  if (a.sc_dev[i] != nullptr) return *a.sc_dev[i];
+  return a.sc_host[i] != 0.0f ? a.sc_host[i] : absent;
+}
+
+// LDS offset of 16-byte chunk `chunk` of K row `row` (ROW_BYTES per row).  The 16 lanes of one
+// ds_read_b128 cycle read one chunk column of 16 consecutive rows: the XOR sends them to 16
+// different 16-byte slots modulo 256 bytes.
+template <int ROW_BYTES>
+__device__ __forceinline__ int k_lds_offset(int row, int chunk) {
+  int sw;
+  if constexpr (ROW_BYTES == 64) sw = (row >> 2) & 3;
+  else if constexpr (ROW_BYTES == 128) sw = (row >> 1) & 7;
+  else sw = row & 15;
+  return row * ROW_BYTES + ((chunk ^ sw) << 4);
+}
+
+// V rows are 256 bytes.  A transposing read covers, per cycle, two 16-lane groups (adjacent chunks)
+// times the 8 keys 8 (2 p' + r / 4) + 4 h + r % 4, r = 0..7: bits 3, 1 and 0 of the key tell them
+// apart, and XORing twice that number into the chunk index gives 8 slots of one parity.
+__device__ __forceinline__ int v_lds_offset(int row, int chunk) {
+  const int key = (((row >> 3) & 1) << 2) | (row & 3);
+  return row * kVRow + ((chunk ^ (key << 1)) << 4);
+}
+
+// 16 bytes of a row of q / k / v starting at byte column d (zero beyond the row's D bytes and for
+// rows outside the tensor).  VEC: the row start and D are multiples of 16.
+__device__ __forceinline__ u32x4 load_chunk(const uint8_t* row_ptr, bool row_ok, int d, int D, bool vec) {
+  u32x4 r = {0u, 0u, 0u, 0u};
+  if (!row_ok || d >= D) return r;
+  if (vec) return *reinterpret_cast<const u32x4*>(row_ptr + d);
+#pragma unroll
+  for (int b = 0; b < 16; ++b) {
+    const uint32_t byte = (d + b < D) ? row_ptr[d + b] : 0u;
+    r[b >> 2] |= byte << (8 * (b & 3));
+  }
+  return r;
+}
+
+template <int FMT>
+__device__ __forceinline__ f32x16 sdpa_mfma(const i32x8& first, const i32x8& second, const f32x16& acc) {
+  constexpr int code = FMT == MI355Q_E5M2 ? 1 : 0;
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(first, second, acc, code, code, 0, 0, 0, 0);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__global__ void sdpa_clear_amax_kernel(float* a, float* b) {
+  if (a != nullptr) *a = 0.0f;
+  if (b != nullptr) *b = 0.0f;
+}
+
+// DKC: 64-byte steps of the q.k depth (head_dim_qk <= 64 DKC); DVT: 32-column tiles of v
+// (head_dim_v <= 32 DVT).
+template <int DKC, int DVT, int FMT>
+__global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd_kernel(const SdpaArgs a) {
+  constexpr int KROW = DKC * 64;
+  constexpr int KCPR = KROW / 16;           // chunks per K row
+  constexpr int VCPR = DVT * 2;             // chunks per V row that carry data
+  constexpr int KBYTES = kSdpaBN * KROW;
+  constexpr int VBYTES = kSdpaBN * kVRow;
+  constexpr int KLOADS = kSdpaBN * KCPR / kSdpaThreads;  // 16-byte loads per thread and block
+  constexpr int VLOADS = kSdpaBN * VCPR / kSdpaThreads;
+  static_assert(KLOADS >= 1 && VLOADS >= 1, "block too small for the workgroup");
+  __shared__ __align__(16) uint8_t lds[2 * (KBYTES + VBYTES)];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lq = lane & 31, h = lane >> 5;
+
+  // Workgroups go to the 8 XCDs round robin: give each XCD a contiguous range of (batch, head,
+  // query block), so that the query blocks that share a K and V meet in one L2.
+  int id = blockIdx.x;
+  const int total = gridDim.x;
+  if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+  int64_t bi = id / a.nqb;
+  const int qb = a.nqb - 1 - (id - (int)bi * a.nqb);  // under a causal mask the long rows start first
+  int64_t q_off = 0, k_off = 0, v_off = 0, m_off = 0, o_off = 0;
+#pragma unroll
+  for (int d = 2; d >= 0; --d) {
+    const int64_t b = bi % a.bdim[d];
+    bi /= a.bdim[d];
+    q_off += b * a.q_bs[d];
+    k_off += b * a.k_bs[d];
+    v_off += b * a.v_bs[d];
+    m_off += b * a.m_bs[d];
+    o_off += b * a.o_bs[d];
+  }
+  const uint8_t* qp = a.q + q_off;
+  const uint8_t* kp = a.k + k_off;
+  const uint8_t* vp = a.v + v_off;
+
+  const int q0 = qb * kSdpaBM;
+  const int wq0 = q0 + wave * 32;  // first query row of this wave
+  const int qrow = wq0 + lq;
+  const bool q_ok = qrow < a.L;
+
+  const float dq = sdpa_scale(a, 0, 1.0f), dk = sdpa_scale(a, 1, 1.0f), dv = sdpa_scale(a, 2, 1.0f);
+  const float qs = sdpa_scale(a, 3, 1.0f);
+  const float ds = sdpa_scale(a, 5, 1.0f / qs);
+  const float sc2 = a.scale * dq * dk * kLog2e;
+  const float lqs = __builtin_log2f(qs);
+  constexpr float kMax8 = FMT == MI355Q_E5M2 ? 57344.0f : 448.0f;
+  const bool clamp_p = !(qs <= kMax8);
+
+  // this lane's query fragments: 32 bytes of depth per 64-byte step
+  i32x8 qf[DKC];
+#pragma unroll
+  for (int c = 0; c < DKC; ++c) {
+    const uint8_t* rp = qp + (int64_t)qrow * a.ldq;
+    const u32x4 lo = load_chunk(rp, q_ok, 64 * c + 32 * h, a.Dk, a.vec_q);
+    const u32x4 hi = load_chunk(rp, q_ok, 64 * c + 32 * h + 16, a.Dk, a.vec_q);
+    qf[c] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+  }
+
+  int nblk = (a.S + kSdpaBN - 1) / kSdpaBN;
+  if (a.causal) {
+    const int last_q = (q0 + kSdpaBM < a.L ? q0 + kSdpaBM : a.L) - 1;
+    const int lim = last_q / kSdpaBN + 1;  // blocks that hold a key <= the last query row
+    nblk = nblk < lim ? nblk : lim;
+  }
+
+  u32x4 kreg[KLOADS], vreg[VLOADS];
+  auto fetch = [&](int blk) {
+    const int kv0 = blk * kSdpaBN;
+#pragma unroll
+    for (int n = 0; n < KLOADS; ++n) {
+      const int ci = tid + n * kSdpaThreads;
+      const int row = ci / KCPR, chunk = ci % KCPR;
+      kreg[n] = load_chunk(kp + (int64_t)(kv0 + row) * a.ldk, kv0 + row < a.S, chunk * 16, a.Dk, a.vec_k);
+    }
+#pragma unroll
+    for (int n = 0; n < VLOADS; ++n) {
+      const int ci = tid + n * kSdpaThreads;
+      const int row = ci / VCPR, chunk = ci % VCPR;
+      vreg[n] = load_chunk(vp + (int64_t)(kv0 + row) * a.ldv, kv0 + row < a.S, chunk * 16, a.Dv, a.vec_v);
+    }
+  };
+  auto commit = [&](int buf) {
+    uint8_t* kb = lds + buf * (KBYTES + VBYTES);
+    uint8_t* vb = kb + KBYTES;
+#pragma unroll
+    for (int n = 0; n < KLOADS; ++n) {
+      const int ci = tid + n * kSdpaThreads;
+      *reinterpret_cast<u32x4*>(kb + k_lds_offset<KROW>(ci / KCPR, ci % KCPR)) = kreg[n];
+    }
+#pragma unroll
+    for (int n = 0; n < VLOADS; ++n) {
+      const int ci = tid + n * kSdpaThreads;
+      *reinterpret_cast<u32x4*>(vb + v_lds_offset(ci / VCPR, ci % VCPR)) = vreg[n];
+    }
+  };
+
+  f32x16 o[DVT];
+#pragma unroll
+  for (int t = 0; t < DVT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[t][r] = 0.0f;
+  float m_run = -__builtin_inff();  // running maximum of the scaled scores, in units of log2
+  float l_run = 0.0f;               // this half-wave's share of the running sum (times q_scale_s)
+
+  if (nblk > 0) {
+    fetch(0);
+    commit(0);
+  }
+  __syncthreads();
+
+  for (int blk = 0; blk < nblk; ++blk) {
+    const int kv0 = blk * kSdpaBN;
+    if (blk + 1 < nblk) fetch(blk + 1);
+    const uint8_t* kb = lds + (blk & 1) * (KBYTES + VBYTES);
+    const uint8_t* vb = kb + KBYTES;
+
+    // a wave whose 32 rows all lie above this block's first key has nothing to add
+    const bool active = !(a.causal && kv0 > wq0 + 31);
+    if (active) {
+      f32x16 s[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[t][r] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < DKC; ++c) {
+          const int row = 32 * t + lq;
+          const u32x4 lo = *reinterpret_cast<const u32x4*>(kb + k_lds_offset<KROW>(row, c * 4 + h * 2));
+          const u32x4 hi = *reinterpret_cast<const u32x4*>(kb + k_lds_offset<KROW>(row, c * 4 + h * 2 + 1));
+          const i32x8 kf = {(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+          s[t] = sdpa_mfma<FMT>(kf, qf[c], s[t]);
+        }
+      }
+
+      // scores in units of log2, masks applied
+      const bool edge = (a.causal && kv0 + kSdpaBN - 1 > wq0) || kv0 + kSdpaBN > a.S || a.mask_kind != kMaskNone;
+      float mx = -__builtin_inff();
+      if (!edge && sc2 >= 0.0f) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, s[t][r]);
+        mx *= sc2;
+      } else {
+        const uint8_t* mrow = a.mask + (m_off + (int64_t)qrow * a.ldm) * (a.mask_kind == kMaskBool ? 1 : a.mask_kind == kMaskBf16 ? 2 : 4);
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int kv = kv0 + 32 * t + 8 * (r >> 2) + 4 * h + (r & 3);
+            float x = s[t][r] * sc2;
+            bool dead = kv >= a.S || (a.causal && kv > qrow);
+            if (a.mask_kind != kMaskNone && q_ok && kv < a.S) {
+              if (a.mask_kind == kMaskBool) dead = dead || mrow[kv] == 0;
+              else if (a.mask_kind == kMaskBf16) x += bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(mrow)[kv]) * kLog2e;
+              else x += reinterpret_cast<const float*>(mrow)[kv] * kLog2e;
+            }
+            x = dead ? -__builtin_inff() : x;
+            s[t][r] = x;
+            mx = __builtin_fmaxf(mx, x);
+          }
+      }
+      mx = __builtin_fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = __builtin_fmaxf(m_run, mx);
+      const float m_use = m_new == -__builtin_inff() ? 0.0f : m_new;
+      const float alpha = fast_exp2(m_run - m_use);
+      m_run = m_new;
+      const float shift = lqs - m_use;  // p * q_scale_s = 2^(x - m + log2 q_scale_s)
+
+      float psum = 0.0f;
+      i32x8 pf;
+      const bool raw = !edge && sc2 >= 0.0f;  // s still holds the unscaled products
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float p[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float x = s[t][4 * j + i];
+            p[i] = fast_exp2(raw ? __builtin_fmaf(x, sc2, shift) : x + shift);
+            psum += p[i];
+            if (clamp_p) p[i] = __builtin_elementwise_minimum(p[i], kMax8);
+          }
+          int w;
+          if constexpr (FMT == MI355Q_E5M2) {
+            w = __builtin_amdgcn_cvt_pk_bf8_f32(p[0], p[1], 0, false);
+            w = __builtin_amdgcn_cvt_pk_bf8_f32(p[2], p[3], w, true);
+          } else {
+            w = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
+            w = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], w, true);
+          }
+          pf[4 * t + j] = w;
+        }
+      l_run = l_run * alpha + psum;
+
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+        for (int t = 0; t < DVT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
+      }
+
+      // O^T += V^T P^T; k-slot 8 p + r' of half-wave h is key 32 (p / 2) + 8 (2 (p % 2) + r' / 4) + 4 h + r' % 4
+      const int g = lane >> 4, gi = lane & 15;
+      const int r8 = gi >> 1, hh = gi & 1;
+#pragma unroll
+      for (int t = 0; t < DVT; ++t) {
+        i32x8 vf;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          const int krow = 32 * (p >> 1) + 8 * (2 * (p & 1) + (r8 >> 2)) + 4 * h + (r8 & 3);
+          const int off = v_lds_offset(krow, 2 * t + (g & 1)) + hh * 8;
+          const i32x2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((SDPA_LDS_AS i32x2*)((SDPA_LDS_AS uint8_t*)vb + off));
+          vf[2 * p] = w[0];
+          vf[2 * p + 1] = w[1];
+        }
+        o[t] = sdpa_mfma<FMT>(vf, pf, o[t]);
+      }
+    }
+
+    if (blk + 1 < nblk) commit((blk + 1) & 1);
+    __syncthreads();
+  }
+
+  // out = O * d_scale_s * d_scale_v / l.  l_run carries the factor q_scale_s that p did.
+  const float l_tot = (l_run + __shfl_xor(l_run, 32, 64)) / qs;
+  const float inv_l = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+  const float f = inv_l * (ds * dv);
+  const float qo = a.out_fp8 ? sdpa_scale(a, 4, 1.0f) : 1.0f;
+  float amax_o = 0.0f;
+  uint8_t* orow = a.out + (o_off + (int64_t)qrow * a.ldo) * (a.out_fp8 ? 1 : 2);
+#pragma unroll
+  for (int t = 0; t < DVT; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int d0 = 32 * t + 8 * j + 4 * h;
+      float val[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        val[i] = o[t][4 * j + i] * f;
+        if (q_ok && d0 + i < a.Dv) amax_o = __builtin_fmaxf(amax_o, __builtin_fabsf(val[i]));
+      }
+      if (!q_ok || d0 >= a.Dv) continue;
+      if (a.out_fp8) {
+        const uint32_t w = cvt_fp8x4<MI355Q_E4M3FN>(val[0] * qo, val[1] * qo, val[2] * qo, val[3] * qo);
+        if (a.vec_o) {
+          *reinterpret_cast<uint32_t*>(orow + d0) = w;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (d0 + i < a.Dv) orow[d0 + i] = (uint8_t)(w >> (8 * i));
+        }
+      } else {
+        const uint32_t w0 = pack_bf16x2(val[0], val[1]), w1 = pack_bf16x2(val[2], val[3]);
+        if (a.vec_o) {
+          *reinterpret_cast<u32x2*>(orow + 2 * d0) = u32x2{w0, w1};
+        } else {
+          uint16_t* o16 = reinterpret_cast<uint16_t*>(orow);
+          const uint32_t ws[2] = {w0, w1};
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (d0 + i < a.Dv) o16[d0 + i] = (uint16_t)(ws[i >> 1] >> (16 * (i & 1)));
+        }
+      }
+    }
+
+  if (a.amax_s != nullptr) {
+    // the largest probability of a row is the one at the row maximum: 1 / l
+    const uint32_t m = wave_max_u32(__float_as_uint(q_ok ? inv_l : 0.0f));
+    if (lane == 0 && m != 0u) atomicMax(reinterpret_cast<unsigned int*>(a.amax_s), m);
+  }
+  if (a.amax_o != nullptr) {
+    const uint32_t m = wave_max_u32(__float_as_uint(amax_o));
+    if (lane == 0 && m != 0u) atomicMax(reinterpret_cast<unsigned int*>(a.amax_o), m);
+  }
+}
+
+template <int DKC, int DVT>
+static int sdpa_launch(const SdpaArgs& a, int fmt, int64_t blocks, hipStream_t st) {
+  if (fmt == MI355Q_E5M2)
+    hipLaunchKernelGGL((fp8_sdpa_fwd_kernel<DKC, DVT, MI355Q_E5M2>), dim3((unsigned)blocks), dim3(kSdpaThreads), 0, st, a);
+  else
+    hipLaunchKernelGGL((fp8_sdpa_fwd_kernel<DKC, DVT, MI355Q_E4M3FN>), dim3((unsigned)blocks), dim3(kSdpaThreads), 0, st, a);
+  return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
+}
+
+static bool aligned_to(const void* p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
+
+}  // namespace mi355q
+
+using namespace mi355q;
+
+extern "C" {
+
+int mi355q_fp8_sdpa_fwd(const void* q, const void* k, const void* v, int fp8_fmt, const void* mask, int mask_kind,
+                        void* out, int out_dtype, const mi355q_sdpa_desc* d, float softmax_scale, int is_causal,
+                        const float* const* scale_dev, const float* scale_host, float* amax_s, float* amax_o,
+                        void* stream) {
+  if (d == nullptr) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (fp8_fmt != MI355Q_E4M3FN && fp8_fmt != MI355Q_E5M2) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (out_dtype != MI355Q_BF16 && out_dtype != MI355Q_E4M3FN) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (mask_kind < MI355Q_SDPA_MASK_NONE || mask_kind > MI355Q_SDPA_MASK_F32) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (d->q_len < 0 || d->kv_len < 0 || d->head_dim_qk <= 0 || d->head_dim_v <= 0) return MI355Q_ERR_INVALID_ARGUMENT;
+  int64_t batches = 1;
+  for (int i = 0; i < 3; ++i) {
+    if (d->batch[i] < 0) return MI355Q_ERR_INVALID_ARGUMENT;
+    batches *= d->batch[i];
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (amax_s != nullptr || amax_o != nullptr) {
+    hipLaunchKernelGGL(sdpa_clear_amax_kernel, dim3(1), dim3(1), 0, st, amax_s, amax_o);
+    if (hipGetLastError() != hipSuccess) return MI355Q_ERR_LAUNCH;
+  }
+  if (batches == 0 || d->q_len == 0) return MI355Q_OK;
+  if (q == nullptr || out == nullptr || (d->kv_len > 0 && (k == nullptr || v == nullptr))) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (mask_kind != MI355Q_SDPA_MASK_NONE && mask == nullptr) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (d->head_dim_qk > 256 || d->head_dim_v > 256) return MI355Q_ERR_UNSUPPORTED;
+  if (d->q_len > (1 << 30) || d->kv_len > (1 << 30)) return MI355Q_ERR_UNSUPPORTED;
+  const int64_t nqb = (d->q_len + kSdpaBM - 1) / kSdpaBM;
+  const int64_t blocks = nqb * batches;
+  if (blocks > 0x7fffffff) return MI355Q_ERR_UNSUPPORTED;
+
+  SdpaArgs a{};
+  a.q = static_cast<const uint8_t*>(q);
+  a.k = static_cast<const uint8_t*>(k);
+  a.v = static_cast<const uint8_t*>(v);
+  a.mask = static_cast<const uint8_t*>(mask);
+  a.out = static_cast<uint8_t*>(out);
+  bool vq = aligned_to(q, 16) && d->head_dim_qk % 16 == 0 && d->ldq % 16 == 0;
+  bool vk = aligned_to(k, 16) && d->head_dim_qk % 16 == 0 && d->ldk % 16 == 0;
+  bool vv = aligned_to(v, 16) && d->head_dim_v % 16 == 0 && d->ldv % 16 == 0;
+  const size_t oel = out_dtype == MI355Q_BF16 ? 2 : 1;
+  bool vo = aligned_to(out, 4 * oel) && d->head_dim_v % 4 == 0 && d->ldo % 4 == 0;
+  for (int i = 0; i < 3; ++i) {
+    a.bdim[i] = d->batch[i];
+    a.q_bs[i] = d->q_bstride[i];
+    a.k_bs[i] = d->k_bstride[i];
+    a.v_bs[i] = d->v_bstride[i];
+    a.m_bs[i] = mask_kind != MI355Q_SDPA_MASK_NONE ? d->mask_bstride[i] : 0;
+    a.o_bs[i] = d->out_bstride[i];
+    vq = vq && d->q_bstride[i] % 16 == 0;
+    vk = vk && d->k_bstride[i] % 16 == 0;
+    vv = vv && d->v_bstride[i] % 16 == 0;
+    vo = vo && d->out_bstride[i] % 4 == 0;
+  }
+  a.ldq = d->ldq; a.ldk = d->ldk; a.ldv = d->ldv; a.ldm = d->ldmask; a.ldo = d->ldo;
+  a.L = (int)d->q_len; a.S = (int)d->kv_len; a.Dk = (int)d->head_dim_qk; a.Dv = (int)d->head_dim_v;
+  a.mask_kind = mask_kind;
+  a.causal = is_causal != 0;
+  a.out_fp8 = out_dtype == MI355Q_E4M3FN;
+  a.vec_q = vq; a.vec_k = vk; a.vec_v = vv; a.vec_o = vo;
+  a.nqb = (int)nqb;
+  a.scale = softmax_scale;
+  for (int i = 0; i < 6; ++i) {
+    a.sc_dev[i] = scale_dev != nullptr ? scale_dev[i] : nullptr;
+    a.sc_host[i] = scale_host != nullptr ? scale_host[i] : 0.0f;
+  }
+  a.amax_s = amax_s;
+  a.amax_o = amax_o;
+
+  const int64_t dmax = d->head_dim_qk > d->head_dim_v ? d->head_dim_qk : d->head_dim_v;
+  if (dmax <= 64) return sdpa_launch<1, 2>(a, fp8_fmt, blocks, st);
+  if (dmax <= 128) return sdpa_launch<2, 4>(a, fp8_fmt, blocks, st);
+  return sdpa_launch<4, 8>(a, fp8_fmt, blocks, st);
+}
+
+}  // extern "C"

@@ -952,6 +952,211 @@ Tensor softmax_fp8_scalar(const Tensor& input, int64_t dim, double input_scale, 
                             fused_add);
 }
 
+// ------------------------------------------------------ fp8_sdpa_recomp_fwd
+
+struct SdpaScale {
+  const float* dev = nullptr;
+  float host = 0.0f;   // 0 = absent
+  Tensor holder;
+  bool given() const { return dev != nullptr || host != 0.0f; }
+};
+
+// A scale counts as given when it is a tensor with elements or a non-zero number
+// (sdpa_add_inputs_and_flags, hpu_ops/backend/sdpa_gen.cpp:868-895).
+SdpaScale sdpa_scale(const c10::optional<Tensor>& t, const Tensor& q, const char* name) {
+  SdpaScale s;
+  if (!t.has_value() || !t->defined() || t->numel() == 0) return s;
+  TORCH_CHECK(t->numel() == 1, "fp8_sdpa_recomp_fwd: ", name, " must have one element, got ", t->sizes());
+  if (q.is_meta()) {
+    s.host = 1.0f;
+    return s;
+  }
+  if (t->is_cpu()) {
+    s.host = t->to(at::kFloat).item<float>();
+    return s;
+  }
+  TORCH_CHECK(t->device() == q.device(), "fp8_sdpa_recomp_fwd: ", name, " must be on the same device as q");
+  s.holder = t->scalar_type() == at::kFloat ? *t : t->to(at::kFloat);
+  s.dev = s.holder.data_ptr<float>();
+  return s;
+}
+SdpaScale sdpa_scale(double v) {
+  SdpaScale s;
+  s.host = (float)v;
+  return s;
+}
+
+using SdpaOut = std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor, Tensor>;
+
+// Strides of the up to three batch dimensions of t (rank = batch rank + 2) against the
+// broadcast batch shape `bshape`, right aligned; 0 where t is broadcast.
+void sdpa_batch_strides(const Tensor& t, const std::vector<int64_t>& bshape, int64_t out[3], const char* name) {
+  const int64_t nb = (int64_t)bshape.size(), tb = t.dim() - 2;
+  TORCH_CHECK(tb <= nb, "fp8_sdpa_recomp_fwd: ", name, " has more batch dimensions than q, k and v");
+  for (int64_t i = 0; i < 3; ++i) out[i] = 0;
+  for (int64_t i = 0; i < tb; ++i) {
+    const int64_t bd = nb - tb + i;  // dimension of bshape this one aligns with
+    TORCH_CHECK(t.size(i) == bshape[bd] || t.size(i) == 1, "fp8_sdpa_recomp_fwd: batch dimension ", i, " of ", name, " (",
+                t.size(i), ") does not broadcast to ", bshape[bd]);
+    out[3 - nb + bd] = t.size(i) == 1 ? 0 : t.stride(i);
+  }
+}
+
+Tensor sdpa_unit_rows(const Tensor& t) { return (t.dim() >= 1 && t.stride(-1) != 1 && t.size(-1) > 1) ? t.contiguous() : t; }
+
+// Fp8SDPARecompFwd::AddNode, hpu_ops/backend/sdpa_gen.cpp:806-1000 (inputs, flags, output types);
+// output shapes SDPARecompFwdOutputShapeCommon / Fp8SDPARecompFwdOutputShape, :597-706.
+SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tensor& v, const c10::optional<Tensor>& attention_mask,
+                                   double p, double scale, bool is_causal, bool requires_backward, c10::string_view softmax_mode,
+                                   const SdpaScale& d_scale_q, const SdpaScale& d_scale_k, const SdpaScale& d_scale_v,
+                                   const SdpaScale& q_scale_s, const SdpaScale& q_scale_o, const SdpaScale& d_scale_s,
+                                   bool is_amax_s, bool is_amax_o, const c10::optional<Tensor>& valid_seq_len,
+                                   c10::string_view seq_padding_type) {
+  TORCH_CHECK(!requires_backward, "fp8_sdpa_recomp_fwd: only the inference forward (requires_backward=False) is implemented");
+  TORCH_CHECK(p == 0.0, "fp8_sdpa_recomp_fwd: dropout is not implemented (p must be 0)");
+  TORCH_CHECK(!(valid_seq_len.has_value() && valid_seq_len->defined()), "fp8_sdpa_recomp_fwd: valid_seq_len is not implemented");
+  TORCH_CHECK(softmax_mode == "none" || softmax_mode == "None" || softmax_mode == "fast", "fp8_sdpa_recomp_fwd: softmax_mode must be \"none\" or \"fast\"");
+  const int64_t rank = q.dim();
+  TORCH_CHECK(rank >= 2 && rank <= 5 && k.dim() == rank && v.dim() == rank,
+              "fp8_sdpa_recomp_fwd: q, k and v must have the same rank, between 2 and 5");
+  const bool has_mask = attention_mask.has_value() && attention_mask->defined();
+  TORCH_CHECK(!(has_mask && is_causal), "fp8_sdpa_recomp_fwd: attention_mask and is_causal exclude each other");
+  const int64_t L = q.size(-2), S = k.size(-2), Dk = q.size(-1), Dv = v.size(-1);
+  TORCH_CHECK(k.size(-1) == Dk, "fp8_sdpa_recomp_fwd: q and k must have the same head dimension");
+  TORCH_CHECK(v.size(-2) == S, "fp8_sdpa_recomp_fwd: k and v must have the same sequence length");
+  const at::ScalarType dt = q.scalar_type();
+  TORCH_CHECK(k.scalar_type() == dt && v.scalar_type() == dt, "fp8_sdpa_recomp_fwd: q, k and v must have the same dtype");
+  // batch dims broadcast like matmul's (SDPARecompFwdOutputShapeCommon)
+  std::vector<int64_t> qb(q.sizes().begin(), q.sizes().end() - 2), kb(k.sizes().begin(), k.sizes().end() - 2),
+      vb(v.sizes().begin(), v.sizes().end() - 2);
+  std::vector<int64_t> bshape = at::infer_size(at::infer_size(qb, kb), vb);
+  std::vector<int64_t> out_shape = bshape;
+  out_shape.push_back(L);
+  out_shape.push_back(Dv);
+  const bool fp8_in = is_fp8(dt);
+  const at::ScalarType out_dt = fp8_in ? (q_scale_o.given() ? at::kFloat8_e4m3fn : at::kBFloat16) : dt;
+  const at::ScalarType stat_dt = fp8_in ? at::kBFloat16 : dt;
+  auto opts = q.options();
+  Tensor out = at::empty(out_shape, opts.dtype(out_dt));
+  Tensor m = at::empty({1}, opts.dtype(stat_dt));
+  Tensor linv = at::empty({1}, opts.dtype(fp8_in || softmax_mode == "fast" ? at::kBFloat16 : at::kFloat));
+  Tensor seed = at::empty({1}, opts.dtype(at::kInt));
+  Tensor amax_s = at::empty({1}, opts.dtype(at::kFloat));
+  Tensor amax_o = at::empty({1}, opts.dtype(at::kFloat));
+  if (q.is_meta()) return SdpaOut(out, m, linv, seed, amax_s, amax_o);
+  DeviceGuard guard(q.device());
+  TORCH_CHECK(k.device() == q.device() && v.device() == q.device(), "fp8_sdpa_recomp_fwd: q, k and v must be on one device");
+  MI355Q_OP_INFO("fp8_sdpa_recomp_fwd : q=" << q.sizes() << " k=" << k.sizes() << " v=" << v.sizes() << " " << dt << " -> " << out_dt
+                                             << (is_causal ? " causal" : "") << (has_mask ? " mask" : ""));
+  m.zero_();
+  linv.zero_();
+  seed.zero_();
+
+  if (!fp8_in) {
+    // The measurement pass of the reference's flow: bf16 / fp32 q, k, v, no fp8 anywhere; only amax_s
+    // (and amax_o) are wanted from it.  It runs on the device's own matmul and softmax.
+    TORCH_CHECK(dt == at::kBFloat16 || dt == at::kFloat, "fp8_sdpa_recomp_fwd: q, k and v must be fp8, bfloat16 or float");
+    Tensor s = at::matmul(q, k.transpose(-2, -1)).to(at::kFloat) * scale;
+    if (has_mask) {
+      if (attention_mask->scalar_type() == at::kBool) s = s.masked_fill(attention_mask->logical_not(), -std::numeric_limits<float>::infinity());
+      else s = s + attention_mask->to(at::kFloat);
+    }
+    if (is_causal) {
+      Tensor keep = at::ones({L, S}, opts.dtype(at::kBool)).tril(0);
+      s = s.masked_fill(keep.logical_not(), -std::numeric_limits<float>::infinity());
+    }
+    Tensor pr = at::softmax(s, -1);
+    pr = at::nan_to_num(pr, 0.0);   // a row with every key masked
+    out.copy_(at::matmul(pr.to(dt), v));
+    if (pr.numel() > 0) amax_s.copy_(pr.max().reshape({1}));
+    else amax_s.zero_();
+    if (out.numel() > 0) amax_o.copy_(out.to(at::kFloat).abs().max().reshape({1}));
+    else amax_o.zero_();
+    return SdpaOut(out, m, linv, seed, amax_s, amax_o);
+  }
+
+  if (!is_amax_s) amax_s.zero_();
+  if (!is_amax_o) amax_o.zero_();
+  if (out.numel() == 0) {
+    amax_s.zero_();
+    amax_o.zero_();
+    return SdpaOut(out, m, linv, seed, amax_s, amax_o);
+  }
+  TORCH_CHECK(Dk <= 256 && Dv <= 256, "fp8_sdpa_recomp_fwd: head dimensions up to 256 are supported, got ", Dk, " and ", Dv);
+  Tensor qc = sdpa_unit_rows(q), kc = sdpa_unit_rows(k), vc = sdpa_unit_rows(v);
+  mi355q_sdpa_desc d{};
+  const int64_t nb = (int64_t)bshape.size();
+  for (int64_t i = 0; i < 3; ++i) d.batch[i] = 1;
+  for (int64_t i = 0; i < nb; ++i) d.batch[3 - nb + i] = bshape[i];
+  sdpa_batch_strides(qc, bshape, d.q_bstride, "q");
+  sdpa_batch_strides(kc, bshape, d.k_bstride, "k");
+  sdpa_batch_strides(vc, bshape, d.v_bstride, "v");
+  sdpa_batch_strides(out, bshape, d.out_bstride, "out");
+  d.q_len = L; d.kv_len = S; d.head_dim_qk = Dk; d.head_dim_v = Dv;
+  d.ldq = qc.stride(-2); d.ldk = kc.stride(-2); d.ldv = vc.stride(-2); d.ldo = out.stride(-2);
+  Tensor mk;
+  int mask_kind = MI355Q_SDPA_MASK_NONE;
+  if (has_mask) {
+    mk = *attention_mask;
+    TORCH_CHECK(mk.device() == q.device(), "fp8_sdpa_recomp_fwd: attention_mask must be on the same device as q");
+    TORCH_CHECK(mk.dim() >= 2 && mk.dim() <= rank, "fp8_sdpa_recomp_fwd: attention_mask must have between 2 and ", rank, " dimensions");
+    TORCH_CHECK((mk.size(-1) == S || mk.size(-1) == 1) && (mk.size(-2) == L || mk.size(-2) == 1),
+                "fp8_sdpa_recomp_fwd: attention_mask ", mk.sizes(), " does not broadcast to [..., ", L, ", ", S, "]");
+    if (mk.scalar_type() == at::kBool) mask_kind = MI355Q_SDPA_MASK_BOOL;
+    else if (mk.scalar_type() == at::kBFloat16) mask_kind = MI355Q_SDPA_MASK_BF16;
+    else {
+      mk = mk.to(at::kFloat);
+      mask_kind = MI355Q_SDPA_MASK_F32;
+    }
+    if (mk.size(-1) != S) {
+      std::vector<int64_t> full(mk.sizes().begin(), mk.sizes().end());
+      full.back() = S;
+      mk = mk.expand(full).contiguous();
+    } else if (mk.stride(-1) != 1 && S > 1) {
+      mk = mk.contiguous();
+    }
+    sdpa_batch_strides(mk, bshape, d.mask_bstride, "attention_mask");
+    d.ldmask = mk.size(-2) == 1 ? 0 : mk.stride(-2);
+  }
+  const SdpaScale* sc[6] = {&d_scale_q, &d_scale_k, &d_scale_v, &q_scale_s, &q_scale_o, &d_scale_s};
+  const float* sc_dev[6];
+  float sc_host[6];
+  for (int i = 0; i < 6; ++i) {
+    sc_dev[i] = sc[i]->dev;
+    sc_host[i] = sc[i]->host;
+  }
+  check_status(mi355q_fp8_sdpa_fwd(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), to_mi355q_dtype(dt), has_mask ? mk.data_ptr() : nullptr,
+                                   mask_kind, out.data_ptr(), to_mi355q_dtype(out_dt), &d, (float)scale, is_causal ? 1 : 0, sc_dev,
+                                   sc_host, is_amax_s ? amax_s.data_ptr<float>() : nullptr,
+                                   is_amax_o ? amax_o.data_ptr<float>() : nullptr, current_stream(q)),
+               "mi355q_fp8_sdpa_fwd");
+  return SdpaOut(out, m, linv, seed, amax_s, amax_o);
+}
+
+SdpaOut fp8_sdpa_recomp_fwd(const Tensor& q, const Tensor& k, const Tensor& v, const c10::optional<Tensor>& attention_mask, double p,
+                            double scale, bool is_causal, bool requires_backward, c10::string_view softmax_mode,
+                            const c10::optional<Tensor>& d_scale_q, const c10::optional<Tensor>& d_scale_k,
+                            const c10::optional<Tensor>& d_scale_v, const c10::optional<Tensor>& q_scale_s,
+                            const c10::optional<Tensor>& q_scale_o, const c10::optional<Tensor>& d_scale_s, bool is_amax_s,
+                            bool is_amax_o, const c10::optional<Tensor>& valid_seq_len, c10::string_view seq_padding_type) {
+  return fp8_sdpa_recomp_fwd_common(q, k, v, attention_mask, p, scale, is_causal, requires_backward, softmax_mode,
+                                    sdpa_scale(d_scale_q, q, "d_scale_q"), sdpa_scale(d_scale_k, q, "d_scale_k"),
+                                    sdpa_scale(d_scale_v, q, "d_scale_v"), sdpa_scale(q_scale_s, q, "q_scale_s"),
+                                    sdpa_scale(q_scale_o, q, "q_scale_o"), sdpa_scale(d_scale_s, q, "d_scale_s"), is_amax_s,
+                                    is_amax_o, valid_seq_len, seq_padding_type);
+}
+
+SdpaOut fp8_sdpa_recomp_fwd_scalar(const Tensor& q, const Tensor& k, const Tensor& v, const c10::optional<Tensor>& attention_mask,
+                                   double p, double scale, bool is_causal, bool requires_backward, c10::string_view softmax_mode,
+                                   double d_scale_q, double d_scale_k, double d_scale_v, double q_scale_s, double q_scale_o,
+                                   double d_scale_s, bool is_amax_s, bool is_amax_o, const c10::optional<Tensor>& valid_seq_len,
+                                   c10::string_view seq_padding_type) {
+  return fp8_sdpa_recomp_fwd_common(q, k, v, attention_mask, p, scale, is_causal, requires_backward, softmax_mode,
+                                    sdpa_scale(d_scale_q), sdpa_scale(d_scale_k), sdpa_scale(d_scale_v), sdpa_scale(q_scale_s),
+                                    sdpa_scale(q_scale_o), sdpa_scale(d_scale_s), is_amax_s, is_amax_o, valid_seq_len,
+                                    seq_padding_type);
+}
+
 // ------------------------------------------------------------- amax helpers
 
 Tensor amax_op(const Tensor& x) {
@@ -1139,6 +1344,8 @@ TORCH_LIBRARY(hpu, m) {
   m.def("hpu::softmax_fp8.Scalar_scales(Tensor input, int dim, float input_scale, float output_scale, Tensor? inv_attn_heads=None, Tensor? fused_add=None) -> Tensor");
   m.def("hpu::softmax_fp8.Scalar(Tensor input, int dim, float input_scale, float output_scale, float inv_attn_heads, Tensor? fused_add=None) -> Tensor");
   m.def("hpu::sum_fp8(Tensor self, int[1]? dim=None, bool keepdim=False, ScalarType? out_dtype=None) -> Tensor");
+  m.def("hpu::fp8_sdpa_recomp_fwd(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, bool requires_backward, str softmax_mode, Tensor? d_scale_q, Tensor? d_scale_k, Tensor? d_scale_v, Tensor? q_scale_s, Tensor? q_scale_o, Tensor? d_scale_s, bool is_amax_s, bool is_amax_0, Tensor? valid_seq_len, str seq_padding_type ) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)");
+  m.def("hpu::fp8_sdpa_recomp_fwd.scalar(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, bool requires_backward, str softmax_mode, float d_scale_q, float d_scale_k, float d_scale_v, float q_scale_s, float q_scale_o, float d_scale_s, bool is_amax_s, bool is_amax_0, Tensor? valid_seq_len, str seq_padding_type ) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)");
 }
 
 // Helpers the reference has no op for: amax alone and per-row amax.
@@ -1169,7 +1376,9 @@ TORCH_LIBRARY(mi355q, m) {
   m.impl("softmax_fp8", softmax_fp8);                                                          \
   m.impl("softmax_fp8.Scalar_scales", softmax_fp8_scalar_scales);                              \
   m.impl("softmax_fp8.Scalar", softmax_fp8_scalar);                                            \
-  m.impl("sum_fp8", sum_fp8);
+  m.impl("sum_fp8", sum_fp8);                                                                  \
+  m.impl("fp8_sdpa_recomp_fwd", fp8_sdpa_recomp_fwd);                                          \
+  m.impl("fp8_sdpa_recomp_fwd.scalar", fp8_sdpa_recomp_fwd_scalar);
 
 TORCH_LIBRARY_IMPL(hpu, CUDA, m) { MI355Q_REGISTER_HPU(m) }
 TORCH_LIBRARY_IMPL(hpu, Meta, m) { MI355Q_REGISTER_HPU(m) }

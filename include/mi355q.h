@@ -306,6 +306,53 @@ int mi355q_softmax_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols,
                        const void* fused_add, int row_dims, const int64_t* row_sizes,
                        const int64_t* fused_add_row_strides, void* y, int y_dtype, void* stream);
 
+/*
+ * Attention forward for inference on fp8 q, k, v:
+ *   S   = (q d_scale_q) (k d_scale_k)^T softmax_scale  [+ float mask | -inf where a bool mask
+ *         is 0 | -inf for key j > query i when is_causal]
+ *   out = softmax(S) (v d_scale_v)
+ * computed with an online softmax over blocks of 64 keys: with m the running row maximum,
+ * p = exp(S - m) in [0, 1] is rounded to fp8 (the format of v) as p * q_scale_s before the
+ * second product, the row sums use the unrounded p, both products accumulate in fp32, and the
+ * result is multiplied by d_scale_s (1 / q_scale_s when absent).  out is bf16, or e4m3fn holding
+ * out * q_scale_o (saturating round-to-nearest-even).  A query row whose keys are all masked
+ * by -inf gives zeros.  Replaces the "sdpa_recomp_fwd" node that hpu::fp8_sdpa_recomp_fwd
+ * builds with requires_backward false and dropout 0 (Fp8SDPARecompFwd::AddNode,
+ * hpu_ops/backend/sdpa_gen.cpp:806-1000; schema habana_eager/eager_custom_op_register.cpp:
+ * 2286-2296; the flags for valid_seq_len and dropout have no counterpart here).
+ *
+ * q is [batch..., q_len, head_dim_qk], k [batch..., kv_len, head_dim_qk], v [batch..., kv_len,
+ * head_dim_v], out [batch..., q_len, head_dim_v], the mask [batch..., q_len, kv_len] with unit
+ * column stride.  The up to three batch extents (outermost first, 1 where unused) are walked
+ * with one stride per tensor and extent, in elements; 0 broadcasts (grouped-query attention:
+ * k and v have stride 0 along the heads of a group).  ld* are row pitches in elements; ldmask 0
+ * repeats one mask row for all queries.  Head dimensions up to 256.
+ *
+ * scale_dev[6] / scale_host[6] hold d_scale_q, d_scale_k, d_scale_v, q_scale_s, q_scale_o,
+ * d_scale_s in that order: a device scalar where the pointer is not NULL, else the host value,
+ * 0 = absent (scale_dev itself may be NULL).  q_scale_o is read only for an e4m3fn out.
+ * amax_s / amax_o, where not NULL, receive max softmax probability and max |out| (before
+ * q_scale_o) as one fp32 each.
+ */
+typedef enum {
+  MI355Q_SDPA_MASK_NONE = 0,
+  MI355Q_SDPA_MASK_BOOL = 1, /* one byte per element, 0 = masked out */
+  MI355Q_SDPA_MASK_BF16 = 2, /* added to the scaled score */
+  MI355Q_SDPA_MASK_F32 = 3
+} mi355q_sdpa_mask_kind;
+
+typedef struct mi355q_sdpa_desc {
+  int64_t batch[3];
+  int64_t q_bstride[3], k_bstride[3], v_bstride[3], mask_bstride[3], out_bstride[3];
+  int64_t q_len, kv_len, head_dim_qk, head_dim_v;
+  int64_t ldq, ldk, ldv, ldmask, ldo;
+} mi355q_sdpa_desc;
+
+int mi355q_fp8_sdpa_fwd(const void* q, const void* k, const void* v, int fp8_fmt, const void* mask,
+                        int mask_kind, void* out, int out_dtype, const mi355q_sdpa_desc* desc,
+                        float softmax_scale, int is_causal, const float* const* scale_dev,
+                        const float* scale_host, float* amax_s, float* amax_o, void* stream);
+
 /* Name of the kernel variant mi355q_fp8_gemm would pick for a problem
  * (for logs and profiles; static string). */
 const char* mi355q_fp8_gemm_variant(int trans_a, int64_t lda, int trans_b, int64_t ldb,

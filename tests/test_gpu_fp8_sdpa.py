@@ -1,0 +1,291 @@
+"""GPU parity of hpu::fp8_sdpa_recomp_fwd (inference forward, fp8 q / k / v) against the CPU oracle.
+
+Floating point, so a tolerance, stated here once.  The oracle follows the kernel's own schedule (online
+softmax over blocks of 64 keys, probabilities rounded to fp8 before the second product) in float64; the
+device accumulates in fp32 and uses the hardware exp2, so two things separate them: the final rounding
+of an output that sits near a rounding boundary (one bf16 step = 2^-8 relative, one e4m3 step = 2^-3),
+and a probability that sits near an fp8 rounding boundary and falls to the other side (one e4m3 step on
+one of kv_len terms: about one probability in 10^4 does, and it moves the 'head_dim_v' outputs of its row
+by up to 2^-3 p_j / l |v_j|).  Bound used for a bf16 output: |out - ref| <= 2^-7 |ref| + 4e-3 max|ref| for
+all but 0.5 % of the values, and <= that + 2^-3 max|v d_scale_v| for every value; for an fp8 output at
+least 97 % of the codes are equal and the values obey the same two bounds with 2^-3 |ref| for 2^-7 |ref|.  The reference's own test
+compares the device with plain bf16 attention at atol 0.4 / rtol 1e-3 (fp8 run) -- that looser check is
+run as well (tests/pytest_working/any_mode/FusedSDPA/test_hpu_sdpa_fp8.py:1046-1052).
+"""
+import ctypes
+import math
+
+import pytest
+import torch
+
+from helpers import E4, E5
+
+pytestmark = pytest.mark.gpu
+
+NONE6 = (None,) * 6
+
+
+def make_qkv(gen, qshape, kshape, vshape, fmt=E4, spread=1.0):
+    q = (torch.randn(*qshape, generator=gen) * spread).to(fmt)
+    k = (torch.randn(*kshape, generator=gen) * spread).to(fmt)
+    v = torch.randn(*vshape, generator=gen).to(fmt)
+    return q, k, v
+
+
+def run_op(dev, q, k, v, mask=None, scale=None, causal=False, scales=NONE6, amax_s=False, amax_o=False, scalar=False):
+    scale = 1.0 / math.sqrt(q.shape[-1]) if scale is None else scale
+    if scalar:
+        sc = [0.0 if s is None else float(s) for s in scales]
+        op = torch.ops.hpu.fp8_sdpa_recomp_fwd.scalar
+    else:
+        sc = [None if s is None else torch.tensor([float(s)], device=dev) for s in scales]
+        op = torch.ops.hpu.fp8_sdpa_recomp_fwd
+    return op(q.to(dev), k.to(dev), v.to(dev), None if mask is None else mask.to(dev), 0.0, scale, causal, False, "None",
+              *sc, amax_s, amax_o, None, "left")
+
+
+def check_bf16(out, ref, what="", vmax=None):
+    """vmax: max |v * d_scale_v| (the largest value an output can take); max |ref| stands in when not given."""
+    out, ref = out.cpu().float(), ref.float()
+    assert out.shape == ref.shape, what
+    tol = ref.abs() * 2.0 ** -7 + 4e-3 * ref.abs().max()
+    err = (out - ref).abs()
+    bad = err > tol
+    assert float(bad.float().mean()) <= 5e-3, f"{what}: {int(bad.sum())} of {bad.numel()} outside the tight bound"
+    loose = tol + 2.0 ** -3 * (float(ref.abs().max()) if vmax is None else vmax)
+    assert not (err > loose).any(), f"{what}: worst {float((err - loose).max())} beyond one flipped probability"
+
+
+def check_fp8(out, ref, what=""):
+    """Codes equal for at least 97 % of the values; the others within one e4m3 step of the reference's
+    magnitude plus the absolute term of the bf16 bound (values near zero have tiny steps)."""
+    a, b = out.cpu().float(), ref.float()
+    same = out.cpu().view(torch.uint8) == ref.view(torch.uint8)
+    assert float(same.float().mean()) >= 0.97, f"{what}: only {float(same.float().mean()):.4f} of the codes agree"
+    tol = b.abs() * 2.0 ** -3 + 4e-3 * b.abs().max()
+    err = (a - b).abs()
+    assert float((err > tol).float().mean()) <= 5e-3, f"{what}: {int((err > tol).sum())} values beyond one step"
+    loose = tol + 2.0 ** -3 * b.abs().max()          # one flipped probability, as for a bf16 output
+    assert not (err > loose).any(), f"{what}: worst {float((err - loose).max())} beyond one flipped probability"
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [
+    # (batch, q_heads, kv_heads, q_len, kv_len, head_dim_qk, head_dim_v)
+    (3, 4, 4, 16, 32, 8, 8),        # the reference test's own case (test_hpu_sdpa_fp8.py:454-476)
+    (2, 3, 3, 128, 128, 64, 64),
+    (1, 2, 2, 200, 333, 128, 128),
+    (2, 2, 2, 257, 257, 128, 128),
+    (1, 2, 2, 130, 190, 256, 256),
+    (1, 2, 2, 96, 160, 72, 40),     # head dimensions that are no multiple of 16, and differ
+    (1, 1, 1, 1, 700, 128, 128),    # one query (decoding)
+    (2, 1, 1, 3, 64, 64, 128),
+])
+def test_against_oracle(oracle, dev, shape, causal):
+    B, H, HK, L, S, DK, DV = shape
+    gen = torch.Generator().manual_seed(L * 1000 + S + DK)
+    q, k, v = make_qkv(gen, (B, H, L, DK), (B, HK, S, DK), (B, HK, S, DV))
+    scales = (0.5, 2.0, 0.25, 128.0, None, 1.0 / 128.0)
+    out, m, linv, seed, amax_s, amax_o = run_op(dev, q, k, v, causal=causal, scales=scales, amax_s=True, amax_o=True)
+    assert out.dtype == torch.bfloat16 and m.shape == (1,) and linv.shape == (1,) and seed.dtype == torch.int32
+    ref, ref_as, ref_ao = oracle.torch_fp8_sdpa(q, k, v, is_causal=causal, d_scale_q=0.5, d_scale_k=2.0, d_scale_v=0.25,
+                                                q_scale_s=128.0, d_scale_s=1.0 / 128.0)
+    check_bf16(out, ref, str(shape))
+    assert abs(float(amax_s.cpu()) - float(ref_as)) <= 1e-4 * float(ref_as)
+    assert abs(float(amax_o.cpu()) - float(ref_ao)) <= 2e-3 * float(ref_ao)
+    # the reference test's own check: plain attention on the dequantised inputs, atol 0.4 / rtol 1e-3
+    keep = torch.ones(L, S, dtype=torch.bool).tril() if causal else None
+    plain = torch.nn.functional.scaled_dot_product_attention(q.float() * 0.5, k.float() * 2.0, v.float() * 0.25, attn_mask=keep)
+    assert torch.allclose(out.cpu().float(), plain, atol=0.4, rtol=1e-3)
+
+
+@pytest.mark.parametrize("scalar", [False, True])
+@pytest.mark.parametrize("causal", [False, True])
+def test_fp8_output(oracle, dev, causal, scalar):
+    """q_scale_o given: the output is e4m3fn holding out * q_scale_o (sdpa_gen.cpp:922-934)."""
+    gen = torch.Generator().manual_seed(5)
+    q, k, v = make_qkv(gen, (2, 4, 150, 128), (2, 4, 210, 128), (2, 4, 210, 128))
+    scales = (1.0, 1.0, 1.0, 128.0, 64.0, 1.0 / 128.0)
+    out = run_op(dev, q, k, v, causal=causal, scales=scales, scalar=scalar)[0]
+    assert out.dtype == E4
+    ref, _, _ = oracle.torch_fp8_sdpa(q, k, v, is_causal=causal, q_scale_s=128.0, q_scale_o=64.0, d_scale_s=1.0 / 128.0)
+    check_fp8(out, ref)
+    plain = torch.nn.functional.scaled_dot_product_attention(
+        q.float(), k.float(), v.float(), attn_mask=torch.ones(150, 210, dtype=torch.bool).tril() if causal else None)
+    assert torch.allclose(out.cpu().float() / 64.0, plain, atol=0.4, rtol=1e-3)
+
+
+def test_defaults_without_scales(oracle, dev):
+    """No scale given: all are 1, d_scale_s = 1 / q_scale_s = 1."""
+    gen = torch.Generator().manual_seed(6)
+    q, k, v = make_qkv(gen, (2, 100, 64), (2, 90, 64), (2, 90, 64))         # rank 3
+    out = run_op(dev, q, k, v)[0]
+    ref, _, _ = oracle.torch_fp8_sdpa(q, k, v)
+    check_bf16(out, ref)
+    # q_scale_s alone: d_scale_s defaults to its inverse
+    out = run_op(dev, q, k, v, scales=(None, None, None, 100.0, None, None))[0]
+    ref, _, _ = oracle.torch_fp8_sdpa(q, k, v, q_scale_s=100.0)
+    check_bf16(out, ref)
+
+
+@pytest.mark.parametrize("kind", ["bool", "bf16", "f32"])
+@pytest.mark.parametrize("mshape", ["Bx1x1xN", "BxHxLxN", "LxN", "1x1xLx1"])
+def test_attention_masks(oracle, dev, kind, mshape):
+    B, H, L, S, D = 2, 3, 70, 150, 64
+    gen = torch.Generator().manual_seed(7)
+    q, k, v = make_qkv(gen, (B, H, L, D), (B, H, S, D), (B, H, S, D))
+    shp = {"Bx1x1xN": (B, 1, 1, S), "BxHxLxN": (B, H, L, S), "LxN": (L, S), "1x1xLx1": (1, 1, L, 1)}[mshape]
+    keep = torch.rand(*shp, generator=gen) > 0.3
+    if mshape != "1x1xLx1":
+        keep[..., 0] = True
+    elif kind != "bool":
+        # a float mask that is -1e9 for every key of a row leaves fp32 no bits for the scores themselves
+        keep[...] = True
+    if kind == "bool":
+        mask = keep
+    else:
+        # the reference's float mask holds 0 and a large negative number (test_hpu_sdpa_fp8.py:272-276)
+        mask = torch.where(keep, 0.0, -1e9) + torch.where(keep, torch.randn(*shp, generator=gen) * 0.5, 0.0)
+        mask = mask.to(torch.bfloat16 if kind == "bf16" else torch.float32)
+    out = run_op(dev, q, k, v, mask=mask, scales=(None, None, None, 128.0, None, 1 / 128.0))[0]
+    ref, _, _ = oracle.torch_fp8_sdpa(q, k, v, attn_mask=mask, q_scale_s=128.0, d_scale_s=1 / 128.0)
+    check_bf16(out, ref, f"{kind} {mshape}")
+
+
+def test_rows_with_every_key_masked_give_zero(oracle, dev):
+    gen = torch.Generator().manual_seed(8)
+    q, k, v = make_qkv(gen, (1, 2, 40, 64), (1, 2, 100, 64), (1, 2, 100, 64))
+    keep = torch.rand(1, 1, 40, 100, generator=gen) > 0.5
+    keep[:, :, 5] = False
+    keep[:, :, 33] = False
+    out, _, _, _, amax_s, _ = run_op(dev, q, k, v, mask=keep, amax_s=True)
+    ref, ref_as, _ = oracle.torch_fp8_sdpa(q, k, v, attn_mask=keep)
+    assert (out.cpu()[:, :, [5, 33]] == 0).all()
+    check_bf16(out, ref)
+    assert abs(float(amax_s.cpu()) - float(ref_as)) <= 1e-4 * float(ref_as)
+
+
+def test_grouped_query_layout(oracle, dev):
+    """The 5-d views the reference's wrapper builds for grouped-query attention: q [B, G, H/G, L, D], k and
+    v [B, G, 1, S, D], mask [B, 1, 1, L, S] (Fp8FusedSDPA.py:49-77); and multi-query, kv_heads == 1."""
+    B, G, HG, L, S, D = 2, 2, 4, 90, 130, 128
+    gen = torch.Generator().manual_seed(9)
+    q, k, v = make_qkv(gen, (B, G, HG, L, D), (B, G, 1, S, D), (B, G, 1, S, D))
+    mask = torch.where(torch.rand(B, 1, 1, L, S, generator=gen) > 0.2, 0.0, -1e9).to(torch.bfloat16)
+    out = run_op(dev, q, k, v, mask=mask, scales=(None, None, None, 128.0, None, 1 / 128.0))[0]
+    assert out.shape == (B, G, HG, L, D)
+    ref, _, _ = oracle.torch_fp8_sdpa(q, k, v, attn_mask=mask, q_scale_s=128.0, d_scale_s=1 / 128.0)
+    check_bf16(out, ref)
+    q4, k4, v4 = make_qkv(gen, (B, 8, L, D), (B, 1, S, D), (B, 1, S, D))
+    out = run_op(dev, q4, k4, v4, causal=True)[0]
+    ref, _, _ = oracle.torch_fp8_sdpa(q4, k4, v4, is_causal=True)
+    check_bf16(out, ref)
+
+
+def test_e5m2_inputs(oracle, dev):
+    gen = torch.Generator().manual_seed(10)
+    q, k, v = make_qkv(gen, (2, 2, 100, 64), (2, 2, 140, 64), (2, 2, 140, 64), fmt=E5)
+    out = run_op(dev, q, k, v, causal=True, scales=(None, None, None, 1024.0, None, 1 / 1024.0))[0]
+    ref, _, _ = oracle.torch_fp8_sdpa(q, k, v, is_causal=True, q_scale_s=1024.0, d_scale_s=1 / 1024.0)
+    # e5m2 probabilities have a 2-bit mantissa: one flipped rounding weighs four times an e4m3 one
+    out, ref = out.cpu().float(), ref.float()
+    assert ((out - ref).abs() <= ref.abs() * 2.0 ** -7 + 1.5e-2 * ref.abs().max()).all()
+
+
+def test_q_scale_s_beyond_the_fp8_range_saturates(oracle, dev):
+    gen = torch.Generator().manual_seed(11)
+    q, k, v = make_qkv(gen, (1, 2, 64, 64), (1, 2, 64, 64), (1, 2, 64, 64), spread=3.0)
+    out = run_op(dev, q, k, v, scales=(None, None, None, 1000.0, None, 1e-3))[0]
+    ref, _, _ = oracle.torch_fp8_sdpa(q, k, v, q_scale_s=1000.0, d_scale_s=1e-3)
+    check_bf16(out, ref)
+
+
+def test_views_into_a_packed_projection(oracle, dev):
+    """q, k, v as strided views of one [B, L, 3, H, D] buffer (row pitch 3 H D), transposed to heads first."""
+    B, L, H, D = 2, 160, 4, 128
+    gen = torch.Generator().manual_seed(12)
+    qkv = torch.randn(B, L, 3, H, D, generator=gen).to(E4).to(dev)
+    q, k, v = (qkv[:, :, i].transpose(1, 2) for i in range(3))
+    assert not q.is_contiguous()
+    scale = 1.0 / math.sqrt(D)
+    out = torch.ops.hpu.fp8_sdpa_recomp_fwd(q, k, v, None, 0.0, scale, True, False, "fast", None, None, None, None, None, None,
+                                            False, False, None, "left")[0]
+    ref, _, _ = oracle.torch_fp8_sdpa(q.cpu(), k.cpu(), v.cpu(), is_causal=True)
+    check_bf16(out, ref)
+
+
+def test_long_sequence_properties(oracle, dev):
+    """At a size the CPU oracle does not finish in seconds: properties that fix the result.  With v = 1
+    everywhere every output is exactly d_scale_s q_scale_s-consistent 1 (a convex combination), rows of a
+    causal run equal the rows of the same keys without the later ones, and sampled rows match the oracle."""
+    B, H, L, D = 1, 4, 4096, 128
+    gen = torch.Generator().manual_seed(13)
+    q, k, v = make_qkv(gen, (B, H, L, D), (B, H, L, D), (B, H, L, D))
+    sc = (None, None, None, 128.0, None, 1 / 128.0)
+    out = run_op(dev, q, k, v, causal=True, scales=sc)[0].cpu()
+    # sampled rows against the oracle: row i of a causal run only sees keys <= i
+    for i in (0, 63, 64, 1000, 4095):
+        # the oracle's blocks must start where the device's do, so give it all keys up to the block's end
+        ref, _, _ = oracle.torch_fp8_sdpa(q[:, :, i:i + 1], k[:, :, :i + 1], v[:, :, :i + 1], q_scale_s=128.0, d_scale_s=1 / 128.0)
+        check_bf16(out[:, :, i:i + 1], ref, f"row {i}")
+    ones = torch.ones_like(v.float()).to(E4)
+    o1 = run_op(dev, q, k, ones, causal=True, scales=sc)[0].cpu().float()
+    # sum of fp8-rounded probabilities over the sum of unrounded ones: within the fp8 rounding, 2^-4
+    assert (o1 - 1.0).abs().max() <= 2.0 ** -4
+
+
+def test_argument_checks(dev):
+    q = torch.zeros(1, 2, 16, 64, device=dev).to(E4)
+    args = (None, 0.0, 0.125, False, False, "None", None, None, None, None, None, None, False, False, None, "left")
+    op = torch.ops.hpu.fp8_sdpa_recomp_fwd
+    with pytest.raises(RuntimeError, match="requires_backward"):
+        op(q, q, q, None, 0.0, 0.125, False, True, *args[5:])
+    with pytest.raises(RuntimeError, match="dropout"):
+        op(q, q, q, None, 0.1, *args[2:])
+    with pytest.raises(RuntimeError, match="valid_seq_len"):
+        op(q, q, q, *args[:14], torch.zeros(1, device=dev, dtype=torch.int32), "left")
+    with pytest.raises(RuntimeError, match="exclude each other"):
+        op(q, q, q, torch.ones(16, 16, device=dev, dtype=torch.bool), 0.0, 0.125, True, *args[4:])
+    with pytest.raises(RuntimeError, match="same head dimension"):
+        op(q, q[..., :32], q, *args)
+    big = torch.zeros(1, 1, 4, 320, device=dev).to(E4)
+    with pytest.raises(RuntimeError, match="up to 256"):
+        op(big, big, big, *args)
+
+
+def test_measurement_pass_with_bf16_inputs(dev):
+    """bf16 q, k, v with is_amax_s: the pass that measures max softmax probability before an fp8 run
+    (test_hpu_sdpa_fp8.py tc_list1).  No fp8 is involved; the device's own matmul and softmax run."""
+    gen = torch.Generator().manual_seed(14)
+    q = torch.randn(3, 4, 16, 8, generator=gen).bfloat16()
+    k = torch.randn(3, 4, 32, 8, generator=gen).bfloat16()
+    v = torch.randn(3, 4, 32, 8, generator=gen).bfloat16()
+    out, _, _, _, amax_s, _ = torch.ops.hpu.fp8_sdpa_recomp_fwd(
+        q.to(dev), k.to(dev), v.to(dev), None, 0.0, 1 / math.sqrt(8), True, False, "fast", None, None, None, None, None, None,
+        True, False, None, "left")
+    keep = torch.ones(16, 32, dtype=torch.bool).tril()
+    s = (q.float() @ k.float().transpose(-2, -1)) / math.sqrt(8)
+    p = torch.softmax(s.masked_fill(~keep, float("-inf")), -1)
+    assert out.dtype == torch.bfloat16
+    assert torch.allclose(out.cpu().float(), p @ v.float(), atol=0.08, rtol=1e-3)
+    assert abs(float(amax_s.cpu()) - float(p.max())) <= 0.05
+
+
+def test_c_entry_point_rejects_bad_arguments(pkg, dev):
+    lib = pkg.capi()
+    q = torch.zeros(16, 64, device=dev).to(E4)
+    out = torch.zeros(16, 64, device=dev, dtype=torch.bfloat16)
+    desc = (ctypes.c_int64 * 27)(*([1, 1, 1] + [0] * 15 + [16, 16, 64, 64] + [64, 64, 64, 0, 64]))
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ok = lib.mi355q_fp8_sdpa_fwd(q.data_ptr(), q.data_ptr(), q.data_ptr(), pkg.E4M3FN, None, 0, out.data_ptr(), pkg.BF16,
+                                 desc, 0.125, 0, None, None, None, None, st)
+    assert ok == 0
+    torch.cuda.synchronize()
+    assert (out == 0).all()          # v = 0
+    assert lib.mi355q_fp8_sdpa_fwd(q.data_ptr(), q.data_ptr(), q.data_ptr(), pkg.BF16, None, 0, out.data_ptr(), pkg.BF16,
+                                   desc, 0.125, 0, None, None, None, None, st) == 1
+    assert lib.mi355q_fp8_sdpa_fwd(q.data_ptr(), q.data_ptr(), q.data_ptr(), pkg.E4M3FN, None, 2, out.data_ptr(), pkg.BF16,
+                                   desc, 0.125, 0, None, None, None, None, st) == 1     # mask kind without a mask
+    desc[20] = 300                   # head_dim_qk
+    assert lib.mi355q_fp8_sdpa_fwd(q.data_ptr(), q.data_ptr(), q.data_ptr(), pkg.E4M3FN, None, 0, out.data_ptr(), pkg.BF16,
+                                   desc, 0.125, 0, None, None, None, None, st) == 2
