@@ -323,6 +323,12 @@ def bench_gemm_c3(ops, oracle, pkg, dev, steps, warmup, cpu):
                   steps, warmup)
     tflops = flop / (ms * 1e-3) / 1e12
     variant = pkg.capi().mi355q_fp8_gemm_variant(0, K, 0, N, M, N, K).decode()
+    # the same product with the weights stored [N, K] (trans_B=True), the layout the vendor library wants
+    w8_nk = w8.t().contiguous()
+    ms_nk = time_gpu(lambda i: ops.fp8_gemm_v2(a8, False, w8_nk, True, None, torch.bfloat16, sa_inv, sw_inv, bias, False),
+                     steps, warmup)
+    variant_nk = pkg.capi().mi355q_fp8_gemm_variant(0, K, 1, K, M, N, K).decode()
+    del w8_nk
     cpu_entry = None
     if cpu:
         rows = M
@@ -344,7 +350,8 @@ def bench_gemm_c3(ops, oracle, pkg, dev, steps, warmup, cpu):
         lib_tflops = round(flop / (lib_ms * 1e-3) / 1e12, 1)
     except Exception:  # noqa: BLE001 - the comparison is optional, the library may refuse the call
         pass
-    return {"ms": ms, "tflops": tflops, "flop": flop, "variant": variant, "cpu": cpu_entry, "library": lib_tflops}
+    return {"ms": ms, "tflops": tflops, "flop": flop, "variant": variant, "cpu": cpu_entry, "library": lib_tflops,
+            "ms_nk": ms_nk, "tflops_nk": flop / (ms_nk * 1e-3) / 1e12, "variant_nk": variant_nk}
 
 
 def bench_gemm_decode(ops, oracle, dev, steps, warmup):
@@ -387,6 +394,74 @@ def bench_gemm_decode(ops, oracle, dev, steps, warmup):
                              f"C4 fp8_gemm_v2 M={M} K=8192 N=28672 per-token x per-channel scales -> bf16",
                              nbytes, ms, steps, "fp8_gemm_skinny_kernel" if M <= 128 else "fp8_gemm_tile_kernel<256,128>",
                              extra={"tflops": round(flop / (ms * 1e-3) / 1e12, 2), "library_gemm_ms_same_shape": lib_ms}))
+    return out
+
+
+def bench_w4a8(oracle, dev, steps, warmup, cpu):
+    """The decode-shaped GEMM of configuration 4 with int4 weights: uint4 nibbles [K, N / 8] int32, bf16 scales and
+    packed zero points per group of 128 along K, per-token e4m3fn activations; the weights are expanded inside the
+    GEMM.  HBM-bound: the algorithmic bytes are the packed weights, their scales and zero points, A and C."""
+    out = []
+    gen = torch.Generator().manual_seed(SEED)
+    K, N, G = 8192, 28672, 128
+    packs = []
+    for _ in range(3):   # three weight sets (3 x 117 MiB) exceed the Infinity Cache
+        packs.append(torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), generator=gen, dtype=torch.int64).to(torch.int32).to(dev))
+    scale = (torch.rand(K // G, N, generator=gen) * 0.019 + 0.001).bfloat16().to(dev)
+    zp = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // G, N // 8), generator=gen, dtype=torch.int64).to(torch.int32).to(dev)
+    cols = torch.randperm(K, generator=gen)[:82]
+    for M in (16, 64, 256):
+        x = torch.randn(M, K, generator=gen)
+        x[:, cols] *= 20
+        x8, sx_inv = torch.ops.mi355q.quantize_rows(x.bfloat16().to(dev), E4)
+        ms = time_gpu(lambda i: torch.ops.mi355q.w4a8_gemm(x8, packs[i % 3], scale, zp, False, torch.bfloat16, sx_inv, None),
+                      steps, warmup)
+        nbytes = K * N // 2 + (K // G) * N * 2 + (K // G) * N // 2 + M * K + 2 * M * N + 4 * M
+        c = None
+        if cpu and M == 16:
+            rows_n = 1024    # a bounded sample: 1024 of the 28672 output columns
+            pk, sc_c, zp_c = packs[0][:, :rows_n // 8].cpu(), scale[:, :rows_n].cpu(), zp[:, :rows_n // 8].cpu()
+            x8c, sxc = x8.cpu(), sx_inv.cpu()
+            t = time_cpu(lambda: oracle.torch_w4a8_gemm(x8c, pk, sc_c, zp_c, False, torch.bfloat16, sxc), min_seconds=3.0)
+            c = {"value": round((K * rows_n // 2) / t / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                 "sample": f"M=16, {rows_n} of the 28672 output columns: unpack, (q - z) * s in float64, matmul, per-row scale"}
+        out.append(hbm_entry(f"w4a8_gemm_M{M}", f"w4a8_gemm M={M} K=8192 N=28672: uint4 weights (group 128, bf16 scales, packed "
+                                                "zero points) x per-token e4m3fn activations -> bf16",
+                             nbytes, ms, steps, "w4a8_gemm_kernel", c,
+                             extra={"tflops": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 2)}))
+    return out
+
+
+def bench_sdpa(oracle, dev, steps, warmup, cpu):
+    """hpu::fp8_sdpa_recomp_fwd, Llama-3-8B attention shapes (32 query heads, 8 key/value heads, head dimension 128),
+    causal, e4m3fn q / k / v, q_scale_s = 128, bf16 output.  MFMA-bound: 4 L S D flop per head, halved by the mask."""
+    import math
+    out = []
+    gen = torch.Generator().manual_seed(SEED)
+    H, HK, D = 32, 8, 128
+    sc = 1.0 / math.sqrt(D)
+    for B, L in ((1, 8192), (4, 4096)):
+        q = torch.randn(B, HK, H // HK, L, D, generator=gen).to(E4).to(dev)     # the grouped-query view of [B, H, L, D]
+        k = torch.randn(B, HK, 1, L, D, generator=gen).to(E4).to(dev)
+        v = torch.randn(B, HK, 1, L, D, generator=gen).to(E4).to(dev)
+        f = lambda i: torch.ops.hpu.fp8_sdpa_recomp_fwd.scalar(q, k, v, None, 0.0, sc, True, False, "None", 1.0, 1.0, 1.0, 128.0,
+                                                               0.0, 1.0 / 128.0, False, False, None, "left")
+        ms = time_gpu(f, steps, warmup)
+        flop = 4.0 * B * H * L * L * D * 0.5
+        tf = flop / (ms * 1e-3) / 1e12
+        e = {"name": f"fp8_sdpa_B{B}_L{L}", "workload": f"fp8_sdpa_recomp_fwd causal, batch {B}, 32 query / 8 kv heads, "
+                                                        f"q_len = kv_len = {L}, head_dim 128, e4m3fn -> bf16",
+             "metric": "TFLOP/s", "value": round(tf, 1), "unit": "TFLOP/s", "ms_per_call": round(ms, 4), "steps": steps,
+             "roofline": {"bound": "mfma", "kernel": "fp8_sdpa_fwd_kernel<2,4,e4m3fn>", "achieved": round(tf, 1),
+                          "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / FP8_PEAK_TFLOPS, 4),
+                          "algorithmic_flop": flop, "traffic": MEASURED_TRAFFIC.get(f"fp8_sdpa_B{B}_L{L}")}}
+        if cpu and B == 1:
+            n = 1024    # a bounded sample: one head, the first 1024 queries and keys
+            qc, kc, vc = q[0, 0, 0, :n].cpu(), k[0, 0, 0, :n].cpu(), v[0, 0, 0, :n].cpu()
+            t = time_cpu(lambda: oracle.torch_fp8_sdpa(qc, kc, vc, is_causal=True, q_scale_s=128.0, d_scale_s=1 / 128.0), min_seconds=3.0)
+            e["cpu_baseline"] = {"value": round(4.0 * n * n * D * 0.5 / t / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                                 "kind": "port", "sample": f"one head, {n} queries x {n} keys, the float64 oracle"}
+        out.append(e)
     return out
 
 
@@ -459,7 +534,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,cast,int4,decode,mlp,reduce")
+    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,cast,int4,decode,mlp,reduce,w4a8,sdpa")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -476,7 +551,7 @@ def main():
     ops = torch.ops.hpu
     dev = torch.device("cuda:0")
     torch.set_num_threads(min(os.cpu_count() or 1, 16))
-    which = set(args.only.split(",")) if args.only else {"gemm", "cast", "int4", "decode", "mlp", "reduce"}
+    which = set(args.only.split(",")) if args.only else {"gemm", "cast", "int4", "decode", "mlp", "reduce", "w4a8", "sdpa"}
     cpu = not args.no_cpu
     k_stream = max(args.steps, 50)      # the microsecond-scale kernels need more calls for a stable mean
     w_stream = max(args.warmup, 10)
@@ -492,6 +567,10 @@ def main():
         ops_out.append(bench_mlp(ops, dev, max(args.steps // 2, 5), args.warmup))
     if "reduce" in which:
         ops_out += bench_reductions(pkg, oracle, dev, args.steps, args.warmup, cpu)
+    if "w4a8" in which:
+        ops_out += bench_w4a8(oracle, dev, args.steps, args.warmup, cpu)
+    if "sdpa" in which:
+        ops_out += bench_sdpa(oracle, dev, args.steps, args.warmup, cpu)
 
     line = {"metric": "cast/dequant GB/s (% HBM peak); fp8_gemm_v2 TFLOP/s (% fp8 MFMA peak)",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
@@ -509,6 +588,13 @@ def main():
                                   "algorithmic_flop": g["flop"], "traffic": MEASURED_TRAFFIC.get("fp8_gemm_v2")}})
         if g["cpu"]:
             line["cpu_baseline"] = g["cpu"]
+        ops_out.insert(0, {"name": "fp8_gemm_v2_B_NK", "workload": "C3 with the weights stored [N=14336, K=4096] (trans_B=True)",
+                           "metric": "TFLOP/s", "value": round(g["tflops_nk"], 1), "unit": "TFLOP/s",
+                           "ms_per_call": round(g["ms_nk"], 4), "steps": args.steps, "kernel_variant": g["variant_nk"],
+                           "roofline": {"bound": "mfma", "kernel": "fp8_gemm_tile_kernel", "achieved": round(g["tflops_nk"], 1),
+                                        "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                        "frac": round(g["tflops_nk"] / FP8_PEAK_TFLOPS, 4), "algorithmic_flop": g["flop"],
+                                        "traffic": MEASURED_TRAFFIC.get("fp8_gemm_v2_B_NK")}})
     else:
         first = ops_out[0]
         line.update({"value": first["value"], "unit": first["unit"], "ms_per_step": first["ms_per_call"],

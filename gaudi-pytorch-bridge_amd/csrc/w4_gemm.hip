@@ -4,31 +4,45 @@
 //
 // The weights are what convert_from_int4 / convert_from_uint4 take (packed int32
 // [K, N / 8], nibble i of word p is column 8 p + i; group-wise scales [K / g, N];
-// packed zero-points [K / g, N / 8]), but they are never written out as bf16 [K, N]:
-// a weight stage travels from HBM to LDS as packed nibbles (half the bytes of fp8
-// weights, a quarter of bf16), the workgroup turns it into fp8 codes of the integers
-// (q - z) in LDS (|q - z| <= 15 is exact in e4m3), the fp8 MFMA accumulates one K
-// group at a time in fp32, and the group's scales multiply the partial sums as they
-// are added to the totals.  So the weights enter the product exactly.
+// packed zero-points [K / g, N / 8]), but they are never written out as bf16 [K, N],
+// nor as fp8: a weight stage travels from HBM to LDS as packed nibbles (half the bytes
+// of fp8 weights, a quarter of bf16) and goes from there into the MFMA as it is.
 //
-// Shaped like the strip kernel of gemm_skinny.h (weights streamed once through a deep
-// LDS ring, one 4-wave workgroup per 128 columns); rows of A beyond 128 run as further
-// row blocks that stream the weights again, which suits decode and small prefill
-// batches, the shapes weight-only quantisation is used for.
+// How a nibble becomes an MFMA operand.  v_mfma_scale_f32_32x32x64_f8f6f4 multiplies an
+// fp8 operand by an fp4 (e2m1) one, and the e2m1 codes 0, 1, 2, 3 stand for 0, 0.5, 1,
+// 1.5: a two-bit integer v, zero-extended to four bits, is the e2m1 code of v / 2.  An
+// unsigned nibble q = 4 hi + lo therefore splits into two planes, (w >> 2) & 0x33333333
+// and w & 0x33333333 on eight nibbles at a time, and two MFMAs with the block scales 2^3
+// and 2^1 accumulate sum_k a q exactly.  The zero-point leaves the inner loop:
+// sum_k a (q - z) = sum_k a q - z sum_k a, and sum_k a comes from a third MFMA against
+// a plane of ones.  (A signed nibble s is q = s ^ 8 = s + 8 with z + 8.)  ds_read_b64_tr_b4
+// turns the packed rows (16 columns in 8 bytes) into the 16 consecutive k of one column
+// that an MFMA lane wants, so the only vector ALU work per 64 x 32 weights is the two
+// masks and a shift per register.
 //
-// Per K stage of 128, one barrier: behind it a wave issues the loads of the stage S - 1
-// ahead, reads the fragments of stage kt (A from the ring, the weights from the fp8 tile
-// that the previous step unpacked) and issues its 2 MFMA blocks into the group's
-// accumulators, then turns the packed tile of stage kt + 1 into the other fp8 tile (a
-// thread converts 8 words: one column word of 8 rows, so its 8 zero-points are set up
-// once per stage) while the MFMAs run, and at the end of a group adds scale * group to
-// the totals.
+// Relative to an fp8 operand whose lane holds k = 32 h + j in byte j (h = lane / 32),
+// the fp4 operand of the same MFMA holds k = 16 h + j in nibble j < 16 and
+// k = 32 + 16 h + (j - 16) in nibble j >= 16.
+//
+// Shaped like the strip kernel of gemm_skinny.h: the weights stream once through a deep LDS
+// ring, one workgroup per 128 columns; rows of A beyond 64 run as further row blocks that
+// stream the weights again, which suits decode and small prefill batches, the shapes
+// weight-only quantisation is used for.  A workgroup has eight waves, two per SIMD, with
+// two roles.  Waves 4..7 are producers: they issue the global -> LDS loads of a stage (packed
+// weights, activations, the scale row and the zero-point row of the stage's group), wait for
+// them, and do nothing else.  Waves 0..3 are consumers: wave w owns columns 32 w .. 32 w + 31
+// and does the LDS reads, the MFMAs and the scaling, with no load, no wait counter and no
+// descriptor arithmetic in its loop.  A wave issues at most one instruction every few cycles,
+// so at 16 useful rows the K loop is bound by the number of instructions per stage, not by the
+// MFMAs: keeping each role's loop short is what the split is for.  The roles meet at one
+// barrier per K stage of 128.  At the end of a group of K the group's scales multiply the
+// partial sums into the totals, in fp32.
 #include "gemm_tile.h"
 
 namespace mi355q {
 
-constexpr int kW4Threads = 256;
-constexpr int kW4Waves = 4;
+constexpr int kW4Threads = 512;
+constexpr int kW4ColWaves = 4;                   // consumer waves side by side along N; as many producers
 constexpr int kW4BN = 128;                       // columns per workgroup
 constexpr int kW4PackedStage = kBK * kW4BN / 2;  // bytes of packed weights per stage (128 k-rows of 64 bytes)
 // The stage's scale row (bf16 or fp32, at most 512 bytes) and its packed zero-points (16 words) each
@@ -52,8 +66,8 @@ constexpr int w4_stage_bytes() { return BM * kBK + kW4PackedStage + kW4ScaleRow 
 
 template <int BM>
 constexpr int w4_stages() {
-  constexpr int s = (160 * 1024 - 2 * kBK * kW4BN) / w4_stage_bytes<BM>();
-  return s > 8 ? 8 : s;
+  constexpr int s = (160 * 1024) / w4_stage_bytes<BM>();
+  return s > 10 ? 10 : s;
 }
 
 // One 16-byte piece per lane, straight copy into LDS (lane l lands at dst + 16 l).  The
@@ -66,34 +80,54 @@ __device__ __forceinline__ void w4_dma16(const i32x4& rsrc, int voff, uint32_t l
                : "memory", "m0");
 }
 
-__device__ __forceinline__ i32x4 w4_rsrc(const uint8_t* base, int64_t bytes) {
-  const uint64_t b = reinterpret_cast<uint64_t>(base);
-  const int64_t rec = bytes < 0 ? 0 : (bytes > 0x7fffffffLL ? 0x7fffffffLL : bytes);
-  i32x4 r;
-  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
-  r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((b >> 32) & 0xffffu));
-  r[2] = __builtin_amdgcn_readfirstlane((int)rec);
-  r[3] = 0x00020000;
-  return r;
+// A buffer descriptor that walks through memory in fixed steps: base and the bytes left behind it.
+struct W4Walker {
+  uint64_t base;
+  int64_t left;   // bytes from base to the end of what may be read; <= 0: every load reads zeros
+  __device__ __forceinline__ void init(const uint8_t* p, int64_t bytes) {
+    base = reinterpret_cast<uint64_t>(p);
+    left = bytes;
+  }
+  __device__ __forceinline__ void step(int64_t d) {
+    base += (uint64_t)d;
+    left -= d;
+  }
+  // at most `cap` bytes from the base on
+  __device__ __forceinline__ i32x4 rsrc(int64_t cap) const {
+    int64_t rec = left < cap ? left : cap;
+    rec = rec < 0 ? 0 : (rec > 0x7fffffffLL ? 0x7fffffffLL : rec);
+    i32x4 r;
+    r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)base);
+    r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((base >> 32) & 0xffffu));
+    r[2] = __builtin_amdgcn_readfirstlane((int)rec);
+    r[3] = 0x00020000;
+    return r;
+  }
+};
+
+// fp4 plane (first operand, its four registers) times fp8 fragment, block scale 2^(E - 127) on the plane
+template <int FMT_A, int E>
+__device__ __forceinline__ f32x16 w4_mfma(const u32x4& plane, const i32x8& fa, const f32x16& c) {
+  const i32x8 b = {(int)plane[0], (int)plane[1], (int)plane[2], (int)plane[3], 0, 0, 0, 0};
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, fa, c, 4, mfma_code<FMT_A>(), 0, E, 0, 127);
 }
 
-template <int BM, int FMT_A>
+// PIPE: the partial sums of a group are folded into the totals one group late, from a second set of
+// accumulators, while the next group's MFMAs run: a wave does not stall on the MFMAs it has just issued.
+template <int BM, int FMT_A, bool PIPE>
 __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
   constexpr int MT = BM / 32;
   constexpr int S = w4_stages<BM>();
   constexpr int kStage = w4_stage_bytes<BM>();
   constexpr int kOffPacked = BM * kBK, kOffScale = kOffPacked + kW4PackedStage, kOffZp = kOffScale + kW4ScaleRow;
-  using LA = DmaLoader<true, BM, kBK, kW4Waves>;
-  using GB = TileGeom<false, kBK, kW4BN>;  // the unpacked weight tile: 128 k-rows of 128 fp8 columns
-  // per wave and stage: its share of A, two 1 KiB regions of packed weights, the scale row, the zero-point row
-  constexpr int kOps = LA::kPerWave + 2 + 2;
-  constexpr int kInFlight = (S - 3) * kOps;  // stage kt + 1 is needed while stage kt is multiplied
-  static_assert(S >= 4 && kInFlight <= 63, "vmcnt holds 6 bits");
+  using LA = DmaLoader<true, BM, kBK, kW4ColWaves>;
+  // loads per producer wave and stage: two 1 KiB regions of packed weights, its share of A, and the scale
+  // row or the zero-point row
+  constexpr int kOps = 2 + LA::kPerWave + 1;
+  static_assert(S >= 3 && (S - 2) * kOps <= 63, "vmcnt holds 6 bits");
   static_assert(kStage % 1024 == 0, "stages stay 1 KiB aligned");
-  static_assert(kW4Waves * epilogue_stage_floats<MT, 1>() * 4 <= S * kStage, "epilogue area overlays the ring");
-  constexpr int kTile = kBK * kW4BN;  // one unpacked fp8 tile
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[S * kStage + 2 * kTile];
-  uint8_t* const unp = lds + S * kStage;  // two tiles, used in turn
+  static_assert(kW4ColWaves * epilogue_stage_floats<MT, 1>() * 4 <= S * kStage, "epilogue area overlays the ring");
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[S * kStage];
 
   // this workgroup's rows and columns
   GemmArgs g = a.g;
@@ -102,180 +136,253 @@ __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
   g.C += (int64_t)m_base * g.ldc * (g.out_bf16 ? 2 : 4);
   if (g.sa_mode == MI355Q_GS_PER_ROW) g.sa += m_base;
   g.M = g.M - m_base < BM ? g.M - m_base : BM;
-  const int n0 = blockIdx.x * kW4BN;
+  // A strip's packed rows are 64 bytes, half a cache line; the other half belongs to the next strip.
+  // Workgroups go to the 8 XCDs round robin: strips 2 j and 2 j + 1 are given to workgroups 8 apart, which
+  // share an XCD (and its L2) and run at the same time.
+  int strip = blockIdx.x;
+  if ((gridDim.x & 15) == 0) strip = (((strip >> 4) << 3) + (strip & 7)) * 2 + ((strip >> 3) & 1);
+  const int n0 = strip * kW4BN;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool producer = wave >= kW4ColWaves;
+  const int wq = wave & 3;
   const int lane = lane_id_here();
-  const int wn = wave * 32;
   const int KT = (g.K + kBK - 1) / kBK;
 
-  LA la;
-  la.init(g.A, g.lda, 0, g.M, g.K);
-  la.clamp_rows(g.lda, g.M);
-  // packed weights: this wave's two regions are k-rows 32 wave .. 32 wave + 31 of the stage (16 rows of 64 bytes each)
-  const int64_t packed_bytes = (int64_t)(g.K - 1) * a.ld_packed + (((g.N + 31) & ~31) - n0) / 2;
-  const uint8_t* const packed0 = a.packed + n0 / 2;
-  const int voff_packed = (wave * 32 + (lane >> 2)) * (int)a.ld_packed + (lane & 3) * 16;
-  const int region_packed = 16 * (int)a.ld_packed;
-  const int es = a.scale_f32 ? 4 : 2;
-  const int64_t scale_row_bytes = (int64_t)(g.N - n0 < kW4BN ? g.N - n0 : kW4BN) * es;
-  const int64_t zp_row_bytes = (int64_t)(g.N - n0 < kW4BN ? g.N - n0 : kW4BN) / 2;
+  if (producer) {
+    LA la;
+    la.set_lane_offsets(g.lda, wq);
+    la.set_tile(g.A, g.lda, 0, g.M, g.K);
+    la.clamp_rows(g.lda, g.M);
+    // Packed weights: producer wq loads k-rows 32 wq .. 32 wq + 31 of the stage, two regions of 16 rows of
+    // 64 bytes.  The 16-byte slots of a row are stored XORed with (row / 4) % 4, which makes the consumers'
+    // transposing reads conflict free; a lane writes slot lane % 4 of row lane / 4 of its region, so it
+    // fetches slot (lane % 4) ^ (lane / 16) of that row.
+    const int voff_packed = (wq * 32 + (lane >> 2)) * (int)a.ld_packed + ((lane & 3) ^ ((lane >> 4) & 3)) * 16;
+    const int region_packed = 16 * (int)a.ld_packed;
+    const int64_t packed_step = (int64_t)kBK * a.ld_packed;
+    W4Walker wp;
+    wp.init(a.packed + n0 / 2, (int64_t)(g.K - 1) * a.ld_packed + (((g.N + 31) & ~31) - n0) / 2);
+    // Producers 0 and 1 bring the scale row, 2 and 3 the zero-point row (the same bytes twice: every
+    // producer then has the same number of loads per stage, all of which go to memory, which the counted
+    // wait below relies on; without zero-points the scale row stands in).
+    const int es = a.scale_f32 ? 4 : 2;
+    const int cols = g.N - n0 < kW4BN ? g.N - n0 : kW4BN;
+    const bool bring_zp = wq >= 2 && a.zp != nullptr;
+    const int64_t row_cap = bring_zp ? cols / 2 : (int64_t)cols * es;
+    const int64_t row_step = bring_zp ? g.N / 2 : (int64_t)g.N * es;
+    const int row_dst = wq < 2 ? kOffScale : kOffZp;
+    W4Walker wr;
+    wr.init(bring_zp ? a.zp + n0 / 2 : a.scale + (int64_t)n0 * es, (int64_t)((KT + a.stages_per_group - 1) / a.stages_per_group - 1) * row_step + row_cap);
+    int in_group = 0;
 
-  int issued = 0;  // stages issued so far: stage `issued` goes out next
-  auto issue_stage = [&](int off) {
-    const int stage = issued;
-    const uint32_t base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)(lds + off);
-    static_for<LA::kPerWave>([&](auto ic) { la.template issue_one<decltype(ic)::value, true>(lds + off, stage * kBK, g.K); });
-    la.advance();
-    // beyond K everything is out of range and arrives as zeros (A's zeros make the products vanish)
-    const int64_t k_off = (int64_t)stage * kBK * a.ld_packed;
-    const i32x4 rp = w4_rsrc(packed0 + k_off, stage < KT ? packed_bytes - k_off : 0);
-    w4_dma16(rp, voff_packed, base + kOffPacked + (wave * 2) * 1024);
-    w4_dma16(rp, voff_packed + region_packed, base + kOffPacked + (wave * 2 + 1) * 1024);
-    const int grp = stage / a.stages_per_group;
-    const i32x4 rs = w4_rsrc(a.scale + ((int64_t)grp * g.N + n0) * es, stage < KT ? scale_row_bytes : 0);
-    w4_dma16(rs, lane * 16, base + kOffScale);
-    // (without zero-points the scale row is fetched once more: every stage's loads are of the same
-    // number and all go to memory, which the counted wait below relies on)
-    const i32x4 rz = a.zp ? w4_rsrc(a.zp + ((int64_t)grp * g.N + n0) / 2, stage < KT ? zp_row_bytes : 0) : rs;
-    w4_dma16(rz, lane * 16, base + kOffZp);
-    ++issued;
-  };
+    auto issue_stage = [&](int off, int stage) {
+      const uint32_t base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)(lds + off);
+      // beyond K everything is out of range and arrives as zeros (A's zeros make the products vanish)
+      const i32x4 rp = wp.rsrc(0x7fffffffLL);
+      w4_dma16(rp, voff_packed, base + kOffPacked + (wq * 2) * 1024);
+      w4_dma16(rp, voff_packed + region_packed, base + kOffPacked + (wq * 2 + 1) * 1024);
+      wp.step(packed_step);
+      static_for<LA::kPerWave>([&](auto ic) { la.template issue_one<decltype(ic)::value, true>(lds + off, stage * kBK, g.K); });
+      la.advance();
+      w4_dma16(wr.rsrc(row_cap), lane * 16, base + row_dst);
+      if (++in_group == a.stages_per_group) {
+        in_group = 0;
+        wr.step(row_step);
+      }
+    };
+    // waits until at most min(later, S - 2) stages' loads of this wave are outstanding
+    auto wait_for_stage = [&](int later) {
+      constexpr int full = (S - 2) * kOps;
+      if (later >= S - 2) {
+        __builtin_amdgcn_s_waitcnt((full & 15) | ((full >> 4) << 14) | 0x0070);
+      } else {
+        static_for<S - 2>([&](auto sc) {
+          constexpr int n = decltype(sc)::value;  // 0 .. S - 3
+          constexpr int cnt = n * kOps;
+          if (later == n || (n == 0 && later < 0)) __builtin_amdgcn_s_waitcnt((cnt & 15) | ((cnt >> 4) << 14) | 0x0070);
+        });
+      }
+    };
 
-  f32x16 total[MT][1], part[MT];
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) issue_stage(s * kStage, s);
+    int wr_off = (S - 1) * kStage;
+    for (int kt = 0; kt < KT; ++kt) {
+      // The loads of stage kt have landed once only those of later stages are outstanding; the
+      // zero-fill loads past K complete at once and are not counted (see gemm_skinny.h).
+      wait_for_stage(KT - 1 - kt);
+      // stage kt is in LDS for the consumers, who are done with stage kt - 1, whose room the next loads take
+      __syncthreads();
+      issue_stage(wr_off, kt + S - 1);
+      wr_off += kStage;
+      if (wr_off == S * kStage) wr_off = 0;
+    }
+    // the ring is idle (zero-fill loads of the stages past K included) before the epilogue overlays it
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    return;
+  }
+
+  // ------------------------------------------------------------------ consumers
+  const int wn = wq * 32;
+  constexpr int NB = PIPE ? 2 : 1;
+  f32x16 total[MT][1], part[NB][MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) total[i][0][e] = 0.0f;
 
-#pragma unroll
-  for (int s = 0; s < S - 1; ++s) issue_stage(s * kStage);
-
-  // unpacking: this thread's column word and its 8 rows of the stage
-  const int uw = threadIdx.x & 15, ur0 = threadIdx.x >> 4;
   const uint32_t flip = a.is_signed ? 0x88888888u : 0u;  // signed nibble s = (q ^ 8) - 8
-  const float zbias = a.is_signed ? 8.0f : 0.0f;
+  const bool has_z = a.zp != nullptr || a.is_signed;
+  // this lane's part in the transposing reads: its 16-lane group covers 16 columns, the lane points at one
+  // k-row; th is the k-half of the MFMA that the lane's rows belong to
+  const int tg = lane >> 4, tr = lane & 15, th = tg >> 1;
+  // byte offsets inside a packed stage of this lane's four reads: k-rows 64 ks + 32 p + 16 th + tr
+  int poff[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = 32 * j + 16 * th + tr;
+    poff[j] = kOffPacked + row * 64 + ((wq ^ ((row >> 2) & 3)) << 4) + (tg & 1) * 8;
+  }
+  const int zoff = kOffZp + ((wn + (lane & 31)) >> 3) * 4, zshift = 4 * (lane & 7);
+  const int soff = kOffScale + (wn + 4 * (lane >> 5)) * (a.scale_f32 ? 4 : 2);
 
-  // packed nibbles of the stage at `st` -> fp8 codes of (q - z) in the tile at `dst`
-  auto unpack = [&](const uint8_t* st, uint8_t* dst) {
-    const uint32_t zw = (a.zp ? *reinterpret_cast<const uint32_t*>(st + kOffZp + uw * 4) : 0u) ^ flip;
-    float z[8];
+  // the scales of this lane's 16 columns (wn + 8 q + 4 (lane / 32) + e) for the group that ended last
+  float sc[16];
+  u32x4 sraw[4];  // as read from the stage's scale row: four fp32, or four bf16 in the first two words
+  auto convert_scales = [&]() {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) z[i] = a.zp ? (float)((zw >> (4 * i)) & 15u) : zbias;
+    for (int q = 0; q < 4; ++q) {
+      if (a.scale_f32) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int r = ur0 + 16 * i;
-      const uint32_t w = *reinterpret_cast<const uint32_t*>(st + kOffPacked + r * 64 + uw * 4) ^ flip;
-      uint32_t ev = w & 0x0f0f0f0fu, od = (w >> 4) & 0x0f0f0f0fu;  // nibbles 0, 2, 4, 6 / 1, 3, 5, 7 as bytes
-      // kept opaque: byte j of these converts in one instruction (v_cvt_f32_ubyte<j>), where the
-      // compiler would otherwise go back to w with a bit-field extract per nibble
-      asm("" : "+v"(ev));
-      asm("" : "+v"(od));
-      const float f0 = (float)(ev & 0xffu) - z[0], f1 = (float)(od & 0xffu) - z[1];
-      const float f2 = (float)((ev >> 8) & 0xffu) - z[2], f3 = (float)((od >> 8) & 0xffu) - z[3];
-      const float f4 = (float)((ev >> 16) & 0xffu) - z[4], f5 = (float)((od >> 16) & 0xffu) - z[5];
-      const float f6 = (float)(ev >> 24) - z[6], f7 = (float)(od >> 24) - z[7];
-      int lo = __builtin_amdgcn_cvt_pk_fp8_f32(f0, f1, 0, false);
-      lo = __builtin_amdgcn_cvt_pk_fp8_f32(f2, f3, lo, true);
-      int hi = __builtin_amdgcn_cvt_pk_fp8_f32(f4, f5, 0, false);
-      hi = __builtin_amdgcn_cvt_pk_fp8_f32(f6, f7, hi, true);
-      *reinterpret_cast<u32x2*>(dst + GB::lds_offset(r, uw >> 1) + (uw & 1) * 8) = u32x2{(uint32_t)lo, (uint32_t)hi};
-    }
-  };
-  // waits until at most min(later, S - 3) stages' loads of this wave are outstanding
-  auto wait_for_stage = [&](int later) {
-    static_for<S - 2>([&](auto sc) {
-      constexpr int n = decltype(sc)::value;  // 0 .. S - 3
-      constexpr int cnt = n * kOps;
-      if (later == n || (n == S - 3 && later > n) || (n == 0 && later < 0))
-        __builtin_amdgcn_s_waitcnt((cnt & 15) | ((cnt >> 4) << 14) | 0x0070);
-    });
-  };
-
-  // stage 0 -> fp8 tile 0
-  wait_for_stage(KT - 2);
-  __syncthreads();
-  unpack(lds, unp);
-
-  int rd_off = 0, wr_off = (S - 1) * kStage;
-  for (int kt = 0; kt < KT; ++kt) {
-    // The loads of stage kt + 1 have landed once only those of later stages are outstanding; the
-    // zero-fill loads past K complete at once and are not counted (see gemm_skinny.h).
-    wait_for_stage(KT - 3 - kt);
-    // everyone's part of stage kt + 1 is in LDS and fp8 tile kt & 1 is complete; everyone is done
-    // with the other fp8 tile and with stage kt - 1
-    __syncthreads();
-    issue_stage(wr_off);
-    const uint8_t* st = lds + rd_off;
-    const uint8_t* tile = unp + (kt & 1) * kTile;
-    int next_off = rd_off + kStage;
-    if (next_off == S * kStage) next_off = 0;
-
-    // ---- the stage's two MFMA blocks into the group's partial sums
-    const bool group_start = kt % a.stages_per_group == 0;
-#pragma unroll
-    for (int ks = 0; ks < kBK / 64; ++ks) {
-      i32x8 fb, fa[MT];
-      static_for<4>([&](auto pc) { read_fragment_part<false, kW4BN, decltype(pc)::value>(tile, wn, ks, fb); });
-      static_for<MT>([&](auto ic) {
-        static_for<2>([&](auto pc) {
-          read_fragment_part<true, BM, decltype(pc)::value>(st, decltype(ic)::value * 32, ks, fa[decltype(ic)::value]);
-        });
-      });
-      static_for<MT>([&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        const f32x16 c = (ks == 0 && group_start) ? zero : part[i];
-        part[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb, fa[i], c, 0, mfma_code<FMT_A>(), 0, 0, 0, 0);
-      });
-    }
-    // ---- the next stage's weights, while the MFMAs run (past K: zeros times A's zeros)
-    unpack(lds + next_off, unp + ((kt + 1) & 1) * kTile);
-    // ---- end of a group: total += scale * partial sums
-    if ((kt + 1) % a.stages_per_group == 0 || kt + 1 == KT) {
-      // this lane's columns: wn + 8 q + 4 (lane / 32) + e, q = 0 .. 3, e = 0 .. 3
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int col = wn + 8 * q + 4 * (lane >> 5);
-        float sc[4];
-        if (a.scale_f32) {
-          const f32x4 v = *reinterpret_cast<const f32x4*>(st + kOffScale + col * 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) sc[e] = v[e];
-        } else {
-          const u32x2 v = *reinterpret_cast<const u32x2*>(st + kOffScale + col * 2);
-          sc[0] = __uint_as_float(v[0] << 16);
-          sc[1] = __uint_as_float(v[0] & 0xffff0000u);
-          sc[2] = __uint_as_float(v[1] << 16);
-          sc[3] = __uint_as_float(v[1] & 0xffff0000u);
-        }
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) total[i][0][4 * q + e] = __builtin_fmaf(part[i][4 * q + e], sc[e], total[i][0][4 * q + e]);
+        for (int e = 0; e < 4; ++e) sc[4 * q + e] = __uint_as_float(sraw[q][e]);
+      } else {
+        sc[4 * q + 0] = __uint_as_float(sraw[q][0] << 16);
+        sc[4 * q + 1] = __uint_as_float(sraw[q][0] & 0xffff0000u);
+        sc[4 * q + 2] = __uint_as_float(sraw[q][1] << 16);
+        sc[4 * q + 3] = __uint_as_float(sraw[q][1] & 0xffff0000u);
       }
     }
-    rd_off = next_off;
-    wr_off += kStage;
-    if (wr_off == S * kStage) wr_off = 0;
+  };
+  // total += scale * sum a (q - z) of a finished group
+  auto fold = [&](auto bc) {
+    constexpr int B = decltype(bc)::value;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) total[i][0][e] = __builtin_fmaf(part[B][i][e], sc[e], total[i][0][e]);
+  };
+
+  int rd_off = 0;
+  int kt = 0;
+  // the stages of one group of K into accumulator set B
+  auto run_group = [&](auto bc, bool have_prev) {
+    constexpr int B = decltype(bc)::value;
+    for (int sg = 0; sg < a.stages_per_group && kt < KT; ++sg, ++kt) {
+      __syncthreads();  // stage kt is in LDS
+      const uint8_t* st = lds + rd_off;
+      const bool last = sg + 1 == a.stages_per_group || kt + 1 == KT;
+      // Every LDS read of the stage goes out before the first result is used: a wave runs its
+      // instructions in order, so a read issued late would find the MFMAs of this stage in its way.
+      uint32_t zw = 0;
+      if (a.zp) zw = *reinterpret_cast<const uint32_t*>(st + zoff);
+      i32x2 wt[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        wt[j] = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LDS_AS i32x2*)((LDS_AS uint8_t*)st + poff[j]));
+      i32x8 fa[2][MT];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+        static_for<MT>([&](auto ic) {
+          static_for<2>([&](auto pc) {
+            read_fragment_part<true, BM, decltype(pc)::value>(st, decltype(ic)::value * 32, ks, fa[ks][decltype(ic)::value]);
+          });
+        });
+      u32x4 snew[4];
+      if (last) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (a.scale_f32) {
+            snew[q] = *reinterpret_cast<const u32x4*>(st + soff + q * 32);
+          } else {
+            const u32x2 v = *reinterpret_cast<const u32x2*>(st + soff + q * 16);
+            snew[q] = u32x4{v[0], v[1], 0u, 0u};
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // the zero-point of this lane's column as two constant planes with the sign bit set: - (4 zhi + zlo)
+      u32x4 zh, zl;
+      if (has_z) {
+        const uint32_t z4 = ((zw ^ flip) >> zshift) & 15u;
+        const uint32_t ph = (8u | (z4 >> 2)) * 0x11111111u, pl = (8u | (z4 & 3u)) * 0x11111111u;
+        zh = u32x4{ph, ph, ph, ph};
+        zl = u32x4{pl, pl, pl, pl};
+      }
+#pragma unroll
+      for (int ks = 0; ks < kBK / 64; ++ks) {
+        u32x4 hi, lo;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const uint32_t w = (uint32_t)wt[2 * ks + (r >> 1)][r & 1] ^ flip;
+          lo[r] = w & 0x33333333u;
+          hi[r] = (w >> 2) & 0x33333333u;
+        }
+        static_for<MT>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          // e2m1 reads the two-bit planes as v / 2: 2^3 and 2^1 give 4 hi + lo
+          if (ks == 0 && sg == 0) part[B][i] = w4_mfma<FMT_A, 130>(hi, fa[ks][i], zero);
+          else part[B][i] = w4_mfma<FMT_A, 130>(hi, fa[ks][i], part[B][i]);
+          part[B][i] = w4_mfma<FMT_A, 128>(lo, fa[ks][i], part[B][i]);
+          if (has_z) {
+            part[B][i] = w4_mfma<FMT_A, 130>(zh, fa[ks][i], part[B][i]);
+            part[B][i] = w4_mfma<FMT_A, 128>(zl, fa[ks][i], part[B][i]);
+          }
+        });
+        if constexpr (PIPE) {
+          // the group before this one, whose MFMAs finished long ago, under the MFMAs just issued
+          if (ks == 0 && sg == 0 && have_prev) fold(std::integral_constant<int, 1 - B>{});
+        }
+      }
+      if (last) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sraw[q] = snew[q];
+        convert_scales();
+        if constexpr (!PIPE) fold(std::integral_constant<int, 0>{});
+      }
+      rd_off += kStage;
+      if (rd_off == S * kStage) rd_off = 0;
+    }
+  };
+  const int groups = (KT + a.stages_per_group - 1) / a.stages_per_group;
+  if constexpr (PIPE) {
+    for (int grp = 0; grp < groups; grp += 2) {
+      run_group(std::integral_constant<int, 0>{}, grp > 0);
+      if (grp + 1 < groups) run_group(std::integral_constant<int, 1>{}, true);
+    }
+    if (groups > 0) {
+      if ((groups - 1) & 1) fold(std::integral_constant<int, 1>{});
+      else fold(std::integral_constant<int, 0>{});
+    }
+  } else {
+    for (int grp = 0; grp < groups; ++grp) run_group(std::integral_constant<int, 0>{}, false);
   }
-  // the ring is idle (zero-fill loads of the stages past K included) before the epilogue overlays it
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-  float* stage_area = reinterpret_cast<float*>(lds) + wave * epilogue_stage_floats<MT, 1>();
+  __syncthreads();  // the producers have seen their last load land: the ring is idle
+  float* stage_area = reinterpret_cast<float*>(lds) + wq * epilogue_stage_floats<MT, 1>();
   epilogue<MT, 1>(g, 0, total, 0, n0 + wn, stage_area);
 }
 
 template <int BM, int FMT_A>
 void w4a8_launch(const W4Args& a, hipStream_t st) {
   dim3 grid((unsigned)((a.g.N + kW4BN - 1) / kW4BN), (unsigned)((a.g.M + BM - 1) / BM));
-  w4a8_gemm_kernel<BM, FMT_A><<<grid, kW4Threads, 0, st>>>(a);
+  w4a8_gemm_kernel<BM, FMT_A, (BM <= 64)><<<grid, kW4Threads, 0, st>>>(a);
 }
 
 template <int FMT_A>
 void w4a8_launch_by_m(const W4Args& a, hipStream_t st) {
   if (a.g.M <= 32) w4a8_launch<32, FMT_A>(a, st);
-  else if (a.g.M <= 64) w4a8_launch<64, FMT_A>(a, st);
-  else w4a8_launch<128, FMT_A>(a, st);
+  else w4a8_launch<64, FMT_A>(a, st);
 }
 
 }  // namespace mi355q
@@ -300,7 +407,7 @@ extern "C" int mi355q_w4a8_gemm(const void* A, int fmt_a, int64_t lda, const int
   const auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
   if (N % 32 != 0 || K % 16 != 0 || lda % 16 != 0 || (ld_packed * 4) % 16 != 0 || group % kBK != 0 ||
       !al16(A) || !al16(packed) || !al16(scale) || (zero_point && !al16(zero_point)) ||
-      M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL || (M + 127) / 128 > 65535)
+      M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL || (M + 63) / 64 > 65535)
     return MI355Q_ERR_UNSUPPORTED;
   W4Args a{};
   a.g.A = static_cast<const uint8_t*>(A);
