@@ -114,7 +114,12 @@ __device__ __forceinline__ f32x16 w4_mfma(const u32x4& plane, const i32x8& fa, c
 
 // PIPE: the partial sums of a group are folded into the totals one group late, from a second set of
 // accumulators, while the next group's MFMAs run: a wave does not stall on the MFMAs it has just issued.
-template <int BM, int FMT_A, bool PIPE>
+//
+// MODE 0 takes any group size and scale type.  MODE 1 (zero-points or signed nibbles) and MODE 2 (neither)
+// are for groups of 128 with bf16 scales: every stage is a whole group, the stage's code has no branch, and
+// the compiler is asked to spread the vector ALU work between the MFMAs (a wave issues in order: what
+// follows an MFMA that has to wait for the matrix unit waits with it).
+template <int BM, int FMT_A, bool PIPE, int MODE>
 __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
   constexpr int MT = BM / 32;
   constexpr int S = w4_stages<BM>();
@@ -275,6 +280,98 @@ __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
 
   int rd_off = 0;
   int kt = 0;
+  if constexpr (MODE != 0) {
+    static_assert(PIPE, "the one-group-per-stage loop folds one stage late");
+    constexpr bool HAS_Z = MODE == 1;
+    const uint32_t zmask = a.zp ? 0xffffffffu : 0u;
+    auto stage = [&](auto bc, auto hpc) {
+      constexpr int B = decltype(bc)::value;
+      constexpr bool HAVE_PREV = decltype(hpc)::value;
+      __syncthreads();  // stage kt is in LDS
+      const uint8_t* st = lds + rd_off;
+      uint32_t zw = 0;
+      if constexpr (HAS_Z) zw = *reinterpret_cast<const uint32_t*>(st + zoff) & zmask;
+      i32x2 wt[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        wt[j] = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LDS_AS i32x2*)((LDS_AS uint8_t*)st + poff[j]));
+      i32x8 fa[2][MT];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+        static_for<MT>([&](auto ic) {
+          static_for<2>([&](auto pc) {
+            read_fragment_part<true, BM, decltype(pc)::value>(st, decltype(ic)::value * 32, ks, fa[ks][decltype(ic)::value]);
+          });
+        });
+      u32x2 snew[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) snew[q] = *reinterpret_cast<const u32x2*>(st + soff + q * 16);
+      __builtin_amdgcn_sched_barrier(0);
+      u32x4 zh, zl;
+      if constexpr (HAS_Z) {
+        const uint32_t z4 = ((zw ^ flip) >> zshift) & 15u;
+        const uint32_t ph = (8u | (z4 >> 2)) * 0x11111111u, pl = (8u | (z4 & 3u)) * 0x11111111u;
+        zh = u32x4{ph, ph, ph, ph};
+        zl = u32x4{pl, pl, pl, pl};
+      }
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        u32x4 hi, lo;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const uint32_t w = (uint32_t)wt[2 * ks + (r >> 1)][r & 1] ^ flip;
+          lo[r] = w & 0x33333333u;
+          hi[r] = (w >> 2) & 0x33333333u;
+        }
+        static_for<MT>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          if (ks == 0) part[B][i] = w4_mfma<FMT_A, 130>(hi, fa[ks][i], zero);
+          else part[B][i] = w4_mfma<FMT_A, 130>(hi, fa[ks][i], part[B][i]);
+          part[B][i] = w4_mfma<FMT_A, 128>(lo, fa[ks][i], part[B][i]);
+          if constexpr (HAS_Z) {
+            part[B][i] = w4_mfma<FMT_A, 130>(zh, fa[ks][i], part[B][i]);
+            part[B][i] = w4_mfma<FMT_A, 128>(zl, fa[ks][i], part[B][i]);
+          }
+        });
+      }
+      if constexpr (HAVE_PREV) fold(std::integral_constant<int, 1 - B>{});
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        sc[4 * q + 0] = __uint_as_float(snew[q][0] << 16);
+        sc[4 * q + 1] = __uint_as_float(snew[q][0] & 0xffff0000u);
+        sc[4 * q + 2] = __uint_as_float(snew[q][1] << 16);
+        sc[4 * q + 3] = __uint_as_float(snew[q][1] & 0xffff0000u);
+      }
+      // one MFMA, then a share of the other vector and scalar work, and so on
+      constexpr int kMfmas = 2 * MT * (HAS_Z ? 4 : 2);
+      constexpr int kOther = (24 + (HAS_Z ? 10 : 0) + (HAVE_PREV ? 16 * MT : 0) + 16 + kMfmas - 1) / kMfmas;
+#pragma unroll
+      for (int n = 0; n < kMfmas; ++n) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x006, kOther, 0);
+      }
+      rd_off += kStage;
+      if (rd_off == S * kStage) rd_off = 0;
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    if (KT > 0) stage(std::integral_constant<int, 0>{}, F{});
+    for (kt = 1; kt + 1 < KT; kt += 2) {
+      stage(std::integral_constant<int, 1>{}, T{});
+      stage(std::integral_constant<int, 0>{}, T{});
+    }
+    if (kt < KT) {
+      stage(std::integral_constant<int, 1>{}, T{});
+      fold(std::integral_constant<int, 1>{});
+    } else if (KT > 0) {
+      fold(std::integral_constant<int, 0>{});
+    }
+    __syncthreads();  // the producers have seen their last load land: the ring is idle
+    float* stage_area = reinterpret_cast<float*>(lds) + wq * epilogue_stage_floats<MT, 1>();
+    epilogue<MT, 1>(g, 0, total, 0, n0 + wn, stage_area);
+    return;
+  }
   // the stages of one group of K into accumulator set B
   auto run_group = [&](auto bc, bool have_prev) {
     constexpr int B = decltype(bc)::value;
@@ -376,7 +473,10 @@ __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
 template <int BM, int FMT_A>
 void w4a8_launch(const W4Args& a, hipStream_t st) {
   dim3 grid((unsigned)((a.g.N + kW4BN - 1) / kW4BN), (unsigned)((a.g.M + BM - 1) / BM));
-  w4a8_gemm_kernel<BM, FMT_A, (BM <= 64)><<<grid, kW4Threads, 0, st>>>(a);
+  const bool fast = a.stages_per_group == 1 && !a.scale_f32 && a.g.K > 0;
+  if (!fast) w4a8_gemm_kernel<BM, FMT_A, true, 0><<<grid, kW4Threads, 0, st>>>(a);
+  else if (a.zp != nullptr || a.is_signed) w4a8_gemm_kernel<BM, FMT_A, true, 1><<<grid, kW4Threads, 0, st>>>(a);
+  else w4a8_gemm_kernel<BM, FMT_A, true, 2><<<grid, kW4Threads, 0, st>>>(a);
 }
 
 template <int FMT_A>
