@@ -137,7 +137,7 @@ def c1_input(gen, rows=4096, cols=4096):
     return x.bfloat16()
 
 
-def bench_cast(pkg, oracle, dev, steps, warmup, cpu):
+def bench_cast(pkg, oracle, dev, steps, warmup, cpu, c1=True, large=True):
     """benchmark configuration 1: amax pass, cast_to_fp8_v2 (scale given), cast_from_fp8.
 
     These kernels run for about ten microseconds, less than the host needs to
@@ -165,6 +165,9 @@ def bench_cast(pkg, oracle, dev, steps, warmup, cpu):
         if status != 0:
             raise RuntimeError(lib.mi355q_status_string(status).decode())
 
+    if not c1:
+        del xs, y8, yb
+        return out + bench_cast_large(lib, pkg, gen, dev, sd, st, ok, steps)
     ms = time_gpu(lambda i: ok(lib.mi355q_amax(xs[i % sets].data_ptr(), pkg.BF16, n, am.data_ptr(), st)), steps, warmup)
     assert am.cpu() == amax
     c = None
@@ -211,16 +214,56 @@ def bench_cast(pkg, oracle, dev, steps, warmup, cpu):
     out.append(hbm_entry("copy_fp8", "cast_to_fp8_v2 of an fp8 tensor: copy of 16 MiB", 2 * n, ms, steps, "copy_vec16"))
     del xs, y8, yb
 
-    # the same cast on a tensor 16x larger: the C1 kernels are so short that launch ramp-up
-    # is a visible share of them; this shows the streaming rate without it
+    if large:
+        out += bench_cast_large(lib, pkg, gen, dev, sd, st, ok, steps)
+    return out
+
+
+def bench_cast_large(lib, pkg, gen, dev, sd, st, ok, steps):
+    """The C1 cast on a tensor 16x larger (not one of the benchmark configurations): the C1 kernels are so
+    short that launch ramp-up is a visible share of them; this shows the streaming rate without it."""
     big = torch.randn(16384, 16384, generator=gen).bfloat16().to(dev) * 3
     nb = big.numel()
     big8 = [torch.empty(big.shape, dtype=E4, device=dev) for _ in range(2)]
     ms = time_gpu(lambda i: ok(lib.mi355q_cast_to_fp8(big.data_ptr(), pkg.BF16, big8[i % 2].data_ptr(), pkg.E4M3FN,
                                                       sd.data_ptr(), 0.0, pkg.SCALE_DEV, nb, 1, 1, None, st)),
                   max(steps // 5, 5), 3)
-    out.append(hbm_entry("cast_to_fp8_v2_large", "cast_to_fp8_v2 bf16 [16384,16384] -> e4m3fn (not one of the benchmark configurations)",
-                         3 * nb, ms, max(steps // 5, 5), "cast_to_fp8_vec8<bf16,e4m3fn,scalar>"))
+    return [hbm_entry("cast_to_fp8_v2_large", "cast_to_fp8_v2 bf16 [16384,16384] -> e4m3fn (not one of the benchmark configurations)",
+                      3 * nb, ms, max(steps // 5, 5), "cast_to_fp8_vec8<bf16,e4m3fn,scalar>")]
+
+
+def bench_ceilings(pkg, dev, steps, warmup):
+    """What this GPU sustains in this run with nothing in the way: back-to-back fp8 MFMAs on register operands
+    (one and two waves per SIMD), and 16-byte read-only / copy streams at three sizes (rotating over enough
+    buffers to exceed the Infinity Cache).  Reference points for the roofline fractions, not workloads."""
+    import ctypes
+    lib = pkg.capi()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sink = torch.zeros(16, device=dev)
+    out = []
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    for wps in (1, 2):
+        per_wave = 4000
+        ms = time_gpu(lambda i: lib.mi355q_probe_mfma(wps, per_wave, cus, sink.data_ptr(), st), max(steps, 20), warmup)
+        flop = 131072.0 * per_wave * 4 * wps * cus
+        out.append({"name": f"ceiling_mfma_fp8_{wps}_wave_per_simd", "workload": f"{per_wave} back-to-back v_mfma_f32_32x32x64_f8f6f4 per wave, "
+                    f"{4 * wps} waves on each of {cus} CUs, register operands", "metric": "TFLOP/s",
+                    "value": round(flop / (ms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "ms_per_call": round(ms, 5), "steps": max(steps, 20),
+                    "implied_clock_ghz": round(per_wave * 64 / (ms * 1e-3) / 1e9 * wps, 3)})
+    for mib in (32, 128, 2048):
+        nbytes = mib << 20
+        sets = 1 if nbytes >= (1 << 30) else n_sets(nbytes)
+        bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev).view(E4) for _ in range(sets)]
+        k = max(steps, 20) if mib < 2048 else 5
+        ms = time_gpu(lambda i: lib.mi355q_probe_read(bufs[i % sets].data_ptr(), nbytes, 2 * cus, sink.data_ptr(), st), k, warmup)
+        out.append(hbm_entry(f"ceiling_read_{mib}MiB", f"read-only stream over {mib} MiB, 16-byte loads, nothing stored", nbytes, ms, k, "probe_read_kernel"))
+        half = nbytes // 2
+        dst = [torch.empty(half, dtype=E4, device=dev) for _ in range(min(sets, 4))]
+        ms = time_gpu(lambda i: lib.mi355q_cast_to_fp8(bufs[i % sets].data_ptr(), pkg.E4M3FN, dst[i % len(dst)].data_ptr(), pkg.E4M3FN, None, 0.0,
+                                                       pkg.SCALE_NONE, half, 1, 1, None, st), k, warmup)
+        out.append(hbm_entry(f"ceiling_copy_{mib}MiB", f"copy of {mib // 2} MiB ({mib} MiB read + written), the library's 16-byte copy kernel",
+                             nbytes, ms, k, "copy_vec16"))
+        del bufs, dst
     return out
 
 
@@ -534,7 +577,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,cast,int4,decode,mlp,reduce,w4a8,sdpa")
+    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,cast,castlarge,int4,decode,mlp,reduce,w4a8,sdpa,ceilings")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -551,14 +594,14 @@ def main():
     ops = torch.ops.hpu
     dev = torch.device("cuda:0")
     torch.set_num_threads(min(os.cpu_count() or 1, 16))
-    which = set(args.only.split(",")) if args.only else {"gemm", "cast", "int4", "decode", "mlp", "reduce", "w4a8", "sdpa"}
+    which = set(args.only.split(",")) if args.only else {"gemm", "cast", "castlarge", "int4", "decode", "mlp", "reduce", "w4a8", "sdpa", "ceilings"}
     cpu = not args.no_cpu
     k_stream = max(args.steps, 50)      # the microsecond-scale kernels need more calls for a stable mean
     w_stream = max(args.warmup, 10)
 
     ops_out = []
-    if "cast" in which:
-        ops_out += bench_cast(pkg, oracle, dev, k_stream, w_stream, cpu)
+    if "cast" in which or "castlarge" in which:
+        ops_out += bench_cast(pkg, oracle, dev, k_stream, w_stream, cpu, c1="cast" in which, large="castlarge" in which)
     if "int4" in which:
         ops_out += bench_int4(pkg, oracle, dev, k_stream, w_stream, cpu)
     if "decode" in which:
@@ -571,6 +614,8 @@ def main():
         ops_out += bench_w4a8(oracle, dev, args.steps, args.warmup, cpu)
     if "sdpa" in which:
         ops_out += bench_sdpa(oracle, dev, args.steps, args.warmup, cpu)
+    if "ceilings" in which:
+        ops_out += bench_ceilings(pkg, dev, args.steps, args.warmup)
 
     line = {"metric": "cast/dequant GB/s (% HBM peak); fp8_gemm_v2 TFLOP/s (% fp8 MFMA peak)",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,

@@ -18,7 +18,7 @@ OBJ = os.path.join(HERE, "build")
 LIB_KERNELS = os.path.join(HERE, "libmi355q.so")
 LIB_TORCH = os.path.join(HERE, "mi355q_torch.so")
 
-HIP_SOURCES = ["cast_kernels.hip", "int4_kernels.hip", "reduce_kernels.hip", "gemm_api.hip", "gemm_inst_kk.hip", "gemm_inst_km.hip", "gemm_inst_mk.hip", "gemm_inst_mm.hip", "w4_gemm.hip", "sdpa_kernels.hip", "api.cpp"]
+HIP_SOURCES = ["cast_kernels.hip", "int4_kernels.hip", "reduce_kernels.hip", "gemm_api.hip", "gemm_inst_kk.hip", "gemm_inst_km.hip", "gemm_inst_mk.hip", "gemm_inst_mm.hip", "w4_gemm.hip", "sdpa_kernels.hip", "probe_kernels.hip", "api.cpp"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

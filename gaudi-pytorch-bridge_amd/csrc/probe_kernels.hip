@@ -1,0 +1,75 @@
+// Measurement aids: what this GPU sustains with nothing in the way.  bench.py times them in the
+// same run as the kernels they bound, so that a roofline fraction can be read against the
+// machine's real ceiling (clocks under load, HBM rate at a given size) as well as against the
+// published peak.  No part of the product path calls these.
+#include "device_common.h"
+
+namespace mi355q {
+
+typedef int probe_i32x8 __attribute__((ext_vector_type(8)));
+typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
+
+// Back-to-back v_mfma_f32_32x32x64_f8f6f4 (e4m3 x e4m3) on register operands: no loads, no LDS.
+// Two accumulators, so no MFMA waits for the one before it.
+__global__ __launch_bounds__(512) void probe_mfma_kernel(int pairs, float* sink) {
+  probe_i32x8 a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = (int)(threadIdx.x * 0x01010101u + i * 0x11u) & 0x37373737;   // small finite e4m3 codes
+    b[i] = (int)(threadIdx.x * 0x03030303u + i * 0x07u) & 0x37373737;
+  }
+  probe_f32x16 c0, c1;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    c0[r] = 0.0f;
+    c1[r] = 0.0f;
+  }
+  for (int it = 0; it < pairs; ++it) {
+    c0 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c0, 0, 0, 0, 0, 0, 0);
+    c1 = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, a, c1, 0, 0, 0, 0, 0, 0);
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s += c0[r] + c1[r];
+  if (s == 123.456f) sink[0] = s;   // keeps the loop alive; practically never true
+}
+
+// 16 bytes per lane, read only: the sum keeps the loads alive, one store per workgroup at most.
+__global__ __launch_bounds__(1024) void probe_read_kernel(const u32x4* __restrict__ x, int64_t n16, uint32_t* sink) {
+  uint32_t acc = 0;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const u32x4 v0 = x[i], v1 = x[i + stride], v2 = x[i + 2 * stride], v3 = x[i + 3 * stride];
+    acc ^= v0[0] ^ v0[1] ^ v0[2] ^ v0[3] ^ v1[0] ^ v1[1] ^ v1[2] ^ v1[3] ^ v2[0] ^ v2[1] ^ v2[2] ^ v2[3] ^ v3[0] ^ v3[1] ^ v3[2] ^ v3[3];
+  }
+  for (; i < n16; i += stride) {
+    const u32x4 v = x[i];
+    acc ^= v[0] ^ v[1] ^ v[2] ^ v[3];
+  }
+  if (acc == 0x9e3779b9u) sink[0] = acc;
+}
+
+}  // namespace mi355q
+
+using namespace mi355q;
+
+extern "C" {
+
+int mi355q_probe_mfma(int waves_per_simd, int mfma_per_wave, int workgroups, float* sink, void* stream) {
+  if ((waves_per_simd != 1 && waves_per_simd != 2) || mfma_per_wave < 2 || workgroups <= 0 || sink == nullptr)
+    return MI355Q_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(probe_mfma_kernel, dim3((unsigned)workgroups), dim3(256u * waves_per_simd), 0, static_cast<hipStream_t>(stream),
+                     mfma_per_wave / 2, sink);
+  return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
+}
+
+int mi355q_probe_read(const void* x, int64_t bytes, int workgroups, void* sink, void* stream) {
+  if (x == nullptr || sink == nullptr || bytes < 0 || workgroups <= 0 || (reinterpret_cast<uintptr_t>(x) & 15u) != 0)
+    return MI355Q_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(probe_read_kernel, dim3((unsigned)workgroups), dim3(1024), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const u32x4*>(x), bytes / 16, static_cast<uint32_t*>(sink));
+  return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
+}
+
+}  // extern "C"

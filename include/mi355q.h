@@ -353,6 +353,18 @@ int mi355q_fp8_sdpa_fwd(const void* q, const void* k, const void* v, int fp8_fmt
                         float softmax_scale, int is_causal, const float* const* scale_dev,
                         const float* scale_host, float* amax_s, float* amax_o, void* stream);
 
+/*
+ * Measurement aids without a counterpart in the reference; the product path never calls them.
+ * mi355q_probe_mfma runs `workgroups` workgroups of 4 * waves_per_simd waves (1 or 2 per SIMD),
+ * each wave issuing mfma_per_wave back-to-back v_mfma_f32_32x32x64_f8f6f4 (131072 flop each) on
+ * register operands: timed, it gives the fp8 MFMA rate this GPU sustains at its clock under load.
+ * mi355q_probe_read reads `bytes` bytes (a multiple of 16, 16-byte aligned) with 16-byte loads
+ * and stores nothing: timed, the HBM read rate at that size.  sink: a few bytes of device memory
+ * that are practically never written.
+ */
+int mi355q_probe_mfma(int waves_per_simd, int mfma_per_wave, int workgroups, float* sink, void* stream);
+int mi355q_probe_read(const void* x, int64_t bytes, int workgroups, void* sink, void* stream);
+
 /* Name of the kernel variant mi355q_fp8_gemm would pick for a problem
  * (for logs and profiles; static string). */
 const char* mi355q_fp8_gemm_variant(int trans_a, int64_t lda, int trans_b, int64_t ldb,
