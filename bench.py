@@ -37,8 +37,8 @@ SEED = 0xC001A1
 MALL_BYTES = 256 << 20
 
 # HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE in two runs of this script, each counter scaled by what it reads for the 16 MiB
-# fp8 copy kernel (fetch x1.9994, write x0.9997); the tables are under profiles/.  Counters
+# WRITE_SIZE in two runs of this script per workload, each counter scaled by what it reads for
+# the 16 MiB fp8 copy kernel (fetch x1.9974, write x1.0000); the tables are under profiles/.  Counters
 # cannot be read from inside the timed run, so these are constants from the committed runs.
 MEASURED_TRAFFIC = {
     "amax": 33.69e6,
@@ -49,10 +49,16 @@ MEASURED_TRAFFIC = {
     "cast_to_fp8_v2_large": 804.67e6,
     "convert_from_uint4": 43.35e6,
     "convert_from_int4": 43.10e6,
-    "fp8_gemm_v2": 939.86e6,
-    "fp8_gemm_v2_decode_M16": 236.93e6,
-    "fp8_gemm_v2_decode_M64": 242.94e6,
-    "fp8_gemm_v2_decode_M256": 266.46e6,
+    "fp8_gemm_v2": 939.65e6,
+    "fp8_gemm_v2_B_NK": 939.17e6,
+    "fp8_gemm_v2_decode_M16": 236.92e6,
+    "fp8_gemm_v2_decode_M64": 243.02e6,
+    "fp8_gemm_v2_decode_M256": 266.45e6,
+    "w4a8_gemm_M16": 124.15e6,
+    "w4a8_gemm_M64": 130.47e6,
+    "w4a8_gemm_M256": 481.35e6,     # four row blocks of 64 stream the weights four times
+    "fp8_sdpa_B1_L8192": 125.08e6,
+    "fp8_sdpa_B4_L4096": 235.42e6,
     "softmax_fp8": 1609.30e6,
     "sum_fp8_rows": 67.32e6,
     "sum_fp8_columns": 73.45e6,   # sum_columns_kernel 69.20 + sum_finish_kernel 4.25

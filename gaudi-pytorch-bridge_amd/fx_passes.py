@@ -27,12 +27,18 @@ def _arg(node, index, name, default=None):
     return node.kwargs.get(name, default)
 
 
+_FP8_MAX = {torch.float8_e4m3fn: 448.0, torch.float8_e5m2: 57344.0}
+
+
 def replace_quantize_with_cast(gm: torch.fx.GraphModule) -> int:
     """quantize_per_tensor(x, s, 0, qmin, qmax, fp8) -> cast_to_fp8_v2(x, 1 / s, False, False, fp8)[0].
 
-    Only fp8 targets with a zero zero-point are rewritten (the cast saturates at
-    the format's maximum, which is what qmin / qmax say for fp8).  Returns the
-    number of nodes replaced.
+    Only fp8 targets with a zero zero-point are rewritten.  The cast saturates at the format's
+    maximum (448 for e4m3fn, 57344 for e5m2).  A node whose [qmin, qmax] is narrower than that --
+    the reference's quantizer asks for +-240, the e4m3 range of the device it was written for
+    (core/quantizer.py:100-123) -- gets a clamp of x to [qmin * s, qmax * s] in front of the cast,
+    so that values beyond the node's range saturate where the node says and not at the format's
+    maximum.  Returns the number of nodes replaced.
     """
     graph = gm.graph
     count = 0
@@ -43,8 +49,15 @@ def replace_quantize_with_cast(gm: torch.fx.GraphModule) -> int:
         zero_point, dtype = _arg(node, 2, "zero_point", 0), _arg(node, 5, "dtype")
         if dtype not in _FP8 or zero_point != 0 or isinstance(scale, torch.fx.Node):
             continue
+        qmin, qmax = _arg(node, 3, "quant_min"), _arg(node, 4, "quant_max")
+        fmax = _FP8_MAX[dtype]
         with graph.inserting_before(node):
-            cast = graph.call_function(torch.ops.hpu.cast_to_fp8_v2.scalar, args=(x, 1.0 / float(scale), False, False, dtype))
+            src = x
+            lo = None if qmin is None or float(qmin) <= -fmax else float(qmin) * float(scale)
+            hi = None if qmax is None or float(qmax) >= fmax else float(qmax) * float(scale)
+            if lo is not None or hi is not None:
+                src = graph.call_function(torch.ops.aten.clamp.default, args=(x, lo, hi))
+            cast = graph.call_function(torch.ops.hpu.cast_to_fp8_v2.scalar, args=(src, 1.0 / float(scale), False, False, dtype))
             out = graph.call_function(operator.getitem, args=(cast, 0))
         node.replace_all_uses_with(out)
         graph.erase_node(node)
@@ -190,6 +203,10 @@ def fold_constant_casts(gm: torch.fx.GraphModule) -> int:
         if not (_is(node, "cast_to_fp8_v2.scalar") or _is(node, "cast_to_fp8_v2.default")):
             continue
         src = node.args[0]
+        # the clamp that replace_quantize_with_cast puts in front of a cast with a narrow range
+        clamp = src if _is(src, "clamp.default") and len(src.users) == 1 else None
+        if clamp is not None:
+            src = clamp.args[0]
         if not (isinstance(src, torch.fx.Node) and src.op == "get_attr"):
             continue
         if any(isinstance(a, torch.fx.Node) for a in node.args[1:]) or any(isinstance(v, torch.fx.Node) for v in node.kwargs.values()):
@@ -202,7 +219,10 @@ def fold_constant_casts(gm: torch.fx.GraphModule) -> int:
         if not isinstance(obj, torch.Tensor) or not obj.is_cuda:
             continue
         with torch.no_grad():
-            value = node.target(obj.detach(), *node.args[1:], **node.kwargs)[0]
+            const_in = obj.detach()
+            if clamp is not None:
+                const_in = clamp.target(const_in, *clamp.args[1:])
+            value = node.target(const_in, *node.args[1:], **node.kwargs)[0]
         name = f"_fp8_const_{sum(1 for _ in gm.buffers())}"
         gm.register_buffer(name, value)
         with graph.inserting_before(node):
@@ -211,6 +231,8 @@ def fold_constant_casts(gm: torch.fx.GraphModule) -> int:
             user.replace_all_uses_with(const)
             graph.erase_node(user)
         graph.erase_node(node)
+        if clamp is not None:
+            graph.erase_node(clamp)
         if not src.users:
             graph.erase_node(src)
         count += 1

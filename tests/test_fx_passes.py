@@ -43,6 +43,38 @@ def test_rewrites_node_counts(pkg):
     assert cast.args[1] == pytest.approx(1.0 / SA) and cast.args[4] == E4
 
 
+def test_a_narrower_quant_range_becomes_a_clamp(pkg):
+    """The reference's quantizer asks for qmin / qmax = -+240 (core/quantizer.py:100-123) where e4m3fn holds
+    448: the rewrite keeps the node's range with a clamp of the input to [qmin * s, qmax * s]."""
+    def narrow(a):
+        return q.quantize_per_tensor.default(a, SA, 0, -240, 240, E4)
+
+    def full(a):
+        return q.quantize_per_tensor.default(a, SA, 0, -448, 448, E4)
+
+    gm = torch.fx.symbolic_trace(narrow)
+    assert passes(pkg).replace_quantize_with_cast(gm) == 1
+    assert count(gm, "clamp.default") == 1 and count(gm, "cast_to_fp8_v2.scalar") == 1
+    clamp = next(n for n in gm.graph.nodes if getattr(n.target, "__name__", "") == "clamp.default")
+    assert clamp.args[1] == pytest.approx(-240 * SA) and clamp.args[2] == pytest.approx(240 * SA)
+    gm = torch.fx.symbolic_trace(full)
+    assert passes(pkg).replace_quantize_with_cast(gm) == 1 and count(gm, "clamp.default") == 0
+
+
+@pytest.mark.gpu
+def test_values_beyond_a_narrow_range_saturate_at_it(pkg, dev):
+    def narrow(a):
+        return q.quantize_per_tensor.default(a, SA, 0, -240, 240, E4)
+
+    x = torch.tensor([[0.5, 13.0, 100.0, -100.0, 11.9, -12.1]], device=dev).bfloat16()     # 240 * SA = 12
+    ref = narrow(x)
+    gm = torch.fx.symbolic_trace(narrow)
+    passes(pkg).replace_quantize_with_cast(gm)
+    out = gm(x)
+    assert out.dtype == E4 and torch.equal(out.float(), ref.float())
+    assert out.float().abs().max().item() == 240.0
+
+
 def test_rewrites_leave_other_graphs_alone(pkg):
     def int8_quant(a):
         return q.quantize_per_tensor.default(a, 0.1, 3, -128, 127, torch.int8)

@@ -142,7 +142,11 @@ def test_flow_node_counts(pkg, dtype, bias):
         s_val = gm.get_buffer(scale.target).item()
         assert getattr(cast.target, "__name__", "") == "cast_to_fp8_v2.scalar" and s_val in allowed
         assert cast.args[1] == 1.0 / s_val and cast.args[2:5] == (False, False, dtype)
-    assert w.args[0].args[0].op == "get_attr"   # the weight parameter itself
+    # the weight parameter itself, behind the clamp that keeps the quantizer's +-240 on a format that holds more
+    w_src = w.args[0].args[0]
+    assert getattr(w_src.target, "__name__", "") == "clamp.default" and w_src.args[2] == pytest.approx(240 * gm.get_buffer(sw.target).item())
+    w_src = w_src.args[0]
+    assert w_src.op == "get_attr"
     _, fx = mods(pkg)
     assert fx.fold_constant_casts(gm) == 0      # parameters on the CPU are left alone
 
@@ -158,7 +162,9 @@ def test_flow_annotates_matmul_and_linear(pkg):
     qk = [n for n in gm.graph.nodes if getattr(n.target, "__name__", "") == "fp8_gemm_v2.default"][-1]
     # k is transposed before it is quantised, so the cast sees the transposed view and the GEMM a plain B
     assert qk.args[3] is False and qk.args[8] is None
-    assert getattr(qk.args[2].args[0].args[0].target, "__name__", "") == "transpose.int"
+    k_src = qk.args[2].args[0].args[0]       # the cast's input: the clamp to the quantizer's +-240, then the view
+    assert getattr(k_src.target, "__name__", "") == "clamp.default"
+    assert getattr(k_src.args[0].target, "__name__", "") == "transpose.int"
 
 
 # ------------------------------------------------------------------ the flow, numerics (GPU)
