@@ -17,14 +17,21 @@
 // and the V^T fragment is gathered from LDS in the same key order by the transposing reads
 // (ds_read_b64_tr_b8 takes each of its 8 k-rows from its own address).
 //
-// K and V blocks go global -> registers -> LDS, double buffered, one barrier per block: the loads
-// of block i + 1 are issued before the arithmetic of block i and written to the other buffer after
-// it.  Rows are XOR-swizzled so that the fragment reads are bank-conflict free.
+// K and V blocks are double buffered in LDS, one barrier per block.  Aligned tensors (16-byte
+// rows and head dimensions) go global -> LDS directly (buffer_load ... lds: the loads of block
+// i + 1 are issued before the arithmetic of block i and waited for after it, and cost the waves
+// neither registers nor vector instructions); anything else goes through registers, byte by
+// byte where it must.  Rows are XOR-swizzled so that the fragment reads are bank-conflict free;
+// for the direct loads the swizzle is applied on the global side (which chunk a lane fetches),
+// since such a load fixes the LDS position of each lane's 16 bytes.
+#include <type_traits>
+
 #include "device_common.h"
 
 namespace mi355q {
 
 typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define SDPA_LDS_AS __attribute__((address_space(3)))
@@ -32,7 +39,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 constexpr int kSdpaThreads = 256;
 constexpr int kSdpaBM = 128;  // query rows per workgroup
 constexpr int kSdpaBN = 64;   // keys per block
-constexpr int kVRow = 256;    // bytes of an LDS row of V, whatever head_dim_v is
 constexpr float kLog2e = 1.44269504088896341f;
 
 enum { kMaskNone = MI355Q_SDPA_MASK_NONE, kMaskBool = MI355Q_SDPA_MASK_BOOL, kMaskBf16 = MI355Q_SDPA_MASK_BF16, kMaskF32 = MI355Q_SDPA_MASK_F32 };
@@ -49,6 +55,7 @@ struct SdpaArgs {
   int L, S, Dk, Dv;
   int mask_kind, causal, out_fp8;
   int vec_q, vec_k, vec_v, vec_o;  // 16-byte (q, k, v) / 4-element (out) accesses are possible
+  int dma;                         // k and v go global -> LDS directly
   int nqb;                         // query blocks per (batch, head)
   float scale;
   const float* sc_dev[6];  // d_scale_q, d_scale_k, d_scale_v, q_scale_s, q_scale_o, d_scale_s
@@ -74,13 +81,51 @@ __device__ __forceinline__ int k_lds_offset(int row, int chunk) {
   return row * ROW_BYTES + ((chunk ^ sw) << 4);
 }
 
-// V rows are 256 bytes.  A transposing read covers, per cycle, two 16-lane groups (adjacent chunks)
-// times the 8 keys 8 (2 p' + r / 4) + 4 h + r % 4, r = 0..7: bits 3, 1 and 0 of the key tell them
-// apart, and XORing twice that number into the chunk index gives 8 slots of one parity.
-__device__ __forceinline__ int v_lds_offset(int row, int chunk) {
-  const int key = (((row >> 3) & 1) << 2) | (row & 3);
-  return row * kVRow + ((chunk ^ (key << 1)) << 4);
+// V rows are 128 or 256 bytes.  A transposing read covers, per cycle, two 16-lane groups (adjacent
+// chunks) times the 8 keys 8 (2 p' + r / 4) + 4 h + r % 4, r = 0..7: bits 3, 1 and 0 of the key tell
+// them apart.  With 256-byte rows, XORing twice that 3-bit number into the chunk index gives 8 slots
+// of one parity; with 128-byte rows two rows share 256 bytes, bit 0 of the key already separates
+// them, and bits 1 and 3 go into the chunk index.
+template <int ROW_BYTES>
+__device__ __forceinline__ int v_swizzle(int row) {
+  if constexpr (ROW_BYTES == 256) return ((((row >> 3) & 1) << 2) | (row & 3)) << 1;
+  else return ((((row >> 3) & 1) << 1) | ((row >> 1) & 1)) << 1;
 }
+template <int ROW_BYTES>
+__device__ __forceinline__ int v_lds_offset(int row, int chunk) {
+  return row * ROW_BYTES + ((chunk ^ v_swizzle<ROW_BYTES>(row)) << 4);
+}
+template <int ROW_BYTES>
+__device__ __forceinline__ int k_swizzle(int row) {
+  if constexpr (ROW_BYTES == 64) return (row >> 2) & 3;
+  else if constexpr (ROW_BYTES == 128) return (row >> 1) & 7;
+  else return row & 15;
+}
+
+// One 16-byte piece per lane, global -> LDS (lane l lands at lds_dst + 16 l; a lane whose offset lies
+// outside the descriptor writes zeros).  The s_nop covers descriptor words that reached their scalar
+// registers through a vector instruction (five wait states before a memory instruction may read them).
+__device__ __forceinline__ void sdpa_dma16(const i32x4& rsrc, int voff, uint32_t lds_dst) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :
+               : "s"(lds_dst), "v"(voff), "s"(rsrc)
+               : "memory", "m0");
+}
+
+// A buffer descriptor that walks down the rows of k or v one block at a time.
+struct SdpaWalker {
+  uint64_t base;
+  int64_t left;  // bytes from base to the end of the tensor's rows; <= 0: every load reads zeros
+  __device__ __forceinline__ i32x4 rsrc() const {
+    int64_t rec = left < 0 ? 0 : (left > 0x7ffffff0LL ? 0x7ffffff0LL : left);
+    i32x4 r;
+    r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)base);
+    r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((base >> 32) & 0xffffu));
+    r[2] = __builtin_amdgcn_readfirstlane((int)rec);
+    r[3] = 0x00020000;
+    return r;
+  }
+};
 
 // 16 bytes of a row of q / k / v starting at byte column d (zero beyond the row's D bytes and for
 // rows outside the tensor).  VEC: the row start and D are multiples of 16.
@@ -114,6 +159,7 @@ __global__ void sdpa_clear_amax_kernel(float* a, float* b) {
 template <int DKC, int DVT, int FMT>
 __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd_kernel(const SdpaArgs a) {
   constexpr int KROW = DKC * 64;
+  constexpr int kVRow = DVT <= 4 ? 128 : 256;  // bytes of an LDS row of V
   constexpr int KCPR = KROW / 16;           // chunks per K row
   constexpr int VCPR = DVT * 2;             // chunks per V row that carry data
   constexpr int KBYTES = kSdpaBN * KROW;
@@ -123,7 +169,8 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
   static_assert(KLOADS >= 1 && VLOADS >= 1, "block too small for the workgroup");
   __shared__ __align__(16) uint8_t lds[2 * (KBYTES + VBYTES)];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in every lane, and known to be
   const int lq = lane & 31, h = lane >> 5;
 
   // Workgroups go to the 8 XCDs round robin: give each XCD a contiguous range of (batch, head,
@@ -205,8 +252,46 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
 #pragma unroll
     for (int n = 0; n < VLOADS; ++n) {
       const int ci = tid + n * kSdpaThreads;
-      *reinterpret_cast<u32x4*>(vb + v_lds_offset(ci / VCPR, ci % VCPR)) = vreg[n];
+      *reinterpret_cast<u32x4*>(vb + v_lds_offset<kVRow>(ci / VCPR, ci % VCPR)) = vreg[n];
     }
+  };
+
+  // Direct loads: the K tile is KBYTES / 1024 regions of 1 KiB (one wave-wide load each), the V tile
+  // VBYTES / 1024; a wave takes every fourth.  The lane's offsets inside a block never change; the
+  // descriptors walk down the rows.
+  constexpr int KREG = KBYTES / 1024 / 4, VREG = VBYTES / 1024 / 4;  // regions per wave
+  static_assert(KBYTES % 4096 == 0 && VBYTES % 4096 == 0, "tiles split into 1 KiB regions over four waves");
+  int kvoff[KREG], vvoff[VREG];
+  SdpaWalker wk{reinterpret_cast<uint64_t>(kp), 0}, wv{reinterpret_cast<uint64_t>(vp), 0};
+  if (a.dma) {
+    wk.left = (int64_t)(a.S - 1) * a.ldk + a.Dk;
+    wv.left = (int64_t)(a.S - 1) * a.ldv + a.Dv;
+#pragma unroll
+    for (int n = 0; n < KREG; ++n) {
+      const int pos = (wave * KREG + n) * 64 + lane;  // 16-byte slot of the tile this lane fills
+      const int row = pos / KCPR, chunk = (pos % KCPR) ^ k_swizzle<KROW>(pos / KCPR);
+      kvoff[n] = chunk * 16 < a.Dk ? row * (int)a.ldk + chunk * 16 : 0x7fffffff;
+    }
+#pragma unroll
+    for (int n = 0; n < VREG; ++n) {
+      const int pos = (wave * VREG + n) * 64 + lane;
+      const int row = pos / (kVRow / 16), chunk = (pos % (kVRow / 16)) ^ v_swizzle<kVRow>(pos / (kVRow / 16));
+      vvoff[n] = chunk * 16 < a.Dv ? row * (int)a.ldv + chunk * 16 : 0x7fffffff;
+    }
+  }
+  // the loads of the next block into buffer `buf`; the descriptors then move on by one block
+  auto issue_block = [&](int buf) {
+    const uint32_t kdst = (uint32_t)(uintptr_t)(SDPA_LDS_AS uint8_t*)(lds + buf * (KBYTES + VBYTES));
+    const i32x4 rk = wk.rsrc();
+#pragma unroll
+    for (int n = 0; n < KREG; ++n) sdpa_dma16(rk, kvoff[n], kdst + (wave * KREG + n) * 1024);
+    const i32x4 rv = wv.rsrc();
+#pragma unroll
+    for (int n = 0; n < VREG; ++n) sdpa_dma16(rv, vvoff[n], kdst + KBYTES + (wave * VREG + n) * 1024);
+    wk.base += (uint64_t)kSdpaBN * a.ldk;
+    wk.left -= (int64_t)kSdpaBN * a.ldk;
+    wv.base += (uint64_t)kSdpaBN * a.ldv;
+    wv.left -= (int64_t)kSdpaBN * a.ldv;
   };
 
   f32x16 o[DVT];
@@ -218,14 +303,22 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
   float l_run = 0.0f;               // this half-wave's share of the running sum (times q_scale_s)
 
   if (nblk > 0) {
-    fetch(0);
-    commit(0);
+    if (a.dma) {
+      issue_block(0);
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    } else {
+      fetch(0);
+      commit(0);
+    }
   }
   __syncthreads();
 
   for (int blk = 0; blk < nblk; ++blk) {
     const int kv0 = blk * kSdpaBN;
-    if (blk + 1 < nblk) fetch(blk + 1);
+    if (blk + 1 < nblk) {
+      if (a.dma) issue_block((blk + 1) & 1);
+      else fetch(blk + 1);
+    }
     const uint8_t* kb = lds + (blk & 1) * (KBYTES + VBYTES);
     const uint8_t* vb = kb + KBYTES;
 
@@ -284,29 +377,40 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
 
       float psum = 0.0f;
       i32x8 pf;
+      // p = 2^(x + shift) for this lane's 32 scores, their sum, and the fp8 codes packed in register
+      // order.  RAW: s still holds the unscaled products (x = s * sc2); CLAMP: q_scale_s exceeds the
+      // format's range.  Compile-time variants, so that the common one is a multiply-add, an exp2 and an
+      // add per score.
+      auto exponentials = [&](auto rawc, auto clampc) {
+        constexpr bool RAW = decltype(rawc)::value, CLAMP = decltype(clampc)::value;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            float p[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float x = s[t][4 * j + i];
+              p[i] = fast_exp2(RAW ? __builtin_fmaf(x, sc2, shift) : x + shift);
+              psum += p[i];
+              if (CLAMP) p[i] = __builtin_elementwise_minimum(p[i], kMax8);
+            }
+            int w;
+            if constexpr (FMT == MI355Q_E5M2) {
+              w = __builtin_amdgcn_cvt_pk_bf8_f32(p[0], p[1], 0, false);
+              w = __builtin_amdgcn_cvt_pk_bf8_f32(p[2], p[3], w, true);
+            } else {
+              w = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
+              w = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], w, true);
+            }
+            pf[4 * t + j] = w;
+          }
+      };
       const bool raw = !edge && sc2 >= 0.0f;  // s still holds the unscaled products
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float p[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float x = s[t][4 * j + i];
-            p[i] = fast_exp2(raw ? __builtin_fmaf(x, sc2, shift) : x + shift);
-            psum += p[i];
-            if (clamp_p) p[i] = __builtin_elementwise_minimum(p[i], kMax8);
-          }
-          int w;
-          if constexpr (FMT == MI355Q_E5M2) {
-            w = __builtin_amdgcn_cvt_pk_bf8_f32(p[0], p[1], 0, false);
-            w = __builtin_amdgcn_cvt_pk_bf8_f32(p[2], p[3], w, true);
-          } else {
-            w = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
-            w = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], w, true);
-          }
-          pf[4 * t + j] = w;
-        }
+      if (raw && !clamp_p) exponentials(std::true_type{}, std::false_type{});
+      else if (raw) exponentials(std::true_type{}, std::true_type{});
+      else if (!clamp_p) exponentials(std::false_type{}, std::false_type{});
+      else exponentials(std::false_type{}, std::true_type{});
       l_run = l_run * alpha + psum;
 
       if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
@@ -325,7 +429,7 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
           const int krow = 32 * (p >> 1) + 8 * (2 * (p & 1) + (r8 >> 2)) + 4 * h + (r8 & 3);
-          const int off = v_lds_offset(krow, 2 * t + (g & 1)) + hh * 8;
+          const int off = v_lds_offset<kVRow>(krow, 2 * t + (g & 1)) + hh * 8;
           const i32x2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((SDPA_LDS_AS i32x2*)((SDPA_LDS_AS uint8_t*)vb + off));
           vf[2 * p] = w[0];
           vf[2 * p + 1] = w[1];
@@ -334,7 +438,8 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
       }
     }
 
-    if (blk + 1 < nblk) commit((blk + 1) & 1);
+    if (a.dma) __builtin_amdgcn_s_waitcnt(0x0f70);  // the next block has landed
+    else if (blk + 1 < nblk) commit((blk + 1) & 1);
     __syncthreads();
   }
 
@@ -465,6 +570,8 @@ int mi355q_fp8_sdpa_fwd(const void* q, const void* k, const void* v, int fp8_fmt
   a.causal = is_causal != 0;
   a.out_fp8 = out_dtype == MI355Q_E4M3FN;
   a.vec_q = vq; a.vec_k = vk; a.vec_v = vv; a.vec_o = vo;
+  // direct loads address a block's rows with 32-bit offsets from a base that moves with the block
+  a.dma = vk && vv && d->ldk < (1 << 24) && d->ldv < (1 << 24);
   a.nqb = (int)nqb;
   a.scale = softmax_scale;
   for (int i = 0; i < 6; ++i) {
