@@ -167,7 +167,10 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
   constexpr int KLOADS = kSdpaBN * KCPR / kSdpaThreads;  // 16-byte loads per thread and block
   constexpr int VLOADS = kSdpaBN * VCPR / kSdpaThreads;
   static_assert(KLOADS >= 1 && VLOADS >= 1, "block too small for the workgroup");
-  __shared__ __align__(16) uint8_t lds[2 * (KBYTES + VBYTES)];
+  // Direct loads run kStages - 1 blocks ahead of the arithmetic (a block's arithmetic takes about a
+  // microsecond, less than a load from HBM under load); the route through registers uses two buffers.
+  constexpr int kStages = 4;
+  __shared__ __align__(1024) uint8_t lds[kStages * (KBYTES + VBYTES)];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in every lane, and known to be
@@ -304,8 +307,13 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
 
   if (nblk > 0) {
     if (a.dma) {
-      issue_block(0);
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+      for (int b = 0; b < kStages - 1 && b < nblk; ++b) issue_block(b);
+      if (nblk >= kStages - 1 && (kStages - 1) * kSdpaBN <= a.S) {
+        constexpr int cnt = (kStages - 2) * (KREG + VREG);
+        __builtin_amdgcn_s_waitcnt((cnt & 15) | ((cnt >> 4) << 14) | 0x0f70);  // block 0 has landed
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+      }
     } else {
       fetch(0);
       commit(0);
@@ -316,10 +324,10 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
   for (int blk = 0; blk < nblk; ++blk) {
     const int kv0 = blk * kSdpaBN;
     if (blk + 1 < nblk) {
-      if (a.dma) issue_block((blk + 1) & 1);
-      else fetch(blk + 1);
+      if (!a.dma) fetch(blk + 1);
     }
-    const uint8_t* kb = lds + (blk & 1) * (KBYTES + VBYTES);
+    if (a.dma && blk + kStages - 1 < nblk) issue_block((blk + kStages - 1) % kStages);
+    const uint8_t* kb = lds + (a.dma ? blk % kStages : blk & 1) * (KBYTES + VBYTES);
     const uint8_t* vb = kb + KBYTES;
 
     // a wave whose 32 rows all lie above this block's first key has nothing to add
@@ -438,8 +446,20 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
       }
     }
 
-    if (a.dma) __builtin_amdgcn_s_waitcnt(0x0f70);  // the next block has landed
-    else if (blk + 1 < nblk) commit((blk + 1) & 1);
+    if (a.dma) {
+      // The next block has landed once only the loads of the blocks after it are outstanding.  Loads
+      // retire in issue order as long as every one of them goes to memory; one whose lanes all lie
+      // beyond kv_len completes at once, so the count is only trusted while every block in flight is
+      // whole, and the tail drains everything.
+      if (blk + kStages <= nblk && (blk + kStages) * kSdpaBN <= a.S) {
+        constexpr int cnt = (kStages - 2) * (KREG + VREG);
+        __builtin_amdgcn_s_waitcnt((cnt & 15) | ((cnt >> 4) << 14) | 0x0f70);
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+      }
+    } else if (blk + 1 < nblk) {
+      commit((blk + 1) & 1);
+    }
     __syncthreads();
   }
 
