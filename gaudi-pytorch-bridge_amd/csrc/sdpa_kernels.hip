@@ -62,6 +62,11 @@ struct SdpaArgs {
   float sc_host[6];        // used where sc_dev is null; 0 = absent
   float* amax_s;
   float* amax_o;
+  // the few-queries kernel only
+  int pack;         // rows of the tile are (innermost batch index, query): k and v are shared along that dimension
+  int rows;         // rows of the tile that hold a query
+  int nsplit, blocks_per_split;
+  float* ws;        // partial results of the key splits when nsplit > 1
 };
 
 __device__ __forceinline__ float sdpa_scale(const SdpaArgs& a, int i, float absent) {
@@ -152,6 +157,129 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __global__ void sdpa_clear_amax_kernel(float* a, float* b) {
   if (a != nullptr) *a = 0.0f;
   if (b != nullptr) *b = 0.0f;
+}
+
+// One block of 64 keys for a wave's 32 query rows: S^T = K Q^T from the K tile at kb, masks, the
+// online-softmax update of (m_run, l_run, o), and O^T += V^T P^T from the V tile at vb.  qpos is the
+// lane's query position (for the causal comparison), mrow its row of the mask; `edge` says that some
+// score of the block may need masking (wave-uniform), otherwise the cheap path runs.
+template <int DKC, int DVT, int FMT>
+__device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb, const uint8_t* vb, int kv0, bool edge, int qpos,
+                                           bool q_ok, const uint8_t* mrow, const i32x8 (&qf)[DKC], float sc2, float lqs, bool clamp_p,
+                                           f32x16 (&o)[DVT], float& m_run, float& l_run) {
+  constexpr int KROW = DKC * 64;
+  constexpr int kVRow = DVT <= 4 ? 128 : 256;
+  constexpr float kMax8 = FMT == MI355Q_E5M2 ? 57344.0f : 448.0f;
+  const int lane = threadIdx.x & 63, lq = lane & 31, h = lane >> 5;
+  f32x16 s[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[t][r] = 0.0f;
+#pragma unroll
+    for (int c = 0; c < DKC; ++c) {
+      const int row = 32 * t + lq;
+      const u32x4 lo = *reinterpret_cast<const u32x4*>(kb + k_lds_offset<KROW>(row, c * 4 + h * 2));
+      const u32x4 hi = *reinterpret_cast<const u32x4*>(kb + k_lds_offset<KROW>(row, c * 4 + h * 2 + 1));
+      const i32x8 kf = {(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+      s[t] = sdpa_mfma<FMT>(kf, qf[c], s[t]);
+    }
+  }
+
+  // scores in units of log2, masks applied
+    float mx = -__builtin_inff();
+  if (!edge && sc2 >= 0.0f) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, s[t][r]);
+    mx *= sc2;
+  } else {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kv = kv0 + 32 * t + 8 * (r >> 2) + 4 * h + (r & 3);
+        float x = s[t][r] * sc2;
+        bool dead = kv >= a.S || (a.causal && kv > qpos);
+        if (a.mask_kind != kMaskNone && q_ok && kv < a.S) {
+          if (a.mask_kind == kMaskBool) dead = dead || mrow[kv] == 0;
+          else if (a.mask_kind == kMaskBf16) x += bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(mrow)[kv]) * kLog2e;
+          else x += reinterpret_cast<const float*>(mrow)[kv] * kLog2e;
+        }
+        x = dead ? -__builtin_inff() : x;
+        s[t][r] = x;
+        mx = __builtin_fmaxf(mx, x);
+      }
+  }
+  mx = __builtin_fmaxf(mx, __shfl_xor(mx, 32, 64));
+  const float m_new = __builtin_fmaxf(m_run, mx);
+  const float m_use = m_new == -__builtin_inff() ? 0.0f : m_new;
+  const float alpha = fast_exp2(m_run - m_use);
+  m_run = m_new;
+  const float shift = lqs - m_use;  // p * q_scale_s = 2^(x - m + log2 q_scale_s)
+
+  float psum = 0.0f;
+  i32x8 pf;
+  // p = 2^(x + shift) for this lane's 32 scores, their sum, and the fp8 codes packed in register
+  // order.  RAW: s still holds the unscaled products (x = s * sc2); CLAMP: q_scale_s exceeds the
+  // format's range.  Compile-time variants, so that the common one is a multiply-add, an exp2 and an
+  // add per score.
+  auto exponentials = [&](auto rawc, auto clampc) {
+    constexpr bool RAW = decltype(rawc)::value, CLAMP = decltype(clampc)::value;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float p[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float x = s[t][4 * j + i];
+          p[i] = fast_exp2(RAW ? __builtin_fmaf(x, sc2, shift) : x + shift);
+          psum += p[i];
+          if (CLAMP) p[i] = __builtin_elementwise_minimum(p[i], kMax8);
+        }
+        int w;
+        if constexpr (FMT == MI355Q_E5M2) {
+          w = __builtin_amdgcn_cvt_pk_bf8_f32(p[0], p[1], 0, false);
+          w = __builtin_amdgcn_cvt_pk_bf8_f32(p[2], p[3], w, true);
+        } else {
+          w = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
+          w = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], w, true);
+        }
+        pf[4 * t + j] = w;
+      }
+  };
+  const bool raw = !edge && sc2 >= 0.0f;  // s still holds the unscaled products
+  if (raw && !clamp_p) exponentials(std::true_type{}, std::false_type{});
+  else if (raw) exponentials(std::true_type{}, std::true_type{});
+  else if (!clamp_p) exponentials(std::false_type{}, std::false_type{});
+  else exponentials(std::false_type{}, std::true_type{});
+  l_run = l_run * alpha + psum;
+
+  if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+    for (int t = 0; t < DVT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
+  }
+
+  // O^T += V^T P^T; k-slot 8 p + r' of half-wave h is key 32 (p / 2) + 8 (2 (p % 2) + r' / 4) + 4 h + r' % 4
+  const int g = lane >> 4, gi = lane & 15;
+  const int r8 = gi >> 1, hh = gi & 1;
+#pragma unroll
+  for (int t = 0; t < DVT; ++t) {
+    i32x8 vf;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int krow = 32 * (p >> 1) + 8 * (2 * (p & 1) + (r8 >> 2)) + 4 * h + (r8 & 3);
+      const int off = v_lds_offset<kVRow>(krow, 2 * t + (g & 1)) + hh * 8;
+      const i32x2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((SDPA_LDS_AS i32x2*)((SDPA_LDS_AS uint8_t*)vb + off));
+      vf[2 * p] = w[0];
+      vf[2 * p + 1] = w[1];
+    }
+    o[t] = sdpa_mfma<FMT>(vf, pf, o[t]);
+  }
 }
 
 // DKC: 64-byte steps of the q.k depth (head_dim_qk <= 64 DKC); DVT: 32-column tiles of v
@@ -305,6 +433,7 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
   float m_run = -__builtin_inff();  // running maximum of the scaled scores, in units of log2
   float l_run = 0.0f;               // this half-wave's share of the running sum (times q_scale_s)
 
+  const uint8_t* mrow = a.mask + (m_off + (int64_t)qrow * a.ldm) * (a.mask_kind == kMaskBool ? 1 : a.mask_kind == kMaskBf16 ? 2 : 4);
   if (nblk > 0) {
     if (a.dma) {
       for (int b = 0; b < kStages - 1 && b < nblk; ++b) issue_block(b);
@@ -333,117 +462,8 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
     // a wave whose 32 rows all lie above this block's first key has nothing to add
     const bool active = !(a.causal && kv0 > wq0 + 31);
     if (active) {
-      f32x16 s[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[t][r] = 0.0f;
-#pragma unroll
-        for (int c = 0; c < DKC; ++c) {
-          const int row = 32 * t + lq;
-          const u32x4 lo = *reinterpret_cast<const u32x4*>(kb + k_lds_offset<KROW>(row, c * 4 + h * 2));
-          const u32x4 hi = *reinterpret_cast<const u32x4*>(kb + k_lds_offset<KROW>(row, c * 4 + h * 2 + 1));
-          const i32x8 kf = {(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-          s[t] = sdpa_mfma<FMT>(kf, qf[c], s[t]);
-        }
-      }
-
-      // scores in units of log2, masks applied
       const bool edge = (a.causal && kv0 + kSdpaBN - 1 > wq0) || kv0 + kSdpaBN > a.S || a.mask_kind != kMaskNone;
-      float mx = -__builtin_inff();
-      if (!edge && sc2 >= 0.0f) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) mx = __builtin_fmaxf(mx, s[t][r]);
-        mx *= sc2;
-      } else {
-        const uint8_t* mrow = a.mask + (m_off + (int64_t)qrow * a.ldm) * (a.mask_kind == kMaskBool ? 1 : a.mask_kind == kMaskBf16 ? 2 : 4);
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int kv = kv0 + 32 * t + 8 * (r >> 2) + 4 * h + (r & 3);
-            float x = s[t][r] * sc2;
-            bool dead = kv >= a.S || (a.causal && kv > qrow);
-            if (a.mask_kind != kMaskNone && q_ok && kv < a.S) {
-              if (a.mask_kind == kMaskBool) dead = dead || mrow[kv] == 0;
-              else if (a.mask_kind == kMaskBf16) x += bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(mrow)[kv]) * kLog2e;
-              else x += reinterpret_cast<const float*>(mrow)[kv] * kLog2e;
-            }
-            x = dead ? -__builtin_inff() : x;
-            s[t][r] = x;
-            mx = __builtin_fmaxf(mx, x);
-          }
-      }
-      mx = __builtin_fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = __builtin_fmaxf(m_run, mx);
-      const float m_use = m_new == -__builtin_inff() ? 0.0f : m_new;
-      const float alpha = fast_exp2(m_run - m_use);
-      m_run = m_new;
-      const float shift = lqs - m_use;  // p * q_scale_s = 2^(x - m + log2 q_scale_s)
-
-      float psum = 0.0f;
-      i32x8 pf;
-      // p = 2^(x + shift) for this lane's 32 scores, their sum, and the fp8 codes packed in register
-      // order.  RAW: s still holds the unscaled products (x = s * sc2); CLAMP: q_scale_s exceeds the
-      // format's range.  Compile-time variants, so that the common one is a multiply-add, an exp2 and an
-      // add per score.
-      auto exponentials = [&](auto rawc, auto clampc) {
-        constexpr bool RAW = decltype(rawc)::value, CLAMP = decltype(clampc)::value;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            float p[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const float x = s[t][4 * j + i];
-              p[i] = fast_exp2(RAW ? __builtin_fmaf(x, sc2, shift) : x + shift);
-              psum += p[i];
-              if (CLAMP) p[i] = __builtin_elementwise_minimum(p[i], kMax8);
-            }
-            int w;
-            if constexpr (FMT == MI355Q_E5M2) {
-              w = __builtin_amdgcn_cvt_pk_bf8_f32(p[0], p[1], 0, false);
-              w = __builtin_amdgcn_cvt_pk_bf8_f32(p[2], p[3], w, true);
-            } else {
-              w = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
-              w = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], w, true);
-            }
-            pf[4 * t + j] = w;
-          }
-      };
-      const bool raw = !edge && sc2 >= 0.0f;  // s still holds the unscaled products
-      if (raw && !clamp_p) exponentials(std::true_type{}, std::false_type{});
-      else if (raw) exponentials(std::true_type{}, std::true_type{});
-      else if (!clamp_p) exponentials(std::false_type{}, std::false_type{});
-      else exponentials(std::false_type{}, std::true_type{});
-      l_run = l_run * alpha + psum;
-
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-        for (int t = 0; t < DVT; ++t)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
-      }
-
-      // O^T += V^T P^T; k-slot 8 p + r' of half-wave h is key 32 (p / 2) + 8 (2 (p % 2) + r' / 4) + 4 h + r' % 4
-      const int g = lane >> 4, gi = lane & 15;
-      const int r8 = gi >> 1, hh = gi & 1;
-#pragma unroll
-      for (int t = 0; t < DVT; ++t) {
-        i32x8 vf;
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-          const int krow = 32 * (p >> 1) + 8 * (2 * (p & 1) + (r8 >> 2)) + 4 * h + (r8 & 3);
-          const int off = v_lds_offset<kVRow>(krow, 2 * t + (g & 1)) + hh * 8;
-          const i32x2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((SDPA_LDS_AS i32x2*)((SDPA_LDS_AS uint8_t*)vb + off));
-          vf[2 * p] = w[0];
-          vf[2 * p + 1] = w[1];
-        }
-        o[t] = sdpa_mfma<FMT>(vf, pf, o[t]);
-      }
+      sdpa_block<DKC, DVT, FMT>(a, kb, vb, kv0, edge, qrow, q_ok, mrow, qf, sc2, lqs, clamp_p, o, m_run, l_run);
     }
 
     if (a.dma) {
@@ -516,6 +536,323 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
   }
 }
 
+// ------------------------------------------------------------------ few queries, many keys
+//
+// Decoding: a handful of queries per head against a long key / value cache.  The 128-row
+// workgroups of the kernel above would hold one useful row each and every query head of a group
+// would stream the group's K and V again.  Here the rows of one 32-row tile are all the queries
+// that share a K and V -- (head of the group, query position) pairs, up to 32 -- and the keys are
+// what is split: over `nsplit` workgroups, and inside a workgroup over its four waves, block by
+// block.  Each wave streams its own blocks through LDS stages of its own (no barrier in the loop)
+// and keeps its own running maximum, sum and O; the four are merged through LDS at the end, and
+// the splits' results (unnormalised O, m, l per row) through a workspace by a second small kernel.
+
+constexpr int kDecodeTileFloats(int DVT) { return 32 * DVT * 32 + 64; }  // O^T [dv][row], m[row], l[row]
+
+// merges `n` partial results for row `row`, columns dv0, dv0 + dvstep, ...; returns the row's 1 / l
+// (0 for a row with nothing to attend to) and leaves the merged, normalised values in `val`
+template <int DVT>
+__device__ __forceinline__ float sdpa_merge(const float* parts, int n, int stride_floats, int row, int dv0, int dvstep, float qs,
+                                            float (&val)[DVT * 32 / 8]) {
+  float M = -__builtin_inff();
+  for (int w = 0; w < n; ++w) M = __builtin_fmaxf(M, parts[(int64_t)w * stride_floats + 32 * DVT * 32 + row]);
+  float L = 0.0f;
+#pragma unroll
+  for (int i = 0; i < DVT * 32 / 8; ++i) val[i] = 0.0f;
+  for (int w = 0; w < n; ++w) {
+    const float* pw = parts + (int64_t)w * stride_floats;
+    const float mw = pw[32 * DVT * 32 + row];
+    const float wgt = mw == -__builtin_inff() ? 0.0f : fast_exp2(mw - M);
+    L += pw[32 * DVT * 32 + 32 + row] * wgt;
+#pragma unroll
+    for (int i = 0; i < DVT * 32 / 8; ++i) val[i] += pw[(dv0 + i * dvstep) * 32 + row] * wgt;
+  }
+  const float l = L / qs;
+  const float inv_l = l > 0.0f ? 1.0f / l : 0.0f;
+#pragma unroll
+  for (int i = 0; i < DVT * 32 / 8; ++i) val[i] *= inv_l;
+  return inv_l;
+}
+
+// final scaling, rounding and store of one row's merged values (columns dv0 + i dvstep), amax updates
+template <int DVT>
+__device__ __forceinline__ void sdpa_store_row(const SdpaArgs& a, uint8_t* orow, bool row_ok, float inv_l, int dv0, int dvstep,
+                                               const float (&val)[DVT * 32 / 8]) {
+  const float dv = sdpa_scale(a, 2, 1.0f), qs = sdpa_scale(a, 3, 1.0f), ds = sdpa_scale(a, 5, 1.0f / qs);
+  const float qo = a.out_fp8 ? sdpa_scale(a, 4, 1.0f) : 1.0f;
+  float amax_o = 0.0f;
+#pragma unroll
+  for (int i = 0; i < DVT * 32 / 8; ++i) {
+    const int d = dv0 + i * dvstep;
+    const float v = val[i] * (ds * dv);
+    if (row_ok && d < a.Dv) {
+      amax_o = __builtin_fmaxf(amax_o, __builtin_fabsf(v));
+      if (a.out_fp8) orow[d] = (uint8_t)(cvt_fp8x4<MI355Q_E4M3FN>(v * qo, 0.f, 0.f, 0.f) & 0xffu);
+      else reinterpret_cast<uint16_t*>(orow)[d] = (uint16_t)(pack_bf16x2(v, 0.f) & 0xffffu);
+    }
+  }
+  const int lane = threadIdx.x & 63;
+  if (a.amax_s != nullptr) {
+    const uint32_t m = wave_max_u32(__float_as_uint(row_ok ? inv_l : 0.0f));
+    if (lane == 0 && m != 0u) atomicMax(reinterpret_cast<unsigned int*>(a.amax_s), m);
+  }
+  if (a.amax_o != nullptr) {
+    const uint32_t m = wave_max_u32(__float_as_uint(amax_o));
+    if (lane == 0 && m != 0u) atomicMax(reinterpret_cast<unsigned int*>(a.amax_o), m);
+  }
+}
+
+// offsets of workgroup `g`'s tensors; with `pack` the innermost batch dimension stays inside the tile
+__device__ __forceinline__ void sdpa_group_offsets(const SdpaArgs& a, int64_t g, int64_t& q_off, int64_t& k_off, int64_t& v_off,
+                                                   int64_t& m_off, int64_t& o_off) {
+  q_off = k_off = v_off = m_off = o_off = 0;
+#pragma unroll
+  for (int d = 2; d >= 0; --d) {
+    if (d == 2 && a.pack) continue;
+    const int64_t b = g % a.bdim[d];
+    g /= a.bdim[d];
+    q_off += b * a.q_bs[d];
+    k_off += b * a.k_bs[d];
+    v_off += b * a.v_bs[d];
+    m_off += b * a.m_bs[d];
+    o_off += b * a.o_bs[d];
+  }
+}
+
+template <int DKC, int DVT, int FMT>
+__global__ __launch_bounds__(kSdpaThreads) void fp8_sdpa_decode_kernel(const SdpaArgs a) {
+  constexpr int KROW = DKC * 64;
+  constexpr int kVRow = 128;
+  static_assert(DVT <= 4, "256-byte V rows do not fit four waves' stages");
+  constexpr int KCPR = KROW / 16;
+  constexpr int KBYTES = kSdpaBN * KROW, VBYTES = kSdpaBN * kVRow;
+  constexpr int KREG = KBYTES / 1024, VREG = VBYTES / 1024;  // regions per block, all loaded by the block's wave
+  constexpr int kStage = KBYTES + VBYTES;
+  constexpr int kOps = KREG + VREG;
+  static_assert(kOps <= 63, "vmcnt holds 6 bits");
+  static_assert(4 * kDecodeTileFloats(DVT) * 4 <= 4 * 2 * kStage, "the merge area overlays the stages");
+  __shared__ __align__(1024) uint8_t lds[4 * 2 * kStage];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lq = lane & 31, h = lane >> 5;
+  const int64_t grp = blockIdx.x / a.nsplit;
+  const int split = blockIdx.x - (int)grp * a.nsplit;
+  int64_t q_off, k_off, v_off, m_off, o_off;
+  sdpa_group_offsets(a, grp, q_off, k_off, v_off, m_off, o_off);
+
+  // this lane's row of the tile: (innermost batch index, query position)
+  const int inner = a.pack ? lq / a.L : 0, qpos = a.pack ? lq - inner * a.L : lq;
+  const bool q_ok = lq < a.rows;
+  const uint8_t* qrowp = a.q + q_off + (int64_t)inner * a.q_bs[2] + (int64_t)qpos * a.ldq;
+  const uint8_t* mrow = a.mask + (m_off + (int64_t)inner * a.m_bs[2] + (int64_t)qpos * a.ldm) *
+                                     (a.mask_kind == kMaskBool ? 1 : a.mask_kind == kMaskBf16 ? 2 : 4);
+
+  const float dq = sdpa_scale(a, 0, 1.0f), dk = sdpa_scale(a, 1, 1.0f);
+  const float qs = sdpa_scale(a, 3, 1.0f);
+  const float sc2 = a.scale * dq * dk * kLog2e;
+  const float lqs = __builtin_log2f(qs);
+  constexpr float kMax8 = FMT == MI355Q_E5M2 ? 57344.0f : 448.0f;
+  const bool clamp_p = !(qs <= kMax8);
+
+  i32x8 qf[DKC];
+#pragma unroll
+  for (int c = 0; c < DKC; ++c) {
+    const u32x4 lo = load_chunk(qrowp, q_ok, 64 * c + 32 * h, a.Dk, a.vec_q);
+    const u32x4 hi = load_chunk(qrowp, q_ok, 64 * c + 32 * h + 16, a.Dk, a.vec_q);
+    qf[c] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+  }
+
+  // this workgroup's blocks of keys, and of those this wave's: first, first + 4, ...
+  const int nblk_all = (a.S + kSdpaBN - 1) / kSdpaBN;
+  const int b0 = split * a.blocks_per_split;
+  const int b1 = b0 + a.blocks_per_split < nblk_all ? b0 + a.blocks_per_split : nblk_all;
+
+  int kvoff[KREG], vvoff[VREG];
+#pragma unroll
+  for (int n = 0; n < KREG; ++n) {
+    const int pos = n * 64 + lane;
+    const int row = pos / KCPR, chunk = (pos % KCPR) ^ k_swizzle<KROW>(pos / KCPR);
+    kvoff[n] = chunk * 16 < a.Dk ? row * (int)a.ldk + chunk * 16 : 0x7fffffff;
+  }
+#pragma unroll
+  for (int n = 0; n < VREG; ++n) {
+    const int pos = n * 64 + lane;
+    const int row = pos / (kVRow / 16), chunk = (pos % (kVRow / 16)) ^ v_swizzle<kVRow>(pos / (kVRow / 16));
+    vvoff[n] = chunk * 16 < a.Dv ? row * (int)a.ldv + chunk * 16 : 0x7fffffff;
+  }
+  const int64_t first_row = (int64_t)(b0 + wave) * kSdpaBN;
+  SdpaWalker wk{reinterpret_cast<uint64_t>(a.k + k_off + first_row * a.ldk), (int64_t)(a.S - 1 - first_row) * a.ldk + a.Dk};
+  SdpaWalker wv{reinterpret_cast<uint64_t>(a.v + v_off + first_row * a.ldv), (int64_t)(a.S - 1 - first_row) * a.ldv + a.Dv};
+  uint8_t* const mine = lds + wave * 2 * kStage;
+  auto issue_block = [&](int buf) {
+    const uint32_t kdst = (uint32_t)(uintptr_t)(SDPA_LDS_AS uint8_t*)(mine + buf * kStage);
+    const i32x4 rk = wk.rsrc();
+#pragma unroll
+    for (int n = 0; n < KREG; ++n) sdpa_dma16(rk, kvoff[n], kdst + n * 1024);
+    const i32x4 rv = wv.rsrc();
+#pragma unroll
+    for (int n = 0; n < VREG; ++n) sdpa_dma16(rv, vvoff[n], kdst + KBYTES + n * 1024);
+    wk.base += (uint64_t)4 * kSdpaBN * a.ldk;
+    wk.left -= (int64_t)4 * kSdpaBN * a.ldk;
+    wv.base += (uint64_t)4 * kSdpaBN * a.ldv;
+    wv.left -= (int64_t)4 * kSdpaBN * a.ldv;
+  };
+
+  f32x16 o[DVT];
+#pragma unroll
+  for (int t = 0; t < DVT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[t][r] = 0.0f;
+  float m_run = -__builtin_inff(), l_run = 0.0f;
+
+  int buf = 0;
+  if (b0 + wave < b1) issue_block(0);
+  for (int blk = b0 + wave; blk < b1; blk += 4) {
+    const int kv0 = blk * kSdpaBN;
+    const bool more = blk + 4 < b1;
+    if (more) issue_block(buf ^ 1);
+    // This block has landed once only the next one's loads are outstanding; a block that reaches beyond
+    // kv_len may hold loads that complete at once, out of order, so the count is used between whole blocks only.
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    const uint8_t* kb = mine + buf * kStage;
+    const bool edge = a.causal || kv0 + kSdpaBN > a.S || a.mask_kind != kMaskNone;
+    sdpa_block<DKC, DVT, FMT>(a, kb, kb + KBYTES, kv0, edge, qpos, q_ok, mrow, qf, sc2, lqs, clamp_p, o, m_run, l_run);
+    buf ^= 1;
+  }
+
+  // ---- merge the four waves: each leaves O^T [dv][row], m[row], l[row] in LDS
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();  // every wave is done with its stages
+  float* tile = reinterpret_cast<float*>(lds) + wave * kDecodeTileFloats(DVT);
+#pragma unroll
+  for (int t = 0; t < DVT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) tile[(32 * t + 8 * (r >> 2) + 4 * h + (r & 3)) * 32 + lq] = o[t][r];
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  if (h == 0) {
+    tile[32 * DVT * 32 + lq] = m_run;
+    tile[32 * DVT * 32 + 32 + lq] = l_tot;
+  }
+  __syncthreads();
+  const int row = tid & 31, dvg = tid >> 5;  // a thread merges columns dvg, dvg + 8, ... of one row
+  const float* parts = reinterpret_cast<const float*>(lds);
+  if (a.nsplit == 1) {
+    float val[DVT * 32 / 8];
+    const float inv_l = sdpa_merge<DVT>(parts, 4, kDecodeTileFloats(DVT), row, dvg, 8, qs, val);
+    const int rin = a.pack ? row / a.L : 0, rq = a.pack ? row - rin * a.L : row;
+    uint8_t* orow = a.out + (o_off + (int64_t)rin * a.o_bs[2] + (int64_t)rq * a.ldo) * (a.out_fp8 ? 1 : 2);
+    sdpa_store_row<DVT>(a, orow, row < a.rows, dvg == 0 ? inv_l : 0.0f, dvg, 8, val);
+  } else {
+    // unnormalised: the merged maximum, the merged sum and O for the second kernel
+    float M = -__builtin_inff();
+    for (int w = 0; w < 4; ++w) M = __builtin_fmaxf(M, parts[w * kDecodeTileFloats(DVT) + 32 * DVT * 32 + row]);
+    float L = 0.0f, val[DVT * 32 / 8];
+#pragma unroll
+    for (int i = 0; i < DVT * 32 / 8; ++i) val[i] = 0.0f;
+    for (int w = 0; w < 4; ++w) {
+      const float* pw = parts + w * kDecodeTileFloats(DVT);
+      const float mw = pw[32 * DVT * 32 + row];
+      const float wgt = mw == -__builtin_inff() ? 0.0f : fast_exp2(mw - M);
+      L += pw[32 * DVT * 32 + 32 + row] * wgt;
+#pragma unroll
+      for (int i = 0; i < DVT * 32 / 8; ++i) val[i] += pw[(dvg + 8 * i) * 32 + row] * wgt;
+    }
+    float* out = a.ws + ((int64_t)grp * a.nsplit + split) * kDecodeTileFloats(DVT);
+#pragma unroll
+    for (int i = 0; i < DVT * 32 / 8; ++i) out[(dvg + 8 * i) * 32 + row] = val[i];
+    if (dvg == 0) {
+      out[32 * DVT * 32 + row] = M;
+      out[32 * DVT * 32 + 32 + row] = L;
+    }
+  }
+}
+
+// The splits of one group merged, normalised and stored: a workgroup takes eight columns of the
+// group's tile, a thread one (row, column) and all the splits.
+template <int DVT>
+__global__ __launch_bounds__(kSdpaThreads) void fp8_sdpa_decode_merge_kernel(const SdpaArgs a) {
+  const int64_t grp = blockIdx.x;
+  int64_t q_off, k_off, v_off, m_off, o_off;
+  sdpa_group_offsets(a, grp, q_off, k_off, v_off, m_off, o_off);
+  const int tid = threadIdx.x, row = tid & 31, d = blockIdx.y * 8 + (tid >> 5);
+  const bool row_ok = row < a.rows;
+  const float* parts = a.ws + grp * a.nsplit * kDecodeTileFloats(DVT);
+  float M = -__builtin_inff(), L = 0.0f, O = 0.0f;
+  if (row_ok) {
+    for (int w = 0; w < a.nsplit; ++w) M = __builtin_fmaxf(M, parts[(int64_t)w * kDecodeTileFloats(DVT) + 32 * DVT * 32 + row]);
+    for (int w = 0; w < a.nsplit; ++w) {
+      const float* pw = parts + (int64_t)w * kDecodeTileFloats(DVT);
+      const float mw = pw[32 * DVT * 32 + row];
+      const float wgt = mw == -__builtin_inff() ? 0.0f : fast_exp2(mw - M);
+      L += pw[32 * DVT * 32 + 32 + row] * wgt;
+      O += pw[d * 32 + row] * wgt;
+    }
+  }
+  const float dv = sdpa_scale(a, 2, 1.0f), qs = sdpa_scale(a, 3, 1.0f), ds = sdpa_scale(a, 5, 1.0f / qs);
+  const float l = L / qs;
+  const float inv_l = l > 0.0f ? 1.0f / l : 0.0f;
+  const float v = O * inv_l * (ds * dv);
+  const bool store = row_ok && d < a.Dv;
+  if (store) {
+    const int rin = a.pack ? row / a.L : 0, rq = a.pack ? row - rin * a.L : row;
+    uint8_t* orow = a.out + (o_off + (int64_t)rin * a.o_bs[2] + (int64_t)rq * a.ldo) * (a.out_fp8 ? 1 : 2);
+    if (a.out_fp8) orow[d] = (uint8_t)(cvt_fp8x4<MI355Q_E4M3FN>(v * sdpa_scale(a, 4, 1.0f), 0.f, 0.f, 0.f) & 0xffu);
+    else reinterpret_cast<uint16_t*>(orow)[d] = (uint16_t)(pack_bf16x2(v, 0.f) & 0xffffu);
+  }
+  const int lane = tid & 63;
+  if (a.amax_s != nullptr && blockIdx.y == 0) {
+    const uint32_t m = wave_max_u32(__float_as_uint(row_ok && tid < 32 ? inv_l : 0.0f));
+    if (lane == 0 && m != 0u) atomicMax(reinterpret_cast<unsigned int*>(a.amax_s), m);
+  }
+  if (a.amax_o != nullptr) {
+    const uint32_t m = wave_max_u32(__float_as_uint(store ? __builtin_fabsf(v) : 0.0f));
+    if (lane == 0 && m != 0u) atomicMax(reinterpret_cast<unsigned int*>(a.amax_o), m);
+  }
+}
+
+template <int DKC, int DVT>
+static int sdpa_decode_launch(const SdpaArgs& a, int fmt, int64_t groups, hipStream_t st) {
+  const dim3 grid((unsigned)(groups * a.nsplit));
+  if (fmt == MI355Q_E5M2) hipLaunchKernelGGL((fp8_sdpa_decode_kernel<DKC, DVT, MI355Q_E5M2>), grid, dim3(kSdpaThreads), 0, st, a);
+  else hipLaunchKernelGGL((fp8_sdpa_decode_kernel<DKC, DVT, MI355Q_E4M3FN>), grid, dim3(kSdpaThreads), 0, st, a);
+  if (hipGetLastError() != hipSuccess) return MI355Q_ERR_LAUNCH;
+  if (a.nsplit > 1) {
+    hipLaunchKernelGGL((fp8_sdpa_decode_merge_kernel<DVT>), dim3((unsigned)groups, DVT * 32 / 8), dim3(kSdpaThreads), 0, st, a);
+    if (hipGetLastError() != hipSuccess) return MI355Q_ERR_LAUNCH;
+  }
+  return MI355Q_OK;
+}
+
+static int compute_units_sdpa();
+
+// How the few-queries kernel would run a problem: rows of the tile, groups, splits (0 groups: it does not apply).
+struct SdpaDecodePlan {
+  int64_t groups = 0;
+  int pack = 0, rows = 0, nsplit = 1, blocks_per_split = 0, dvt = 0;
+  size_t ws_bytes = 0;
+};
+static SdpaDecodePlan sdpa_decode_plan(const mi355q_sdpa_desc* d, int cus) {
+  SdpaDecodePlan p;
+  const bool shared = d->batch[2] > 1 && d->k_bstride[2] == 0 && d->v_bstride[2] == 0;
+  const int64_t inner = shared ? d->batch[2] : 1;
+  if (inner * d->q_len > 32 || d->kv_len < 512 || d->head_dim_qk > 128 || d->head_dim_v > 128) return p;
+  p.pack = shared;
+  p.rows = (int)(inner * d->q_len);
+  p.groups = d->batch[0] * d->batch[1] * (shared ? 1 : d->batch[2]);
+  p.dvt = (d->head_dim_qk > 64 || d->head_dim_v > 64) ? 4 : 2;
+  const int nblk = (int)((d->kv_len + kSdpaBN - 1) / kSdpaBN);
+  // enough workgroups for one per CU (a workgroup's LDS stages leave no room for a second), at least 8
+  // blocks (two per wave) in each
+  int64_t want = ((int64_t)cus + p.groups - 1) / p.groups;
+  const int64_t most = nblk / 8 > 0 ? nblk / 8 : 1;
+  want = want < 1 ? 1 : (want > most ? most : want);
+  p.blocks_per_split = (int)((nblk + want - 1) / want);
+  p.nsplit = (nblk + p.blocks_per_split - 1) / p.blocks_per_split;
+  p.ws_bytes = p.nsplit > 1 ? (size_t)p.groups * p.nsplit * kDecodeTileFloats(p.dvt) * sizeof(float) : 0;
+  return p;
+}
+
 template <int DKC, int DVT>
 static int sdpa_launch(const SdpaArgs& a, int fmt, int64_t blocks, hipStream_t st) {
   if (fmt == MI355Q_E5M2)
@@ -527,16 +864,44 @@ static int sdpa_launch(const SdpaArgs& a, int fmt, int64_t blocks, hipStream_t s
 
 static bool aligned_to(const void* p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
 
+static int compute_units_sdpa() {
+  static const int n = [] {
+    int dev = 0, cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0)
+      cu = 256;
+    return cu;
+  }();
+  return n;
+}
+
 }  // namespace mi355q
 
 using namespace mi355q;
 
 extern "C" {
 
+size_t mi355q_fp8_sdpa_workspace_bytes(const mi355q_sdpa_desc* d) {
+  if (d == nullptr || d->q_len <= 0 || d->kv_len <= 0 || d->head_dim_qk <= 0 || d->head_dim_v <= 0) return 0;
+  for (int i = 0; i < 3; ++i)
+    if (d->batch[i] <= 0) return 0;
+  return sdpa_decode_plan(d, compute_units_sdpa()).ws_bytes;
+}
+
+int mi355q_fp8_sdpa_key_splits(const mi355q_sdpa_desc* d, int64_t* blocks_per_split) {
+  if (blocks_per_split != nullptr) *blocks_per_split = 0;
+  if (d == nullptr || d->q_len <= 0 || d->kv_len <= 0 || d->head_dim_qk <= 0 || d->head_dim_v <= 0) return 0;
+  for (int i = 0; i < 3; ++i)
+    if (d->batch[i] <= 0) return 0;
+  const SdpaDecodePlan p = sdpa_decode_plan(d, compute_units_sdpa());
+  if (p.groups == 0) return 0;
+  if (blocks_per_split != nullptr) *blocks_per_split = p.blocks_per_split;
+  return p.nsplit;
+}
+
 int mi355q_fp8_sdpa_fwd(const void* q, const void* k, const void* v, int fp8_fmt, const void* mask, int mask_kind,
                         void* out, int out_dtype, const mi355q_sdpa_desc* d, float softmax_scale, int is_causal,
                         const float* const* scale_dev, const float* scale_host, float* amax_s, float* amax_o,
-                        void* stream) {
+                        void* workspace, size_t workspace_bytes, void* stream) {
   if (d == nullptr) return MI355Q_ERR_INVALID_ARGUMENT;
   if (fp8_fmt != MI355Q_E4M3FN && fp8_fmt != MI355Q_E5M2) return MI355Q_ERR_INVALID_ARGUMENT;
   if (out_dtype != MI355Q_BF16 && out_dtype != MI355Q_E4M3FN) return MI355Q_ERR_INVALID_ARGUMENT;
@@ -602,6 +967,20 @@ int mi355q_fp8_sdpa_fwd(const void* q, const void* k, const void* v, int fp8_fmt
   a.amax_o = amax_o;
 
   const int64_t dmax = d->head_dim_qk > d->head_dim_v ? d->head_dim_qk : d->head_dim_v;
+  // a few queries against many keys: the kernel that splits the keys (direct loads only)
+  SdpaDecodePlan plan = sdpa_decode_plan(d, compute_units_sdpa());
+  if (plan.groups > 0 && a.dma && plan.groups * (int64_t)plan.nsplit <= 0x7fffffff) {
+    if (plan.nsplit > 1 && (workspace == nullptr || workspace_bytes < plan.ws_bytes || !aligned_to(workspace, 4))) {
+      plan.nsplit = 1;  // no room for partial results: one workgroup per group walks all the keys
+      plan.blocks_per_split = (int)((d->kv_len + kSdpaBN - 1) / kSdpaBN);
+    }
+    a.pack = plan.pack;
+    a.rows = plan.rows;
+    a.nsplit = plan.nsplit;
+    a.blocks_per_split = plan.blocks_per_split;
+    a.ws = static_cast<float*>(workspace);
+    return plan.dvt == 2 ? sdpa_decode_launch<1, 2>(a, fp8_fmt, plan.groups, st) : sdpa_decode_launch<2, 4>(a, fp8_fmt, plan.groups, st);
+  }
   if (dmax <= 64) return sdpa_launch<1, 2>(a, fp8_fmt, blocks, st);
   if (dmax <= 128) return sdpa_launch<2, 4>(a, fp8_fmt, blocks, st);
   return sdpa_launch<4, 8>(a, fp8_fmt, blocks, st);

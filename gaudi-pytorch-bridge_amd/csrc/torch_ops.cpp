@@ -1038,19 +1038,19 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
   const at::ScalarType stat_dt = fp8_in ? at::kBFloat16 : dt;
   auto opts = q.options();
   Tensor out = at::empty(out_shape, opts.dtype(out_dt));
-  Tensor m = at::empty({1}, opts.dtype(stat_dt));
-  Tensor linv = at::empty({1}, opts.dtype(fp8_in || softmax_mode == "fast" ? at::kBFloat16 : at::kFloat));
-  Tensor seed = at::empty({1}, opts.dtype(at::kInt));
-  Tensor amax_s = at::empty({1}, opts.dtype(at::kFloat));
-  Tensor amax_o = at::empty({1}, opts.dtype(at::kFloat));
-  if (q.is_meta()) return SdpaOut(out, m, linv, seed, amax_s, amax_o);
+  const at::ScalarType linv_dt = fp8_in || softmax_mode == "fast" ? at::kBFloat16 : at::kFloat;
+  if (q.is_meta())
+    return SdpaOut(out, at::empty({1}, opts.dtype(stat_dt)), at::empty({1}, opts.dtype(linv_dt)), at::empty({1}, opts.dtype(at::kInt)),
+                   at::empty({1}, opts.dtype(at::kFloat)), at::empty({1}, opts.dtype(at::kFloat)));
+  // the five one-element outputs (placeholders in inference, sdpa_gen.cpp:944-965) share one zeroed
+  // allocation: one fill instead of five
+  Tensor pool = at::zeros({40}, opts.dtype(at::kByte));
+  auto one = [&](int slot, at::ScalarType t) { return pool.slice(0, 8 * slot, 8 * slot + (int64_t)c10::elementSize(t)).view(t); };
+  Tensor m = one(0, stat_dt), linv = one(1, linv_dt), seed = one(2, at::kInt), amax_s = one(3, at::kFloat), amax_o = one(4, at::kFloat);
   DeviceGuard guard(q.device());
   TORCH_CHECK(k.device() == q.device() && v.device() == q.device(), "fp8_sdpa_recomp_fwd: q, k and v must be on one device");
   MI355Q_OP_INFO("fp8_sdpa_recomp_fwd : q=" << q.sizes() << " k=" << k.sizes() << " v=" << v.sizes() << " " << dt << " -> " << out_dt
                                              << (is_causal ? " causal" : "") << (has_mask ? " mask" : ""));
-  m.zero_();
-  linv.zero_();
-  seed.zero_();
 
   if (!fp8_in) {
     // The measurement pass of the reference's flow: bf16 / fp32 q, k, v, no fp8 anywhere; only amax_s
@@ -1069,19 +1069,11 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
     pr = at::nan_to_num(pr, 0.0);   // a row with every key masked
     out.copy_(at::matmul(pr.to(dt), v));
     if (pr.numel() > 0) amax_s.copy_(pr.max().reshape({1}));
-    else amax_s.zero_();
     if (out.numel() > 0) amax_o.copy_(out.to(at::kFloat).abs().max().reshape({1}));
-    else amax_o.zero_();
     return SdpaOut(out, m, linv, seed, amax_s, amax_o);
   }
 
-  if (!is_amax_s) amax_s.zero_();
-  if (!is_amax_o) amax_o.zero_();
-  if (out.numel() == 0) {
-    amax_s.zero_();
-    amax_o.zero_();
-    return SdpaOut(out, m, linv, seed, amax_s, amax_o);
-  }
+  if (out.numel() == 0) return SdpaOut(out, m, linv, seed, amax_s, amax_o);
   TORCH_CHECK(Dk <= 256 && Dv <= 256, "fp8_sdpa_recomp_fwd: head dimensions up to 256 are supported, got ", Dk, " and ", Dv);
   Tensor qc = sdpa_unit_rows(q), kc = sdpa_unit_rows(k), vc = sdpa_unit_rows(v);
   mi355q_sdpa_desc d{};
@@ -1125,10 +1117,15 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
     sc_dev[i] = sc[i]->dev;
     sc_host[i] = sc[i]->host;
   }
+  // few queries against many keys: the partial results of the key splits pass through a workspace
+  const size_t ws_bytes = mi355q_fp8_sdpa_workspace_bytes(&d);
+  Tensor ws;
+  if (ws_bytes > 0) ws = at::empty({(int64_t)ws_bytes}, opts.dtype(at::kByte));
   check_status(mi355q_fp8_sdpa_fwd(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), to_mi355q_dtype(dt), has_mask ? mk.data_ptr() : nullptr,
                                    mask_kind, out.data_ptr(), to_mi355q_dtype(out_dt), &d, (float)scale, is_causal ? 1 : 0, sc_dev,
                                    sc_host, is_amax_s ? amax_s.data_ptr<float>() : nullptr,
-                                   is_amax_o ? amax_o.data_ptr<float>() : nullptr, current_stream(q)),
+                                   is_amax_o ? amax_o.data_ptr<float>() : nullptr, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes,
+                                   current_stream(q)),
                "mi355q_fp8_sdpa_fwd");
   return SdpaOut(out, m, linv, seed, amax_s, amax_o);
 }

@@ -348,10 +348,26 @@ typedef struct mi355q_sdpa_desc {
   int64_t ldq, ldk, ldv, ldmask, ldo;
 } mi355q_sdpa_desc;
 
+/*
+ * Few queries against many keys (decoding: at most 32 rows of (innermost batch index, query) that
+ * share a k and v, kv_len >= 512, head dimensions up to 128, 16-byte aligned rows) run on a kernel
+ * that splits the keys over workgroups; the splits' partial results pass through `workspace`
+ * (device memory, mi355q_fp8_sdpa_workspace_bytes(desc) bytes, 0 when the problem does not split).
+ * Without a workspace of that size the call still works, one workgroup per group of rows.
+ * Nothing is allocated here.
+ */
+size_t mi355q_fp8_sdpa_workspace_bytes(const mi355q_sdpa_desc* desc);
+/* How the few-queries kernel would walk the keys of a problem with a workspace of that size:
+ * returns the number of key splits and stores the 64-key blocks per split (0 and 0 when the
+ * problem takes the other kernel).  Inside a split the four waves take every fourth block.  The
+ * probabilities are rounded to fp8 against each wave's own running maximum, so results depend
+ * on this walk in their last fp8-rounding digit; for logs, and for tests that restate it. */
+int mi355q_fp8_sdpa_key_splits(const mi355q_sdpa_desc* desc, int64_t* blocks_per_split);
 int mi355q_fp8_sdpa_fwd(const void* q, const void* k, const void* v, int fp8_fmt, const void* mask,
                         int mask_kind, void* out, int out_dtype, const mi355q_sdpa_desc* desc,
                         float softmax_scale, int is_causal, const float* const* scale_dev,
-                        const float* scale_host, float* amax_s, float* amax_o, void* stream);
+                        const float* scale_host, float* amax_s, float* amax_o, void* workspace,
+                        size_t workspace_bytes, void* stream);
 
 /*
  * Measurement aids without a counterpart in the reference; the product path never calls them.

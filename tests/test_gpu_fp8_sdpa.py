@@ -44,6 +44,28 @@ def run_op(dev, q, k, v, mask=None, scale=None, causal=False, scales=NONE6, amax
               *sc, amax_s, amax_o, None, "left")
 
 
+def key_walk(pkg, q, k, v, workspace=True):
+    """How the device walks the keys of this problem (None: block after block): asked of the library with the
+    description the torch layer builds (batch extents right-aligned to three, stride 0 where k / v are broadcast)."""
+    nb = q.dim() - 2
+    bshape = list(torch.broadcast_shapes(q.shape[:-2], k.shape[:-2], v.shape[:-2]))
+    batch = [1] * (3 - nb) + bshape
+
+    def strides(t):
+        st = [0] * (3 - nb) + [0 if t.shape[i] == 1 else t.stride(i) for i in range(nb)]
+        return st
+    desc = (ctypes.c_int64 * 27)(*batch, *strides(q), *strides(k), *strides(v), 0, 0, 0, 0, 0, 0,
+                                 q.shape[-2], k.shape[-2], q.shape[-1], v.shape[-1],
+                                 q.stride(-2), k.stride(-2), v.stride(-2), 0, v.shape[-1])
+    per = ctypes.c_int64(0)
+    n = pkg.capi().mi355q_fp8_sdpa_key_splits(desc, ctypes.byref(per))
+    if n == 0:
+        return None
+    if not workspace:
+        return (1, -(-k.shape[-2] // 64), 4)
+    return (n, per.value, 4)
+
+
 def check_bf16(out, ref, what="", vmax=None):
     """vmax: max |v * d_scale_v| (the largest value an output can take); max |ref| stands in when not given."""
     out, ref = out.cpu().float(), ref.float()
@@ -81,7 +103,7 @@ def check_fp8(out, ref, what=""):
     (1, 1, 1, 1, 700, 128, 128),    # one query (decoding)
     (2, 1, 1, 3, 64, 64, 128),
 ])
-def test_against_oracle(oracle, dev, shape, causal):
+def test_against_oracle(oracle, pkg, dev, shape, causal):
     B, H, HK, L, S, DK, DV = shape
     gen = torch.Generator().manual_seed(L * 1000 + S + DK)
     q, k, v = make_qkv(gen, (B, H, L, DK), (B, HK, S, DK), (B, HK, S, DV))
@@ -89,7 +111,7 @@ def test_against_oracle(oracle, dev, shape, causal):
     out, m, linv, seed, amax_s, amax_o = run_op(dev, q, k, v, causal=causal, scales=scales, amax_s=True, amax_o=True)
     assert out.dtype == torch.bfloat16 and m.shape == (1,) and linv.shape == (1,) and seed.dtype == torch.int32
     ref, ref_as, ref_ao = oracle.torch_fp8_sdpa(q, k, v, is_causal=causal, d_scale_q=0.5, d_scale_k=2.0, d_scale_v=0.25,
-                                                q_scale_s=128.0, d_scale_s=1.0 / 128.0)
+                                                q_scale_s=128.0, d_scale_s=1.0 / 128.0, key_streams=key_walk(pkg, q, k, v))
     check_bf16(out, ref, str(shape))
     assert abs(float(amax_s.cpu()) - float(ref_as)) <= 1e-4 * float(ref_as)
     assert abs(float(amax_o.cpu()) - float(ref_ao)) <= 2e-3 * float(ref_ao)
@@ -234,6 +256,60 @@ def test_long_sequence_properties(oracle, dev):
     assert (o1 - 1.0).abs().max() <= 2.0 ** -4
 
 
+@pytest.mark.parametrize("case", [
+    # (batch, kv heads, query heads per kv head, q_len, kv_len, head_dim, causal, mask)
+    (2, 2, 4, 1, 1000, 128, False, None),        # grouped-query decoding, keys split over workgroups
+    (1, 1, 8, 4, 4096, 128, False, "bf16"),      # 32 rows: 8 heads x 4 queries, float mask
+    (3, 2, 4, 1, 700, 64, False, "bool"),        # head dimension 64, ragged last block, bool mask
+    (2, 3, 1, 5, 900, 128, True, None),          # no sharing (one query head per kv head), causal from the top left
+    (1, 2, 4, 2, 8192, 128, False, None),        # long cache
+    (16, 8, 4, 1, 2048, 128, False, None),       # many groups: no split, one workgroup each
+    (1, 1, 4, 1, 520, 80, False, None),          # head dimension 80 (padded to 128 in LDS)
+])
+def test_few_queries_against_many_keys(oracle, pkg, dev, case):
+    """Decoding shapes take the kernel that packs the queries sharing a k / v into one tile and splits the keys:
+    same results as the oracle, in the reference wrapper's grouped layout, with and without fp8 output and amax."""
+    B, G, HG, L, S, D, causal, mk = case
+    gen = torch.Generator().manual_seed(S + D + L)
+    q, k, v = make_qkv(gen, (B, G, HG, L, D), (B, G, 1, S, D), (B, G, 1, S, D))
+    mask = None
+    if mk is not None:
+        keep = torch.rand(B, 1, 1, L, S, generator=gen) > 0.3
+        keep[..., 0] = True
+        mask = keep if mk == "bool" else torch.where(keep, 0.0, -1e9).to(torch.bfloat16)
+    sc = (0.5, 2.0, 0.25, 128.0, None, 1 / 128.0)
+    out, _, _, _, amax_s, amax_o = run_op(dev, q, k, v, mask=mask, causal=causal, scales=sc, amax_s=True, amax_o=True)
+    walk = key_walk(pkg, q, k, v)
+    assert walk is not None
+    ref, ref_as, ref_ao = oracle.torch_fp8_sdpa(q, k, v, attn_mask=mask, is_causal=causal, d_scale_q=0.5, d_scale_k=2.0,
+                                                d_scale_v=0.25, q_scale_s=128.0, d_scale_s=1 / 128.0, key_streams=walk)
+    check_bf16(out, ref, str(case))
+    assert abs(float(amax_s.cpu()) - float(ref_as)) <= 1e-4 * float(ref_as)
+    assert abs(float(amax_o.cpu()) - float(ref_ao)) <= 2e-3 * float(ref_ao)
+    out8 = run_op(dev, q, k, v, mask=mask, causal=causal, scales=(0.5, 2.0, 0.25, 128.0, 32.0, 1 / 128.0))[0]
+    ref8, _, _ = oracle.torch_fp8_sdpa(q, k, v, attn_mask=mask, is_causal=causal, d_scale_q=0.5, d_scale_k=2.0, d_scale_v=0.25,
+                                       q_scale_s=128.0, q_scale_o=32.0, d_scale_s=1 / 128.0, key_streams=walk)
+    check_fp8(out8, ref8, str(case))
+
+
+def test_few_queries_without_a_workspace(oracle, pkg, dev):
+    """The C entry point without the workspace it asks for: one workgroup per group walks all the keys."""
+    gen = torch.Generator().manual_seed(21)
+    B, G, HG, S, D = 1, 2, 4, 3000, 128
+    q, k, v = make_qkv(gen, (B, G, HG, 1, D), (B, G, 1, S, D), (B, G, 1, S, D))
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    out = torch.empty(B, G, HG, 1, D, dtype=torch.bfloat16, device=dev)
+    lib = pkg.capi()
+    desc = (ctypes.c_int64 * 27)(B, G, HG, 0, HG * D, D, 0, S * D, 0, 0, S * D, 0, 0, 0, 0, 0, HG * D, D, 1, S, D, D, D, D, D, 0, D)
+    assert lib.mi355q_fp8_sdpa_workspace_bytes(desc) > 0
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert lib.mi355q_fp8_sdpa_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), pkg.E4M3FN, None, 0, out.data_ptr(), pkg.BF16, desc,
+                                   1 / math.sqrt(D), 0, None, None, None, None, None, 0, st) == 0
+    torch.cuda.synchronize()
+    ref, _, _ = oracle.torch_fp8_sdpa(q, k, v, key_streams=key_walk(pkg, q, k, v, workspace=False))
+    check_bf16(out, ref)
+
+
 def test_argument_checks(dev):
     q = torch.zeros(1, 2, 16, 64, device=dev).to(E4)
     args = (None, 0.0, 0.125, False, False, "None", None, None, None, None, None, None, False, False, None, "left")
@@ -278,14 +354,14 @@ def test_c_entry_point_rejects_bad_arguments(pkg, dev):
     desc = (ctypes.c_int64 * 27)(*([1, 1, 1] + [0] * 15 + [16, 16, 64, 64] + [64, 64, 64, 0, 64]))
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     ok = lib.mi355q_fp8_sdpa_fwd(q.data_ptr(), q.data_ptr(), q.data_ptr(), pkg.E4M3FN, None, 0, out.data_ptr(), pkg.BF16,
-                                 desc, 0.125, 0, None, None, None, None, st)
+                                 desc, 0.125, 0, None, None, None, None, None, 0, st)
     assert ok == 0
     torch.cuda.synchronize()
     assert (out == 0).all()          # v = 0
     assert lib.mi355q_fp8_sdpa_fwd(q.data_ptr(), q.data_ptr(), q.data_ptr(), pkg.BF16, None, 0, out.data_ptr(), pkg.BF16,
-                                   desc, 0.125, 0, None, None, None, None, st) == 1
+                                   desc, 0.125, 0, None, None, None, None, None, 0, st) == 1
     assert lib.mi355q_fp8_sdpa_fwd(q.data_ptr(), q.data_ptr(), q.data_ptr(), pkg.E4M3FN, None, 2, out.data_ptr(), pkg.BF16,
-                                   desc, 0.125, 0, None, None, None, None, st) == 1     # mask kind without a mask
+                                   desc, 0.125, 0, None, None, None, None, None, 0, st) == 1     # mask kind without a mask
     desc[20] = 300                   # head_dim_qk
     assert lib.mi355q_fp8_sdpa_fwd(q.data_ptr(), q.data_ptr(), q.data_ptr(), pkg.E4M3FN, None, 0, out.data_ptr(), pkg.BF16,
-                                   desc, 0.125, 0, None, None, None, None, st) == 2
+                                   desc, 0.125, 0, None, None, None, None, None, 0, st) == 2

@@ -44,6 +44,23 @@ def test_without_rounding_it_is_plain_attention(oracle, block, causal):
     assert abs(float(amax_o) - float(ref.abs().max())) < 1e-6
 
 
+def test_the_walk_over_the_keys_does_not_matter_without_rounding(oracle):
+    """key_streams (several streams of blocks, each with its own running maximum, merged at the end) is the same
+    function as one pass when the probabilities are not rounded; with rounding it moves the result by no more than
+    the rounding does."""
+    gen = torch.Generator().manual_seed(11)
+    q = torch.randn(2, 3, 64, generator=gen).to(E4)
+    k = torch.randn(2, 1000, 64, generator=gen).to(E4)
+    v = torch.randn(2, 1000, 64, generator=gen).to(E4)
+    ref, w = plain(q.float(), k.float(), v.float())
+    for walk in ((1, 16, 4), (3, 6, 4), (16, 1, 4), (2, 8, 1)):
+        out, amax_s, _ = oracle.torch_fp8_sdpa(q, k, v, q_scale_s=128.0, quantize_p=False, key_streams=walk)
+        assert torch.equal(out, ref.float().to(torch.bfloat16))
+        assert abs(float(amax_s) - float(w.max())) < 1e-6
+        rounded, _, _ = oracle.torch_fp8_sdpa(q, k, v, q_scale_s=128.0, key_streams=walk)
+        assert (rounded.float() - ref.float()).abs().max() <= 2.0 ** -4 * v.float().abs().max()
+
+
 @pytest.mark.parametrize("kind", ["bool", "float"])
 def test_masks_and_broadcast_batches(oracle, kind):
     gen = torch.Generator().manual_seed(2)
