@@ -511,6 +511,20 @@ def bench_sdpa(oracle, dev, steps, warmup, cpu):
             e["cpu_baseline"] = {"value": round(4.0 * n * n * D * 0.5 / t / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
                                  "kind": "port", "sample": f"one head, {n} queries x {n} keys, the float64 oracle"}
         out.append(e)
+    # decoding: one query per head against a long cache; bound by reading k and v once
+    for B, S in ((64, 4096), (8, 8192)):
+        q = torch.randn(B, HK, H // HK, 1, D, generator=gen).to(E4).to(dev)
+        sets = n_sets(2 * B * HK * S * D)
+        ks = [torch.randn(B, HK, 1, S, D, generator=gen).to(E4).to(dev) for _ in range(sets)]
+        vs = [torch.randn(B, HK, 1, S, D, generator=gen).to(E4).to(dev) for _ in range(sets)]
+        f = lambda i: torch.ops.hpu.fp8_sdpa_recomp_fwd.scalar(q, ks[i % sets], vs[i % sets], None, 0.0, sc, False, False, "None", 1.0, 1.0,
+                                                               1.0, 128.0, 0.0, 1.0 / 128.0, False, False, None, "left")
+        ms = time_gpu(f, max(steps, 50), warmup)
+        nbytes = 2 * B * HK * S * D + B * H * D + 2 * B * H * D
+        out.append(hbm_entry(f"fp8_sdpa_decode_B{B}_S{S}", f"fp8_sdpa_recomp_fwd, one query per head, batch {B}, 32 query / 8 kv heads, "
+                                                           f"kv_len = {S}, head_dim 128, e4m3fn -> bf16", nbytes, ms, max(steps, 50),
+                             "fp8_sdpa_decode_kernel<2,4,e4m3fn> + fp8_sdpa_decode_merge_kernel"))
+        del ks, vs
     return out
 
 

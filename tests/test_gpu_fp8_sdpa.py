@@ -101,6 +101,10 @@ def check_fp8(out, ref, what=""):
     (1, 2, 2, 130, 190, 256, 256),
     (1, 2, 2, 96, 160, 72, 40),     # head dimensions that are no multiple of 16, and differ
     (1, 1, 1, 1, 700, 128, 128),    # one query (decoding)
+    (1, 2, 2, 300, 1500, 64, 64),   # many blocks: the ring of K / V stages in steady state, 64-byte K rows
+    (1, 2, 1, 260, 1100, 128, 128),
+    (1, 1, 1, 140, 900, 256, 256),
+    (1, 1, 1, 200, 1000, 96, 48),
     (2, 1, 1, 3, 64, 64, 128),
 ])
 def test_against_oracle(oracle, pkg, dev, shape, causal):
