@@ -57,8 +57,10 @@ MEASURED_TRAFFIC = {
     "w4a8_gemm_M16": 124.15e6,
     "w4a8_gemm_M64": 130.47e6,
     "w4a8_gemm_M256": 481.35e6,     # four row blocks of 64 stream the weights four times
-    "fp8_sdpa_B1_L8192": 125.08e6,
-    "fp8_sdpa_B4_L4096": 235.42e6,
+    "fp8_sdpa_B1_L8192": 130.55e6,
+    "fp8_sdpa_B4_L4096": 235.41e6,
+    "fp8_sdpa_decode_B64_S4096": 537.35e6,
+    "fp8_sdpa_decode_B8_S8192": 143.14e6,   # fp8_sdpa_decode_kernel 138.75 + fp8_sdpa_decode_merge_kernel 4.39
     "softmax_fp8": 1609.30e6,
     "sum_fp8_rows": 67.32e6,
     "sum_fp8_columns": 73.45e6,   # sum_columns_kernel 69.20 + sum_finish_kernel 4.25
