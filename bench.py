@@ -461,7 +461,7 @@ def bench_w4a8(oracle, dev, steps, warmup, cpu):
     scale = (torch.rand(K // G, N, generator=gen) * 0.019 + 0.001).bfloat16().to(dev)
     zp = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // G, N // 8), generator=gen, dtype=torch.int64).to(torch.int32).to(dev)
     cols = torch.randperm(K, generator=gen)[:82]
-    for M in (16, 64, 256):
+    for M in (16, 32, 64, 256):
         x = torch.randn(M, K, generator=gen)
         x[:, cols] *= 20
         x8, sx_inv = torch.ops.mi355q.quantize_rows(x.bfloat16().to(dev), E4)
@@ -478,7 +478,7 @@ def bench_w4a8(oracle, dev, steps, warmup, cpu):
                  "sample": f"M=16, {rows_n} of the 28672 output columns: unpack, (q - z) * s in float64, matmul, per-row scale"}
         out.append(hbm_entry(f"w4a8_gemm_M{M}", f"w4a8_gemm M={M} K=8192 N=28672: uint4 weights (group 128, bf16 scales, packed "
                                                 "zero points) x per-token e4m3fn activations -> bf16",
-                             nbytes, ms, steps, "w4a8_gemm_kernel", c,
+                             nbytes, ms, steps, "w4a8_wide_kernel" if M <= 32 else "w4a8_gemm_kernel", c,
                              extra={"tflops": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 2)}))
     return out
 

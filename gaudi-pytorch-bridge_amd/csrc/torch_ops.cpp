@@ -16,10 +16,13 @@
 #include <ATen/hip/HIPGeneratorImpl.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/hip/HIPGraphsC10Utils.h>
 #include <torch/library.h>
 
 #include <cstdlib>
 #include <iostream>
+#include <map>
+#include <mutex>
 #include <sstream>
 
 #include "../../include/mi355q.h"
@@ -730,6 +733,24 @@ Tensor convert_from_uint4(const Tensor& input, const Tensor& scale,
 // hpu::convert_from_int4 / convert_from_uint4 take (int4_ops.cpp:40-56), without the bf16 [K, N]
 // matrix in between.  out = out_dtype((A @ ((q - z) * s)) * A_scale_inv + bias).  The reference has no
 // fused op; shapes the kernel does not take raise (there is no second route to the same bits).
+//
+// The kernel's split over K keeps arrival counters in its workspace, which have to be zero when a
+// call starts and are left zero by every call: one zero-filled buffer per (device, stream) is kept
+// here and grown on demand, so that a call launches one kernel and nothing else.  Calls on one
+// stream run in order, which is all the sharing the buffer allows.  While a stream is being
+// captured into a graph no buffer is handed out (its memory would belong to the graph's pool, and
+// replays of two graphs could overlap): the kernel then runs without the split.
+Tensor w4a8_workspace(const Tensor& like, size_t bytes) {
+  if (bytes == 0 || c10::hip::currentStreamCaptureStatusMayInitCtx() != c10::hip::CaptureStatus::None) return Tensor();
+  static std::mutex mu;
+  // never destroyed: a static Tensor would be freed after the HIP runtime has shut down
+  static auto* cache = new std::map<std::pair<int, void*>, Tensor>();
+  std::lock_guard<std::mutex> lock(mu);
+  Tensor& t = (*cache)[std::make_pair((int)like.device().index(), current_stream(like))];
+  if (!t.defined() || (size_t)t.numel() < bytes) t = at::zeros({(int64_t)bytes}, like.options().dtype(at::kByte));
+  return t;
+}
+
 Tensor w4a8_gemm(const Tensor& A, const Tensor& packed, const Tensor& scale, const c10::optional<Tensor>& zero_point,
                  bool is_signed, at::ScalarType out_dtype, const c10::optional<Tensor>& A_scale_inv,
                  const c10::optional<Tensor>& bias) {
@@ -778,10 +799,12 @@ Tensor w4a8_gemm(const Tensor& A, const Tensor& packed, const Tensor& scale, con
     b = bias->to(out_dtype).contiguous();
   }
   MI355Q_OP_INFO("w4a8_gemm : A=" << A.sizes() << " packed=" << packed.sizes() << " group=" << group << " signed=" << is_signed);
+  Tensor ws = w4a8_workspace(a, mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, to_mi355q_dtype(s.scalar_type())));
   const int st = mi355q_w4a8_gemm(a.data_ptr(), to_mi355q_dtype(a.scalar_type()), K, w.data_ptr<int32_t>(), N / 8, s.data_ptr(),
                                   to_mi355q_dtype(s.scalar_type()), has_zp ? z.data_ptr<int32_t>() : nullptr, is_signed ? 1 : 0,
                                   group, out.data_ptr(), to_mi355q_dtype(out_dtype), N, M, N, K, sa_dev, 1.0f, sa_mode,
-                                  b.defined() ? b.data_ptr() : nullptr, current_stream(a));
+                                  b.defined() ? b.data_ptr() : nullptr, ws.defined() ? ws.data_ptr() : nullptr,
+                                  ws.defined() ? (size_t)ws.numel() : 0, current_stream(a));
   TORCH_CHECK(st != MI355Q_ERR_UNSUPPORTED,
               "mi355q::w4a8_gemm takes groups that are multiples of 128, N a multiple of 32 and K a multiple of 16 (got group ",
               group, ", N ", N, ", K ", K, "); expand the weights with hpu::convert_from_", is_signed ? "int4" : "uint4", " for other shapes");

@@ -59,6 +59,10 @@ struct W4Args {
   const uint8_t* zp;       // packed int32 [K / group, N / 8] or nullptr
   int scale_f32, is_signed;
   int stages_per_group;    // group / 128
+  // wide kernel: K is walked in `ksplit` parts by as many workgroups per strip
+  int ksplit;
+  uint32_t* tickets;       // one per strip, zero between launches
+  float* partials;         // [ksplit][strips] partial sums of 32 x 256, in the consumers' register order
 };
 
 template <int BM>
@@ -470,6 +474,456 @@ __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
   epilogue<MT, 1>(g, 0, total, 0, n0 + wn, stage_area);
 }
 
+// ---------------------------------------------------------------------------------- wide strips
+// For at most 32 rows of A, groups of 128 and bf16 scales.  A workgroup takes 256 columns: a k-row
+// of its packed weights is a whole 128-byte line (the 64-byte rows of the 128-column strips move
+// at about 3.2 TB/s, whole lines at 4.3), and K is cut into `ksplit` parts walked by as many
+// workgroups, so that a launch fills the chip whatever N is.  The parts of a strip meet through
+// memory: every workgroup stores its partial sums (already scaled by the groups' scales, fp32, in
+// register order), and the one that draws the last ticket of the strip adds them up in the order
+// of the parts, whoever came last, and runs the epilogue.  The last one also returns the ticket
+// counter to zero for the next launch.
+//
+// Roles and the stage pipeline are those of the kernel above, with eight consumer waves of 32
+// columns and four producers.  The 16-byte slots of a packed row in LDS are XORed with
+// (row / 2) % 8, which spreads the 16 rows of a transposing read over all banks.
+//
+// The loads of this kernel run close to what HBM gives, and every MFMA costs time on top of them
+// (the chip clocks lower while the matrix units work): a stage with sixteen 32x32x64 MFMAs per SIMD
+// takes a third longer than one with none.  Two things keep their number down:
+//  * the zero-points are not two more planes: sum_k a (q - z) = sum_k a q - z sum_k a, and the row
+//    sums of the stage's A tile come from one producer wave (one MFMA against a plane of ones, the
+//    producers taking turns), which leaves them in a small ring in LDS for the consumers' fold of
+//    the next stage;
+//  * with at most 16 rows (M16) the consumers use v_mfma_scale_f32_16x16x128_f8f6f4, half the
+//    matrix work of the 32x32x64 form, which would multiply 16 rows of padding.
+// In the 16x16x128 form with an fp4 first and an fp8 second operand, lane group g = lane / 16 of the
+// fp8 operand holds k = 32 g .. 32 g + 31 in its 32 bytes, and nibbles 16 p .. 16 p + 15 (p = 0, 1) of
+// the fp4 operand of lane group g pair with k = 16 (4 (g % 2) + g / 2 + 2 p) .. + 15.  Row i of the
+// first operand and column j of the second meet in lane j + 16 (i / 4), register i % 4.
+constexpr int kW4WideBN = 256;
+constexpr int kW4WidePacked = kBK * kW4WideBN / 2;
+constexpr int kW4WideStage = 32 * kBK + kW4WidePacked + kW4ScaleRow + kW4ZpRow;
+constexpr int kW4WideStages = (160 * 1024 - 1024) / kW4WideStage;
+constexpr int kW4WidePartialBytes = 32 * kW4WideBN * 4;
+constexpr int kW4WideConsumers = 8;
+constexpr int kW4WideThreads = (kW4WideConsumers + kW4ColWaves) * 64;
+constexpr int kW4SumRing = 4;  // stages of row sums kept
+
+template <int FMT_A>
+__device__ __forceinline__ f32x4 w4_mfma16(const u32x4& plane, const i32x8& fa, const f32x4& c, int e) {
+  const i32x8 b = {(int)plane[0], (int)plane[1], (int)plane[2], (int)plane[3], 0, 0, 0, 0};
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b, fa, c, 4, mfma_code<FMT_A>(), 0, e, 0, 127);
+}
+
+template <int FMT_A, bool HAS_Z, bool M16>
+__global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
+  constexpr int BM = 32;
+  constexpr int kConsumers = kW4WideConsumers;
+  constexpr int S = kW4WideStages, kStage = kW4WideStage;
+  constexpr int kOffPacked = BM * kBK, kOffScale = kOffPacked + kW4WidePacked, kOffZp = kOffScale + kW4ScaleRow;
+  constexpr int NV = M16 ? 8 : 16;  // results per consumer lane
+  using LA = DmaLoader<true, BM, kBK, kW4ColWaves>;
+  using GA = TileGeom<true, BM, kBK>;
+  constexpr int kOps = 4 + LA::kPerWave + 1;  // four 1 KiB regions of weights, A, and the scale or zero-point row
+  static_assert(S >= 3 && (S - 2) * kOps <= 63, "vmcnt holds 6 bits");
+  static_assert(kStage % 1024 == 0, "stages stay 1 KiB aligned");
+  static_assert(kConsumers * epilogue_stage_floats<1, 1>() * 4 <= S * kStage, "epilogue area overlays the ring");
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[S * kStage];
+  __shared__ float row_sums[kW4SumRing][32];
+  __shared__ uint32_t ticket_drawn;
+
+  GemmArgs g = a.g;
+  const int part = blockIdx.x % a.ksplit, strip = blockIdx.x / a.ksplit;
+  const int n0 = strip * kW4WideBN;
+  // this workgroup's part of K, whole stages (= groups)
+  const int kt_all = (g.K + kBK - 1) / kBK;
+  const int kt0 = (int)((int64_t)part * kt_all / a.ksplit), kt1 = (int)((int64_t)(part + 1) * kt_all / a.ksplit);
+  const int KT = kt1 - kt0;
+  const int k_begin = kt0 * kBK;
+  g.K = (g.K < kt1 * kBK ? g.K : kt1 * kBK) - k_begin;
+  g.A += k_begin;
+  const uint8_t* packed = a.packed + (int64_t)k_begin * a.ld_packed;
+  const uint8_t* scale = a.scale + (int64_t)kt0 * g.N * 2;
+  const uint8_t* zp = a.zp ? a.zp + (int64_t)kt0 * (g.N / 2) : nullptr;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool producer = wave >= kConsumers;
+  const int wq = producer ? wave - kConsumers : wave;  // index among the waves of its role
+  const int lane = lane_id_here();
+  float total[NV];
+#pragma unroll
+  for (int e = 0; e < NV; ++e) total[e] = 0.0f;
+
+  if (producer) {
+    LA la;
+    la.set_lane_offsets(g.lda, wq);
+    la.set_tile(g.A, g.lda, 0, g.M, g.K);
+    la.clamp_rows(g.lda, g.M);
+    // Producer wq loads k-rows 32 wq .. 32 wq + 31, four regions of 8 rows of 128 bytes.  A lane writes
+    // slot lane % 8 of row lane / 8 of its region; rows 8 r + lane / 8 have (row / 2) % 8 = 4 (r % 2) +
+    // lane / 16, so that is what the lane's slot is XORed with on the memory side.
+    const int ld = (int)a.ld_packed;
+    const int vo_even = (wq * 32 + (lane >> 3)) * ld + (((lane & 7) ^ (lane >> 4)) << 4);
+    const int vo_odd = (wq * 32 + 8 + (lane >> 3)) * ld + (((lane & 7) ^ (4 | (lane >> 4))) << 4);
+    const int64_t packed_step = (int64_t)kBK * a.ld_packed;
+    W4Walker wp;
+    wp.init(packed + n0 / 2, (int64_t)(g.K - 1) * a.ld_packed + (((g.N + 31) & ~31) - n0) / 2);
+    // producers 0 and 1 bring the scale row, 2 and 3 the zero-point row (the scale row again without one)
+    const int cols = g.N - n0 < kW4WideBN ? g.N - n0 : kW4WideBN;
+    const bool bring_zp = wq >= 2 && zp != nullptr;
+    const int64_t row_cap = bring_zp ? cols / 2 : (int64_t)cols * 2;
+    const int64_t row_step = bring_zp ? g.N / 2 : (int64_t)g.N * 2;
+    const int row_dst = wq < 2 ? kOffScale : kOffZp;
+    W4Walker wr;
+    wr.init(bring_zp ? zp + n0 / 2 : scale + (int64_t)n0 * 2, (int64_t)(KT - 1) * row_step + row_cap);
+
+    auto issue_stage = [&](int off, int stage) {
+      const uint32_t base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)(lds + off);
+      const i32x4 rp = wp.rsrc(0x7fffffffLL);
+      w4_dma16(rp, vo_even, base + kOffPacked + (wq * 4) * 1024);
+      w4_dma16(rp, vo_odd, base + kOffPacked + (wq * 4 + 1) * 1024);
+      w4_dma16(rp, vo_even + 16 * ld, base + kOffPacked + (wq * 4 + 2) * 1024);
+      w4_dma16(rp, vo_odd + 16 * ld, base + kOffPacked + (wq * 4 + 3) * 1024);
+      wp.step(packed_step);
+      static_for<LA::kPerWave>([&](auto ic) { la.template issue_one<decltype(ic)::value, true>(lds + off, stage * kBK, g.K); });
+      la.advance();
+      w4_dma16(wr.rsrc(row_cap), lane * 16, base + row_dst);
+      wr.step(row_step);
+    };
+    auto wait_for_stage = [&](int later) {
+      constexpr int full = (S - 2) * kOps;
+      if (later >= S - 2) {
+        __builtin_amdgcn_s_waitcnt((full & 15) | ((full >> 4) << 14) | 0x0070);
+      } else {
+        static_for<S - 2>([&](auto sc) {
+          constexpr int n = decltype(sc)::value;
+          constexpr int cnt = n * kOps;
+          if (later == n || (n == 0 && later < 0)) __builtin_amdgcn_s_waitcnt((cnt & 15) | ((cnt >> 4) << 14) | 0x0070);
+        });
+      }
+    };
+    // sum_k a[m, k] over the stage at `off`, for the consumers' fold one stage later
+    const u32x4 ones = {0x22222222u, 0x22222222u, 0x22222222u, 0x22222222u};  // e2m1 1.0
+    auto sum_rows = [&](int off, int slot) {
+      const uint8_t* st = lds + off;
+      if constexpr (M16) {
+        const int m = lane & 15, gk = lane >> 4;
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(st + GA::lds_offset(m, 2 * gk));
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(st + GA::lds_offset(m, 2 * gk + 1));
+        const i32x8 fa = {(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+        const f32x4 r = w4_mfma16<FMT_A>(ones, fa, f32x4{0.f, 0.f, 0.f, 0.f}, 127);
+        // every lane holds the sum of its row (lane % 16) and every lane stores it: a store under a lane mask would
+        // take the MFMA, whose result only those lanes used, under the mask with it
+        row_sums[slot][lane & 15] = r[0];
+      } else {
+        i32x8 fa[2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+          static_for<2>([&](auto pc) { read_fragment_part<true, BM, decltype(pc)::value>(st, 0, ks, fa[ks]); });
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        f32x16 r = w4_mfma<FMT_A, 127>(ones, fa[0], zero);
+        r = w4_mfma<FMT_A, 127>(ones, fa[1], r);
+        row_sums[slot][lane & 31] = r[0];  // by every lane, as above
+      }
+    };
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s) issue_stage(s * kStage, s);
+    int wr_off = (S - 1) * kStage, rd_off = 0;
+    for (int kt = 0; kt < KT; ++kt) {
+      // the loads past this part of K fall outside their descriptors, complete at once and are not counted
+      wait_for_stage(KT - 1 - kt);
+      __syncthreads();
+      issue_stage(wr_off, kt + S - 1);
+      if (HAS_Z && (kt & 3) == wq) sum_rows(rd_off, kt & (kW4SumRing - 1));
+      wr_off += kStage;
+      if (wr_off == S * kStage) wr_off = 0;
+      rd_off += kStage;
+      if (rd_off == S * kStage) rd_off = 0;
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();  // the consumers' barrier of the fold that follows the last stage
+  } else {
+    const int wn = wq * 32;
+    const uint32_t flip = a.is_signed ? 0x88888888u : 0u;
+    const uint32_t zmask = a.zp ? 0xffffffffu : 0u;
+    int rd_off = 0, slot = 0;
+    using T = std::true_type;
+    using F = std::false_type;
+    if constexpr (M16) {
+      // lane: row m = lane % 16 of A; columns wn + 16 t + 4 gk + e (t = 0, 1; e = 0 .. 3); k block gk = lane / 16
+      const int gk = lane >> 4, r16 = lane & 15;
+      int poff[2][2];
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        const int row = 16 * (4 * (gk & 1) + (gk >> 1) + 2 * p) + r16;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) poff[t][p] = kOffPacked + row * 128 + ((wq ^ ((row >> 1) & 7)) << 4) + t * 8;
+      }
+      const int aoff0 = GA::lds_offset(r16, 2 * gk), aoff1 = GA::lds_offset(r16, 2 * gk + 1);
+      const int soff = kOffScale + (wn + 4 * gk) * 2;             // + 32 t: four bf16
+      const int zoff = kOffZp + (wn / 8 + (gk >> 1)) * 4;         // + 8 t: the word of these columns
+      const int zshift = 16 * (gk & 1);
+      f32x4 acc[2][2];
+      float sc[2][4];
+      uint32_t zprev[2] = {0u, 0u};
+      auto fold = [&](auto bc, int sum_slot) {
+        constexpr int B = decltype(bc)::value;
+        float rs = 0.0f;
+        if constexpr (HAS_Z) rs = row_sums[sum_slot][r16];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float v = acc[B][t][e];
+            if constexpr (HAS_Z) v = __builtin_fmaf(-(float)((zprev[t] >> (4 * e)) & 15u), rs, v);
+            total[4 * t + e] = __builtin_fmaf(v, sc[t][e], total[4 * t + e]);
+          }
+      };
+      auto stage = [&](auto bc, auto hpc) {
+        constexpr int B = decltype(bc)::value;
+        constexpr bool HAVE_PREV = decltype(hpc)::value;
+        __syncthreads();  // the stage is in LDS, and so are the row sums of the one before
+        const uint8_t* st = lds + rd_off;
+        i32x2 wt[2][2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int p = 0; p < 2; ++p)
+            wt[t][p] = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LDS_AS i32x2*)((LDS_AS uint8_t*)st + poff[t][p]));
+        const u32x4 alo = *reinterpret_cast<const u32x4*>(st + aoff0), ahi = *reinterpret_cast<const u32x4*>(st + aoff1);
+        u32x2 snew[2];
+        uint32_t znew[2] = {0u, 0u};
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          snew[t] = *reinterpret_cast<const u32x2*>(st + soff + 32 * t);
+          if constexpr (HAS_Z) znew[t] = *reinterpret_cast<const uint32_t*>(st + zoff + 8 * t);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        const i32x8 fa = {(int)alo[0], (int)alo[1], (int)alo[2], (int)alo[3], (int)ahi[0], (int)ahi[1], (int)ahi[2], (int)ahi[3]};
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          u32x4 hi, lo;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const uint32_t w = (uint32_t)wt[t][r >> 1][r & 1] ^ flip;
+            lo[r] = w & 0x33333333u;
+            hi[r] = (w >> 2) & 0x33333333u;
+          }
+          acc[B][t] = w4_mfma16<FMT_A>(hi, fa, f32x4{0.f, 0.f, 0.f, 0.f}, 130);
+          acc[B][t] = w4_mfma16<FMT_A>(lo, fa, acc[B][t], 128);
+        }
+        // the stage before this one, whose MFMAs finished long ago, behind the MFMAs just issued
+        if constexpr (HAVE_PREV) fold(std::integral_constant<int, 1 - B>{}, (slot - 1) & (kW4SumRing - 1));
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          sc[t][0] = __uint_as_float(snew[t][0] << 16);
+          sc[t][1] = __uint_as_float(snew[t][0] & 0xffff0000u);
+          sc[t][2] = __uint_as_float(snew[t][1] << 16);
+          sc[t][3] = __uint_as_float(snew[t][1] & 0xffff0000u);
+          zprev[t] = (((znew[t] & zmask) ^ flip) >> zshift) & 0xffffu;
+        }
+        rd_off += kStage;
+        if (rd_off == S * kStage) rd_off = 0;
+        ++slot;
+      };
+      int kt = 1;
+      if (KT > 0) stage(std::integral_constant<int, 0>{}, F{});
+      for (; kt + 1 < KT; kt += 2) {
+        stage(std::integral_constant<int, 1>{}, T{});
+        stage(std::integral_constant<int, 0>{}, T{});
+      }
+      if (kt < KT) stage(std::integral_constant<int, 1>{}, T{});
+      __syncthreads();  // the row sums of the last stage
+      if (KT > 0) {
+        if (KT & 1) fold(std::integral_constant<int, 0>{}, (slot - 1) & (kW4SumRing - 1));
+        else fold(std::integral_constant<int, 1>{}, (slot - 1) & (kW4SumRing - 1));
+      }
+    } else {
+      // lane: row m = lane % 32 of A; columns wn + 8 q + 4 (lane / 32) + i, e = 4 q + i
+      const int tg = lane >> 4, tr = lane & 15, th = tg >> 1;
+      int poff[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int row = 32 * j + 16 * th + tr;
+        poff[j] = kOffPacked + row * 128 + ((wq ^ ((row >> 1) & 7)) << 4) + (tg & 1) * 8;
+      }
+      const int zoff = kOffZp + (wn / 8) * 4;  // the four words of this wave's columns
+      const int zshift = 16 * (lane >> 5);
+      const int soff = kOffScale + (wn + 4 * (lane >> 5)) * 2;
+      f32x16 acc[2];
+      float sc[16];
+      u32x4 zprev = {0u, 0u, 0u, 0u};
+      auto fold = [&](auto bc, int sum_slot) {
+        constexpr int B = decltype(bc)::value;
+        float rs = 0.0f;
+        if constexpr (HAS_Z) rs = row_sums[sum_slot][lane & 31];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          float v = acc[B][e];
+          if constexpr (HAS_Z) v = __builtin_fmaf(-(float)((zprev[e >> 2] >> (4 * (e & 3))) & 15u), rs, v);
+          total[e] = __builtin_fmaf(v, sc[e], total[e]);
+        }
+      };
+      auto stage = [&](auto bc, auto hpc) {
+        constexpr int B = decltype(bc)::value;
+        constexpr bool HAVE_PREV = decltype(hpc)::value;
+        __syncthreads();  // the stage is in LDS, and so are the row sums of the one before
+        const uint8_t* st = lds + rd_off;
+        i32x2 wt[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          wt[j] = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LDS_AS i32x2*)((LDS_AS uint8_t*)st + poff[j]));
+        i32x8 fa[2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+          static_for<2>([&](auto pc) { read_fragment_part<true, BM, decltype(pc)::value>(st, 0, ks, fa[ks]); });
+        u32x2 snew[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) snew[q] = *reinterpret_cast<const u32x2*>(st + soff + q * 16);
+        u32x4 znew = {0u, 0u, 0u, 0u};
+        if constexpr (HAS_Z) znew = *reinterpret_cast<const u32x4*>(st + zoff);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          u32x4 hi, lo;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const uint32_t w = (uint32_t)wt[2 * ks + (r >> 1)][r & 1] ^ flip;
+            lo[r] = w & 0x33333333u;
+            hi[r] = (w >> 2) & 0x33333333u;
+          }
+          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          if (ks == 0) acc[B] = w4_mfma<FMT_A, 130>(hi, fa[ks], zero);
+          else acc[B] = w4_mfma<FMT_A, 130>(hi, fa[ks], acc[B]);
+          acc[B] = w4_mfma<FMT_A, 128>(lo, fa[ks], acc[B]);
+        }
+        // the stage before this one, whose MFMAs finished long ago, behind the MFMAs just issued
+        if constexpr (HAVE_PREV) fold(std::integral_constant<int, 1 - B>{}, (slot - 1) & (kW4SumRing - 1));
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          sc[4 * q + 0] = __uint_as_float(snew[q][0] << 16);
+          sc[4 * q + 1] = __uint_as_float(snew[q][0] & 0xffff0000u);
+          sc[4 * q + 2] = __uint_as_float(snew[q][1] << 16);
+          sc[4 * q + 3] = __uint_as_float(snew[q][1] & 0xffff0000u);
+          zprev[q] = (((znew[q] & zmask) ^ flip) >> zshift) & 0xffffu;
+        }
+        rd_off += kStage;
+        if (rd_off == S * kStage) rd_off = 0;
+        ++slot;
+      };
+      int kt = 1;
+      if (KT > 0) stage(std::integral_constant<int, 0>{}, F{});
+      for (; kt + 1 < KT; kt += 2) {
+        stage(std::integral_constant<int, 1>{}, T{});
+        stage(std::integral_constant<int, 0>{}, T{});
+      }
+      if (kt < KT) stage(std::integral_constant<int, 1>{}, T{});
+      __syncthreads();  // the row sums of the last stage
+      if (KT > 0) {
+        if (KT & 1) fold(std::integral_constant<int, 0>{}, (slot - 1) & (kW4SumRing - 1));
+        else fold(std::integral_constant<int, 1>{}, (slot - 1) & (kW4SumRing - 1));
+      }
+    }
+  }
+  __syncthreads();  // every load has landed and every stage is consumed: the ring is idle
+
+  if (a.ksplit > 1) {
+    // Partial sums in register order: 64-bit word number h 64 + lane (h < NV / 2) of consumer wave wq.  They are
+    // written and read with device-scope atomic accesses, which go past the caches of this XCD to where the other
+    // XCDs see them: no cache has to be written back or invalidated as a whole, which a fence would do (and
+    // which, done by every workgroup while the others still stream, costs more than the kernel).
+    const int strips = gridDim.x / a.ksplit;
+    constexpr int kWords = 8 * 64;  // per consumer wave (half of them used with M16)
+    unsigned long long* mine = reinterpret_cast<unsigned long long*>(a.partials) + ((int64_t)(part * strips + strip) * kConsumers + wq) * kWords + lane;
+    if (!producer) {
+#pragma unroll
+      for (int h = 0; h < NV / 2; ++h) {
+        const unsigned long long v = (unsigned long long)__float_as_uint(total[2 * h]) | ((unsigned long long)__float_as_uint(total[2 * h + 1]) << 32);
+        __hip_atomic_store(mine + h * 64, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __builtin_amdgcn_s_waitcnt(0);  // the stores have been acknowledged before the ticket is drawn
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const uint32_t t = __hip_atomic_fetch_add(a.tickets + strip, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (t == (uint32_t)a.ksplit - 1) __hip_atomic_store(a.tickets + strip, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+      ticket_drawn = t;
+    }
+    __syncthreads();
+    if (ticket_drawn != (uint32_t)a.ksplit - 1) return;
+    if (!producer) {
+#pragma unroll
+      for (int e = 0; e < NV; ++e) total[e] = 0.0f;
+      const unsigned long long* from = reinterpret_cast<const unsigned long long*>(a.partials) + ((int64_t)strip * kConsumers + wq) * kWords + lane;
+      for (int p = 0; p < a.ksplit; ++p) {
+        unsigned long long v[NV / 2];
+#pragma unroll
+        for (int h = 0; h < NV / 2; ++h) v[h] = __hip_atomic_load(from + h * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int h = 0; h < NV / 2; ++h) {
+          total[2 * h] += __uint_as_float((uint32_t)v[h]);
+          total[2 * h + 1] += __uint_as_float((uint32_t)(v[h] >> 32));
+        }
+        from += (int64_t)strips * kConsumers * kWords;
+      }
+    }
+  }
+  if (producer) return;
+  if constexpr (M16) {
+    // C[m, n .. n + 3] for this lane's row and its two sets of four columns
+    const int gk = lane >> 4, m = lane & 15;
+    const ScalarScales scalars = load_scalar_scales(g);
+    if (m >= g.M) return;
+    const float sa = g.sa_mode == MI355Q_GS_PER_ROW ? g.sa[m] : scalars.sa;
+    const int es = g.out_bf16 ? 2 : 4;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int n = n0 + wq * 32 + 16 * t + 4 * gk;
+      if (n >= g.N) continue;  // N is a multiple of 32: the four columns are inside or outside together
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float bias = g.bias_mode == MI355Q_BIAS_ROW_VECTOR ? load_out_as_f32(g.bias, n + e, g.out_bf16) : 0.0f;
+        v[e] = __fmul_rn(total[4 * t + e], sa) + bias;  // rounded as the other epilogues round
+      }
+      uint8_t* cp = g.C + ((int64_t)m * g.ldc + n) * es;
+      const bool vec_ok = (reinterpret_cast<uintptr_t>(cp) % (4 * es)) == 0;
+      if (g.out_bf16) {
+        if (vec_ok) {
+          *reinterpret_cast<u32x2*>(cp) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) reinterpret_cast<uint16_t*>(cp)[e] = (uint16_t)(pack_bf16x2(v[e], v[e]) & 0xffffu);
+        }
+      } else {
+        if (vec_ok) {
+          *reinterpret_cast<f32x4*>(cp) = f32x4{v[0], v[1], v[2], v[3]};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) reinterpret_cast<float*>(cp)[e] = v[e];
+        }
+      }
+    }
+  } else {
+    f32x16 out[1][1];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) out[0][0][e] = total[e];
+    float* stage_area = reinterpret_cast<float*>(lds) + wq * epilogue_stage_floats<1, 1>();
+    epilogue<1, 1>(g, 0, out, 0, n0 + wq * 32, stage_area);
+  }
+}
+
+// How the wide kernel would split a problem: parts of K per strip (0: the wide kernel does not apply).
+inline int w4a8_wide_parts(int64_t M, int64_t N, int64_t K, int64_t group, int scale_f32) {
+  if (M > 32 || group != kBK || scale_f32 || K <= 0) return 0;
+  const int64_t strips = (N + kW4WideBN - 1) / kW4WideBN, kt = (K + kBK - 1) / kBK;
+  int64_t parts = 256 / strips;
+  if (parts > kt / 8) parts = kt / 8;
+  if (parts < 2) return strips >= 128 ? 1 : 0;
+  return (int)parts;
+}
+
 template <int BM, int FMT_A>
 void w4a8_launch(const W4Args& a, hipStream_t st) {
   dim3 grid((unsigned)((a.g.N + kW4BN - 1) / kW4BN), (unsigned)((a.g.M + BM - 1) / BM));
@@ -481,18 +935,46 @@ void w4a8_launch(const W4Args& a, hipStream_t st) {
 
 template <int FMT_A>
 void w4a8_launch_by_m(const W4Args& a, hipStream_t st) {
-  if (a.g.M <= 32) w4a8_launch<32, FMT_A>(a, st);
-  else w4a8_launch<64, FMT_A>(a, st);
+  if (a.ksplit > 0) {
+    const unsigned grid = (unsigned)((a.g.N + kW4WideBN - 1) / kW4WideBN) * (unsigned)a.ksplit;
+    const bool z = a.zp != nullptr || a.is_signed;
+    if (a.g.M <= 16) {
+      if (z) w4a8_wide_kernel<FMT_A, true, true><<<grid, kW4WideThreads, 0, st>>>(a);
+      else w4a8_wide_kernel<FMT_A, false, true><<<grid, kW4WideThreads, 0, st>>>(a);
+    } else {
+      if (z) w4a8_wide_kernel<FMT_A, true, false><<<grid, kW4WideThreads, 0, st>>>(a);
+      else w4a8_wide_kernel<FMT_A, false, false><<<grid, kW4WideThreads, 0, st>>>(a);
+    }
+  } else if (a.g.M <= 32) {
+    w4a8_launch<32, FMT_A>(a, st);
+  } else {
+    w4a8_launch<64, FMT_A>(a, st);
+  }
+}
+
+constexpr size_t kW4TicketAlign = 256;
+inline size_t w4a8_ticket_bytes(int64_t N) {
+  const size_t strips = (size_t)((N + kW4WideBN - 1) / kW4WideBN);
+  return (strips * 4 + kW4TicketAlign - 1) / kW4TicketAlign * kW4TicketAlign;
 }
 
 }  // namespace mi355q
 
 using namespace mi355q;
 
+extern "C" size_t mi355q_w4a8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group, int scale_dtype) {
+  if (M <= 0 || N <= 0 || K <= 0 || group <= 0) return 0;
+  const int parts = w4a8_wide_parts(M, N, K, group, scale_dtype == MI355Q_F32);
+  if (parts < 2) return 0;
+  const size_t strips = (size_t)((N + kW4WideBN - 1) / kW4WideBN);
+  return w4a8_ticket_bytes(N) + (size_t)parts * strips * kW4WidePartialBytes;
+}
+
 extern "C" int mi355q_w4a8_gemm(const void* A, int fmt_a, int64_t lda, const int32_t* packed, int64_t ld_packed,
                                 const void* scale, int scale_dtype, const int32_t* zero_point, int is_signed,
                                 int64_t group, void* C, int out_dtype, int64_t ldc, int64_t M, int64_t N, int64_t K,
-                                const float* sa_dev, float sa_host, int sa_mode, const void* bias, void* stream) {
+                                const float* sa_dev, float sa_host, int sa_mode, const void* bias,
+                                void* workspace, size_t workspace_bytes, void* stream) {
   if (fmt_a != MI355Q_E4M3FN && fmt_a != MI355Q_E5M2) return MI355Q_ERR_INVALID_ARGUMENT;
   if (out_dtype != MI355Q_F32 && out_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
   if (scale_dtype != MI355Q_F32 && scale_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
@@ -532,6 +1014,16 @@ extern "C" int mi355q_w4a8_gemm(const void* A, int fmt_a, int64_t lda, const int
   a.scale_f32 = scale_dtype == MI355Q_F32;
   a.is_signed = is_signed != 0;
   a.stages_per_group = (int)(group / kBK);
+  // the wide kernel where it applies: K in parts if the caller brought the room for the partial sums
+  const int parts = w4a8_wide_parts(M, N, K, group, a.scale_f32);
+  if (parts >= 2 && workspace != nullptr) {
+    if (!al16(workspace) || workspace_bytes < mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, scale_dtype)) return MI355Q_ERR_WORKSPACE;
+    a.ksplit = parts;
+    a.tickets = static_cast<uint32_t*>(workspace);
+    a.partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + w4a8_ticket_bytes(N));
+  } else if (parts == 1) {
+    a.ksplit = 1;
+  }
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (K == 0) {
     // an empty sum: bias (or zero) through the same epilogue, with no stage to walk

@@ -249,11 +249,24 @@ int mi355q_fp8_gemm(const void* A, int fmt_a, int trans_a, int64_t lda,
  * group must be a multiple of 128 that divides K; N a multiple of 32; K, lda multiples of 16; all
  * pointers 16-byte aligned; otherwise MI355Q_ERR_UNSUPPORTED, and the caller expands the weights
  * with mi355q_dequant_4bit.
+ *
+ * workspace: with at most 32 rows of A, groups of 128 and bf16 scales, K is walked in parts by
+ * several workgroups per 256 columns, which meet through `workspace`:
+ * mi355q_w4a8_gemm_workspace_bytes() of device memory, 16-byte aligned (0: the shape is not split
+ * and no workspace is read).  Its first (N / 256 rounded up) 32-bit words, rounded up to 256 bytes,
+ * are arrival counters: they have to be zero when a call starts and every call leaves them zero, so
+ * a workspace is zero-filled once, when it is allocated, and then reused.  Calls that share a
+ * workspace must not overlap (one stream, or an order between the streams).  NULL is allowed: the
+ * call then runs without the split, slower for these shapes.  Too small or misaligned:
+ * MI355Q_ERR_WORKSPACE.  The parts are added in a fixed order: a result does not depend on which
+ * workgroup finished last.
  */
+size_t mi355q_w4a8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group, int scale_dtype);
 int mi355q_w4a8_gemm(const void* A, int fmt_a, int64_t lda, const int32_t* packed, int64_t ld_packed,
                      const void* scale, int scale_dtype, const int32_t* zero_point, int is_signed,
                      int64_t group, void* C, int out_dtype, int64_t ldc, int64_t M, int64_t N, int64_t K,
-                     const float* sa_dev, float sa_host, int sa_mode, const void* bias, void* stream);
+                     const float* sa_dev, float sa_host, int sa_mode, const void* bias,
+                     void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Sum over the middle dimension of an fp8 tensor viewed as [outer, reduce, inner]

@@ -33,6 +33,10 @@ def weights(oracle, gen, K, N, group, signed, zp, scale_dtype=torch.bfloat16, po
     (100, 384, 1056, 384),    # 128-row strip, one group
     (300, 256, 288, 128),     # three row blocks
     (64, 4096, 128, 4096),    # per-channel scales, a ring walked several times
+    (16, 2048, 512, 128),     # 256-column strips, K in two parts
+    (7, 4224, 1056, 128),     # ... in four uneven parts (33 stages), the last strip 32 columns wide
+    (32, 8192, 256, 128),     # ... one strip, K in eight parts
+    (3, 256, 32800, 128),     # ... 129 strips, K in one part
 ])
 def test_exact(oracle, dev, M, K, N, group, signed, zp):
     gen = torch.Generator().manual_seed(M * 3 + K + N + signed * 7 + zp)
@@ -98,7 +102,7 @@ def test_batched_activations_scalar_scale_and_c_abi(oracle, pkg, dev):
     Ad, pkd, sd, pzd = A.to(dev), pk.to(dev), s.to(dev), pz.to(dev)
     C = torch.full((M, N + 32), -5.0, device=dev)
     st = lib.mi355q_w4a8_gemm(Ad.data_ptr(), pkg.E4M3FN, K + 64, pkd.data_ptr(), N // 8, sd.data_ptr(), pkg.BF16, pzd.data_ptr(), 0,
-                              group, C.data_ptr(), pkg.F32, N + 32, M, N, K, None, 0.5, pkg.GS_HOST, None, stream)
+                              group, C.data_ptr(), pkg.F32, N + 32, M, N, K, None, 0.5, pkg.GS_HOST, None, None, 0, stream)
     assert st == 0
     torch.cuda.synchronize()
     ref = oracle.torch_w4a8_gemm(A[:, :K].view(E4), pk, s, pz, False, torch.float32, 0.5)
@@ -107,11 +111,72 @@ def test_batched_activations_scalar_scale_and_c_abi(oracle, pkg, dev):
     assert (C[:, N:] == -5.0).all()
     # refused shapes launch nothing: a group of 64, N not a multiple of 32
     assert lib.mi355q_w4a8_gemm(Ad.data_ptr(), pkg.E4M3FN, K + 64, pkd.data_ptr(), N // 8, sd.data_ptr(), pkg.BF16, None, 0,
-                                64, C.data_ptr(), pkg.F32, N + 32, M, N, K, None, 1.0, pkg.GS_NONE, None, stream) == 2
+                                64, C.data_ptr(), pkg.F32, N + 32, M, N, K, None, 1.0, pkg.GS_NONE, None, None, 0, stream) == 2
     assert lib.mi355q_w4a8_gemm(Ad.data_ptr(), pkg.E4M3FN, K + 64, pkd.data_ptr(), N // 8, sd.data_ptr(), pkg.BF16, None, 0,
-                                128, C.data_ptr(), pkg.F32, N + 32, M, N - 8, K, None, 1.0, pkg.GS_NONE, None, stream) == 2
+                                128, C.data_ptr(), pkg.F32, N + 32, M, N - 8, K, None, 1.0, pkg.GS_NONE, None, None, 0, stream) == 2
     with pytest.raises(RuntimeError, match="multiples of 128"):
         torch.ops.mi355q.w4a8_gemm(a8.to(dev), pk.to(dev), s.repeat(2, 1).to(dev), None, False, torch.float32, None, None)
+
+
+def test_split_k_workspace_c_abi(oracle, pkg, dev):
+    """The C entry point with and without the workspace of the split over K: the same exact result, arrival
+    counters back at zero after every call, repeated calls bit-identical, sizes checked."""
+    lib = pkg.capi()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    gen = torch.Generator().manual_seed(11)
+    M, K, N, group = 24, 4096, 1312, 128
+    need = lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, pkg.BF16)
+    strips = (N + 255) // 256
+    assert need == 256 + 4 * strips * 32 * 256 * 4                        # K / 128 / 8 = 4 parts
+    assert lib.mi355q_w4a8_gemm_workspace_bytes(33, N, K, group, pkg.BF16) == 0     # more than 32 rows
+    assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, 256, pkg.BF16) == 0       # groups of two stages
+    assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, pkg.F32) == 0      # fp32 scales
+    assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, 1024, group, pkg.BF16) == 0  # too few stages to split
+    q, z, s, pk, pz = weights(oracle, gen, K, N, group, False, True, pow2=True)
+    a = torch.randint(-4, 5, (M, K), generator=gen).float()
+    w = (q - z.repeat_interleave(group, 0)).double() * s.double().repeat_interleave(group, 0)
+    expect = a.double() @ w
+    Ad, pkd, sd, pzd = a.to(E4).to(dev), pk.to(dev), s.to(dev), pz.to(dev)
+    ws = torch.zeros(need + 64, dtype=torch.uint8, device=dev)
+
+    def call(C, Adev, workspace, nbytes):
+        return lib.mi355q_w4a8_gemm(Adev.data_ptr(), pkg.E4M3FN, K, pkd.data_ptr(), N // 8, sd.data_ptr(), pkg.BF16, pzd.data_ptr(), 0,
+                                    group, C.data_ptr(), pkg.F32, N, M, N, K, None, 1.0, pkg.GS_NONE, None,
+                                    workspace.data_ptr() if workspace is not None else None, nbytes, stream)
+    for workspace, nbytes in ((ws, need), (None, 0), (ws, need + 64)):
+        C = torch.full((M, N), -5.0, device=dev)
+        assert call(C, Ad, workspace, nbytes) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.cpu().double(), expect)
+        assert int(ws[:256].view(torch.int32).abs().sum()) == 0
+    C = torch.full((M, N), -5.0, device=dev)
+    assert call(C, Ad, ws, need - 1) == 4 and call(C, Ad, ws[1:], need) == 4      # too small, misaligned
+    torch.cuda.synchronize()
+    assert (C == -5.0).all()
+    # values whose fp32 sums depend on the order: the parts are added in a fixed order
+    x8 = torch.randn(M, K, generator=gen).to(E4).to(dev)
+    outs = []
+    for _ in range(4):
+        C = torch.empty(M, N, device=dev)
+        assert call(C, x8, ws, need) == 0
+        outs.append(C)
+    torch.cuda.synchronize()
+    assert all(torch.equal(outs[0], o) for o in outs[1:])
+    ref = oracle.torch_w4a8_gemm(x8.cpu(), pk, s, pz, False, torch.float32, None)
+    rel, ok = gemm_errors(outs[0], ref)
+    assert rel < 1e-5 and ok, rel
+    # at most 16 rows (the 16x16x128 form): bf16 output whose rows start at odd element offsets, per-row scales, bias
+    M2 = 10
+    sa = torch.exp2(torch.randint(-2, 3, (M2,), generator=gen).float())
+    bias = torch.randint(-8, 9, (N,), generator=gen).float()
+    C = torch.full((M2, N + 2), -5.0, dtype=torch.bfloat16, device=dev)
+    sad, biasd = sa.to(dev), bias.bfloat16().to(dev)
+    assert lib.mi355q_w4a8_gemm(Ad.data_ptr(), pkg.E4M3FN, K, pkd.data_ptr(), N // 8, sd.data_ptr(), pkg.BF16, pzd.data_ptr(), 0,
+                                group, C.data_ptr(), pkg.BF16, N + 2, M2, N, K, sad.data_ptr(), 1.0, pkg.GS_PER_ROW, biasd.data_ptr(),
+                                ws.data_ptr(), need, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(C[:, :N].cpu(), (expect[:M2] * sa.double()[:, None] + bias.double()).float().bfloat16())
+    assert (C[:, N:] == -5.0).all()
 
 
 def test_meta_and_checks(dev):
