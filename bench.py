@@ -478,7 +478,7 @@ def bench_w4a8(oracle, dev, steps, warmup, cpu):
                  "sample": f"M=16, {rows_n} of the 28672 output columns: unpack, (q - z) * s in float64, matmul, per-row scale"}
         out.append(hbm_entry(f"w4a8_gemm_M{M}", f"w4a8_gemm M={M} K=8192 N=28672: uint4 weights (group 128, bf16 scales, packed "
                                                 "zero points) x per-token e4m3fn activations -> bf16",
-                             nbytes, ms, steps, "w4a8_wide_kernel" if M <= 32 else "w4a8_gemm_kernel", c,
+                             nbytes, ms, steps, "w4a8_wide_kernel", c,
                              extra={"tflops": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 2)}))
     return out
 

@@ -503,9 +503,9 @@ __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
 // first operand and column j of the second meet in lane j + 16 (i / 4), register i % 4.
 constexpr int kW4WideBN = 256;
 constexpr int kW4WidePacked = kBK * kW4WideBN / 2;
-constexpr int kW4WideStage = 32 * kBK + kW4WidePacked + kW4ScaleRow + kW4ZpRow;
-constexpr int kW4WideStages = (160 * 1024 - 1024) / kW4WideStage;
-constexpr int kW4WidePartialBytes = 32 * kW4WideBN * 4;
+constexpr int w4_wide_stage(int bm) { return bm * kBK + kW4WidePacked + kW4ScaleRow + kW4ZpRow; }
+constexpr int w4_wide_stages(int bm) { return (160 * 1024 - 1024) / w4_wide_stage(bm); }
+constexpr int w4_wide_partial_bytes(int bm) { return bm * kW4WideBN * 4; }  // per workgroup and part of K
 constexpr int kW4WideConsumers = 8;
 constexpr int kW4WideThreads = (kW4WideConsumers + kW4ColWaves) * 64;
 constexpr int kW4SumRing = 4;  // stages of row sums kept
@@ -516,24 +516,32 @@ __device__ __forceinline__ f32x4 w4_mfma16(const u32x4& plane, const i32x8& fa, 
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b, fa, c, 4, mfma_code<FMT_A>(), 0, e, 0, 127);
 }
 
-template <int FMT_A, bool HAS_Z, bool M16>
+// ROWS: 16 (the 16x16x128 form), 32, or 64 (row blocks of 64 along grid.y; one set of accumulators, folded into
+// the totals at the start of the next stage, for the registers of three waves per SIMD).
+template <int FMT_A, bool HAS_Z, int ROWS>
 __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
-  constexpr int BM = 32;
+  constexpr bool M16 = ROWS == 16;
+  constexpr int BM = ROWS == 64 ? 64 : 32, MT = BM / 32;
   constexpr int kConsumers = kW4WideConsumers;
-  constexpr int S = kW4WideStages, kStage = kW4WideStage;
+  constexpr int S = w4_wide_stages(BM), kStage = w4_wide_stage(BM);
   constexpr int kOffPacked = BM * kBK, kOffScale = kOffPacked + kW4WidePacked, kOffZp = kOffScale + kW4ScaleRow;
-  constexpr int NV = M16 ? 8 : 16;  // results per consumer lane
+  constexpr int NV = M16 ? 8 : 16 * MT;  // results per consumer lane
   using LA = DmaLoader<true, BM, kBK, kW4ColWaves>;
   using GA = TileGeom<true, BM, kBK>;
   constexpr int kOps = 4 + LA::kPerWave + 1;  // four 1 KiB regions of weights, A, and the scale or zero-point row
   static_assert(S >= 3 && (S - 2) * kOps <= 63, "vmcnt holds 6 bits");
   static_assert(kStage % 1024 == 0, "stages stay 1 KiB aligned");
-  static_assert(kConsumers * epilogue_stage_floats<1, 1>() * 4 <= S * kStage, "epilogue area overlays the ring");
+  static_assert(kConsumers * epilogue_stage_floats<MT, 1>() * 4 <= S * kStage, "epilogue area overlays the ring");
   __shared__ __attribute__((aligned(1024))) uint8_t lds[S * kStage];
-  __shared__ float row_sums[kW4SumRing][32];
+  __shared__ float row_sums[kW4SumRing][BM];
   __shared__ uint32_t ticket_drawn;
 
   GemmArgs g = a.g;
+  const int m_base = blockIdx.y * BM;
+  g.A += (int64_t)m_base * g.lda;
+  g.C += (int64_t)m_base * g.ldc * (g.out_bf16 ? 2 : 4);
+  if (g.sa_mode == MI355Q_GS_PER_ROW) g.sa += m_base;
+  g.M = g.M - m_base < BM ? g.M - m_base : BM;
   const int part = blockIdx.x % a.ksplit, strip = blockIdx.x / a.ksplit;
   const int n0 = strip * kW4WideBN;
   // this workgroup's part of K, whole stages (= groups)
@@ -617,14 +625,17 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         // take the MFMA, whose result only those lanes used, under the mask with it
         row_sums[slot][lane & 15] = r[0];
       } else {
-        i32x8 fa[2];
+        static_for<MT>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          i32x8 fa[2];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
-          static_for<2>([&](auto pc) { read_fragment_part<true, BM, decltype(pc)::value>(st, 0, ks, fa[ks]); });
-        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        f32x16 r = w4_mfma<FMT_A, 127>(ones, fa[0], zero);
-        r = w4_mfma<FMT_A, 127>(ones, fa[1], r);
-        row_sums[slot][lane & 31] = r[0];  // by every lane, as above
+          for (int ks = 0; ks < 2; ++ks)
+            static_for<2>([&](auto pc) { read_fragment_part<true, BM, decltype(pc)::value>(st, 32 * i, ks, fa[ks]); });
+          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          f32x16 r = w4_mfma<FMT_A, 127>(ones, fa[0], zero);
+          r = w4_mfma<FMT_A, 127>(ones, fa[1], r);
+          row_sums[slot][32 * i + (lane & 31)] = r[0];  // by every lane, as above
+        });
       }
     };
 #pragma unroll
@@ -740,7 +751,7 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         else fold(std::integral_constant<int, 1>{}, (slot - 1) & (kW4SumRing - 1));
       }
     } else {
-      // lane: row m = lane % 32 of A; columns wn + 8 q + 4 (lane / 32) + i, e = 4 q + i
+      // lane: rows m = 32 i + lane % 32 of A (i < MT); columns wn + 8 q + 4 (lane / 32) + c, e = 4 q + c
       const int tg = lane >> 4, tr = lane & 15, th = tg >> 1;
       int poff[4];
 #pragma unroll
@@ -751,22 +762,28 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
       const int zoff = kOffZp + (wn / 8) * 4;  // the four words of this wave's columns
       const int zshift = 16 * (lane >> 5);
       const int soff = kOffScale + (wn + 4 * (lane >> 5)) * 2;
-      f32x16 acc[2];
+      // two sets of partial sums, folded one stage late behind the next stage's MFMAs; with 64 rows there are
+      // registers for one set only, folded at the start of the next stage, before its MFMAs overwrite it
+      constexpr int NB = MT == 1 ? 2 : 1;
+      f32x16 acc[NB][MT];
       float sc[16];
       u32x4 zprev = {0u, 0u, 0u, 0u};
       auto fold = [&](auto bc, int sum_slot) {
-        constexpr int B = decltype(bc)::value;
-        float rs = 0.0f;
-        if constexpr (HAS_Z) rs = row_sums[sum_slot][lane & 31];
+        constexpr int B = decltype(bc)::value % NB;
+        static_for<MT>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          float rs = 0.0f;
+          if constexpr (HAS_Z) rs = row_sums[sum_slot][32 * i + (lane & 31)];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          float v = acc[B][e];
-          if constexpr (HAS_Z) v = __builtin_fmaf(-(float)((zprev[e >> 2] >> (4 * (e & 3))) & 15u), rs, v);
-          total[e] = __builtin_fmaf(v, sc[e], total[e]);
-        }
+          for (int e = 0; e < 16; ++e) {
+            float v = acc[B][i][e];
+            if constexpr (HAS_Z) v = __builtin_fmaf(-(float)((zprev[e >> 2] >> (4 * (e & 3))) & 15u), rs, v);
+            total[16 * i + e] = __builtin_fmaf(v, sc[e], total[16 * i + e]);
+          }
+        });
       };
       auto stage = [&](auto bc, auto hpc) {
-        constexpr int B = decltype(bc)::value;
+        constexpr int B = decltype(bc)::value % NB;
         constexpr bool HAVE_PREV = decltype(hpc)::value;
         __syncthreads();  // the stage is in LDS, and so are the row sums of the one before
         const uint8_t* st = lds + rd_off;
@@ -774,15 +791,24 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           wt[j] = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LDS_AS i32x2*)((LDS_AS uint8_t*)st + poff[j]));
-        i32x8 fa[2];
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
-          static_for<2>([&](auto pc) { read_fragment_part<true, BM, decltype(pc)::value>(st, 0, ks, fa[ks]); });
+        // the A fragments of both halves of the stage up front, or (64 rows) of the second half behind the MFMAs of
+        // the first, for the registers
+        i32x8 fa[2][MT];
+        auto read_a = [&](int ks) {
+          static_for<MT>([&](auto ic) {
+            static_for<2>([&](auto pc) {
+              read_fragment_part<true, BM, decltype(pc)::value>(st, 32 * decltype(ic)::value, ks, fa[MT == 1 ? ks : 0][decltype(ic)::value]);
+            });
+          });
+        };
+        read_a(0);
+        if constexpr (MT == 1) read_a(1);
         u32x2 snew[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) snew[q] = *reinterpret_cast<const u32x2*>(st + soff + q * 16);
         u32x4 znew = {0u, 0u, 0u, 0u};
         if constexpr (HAS_Z) znew = *reinterpret_cast<const u32x4*>(st + zoff);
+        if constexpr (HAVE_PREV && NB == 1) fold(std::integral_constant<int, 0>{}, (slot - 1) & (kW4SumRing - 1));
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
@@ -793,13 +819,20 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
             lo[r] = w & 0x33333333u;
             hi[r] = (w >> 2) & 0x33333333u;
           }
-          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          if (ks == 0) acc[B] = w4_mfma<FMT_A, 130>(hi, fa[ks], zero);
-          else acc[B] = w4_mfma<FMT_A, 130>(hi, fa[ks], acc[B]);
-          acc[B] = w4_mfma<FMT_A, 128>(lo, fa[ks], acc[B]);
+          const int f = MT == 1 ? ks : 0;
+          static_for<MT>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            if (ks == 0) acc[B][i] = w4_mfma<FMT_A, 130>(hi, fa[f][i], zero);
+            else acc[B][i] = w4_mfma<FMT_A, 130>(hi, fa[f][i], acc[B][i]);
+            acc[B][i] = w4_mfma<FMT_A, 128>(lo, fa[f][i], acc[B][i]);
+          });
+          if constexpr (MT == 2) {
+            if (ks == 0) read_a(1);
+          }
         }
         // the stage before this one, whose MFMAs finished long ago, behind the MFMAs just issued
-        if constexpr (HAVE_PREV) fold(std::integral_constant<int, 1 - B>{}, (slot - 1) & (kW4SumRing - 1));
+        if constexpr (HAVE_PREV && NB == 2) fold(std::integral_constant<int, 1 - B>{}, (slot - 1) & (kW4SumRing - 1));
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           sc[4 * q + 0] = __uint_as_float(snew[q][0] << 16);
@@ -833,9 +866,10 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
     // written and read with device-scope atomic accesses, which go past the caches of this XCD to where the other
     // XCDs see them: no cache has to be written back or invalidated as a whole, which a fence would do (and
     // which, done by every workgroup while the others still stream, costs more than the kernel).
-    const int strips = gridDim.x / a.ksplit;
-    constexpr int kWords = 8 * 64;  // per consumer wave (half of them used with M16)
-    unsigned long long* mine = reinterpret_cast<unsigned long long*>(a.partials) + ((int64_t)(part * strips + strip) * kConsumers + wq) * kWords + lane;
+    const int strips = gridDim.x / a.ksplit * gridDim.y;         // strips of all row blocks
+    const int strip_rb = blockIdx.y * (gridDim.x / a.ksplit) + strip;
+    constexpr int kWords = 8 * MT * 64;  // per consumer wave (half of them used with 16 rows)
+    unsigned long long* mine = reinterpret_cast<unsigned long long*>(a.partials) + ((int64_t)(part * strips + strip_rb) * kConsumers + wq) * kWords + lane;
     if (!producer) {
 #pragma unroll
       for (int h = 0; h < NV / 2; ++h) {
@@ -846,8 +880,8 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-      const uint32_t t = __hip_atomic_fetch_add(a.tickets + strip, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (t == (uint32_t)a.ksplit - 1) __hip_atomic_store(a.tickets + strip, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+      const uint32_t t = __hip_atomic_fetch_add(a.tickets + strip_rb, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (t == (uint32_t)a.ksplit - 1) __hip_atomic_store(a.tickets + strip_rb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
       ticket_drawn = t;
     }
     __syncthreads();
@@ -855,7 +889,7 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
     if (!producer) {
 #pragma unroll
       for (int e = 0; e < NV; ++e) total[e] = 0.0f;
-      const unsigned long long* from = reinterpret_cast<const unsigned long long*>(a.partials) + ((int64_t)strip * kConsumers + wq) * kWords + lane;
+      const unsigned long long* from = reinterpret_cast<const unsigned long long*>(a.partials) + ((int64_t)strip_rb * kConsumers + wq) * kWords + lane;
       for (int p = 0; p < a.ksplit; ++p) {
         unsigned long long v[NV / 2];
 #pragma unroll
@@ -906,22 +940,40 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
       }
     }
   } else {
-    f32x16 out[1][1];
+    f32x16 out[MT][1];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) out[0][0][e] = total[e];
-    float* stage_area = reinterpret_cast<float*>(lds) + wq * epilogue_stage_floats<1, 1>();
-    epilogue<1, 1>(g, 0, out, 0, n0 + wq * 32, stage_area);
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) out[i][0][e] = total[16 * i + e];
+    float* stage_area = reinterpret_cast<float*>(lds) + wq * epilogue_stage_floats<MT, 1>();
+    epilogue<MT, 1>(g, 0, out, 0, n0 + wq * 32, stage_area);
   }
 }
 
-// How the wide kernel would split a problem: parts of K per strip (0: the wide kernel does not apply).
-inline int w4a8_wide_parts(int64_t M, int64_t N, int64_t K, int64_t group, int scale_f32) {
-  if (M > 32 || group != kBK || scale_f32 || K <= 0) return 0;
-  const int64_t strips = (N + kW4WideBN - 1) / kW4WideBN, kt = (K + kBK - 1) / kBK;
-  int64_t parts = 256 / strips;
+// How the wide kernel takes a problem: rows per workgroup (16 selects the 16x16x128 form of the 32-row tile), row
+// blocks, strips, and the parts K is walked in (0: the wide kernel does not apply).
+struct W4WidePlan {
+  int rows, row_blocks, strips, parts;
+  int tile_rows() const { return rows == 64 ? 64 : 32; }
+  size_t ticket_bytes() const { return ((size_t)strips * row_blocks * 4 + 255) / 256 * 256; }
+  size_t workspace_bytes() const {
+    return parts < 2 ? 0 : ticket_bytes() + (size_t)parts * strips * row_blocks * w4_wide_partial_bytes(tile_rows());
+  }
+};
+inline W4WidePlan w4a8_wide_plan(int64_t M, int64_t N, int64_t K, int64_t group, int scale_f32) {
+  W4WidePlan p{0, 0, 0, 0};
+  if (group != kBK || scale_f32 || K <= 0 || M <= 0 || N <= 0) return p;
+  p.rows = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
+  p.row_blocks = (int)((M + p.tile_rows() - 1) / p.tile_rows());
+  p.strips = (int)((N + kW4WideBN - 1) / kW4WideBN);
+  const int64_t kt = (K + kBK - 1) / kBK, groups = (int64_t)p.strips * p.row_blocks;
+  int64_t parts = 256 / groups;
   if (parts > kt / 8) parts = kt / 8;
-  if (parts < 2) return strips >= 128 ? 1 : 0;
-  return (int)parts;
+  // too few workgroups for the chip even so: the 128-column strips have twice as many
+  if (parts < 2) parts = groups >= 100 ? 1 : 0;
+  if (p.row_blocks > 65535) parts = 0;
+  p.parts = (int)parts;
+  return p;
 }
 
 template <int BM, int FMT_A>
@@ -936,14 +988,20 @@ void w4a8_launch(const W4Args& a, hipStream_t st) {
 template <int FMT_A>
 void w4a8_launch_by_m(const W4Args& a, hipStream_t st) {
   if (a.ksplit > 0) {
-    const unsigned grid = (unsigned)((a.g.N + kW4WideBN - 1) / kW4WideBN) * (unsigned)a.ksplit;
     const bool z = a.zp != nullptr || a.is_signed;
+    const unsigned strips = (unsigned)((a.g.N + kW4WideBN - 1) / kW4WideBN);
     if (a.g.M <= 16) {
-      if (z) w4a8_wide_kernel<FMT_A, true, true><<<grid, kW4WideThreads, 0, st>>>(a);
-      else w4a8_wide_kernel<FMT_A, false, true><<<grid, kW4WideThreads, 0, st>>>(a);
+      const dim3 grid(strips * (unsigned)a.ksplit);
+      if (z) w4a8_wide_kernel<FMT_A, true, 16><<<grid, kW4WideThreads, 0, st>>>(a);
+      else w4a8_wide_kernel<FMT_A, false, 16><<<grid, kW4WideThreads, 0, st>>>(a);
+    } else if (a.g.M <= 32) {
+      const dim3 grid(strips * (unsigned)a.ksplit);
+      if (z) w4a8_wide_kernel<FMT_A, true, 32><<<grid, kW4WideThreads, 0, st>>>(a);
+      else w4a8_wide_kernel<FMT_A, false, 32><<<grid, kW4WideThreads, 0, st>>>(a);
     } else {
-      if (z) w4a8_wide_kernel<FMT_A, true, false><<<grid, kW4WideThreads, 0, st>>>(a);
-      else w4a8_wide_kernel<FMT_A, false, false><<<grid, kW4WideThreads, 0, st>>>(a);
+      const dim3 grid(strips * (unsigned)a.ksplit, (unsigned)((a.g.M + 63) / 64));
+      if (z) w4a8_wide_kernel<FMT_A, true, 64><<<grid, kW4WideThreads, 0, st>>>(a);
+      else w4a8_wide_kernel<FMT_A, false, 64><<<grid, kW4WideThreads, 0, st>>>(a);
     }
   } else if (a.g.M <= 32) {
     w4a8_launch<32, FMT_A>(a, st);
@@ -952,22 +1010,12 @@ void w4a8_launch_by_m(const W4Args& a, hipStream_t st) {
   }
 }
 
-constexpr size_t kW4TicketAlign = 256;
-inline size_t w4a8_ticket_bytes(int64_t N) {
-  const size_t strips = (size_t)((N + kW4WideBN - 1) / kW4WideBN);
-  return (strips * 4 + kW4TicketAlign - 1) / kW4TicketAlign * kW4TicketAlign;
-}
-
 }  // namespace mi355q
 
 using namespace mi355q;
 
 extern "C" size_t mi355q_w4a8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group, int scale_dtype) {
-  if (M <= 0 || N <= 0 || K <= 0 || group <= 0) return 0;
-  const int parts = w4a8_wide_parts(M, N, K, group, scale_dtype == MI355Q_F32);
-  if (parts < 2) return 0;
-  const size_t strips = (size_t)((N + kW4WideBN - 1) / kW4WideBN);
-  return w4a8_ticket_bytes(N) + (size_t)parts * strips * kW4WidePartialBytes;
+  return w4a8_wide_plan(M, N, K, group, scale_dtype == MI355Q_F32).workspace_bytes();
 }
 
 extern "C" int mi355q_w4a8_gemm(const void* A, int fmt_a, int64_t lda, const int32_t* packed, int64_t ld_packed,
@@ -1015,13 +1063,13 @@ extern "C" int mi355q_w4a8_gemm(const void* A, int fmt_a, int64_t lda, const int
   a.is_signed = is_signed != 0;
   a.stages_per_group = (int)(group / kBK);
   // the wide kernel where it applies: K in parts if the caller brought the room for the partial sums
-  const int parts = w4a8_wide_parts(M, N, K, group, a.scale_f32);
-  if (parts >= 2 && workspace != nullptr) {
-    if (!al16(workspace) || workspace_bytes < mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, scale_dtype)) return MI355Q_ERR_WORKSPACE;
-    a.ksplit = parts;
+  const W4WidePlan plan = w4a8_wide_plan(M, N, K, group, a.scale_f32);
+  if (plan.parts >= 2 && workspace != nullptr) {
+    if (!al16(workspace) || workspace_bytes < plan.workspace_bytes()) return MI355Q_ERR_WORKSPACE;
+    a.ksplit = plan.parts;
     a.tickets = static_cast<uint32_t*>(workspace);
-    a.partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + w4a8_ticket_bytes(N));
-  } else if (parts == 1) {
+    a.partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + plan.ticket_bytes());
+  } else if (plan.parts == 1) {
     a.ksplit = 1;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);

@@ -37,6 +37,9 @@ def weights(oracle, gen, K, N, group, signed, zp, scale_dtype=torch.bfloat16, po
     (7, 4224, 1056, 128),     # ... in four uneven parts (33 stages), the last strip 32 columns wide
     (32, 8192, 256, 128),     # ... one strip, K in eight parts
     (3, 256, 32800, 128),     # ... 129 strips, K in one part
+    (64, 4096, 1056, 128),    # ... 64-row tiles, K in four parts
+    (100, 2048, 512, 128),    # ... two row blocks (the second ragged), K in two parts
+    (130, 256, 8992, 128),    # ... three row blocks, 36 strips, K in one part
 ])
 def test_exact(oracle, dev, M, K, N, group, signed, zp):
     gen = torch.Generator().manual_seed(M * 3 + K + N + signed * 7 + zp)
@@ -128,7 +131,8 @@ def test_split_k_workspace_c_abi(oracle, pkg, dev):
     need = lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, pkg.BF16)
     strips = (N + 255) // 256
     assert need == 256 + 4 * strips * 32 * 256 * 4                        # K / 128 / 8 = 4 parts
-    assert lib.mi355q_w4a8_gemm_workspace_bytes(33, N, K, group, pkg.BF16) == 0     # more than 32 rows
+    assert lib.mi355q_w4a8_gemm_workspace_bytes(33, N, K, group, pkg.BF16) == 256 + 4 * strips * 64 * 256 * 4    # 64-row tiles
+    assert lib.mi355q_w4a8_gemm_workspace_bytes(130, N, K, group, pkg.BF16) == 256 + 4 * strips * 3 * 64 * 256 * 4  # three row blocks
     assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, 256, pkg.BF16) == 0       # groups of two stages
     assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, pkg.F32) == 0      # fp32 scales
     assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, 1024, group, pkg.BF16) == 0  # too few stages to split
