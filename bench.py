@@ -54,9 +54,10 @@ MEASURED_TRAFFIC = {
     "fp8_gemm_v2_decode_M16": 236.92e6,
     "fp8_gemm_v2_decode_M64": 243.02e6,
     "fp8_gemm_v2_decode_M256": 266.45e6,
-    "w4a8_gemm_M16": 124.15e6,
-    "w4a8_gemm_M64": 130.47e6,
-    "w4a8_gemm_M256": 481.35e6,     # four row blocks of 64 stream the weights four times
+    "w4a8_gemm_M16": 130.86e6,      # the partial sums of the two K parts on top of the 124 MB of operands
+    "w4a8_gemm_M32": 140.24e6,
+    "w4a8_gemm_M64": 159.36e6,
+    "w4a8_gemm_M256": 284.69e6,     # four row blocks of 64 stream the weights; the caches catch half of it
     "fp8_sdpa_B1_L8192": 130.55e6,
     "fp8_sdpa_B4_L4096": 235.41e6,
     "fp8_sdpa_decode_B64_S4096": 537.35e6,
