@@ -82,7 +82,7 @@ __global__ __launch_bounds__(kSkThreads) void fp8_gemm_skinny_kernel(GemmArgs g)
       at = stage;
     }
     static_for<LA::kPerWave>([&](auto ic) { la.template issue_one<decltype(ic)::value, A_KMAJOR>(lds + off, stage * kBK, g.K); });
-    static_for<LB::kPerWave>([&](auto ic) { lb.template issue_one<decltype(ic)::value, B_KMAJOR>(lds + off + BM * kBK, stage * kBK, g.K); });
+    static_for<LB::kPerWave>([&](auto ic) { lb.template issue_one<decltype(ic)::value, B_KMAJOR, true>(lds + off + BM * kBK, stage * kBK, g.K); });  // B is read once
     la.advance();
     lb.advance();
     ++at;

@@ -256,7 +256,9 @@ struct DmaLoader {
 
   // Issues load I of this wave's share of the stage the descriptor points at,
   // which starts at k0.
-  template <int I, bool CLAMP_ROWS = false>
+  // NT: the nontemporal hint, for an operand that is read once (the weights of a decode-shaped call): a strip
+  // read of a 235 MB matrix runs 8 % faster with it (41 against 45 us), through registers or into LDS alike.
+  template <int I, bool CLAMP_ROWS = false, bool NT = false>
   __device__ __forceinline__ void issue_one(uint8_t* lds_tile, int k0, int K) const {
     const uint32_t lds_base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)lds_tile;
     {
@@ -269,10 +271,17 @@ struct DmaLoader {
       // Written as asm so that the compiler, which would otherwise make every later
       // LDS read wait for all outstanding global->LDS loads, leaves the waiting to
       // the explicit vmcnt drain before each barrier.
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                   :
-                   : "s"(dst), "v"(vo), "s"(rsrc)
-                   : "memory", "m0");
+      if constexpr (NT) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen nt lds"
+                     :
+                     : "s"(dst), "v"(vo), "s"(rsrc)
+                     : "memory", "m0");
+      } else {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                     :
+                     : "s"(dst), "v"(vo), "s"(rsrc)
+                     : "memory", "m0");
+      }
     }
   }
 

@@ -110,11 +110,20 @@ __device__ __forceinline__ int k_swizzle(int row) {
 // One 16-byte piece per lane, global -> LDS (lane l lands at lds_dst + 16 l; a lane whose offset lies
 // outside the descriptor writes zeros).  The s_nop covers descriptor words that reached their scalar
 // registers through a vector instruction (five wait states before a memory instruction may read them).
+// STREAM adds the nontemporal hint: for keys and values that the launch reads once (the decoding kernel).
+template <bool STREAM = false>
 __device__ __forceinline__ void sdpa_dma16(const i32x4& rsrc, int voff, uint32_t lds_dst) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-               :
-               : "s"(lds_dst), "v"(voff), "s"(rsrc)
-               : "memory", "m0");
+  if constexpr (STREAM) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, 0 offen nt lds"
+                 :
+                 : "s"(lds_dst), "v"(voff), "s"(rsrc)
+                 : "memory", "m0");
+  } else {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_dst), "v"(voff), "s"(rsrc)
+                 : "memory", "m0");
+  }
 }
 
 // A buffer descriptor that walks down the rows of k or v one block at a time.
@@ -689,10 +698,10 @@ __global__ __launch_bounds__(kSdpaThreads) void fp8_sdpa_decode_kernel(const Sdp
     const uint32_t kdst = (uint32_t)(uintptr_t)(SDPA_LDS_AS uint8_t*)(mine + buf * kStage);
     const i32x4 rk = wk.rsrc();
 #pragma unroll
-    for (int n = 0; n < KREG; ++n) sdpa_dma16(rk, kvoff[n], kdst + n * 1024);
+    for (int n = 0; n < KREG; ++n) sdpa_dma16<true>(rk, kvoff[n], kdst + n * 1024);
     const i32x4 rv = wv.rsrc();
 #pragma unroll
-    for (int n = 0; n < VREG; ++n) sdpa_dma16(rv, vvoff[n], kdst + KBYTES + n * 1024);
+    for (int n = 0; n < VREG; ++n) sdpa_dma16<true>(rv, vvoff[n], kdst + KBYTES + n * 1024);
     wk.base += (uint64_t)4 * kSdpaBN * a.ldk;
     wk.left -= (int64_t)4 * kSdpaBN * a.ldk;
     wv.base += (uint64_t)4 * kSdpaBN * a.ldv;
