@@ -121,6 +121,34 @@ def test_batched_activations_scalar_scale_and_c_abi(oracle, pkg, dev):
         torch.ops.mi355q.w4a8_gemm(a8.to(dev), pk.to(dev), s.repeat(2, 1).to(dev), None, False, torch.float32, None, None)
 
 
+@pytest.mark.parametrize("seed", range(32))
+def test_random_shapes_exact(oracle, dev, seed):
+    """Shapes drawn at random across the kernels' regimes (rows up to 300, K up to 64 stages, strips of every width,
+    groups of one or more stages, both scale types), small-integer values: every output exact."""
+    gen = torch.Generator().manual_seed(1000 + seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=gen))
+    M = [r(1, 16), r(17, 32), r(33, 64), r(65, 300)][seed % 4]
+    stages = r(1, 64)
+    per_group = [1, 1, 1, 2, stages][r(0, 4)]
+    stages -= stages % per_group
+    stages = max(stages, per_group)
+    K, group = 128 * stages, 128 * per_group
+    N = 32 * r(1, 80)
+    signed, zp = bool(r(0, 1)), bool(r(0, 1))
+    scale_dtype = torch.float32 if r(0, 5) == 0 else torch.bfloat16
+    q, z, s, pk, pz = weights(oracle, gen, K, N, group, signed, zp, scale_dtype, pow2=True)
+    a = torch.randint(-3, 4, (M, K), generator=gen).float()
+    sa = torch.exp2(torch.randint(-2, 3, (M, 1), generator=gen).float())
+    bias = torch.randint(-8, 9, (N,), generator=gen).float()
+    w = (q - (z.repeat_interleave(group, 0) if zp else 0)).double() * s.double().repeat_interleave(group, 0)
+    expect = (a.double() @ w) * sa.double() + bias.double()
+    assert expect.abs().max() < 2 ** 24
+    fmt = E5 if r(0, 3) == 0 else E4
+    out = torch.ops.mi355q.w4a8_gemm(a.to(fmt).to(dev), pk.to(dev), s.to(dev), pz.to(dev) if zp else None, signed,
+                                     torch.float32, sa.to(dev), bias.to(dev))
+    assert torch.equal(out.cpu().double(), expect), (M, K, N, group, signed, zp, scale_dtype, fmt)
+
+
 def test_split_k_workspace_c_abi(oracle, pkg, dev):
     """The C entry point with and without the workspace of the split over K: the same exact result, arrival
     counters back at zero after every call, repeated calls bit-identical, sizes checked."""
