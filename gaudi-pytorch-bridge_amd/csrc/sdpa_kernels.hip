@@ -293,7 +293,12 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
 
 // DKC: 64-byte steps of the q.k depth (head_dim_qk <= 64 DKC); DVT: 32-column tiles of v
 // (head_dim_v <= 32 DVT).
-template <int DKC, int DVT, int FMT>
+// DMA: K and V blocks go from global memory straight into LDS (aligned tensors), a ring of kStages blocks;
+// otherwise through registers, two buffers.  A compile-time choice: with both routes in one loop the compiler
+// has to assume the register route's loads outstanding wherever their registers are reused, and the wait it
+// puts there (vmcnt(0), in front of the first MFMA of every block) also waits for the blocks just requested
+// by the direct route.
+template <int DKC, int DVT, int FMT, bool DMA>
 __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd_kernel(const SdpaArgs a) {
   constexpr int KROW = DKC * 64;
   constexpr int kVRow = DVT <= 4 ? 128 : 256;  // bytes of an LDS row of V
@@ -357,6 +362,13 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
     const u32x4 hi = load_chunk(rp, q_ok, 64 * c + 32 * h + 16, a.Dk, a.vec_q);
     qf[c] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
   }
+  // The fragments are first used by an MFMA inside the block loop, and the wait for their loads would be placed
+  // there: a vmcnt(0) in every pass, which also waits for the K / V blocks just requested.  Naming them here
+  // puts that wait in front of the loop.
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass, which compiles this body for the launch stub, knows no "v"
+#pragma unroll
+  for (int c = 0; c < DKC; ++c) asm volatile("" : : "v"(qf[c]));
+#endif
 
   int nblk = (a.S + kSdpaBN - 1) / kSdpaBN;
   if (a.causal) {
@@ -403,7 +415,7 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
   static_assert(KBYTES % 4096 == 0 && VBYTES % 4096 == 0, "tiles split into 1 KiB regions over four waves");
   int kvoff[KREG], vvoff[VREG];
   SdpaWalker wk{reinterpret_cast<uint64_t>(kp), 0}, wv{reinterpret_cast<uint64_t>(vp), 0};
-  if (a.dma) {
+  if constexpr (DMA) {
     wk.left = (int64_t)(a.S - 1) * a.ldk + a.Dk;
     wv.left = (int64_t)(a.S - 1) * a.ldv + a.Dv;
 #pragma unroll
@@ -444,7 +456,7 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
 
   const uint8_t* mrow = a.mask + (m_off + (int64_t)qrow * a.ldm) * (a.mask_kind == kMaskBool ? 1 : a.mask_kind == kMaskBf16 ? 2 : 4);
   if (nblk > 0) {
-    if (a.dma) {
+    if constexpr (DMA) {
       for (int b = 0; b < kStages - 1 && b < nblk; ++b) issue_block(b);
       if (nblk >= kStages - 1 && (kStages - 1) * kSdpaBN <= a.S) {
         constexpr int cnt = (kStages - 2) * (KREG + VREG);
@@ -461,11 +473,12 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
 
   for (int blk = 0; blk < nblk; ++blk) {
     const int kv0 = blk * kSdpaBN;
-    if (blk + 1 < nblk) {
-      if (!a.dma) fetch(blk + 1);
+    if constexpr (DMA) {
+      if (blk + kStages - 1 < nblk) issue_block((blk + kStages - 1) % kStages);
+    } else {
+      if (blk + 1 < nblk) fetch(blk + 1);
     }
-    if (a.dma && blk + kStages - 1 < nblk) issue_block((blk + kStages - 1) % kStages);
-    const uint8_t* kb = lds + (a.dma ? blk % kStages : blk & 1) * (KBYTES + VBYTES);
+    const uint8_t* kb = lds + (DMA ? blk % kStages : blk & 1) * (KBYTES + VBYTES);
     const uint8_t* vb = kb + KBYTES;
 
     // a wave whose 32 rows all lie above this block's first key has nothing to add
@@ -475,7 +488,7 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
       sdpa_block<DKC, DVT, FMT>(a, kb, vb, kv0, edge, qrow, q_ok, mrow, qf, sc2, lqs, clamp_p, o, m_run, l_run);
     }
 
-    if (a.dma) {
+    if constexpr (DMA) {
       // The next block has landed once only the loads of the blocks after it are outstanding.  Loads
       // retire in issue order as long as every one of them goes to memory; one whose lanes all lie
       // beyond kv_len completes at once, so the count is only trusted while every block in flight is
@@ -486,8 +499,8 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
       } else {
         __builtin_amdgcn_s_waitcnt(0x0f70);
       }
-    } else if (blk + 1 < nblk) {
-      commit((blk + 1) & 1);
+    } else {
+      if (blk + 1 < nblk) commit((blk + 1) & 1);
     }
     __syncthreads();
   }
@@ -671,6 +684,12 @@ __global__ __launch_bounds__(kSdpaThreads) void fp8_sdpa_decode_kernel(const Sdp
     const u32x4 hi = load_chunk(qrowp, q_ok, 64 * c + 32 * h + 16, a.Dk, a.vec_q);
     qf[c] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
   }
+  // the wait for these loads belongs in front of the block loop, not at their first use inside it (see the
+  // kernel above)
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+  for (int c = 0; c < DKC; ++c) asm volatile("" : : "v"(qf[c]));
+#endif
 
   // this workgroup's blocks of keys, and of those this wave's: first, first + 4, ...
   const int nblk_all = (a.S + kSdpaBN - 1) / kSdpaBN;
@@ -721,9 +740,16 @@ __global__ __launch_bounds__(kSdpaThreads) void fp8_sdpa_decode_kernel(const Sdp
     const int kv0 = blk * kSdpaBN;
     const bool more = blk + 4 < b1;
     if (more) issue_block(buf ^ 1);
-    // This block has landed once only the next one's loads are outstanding; a block that reaches beyond
-    // kv_len may hold loads that complete at once, out of order, so the count is used between whole blocks only.
-    __builtin_amdgcn_s_waitcnt(0x0f70);
+    // This block has landed once only the next one's loads are outstanding.  A block that reaches beyond
+    // kv_len may hold loads that complete at once, ahead of older ones, so the count is only trusted when the
+    // block just requested is whole; otherwise everything is waited for.
+    if (more && (blk + 5) * kSdpaBN <= a.S) {
+      constexpr int cnt = KREG + VREG;
+      static_assert(cnt <= 63, "vmcnt holds 6 bits");
+      __builtin_amdgcn_s_waitcnt((cnt & 15) | ((cnt >> 4) << 14) | 0x0f70);
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+    }
     const uint8_t* kb = mine + buf * kStage;
     const bool edge = a.causal || kv0 + kSdpaBN > a.S || a.mask_kind != kMaskNone;
     sdpa_block<DKC, DVT, FMT>(a, kb, kb + KBYTES, kv0, edge, qpos, q_ok, mrow, qf, sc2, lqs, clamp_p, o, m_run, l_run);
@@ -864,10 +890,14 @@ static SdpaDecodePlan sdpa_decode_plan(const mi355q_sdpa_desc* d, int cus) {
 
 template <int DKC, int DVT>
 static int sdpa_launch(const SdpaArgs& a, int fmt, int64_t blocks, hipStream_t st) {
-  if (fmt == MI355Q_E5M2)
-    hipLaunchKernelGGL((fp8_sdpa_fwd_kernel<DKC, DVT, MI355Q_E5M2>), dim3((unsigned)blocks), dim3(kSdpaThreads), 0, st, a);
-  else
-    hipLaunchKernelGGL((fp8_sdpa_fwd_kernel<DKC, DVT, MI355Q_E4M3FN>), dim3((unsigned)blocks), dim3(kSdpaThreads), 0, st, a);
+  const dim3 grid((unsigned)blocks), block(kSdpaThreads);
+  if (fmt == MI355Q_E5M2) {
+    if (a.dma) hipLaunchKernelGGL((fp8_sdpa_fwd_kernel<DKC, DVT, MI355Q_E5M2, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((fp8_sdpa_fwd_kernel<DKC, DVT, MI355Q_E5M2, false>), grid, block, 0, st, a);
+  } else {
+    if (a.dma) hipLaunchKernelGGL((fp8_sdpa_fwd_kernel<DKC, DVT, MI355Q_E4M3FN, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((fp8_sdpa_fwd_kernel<DKC, DVT, MI355Q_E4M3FN, false>), grid, block, 0, st, a);
+  }
   return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
 }
 
