@@ -229,7 +229,7 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
   const float shift = lqs - m_use;  // p * q_scale_s = 2^(x - m + log2 q_scale_s)
 
   float psum = 0.0f;
-  i32x8 pf;
+  i32x8 pf = {0, 0, 0, 0, 0, 0, 0, 0};
   // p = 2^(x + shift) for this lane's 32 scores, their sum, and the fp8 codes packed in register
   // order.  RAW: s still holds the unscaled products (x = s * sc2); CLAMP: q_scale_s exceeds the
   // format's range.  Compile-time variants, so that the common one is a multiply-add, an exp2 and an
@@ -248,12 +248,14 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
           psum += p[i];
           if (CLAMP) p[i] = __builtin_elementwise_minimum(p[i], kMax8);
         }
-        int w;
+        // both halves of the word are written: what it held before does not matter, and taking the register's
+        // previous contents as the "old" value saves the move that a zero would cost
+        int w = pf[4 * t + j];
         if constexpr (FMT == MI355Q_E5M2) {
-          w = __builtin_amdgcn_cvt_pk_bf8_f32(p[0], p[1], 0, false);
+          w = __builtin_amdgcn_cvt_pk_bf8_f32(p[0], p[1], w, false);
           w = __builtin_amdgcn_cvt_pk_bf8_f32(p[2], p[3], w, true);
         } else {
-          w = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
+          w = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], w, false);
           w = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], w, true);
         }
         pf[4 * t + j] = w;
