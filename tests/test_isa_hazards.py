@@ -80,12 +80,35 @@ def test_scanner_flags_m0_used_at_once():
 
 @pytest.mark.timeout(900)
 def test_gemm_kernels_have_no_uncovered_hazard():
-    sources = ["gemm_inst_kk.hip", "gemm_inst_km.hip", "gemm_inst_mk.hip", "gemm_inst_mm.hip", "w4_gemm.hip"]
-    with ThreadPoolExecutor(max_workers=5) as ex:
+    sources = ["gemm_inst_kk.hip", "gemm_inst_km.hip", "gemm_inst_mk.hip", "gemm_inst_mm.hip", "w4_gemm.hip", "sdpa_kernels.hip"]
+    with ThreadPoolExecutor(max_workers=6) as ex:
         texts = list(ex.map(isa_check.compile_to_isa, sources))
     for src, text in zip(sources, texts):
         assert text.count("#ASMSTART") > 100, f"{src}: the asm statements are gone?"
         assert isa_check.scan(text) == [], src
+
+
+@pytest.mark.timeout(600)
+def test_attention_block_loop_does_not_wait_for_its_own_prefetch():
+    """The compiler places the wait for a load at its first use.  The query fragments of the attention kernels
+    are loaded once and first used by the first MFMA of the block loop: left alone, that is a vmcnt(0) in every
+    pass, which also waits for the K / V blocks the pass has just requested (global -> LDS loads share the
+    counter).  The kernels name the fragments in front of the loop; here the basic block that ends in the first
+    MFMA must hold no wait on vmcnt."""
+    import re
+    text = isa_check.compile_to_isa("sdpa_kernels.hip")
+    seen = 0
+    for name, body in re.findall(r"^(_ZN6mi355q\w+):.*?\n(.*?)s_endpgm", text, flags=re.S | re.M):
+        if "fp8_sdpa_fwd_kernel" not in name and "fp8_sdpa_decode_kernel" not in name:
+            continue
+        lines = body.split("\n")
+        first = next(k for k, line in enumerate(lines) if "v_mfma" in line)
+        start = first
+        while start > 0 and not lines[start].startswith(".LBB"):
+            start -= 1
+        assert not any("vmcnt" in line for line in lines[start:first]), name
+        seen += 1
+    assert seen >= 16
 
 
 def test_memory_order_reads_a_kernel():
