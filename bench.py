@@ -273,6 +273,18 @@ def bench_ceilings(pkg, dev, steps, warmup):
         out.append(hbm_entry(f"ceiling_copy_{mib}MiB", f"copy of {mib // 2} MiB ({mib} MiB read + written), the library's 16-byte copy kernel",
                              nbytes, ms, k, "copy_vec16"))
         del bufs, dst
+    # the weights of the decode GEMMs ([8192, 28672] fp8 bytes) read in strips, as those kernels read them
+    pitch, rows = 28672, 8192
+    sets = n_sets(pitch * rows)
+    bufs = [torch.randint(0, 255, (rows * pitch,), dtype=torch.uint8, device=dev) for _ in range(sets)]
+    for strip, parts, nt in ((64, 1, 1), (128, 1, 0), (128, 1, 1), (256, 2, 1)):
+        k = max(steps, 20)
+        ms = time_gpu(lambda i: lib.mi355q_probe_strip_read(bufs[i % sets].data_ptr(), pitch, rows, strip, parts, nt, sink.data_ptr(), st), k, warmup)
+        out.append(hbm_entry(f"ceiling_strip_read_{strip}B" + ("_nt" if nt else "") + (f"_K{parts}" if parts > 1 else ""),
+                             f"[{rows}, {pitch}] bytes read in strips of {strip} bytes per row, {pitch // strip * parts} workgroups"
+                             + (f", the rows in {parts} ranges" if parts > 1 else "") + (", nontemporal loads" if nt else ""),
+                             pitch * rows, ms, k, "probe_strip_read_kernel"))
+    del bufs
     return out
 
 

@@ -50,6 +50,31 @@ __global__ __launch_bounds__(1024) void probe_read_kernel(const u32x4* __restric
   if (acc == 0x9e3779b9u) sink[0] = acc;
 }
 
+// A row-major byte matrix read the way the decode-shaped GEMMs read their weights: a workgroup takes a strip of
+// R bytes of every row (of its part of the rows), 16 bytes per lane, 8 loads in flight per lane, nothing else.
+// NT: with the nontemporal hint.
+template <int R, bool NT>
+__global__ __launch_bounds__(256) void probe_strip_read_kernel(const uint8_t* base, int64_t pitch, int rows, int parts, uint32_t* sink) {
+  const int strip = blockIdx.x / parts, part = blockIdx.x % parts;
+  const int r0 = (int)((int64_t)rows * part / parts), r1 = (int)((int64_t)rows * (part + 1) / parts);
+  constexpr int kLanesPerRow = R / 16, kRowsPerLoad = 256 / kLanesPerRow, kLoads = 8;
+  const int lr = threadIdx.x / kLanesPerRow, lc = threadIdx.x % kLanesPerRow;
+  const uint8_t* p = base + (int64_t)strip * R + lc * 16 + (int64_t)(r0 + lr) * pitch;
+  u32x4 acc = {0u, 0u, 0u, 0u};
+  for (int r = r0; r + kLoads * kRowsPerLoad <= r1; r += kLoads * kRowsPerLoad) {
+    u32x4 v[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      const u32x4* q = reinterpret_cast<const u32x4*>(p + (int64_t)i * kRowsPerLoad * pitch);
+      v[i] = NT ? __builtin_nontemporal_load(q) : *q;
+    }
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) acc ^= v[i];
+    p += (int64_t)kLoads * kRowsPerLoad * pitch;
+  }
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u) sink[0] = acc[0];
+}
+
 }  // namespace mi355q
 
 using namespace mi355q;
@@ -69,6 +94,30 @@ int mi355q_probe_read(const void* x, int64_t bytes, int workgroups, void* sink, 
     return MI355Q_ERR_INVALID_ARGUMENT;
   hipLaunchKernelGGL(probe_read_kernel, dim3((unsigned)workgroups), dim3(1024), 0, static_cast<hipStream_t>(stream),
                      static_cast<const u32x4*>(x), bytes / 16, static_cast<uint32_t*>(sink));
+  return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
+}
+
+int mi355q_probe_strip_read(const void* x, int64_t pitch, int64_t rows, int strip_bytes, int parts, int nontemporal, void* sink,
+                            void* stream) {
+  if (x == nullptr || sink == nullptr || pitch <= 0 || rows <= 0 || parts <= 0 || rows > 0x7fffffffLL ||
+      (reinterpret_cast<uintptr_t>(x) & 15u) != 0 || (strip_bytes != 64 && strip_bytes != 128 && strip_bytes != 256) ||
+      pitch % strip_bytes != 0 || pitch / strip_bytes * parts > 0x7fffffffLL)
+    return MI355Q_ERR_INVALID_ARGUMENT;
+  const dim3 grid((unsigned)(pitch / strip_bytes * parts)), block(256);
+  const uint8_t* p = static_cast<const uint8_t*>(x);
+  uint32_t* s = static_cast<uint32_t*>(sink);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int r = (int)rows;
+  if (strip_bytes == 64) {
+    if (nontemporal) hipLaunchKernelGGL((probe_strip_read_kernel<64, true>), grid, block, 0, st, p, pitch, r, parts, s);
+    else hipLaunchKernelGGL((probe_strip_read_kernel<64, false>), grid, block, 0, st, p, pitch, r, parts, s);
+  } else if (strip_bytes == 128) {
+    if (nontemporal) hipLaunchKernelGGL((probe_strip_read_kernel<128, true>), grid, block, 0, st, p, pitch, r, parts, s);
+    else hipLaunchKernelGGL((probe_strip_read_kernel<128, false>), grid, block, 0, st, p, pitch, r, parts, s);
+  } else {
+    if (nontemporal) hipLaunchKernelGGL((probe_strip_read_kernel<256, true>), grid, block, 0, st, p, pitch, r, parts, s);
+    else hipLaunchKernelGGL((probe_strip_read_kernel<256, false>), grid, block, 0, st, p, pitch, r, parts, s);
+  }
   return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
 }
 

@@ -393,6 +393,12 @@ int mi355q_fp8_sdpa_fwd(const void* q, const void* k, const void* v, int fp8_fmt
  */
 int mi355q_probe_mfma(int waves_per_simd, int mfma_per_wave, int workgroups, float* sink, void* stream);
 int mi355q_probe_read(const void* x, int64_t bytes, int workgroups, void* sink, void* stream);
+/* mi355q_probe_strip_read reads a row-major byte matrix [rows, pitch] the way the decode-shaped GEMMs read
+ * their weights: pitch / strip_bytes strips (64, 128 or 256 bytes of every row), the rows of a strip cut
+ * into `parts` ranges, one workgroup per strip and range, 16-byte loads with or without the nontemporal
+ * hint, nothing stored. */
+int mi355q_probe_strip_read(const void* x, int64_t pitch, int64_t rows, int strip_bytes, int parts, int nontemporal,
+                            void* sink, void* stream);
 
 /* Name of the kernel variant mi355q_fp8_gemm would pick for a problem
  * (for logs and profiles; static string). */
