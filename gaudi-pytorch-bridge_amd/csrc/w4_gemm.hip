@@ -77,11 +77,20 @@ constexpr int w4_stages() {
 // One 16-byte piece per lane, straight copy into LDS (lane l lands at dst + 16 l).  The
 // s_nop covers a descriptor word that reached its scalar register through a vector
 // instruction (five wait states before a memory instruction may read it).
+// STREAM adds the nontemporal hint, for weights that the launch reads once.
+template <bool STREAM = false>
 __device__ __forceinline__ void w4_dma16(const i32x4& rsrc, int voff, uint32_t lds_dst) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-               :
-               : "s"(lds_dst), "v"(voff), "s"(rsrc)
-               : "memory", "m0");
+  if constexpr (STREAM) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, 0 offen nt lds"
+                 :
+                 : "s"(lds_dst), "v"(voff), "s"(rsrc)
+                 : "memory", "m0");
+  } else {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_dst), "v"(voff), "s"(rsrc)
+                 : "memory", "m0");
+  }
 }
 
 // A buffer descriptor that walks through memory in fixed steps: base and the bytes left behind it.
@@ -589,10 +598,13 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
     auto issue_stage = [&](int off, int stage) {
       const uint32_t base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)(lds + off);
       const i32x4 rp = wp.rsrc(0x7fffffffLL);
-      w4_dma16(rp, vo_even, base + kOffPacked + (wq * 4) * 1024);
-      w4_dma16(rp, vo_odd, base + kOffPacked + (wq * 4 + 1) * 1024);
-      w4_dma16(rp, vo_even + 16 * ld, base + kOffPacked + (wq * 4 + 2) * 1024);
-      w4_dma16(rp, vo_odd + 16 * ld, base + kOffPacked + (wq * 4 + 3) * 1024);
+      // with tiles of 16 or 32 rows there is one row block: the weights are read once (with 64-row tiles further
+      // row blocks read them again, out of the caches)
+      constexpr bool kOnce = ROWS != 64;
+      w4_dma16<kOnce>(rp, vo_even, base + kOffPacked + (wq * 4) * 1024);
+      w4_dma16<kOnce>(rp, vo_odd, base + kOffPacked + (wq * 4 + 1) * 1024);
+      w4_dma16<kOnce>(rp, vo_even + 16 * ld, base + kOffPacked + (wq * 4 + 2) * 1024);
+      w4_dma16<kOnce>(rp, vo_odd + 16 * ld, base + kOffPacked + (wq * 4 + 3) * 1024);
       wp.step(packed_step);
       static_for<LA::kPerWave>([&](auto ic) { la.template issue_one<decltype(ic)::value, true>(lds + off, stage * kBK, g.K); });
       la.advance();
