@@ -24,7 +24,8 @@
 // the fp4 operand of the same MFMA holds k = 16 h + j in nibble j < 16 and
 // k = 32 + 16 h + (j - 16) in nibble j >= 16.
 //
-// Shaped like the strip kernel of gemm_skinny.h: the weights stream once through a deep LDS
+// Two kernels.  The first, below, is shaped like the strip kernel of gemm_skinny.h (the second, for groups of
+// 128 with bf16 scales, follows it: 256-column strips, K split over workgroups): the weights stream once through a deep LDS
 // ring, one workgroup per 128 columns; rows of A beyond 64 run as further row blocks that
 // stream the weights again, which suits decode and small prefill batches, the shapes
 // weight-only quantisation is used for.  A workgroup has eight waves, two per SIMD, with
@@ -484,7 +485,8 @@ __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
 }
 
 // ---------------------------------------------------------------------------------- wide strips
-// For at most 32 rows of A, groups of 128 and bf16 scales.  A workgroup takes 256 columns: a k-row
+// For groups of 128 and bf16 scales (tiles of 16, 32 or 64 rows; more rows are further row blocks of 64).
+// A workgroup takes 256 columns: a k-row
 // of its packed weights is a whole 128-byte line (the 64-byte rows of the 128-column strips move
 // at about 3.2 TB/s, whole lines at 4.3), and K is cut into `ksplit` parts walked by as many
 // workgroups, so that a launch fills the chip whatever N is.  The parts of a strip meet through
