@@ -195,8 +195,33 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
     }
   }
 
+  // The V fragments do not depend on the scores: for up to four tiles their LDS reads go out here, under the
+  // score MFMAs and the softmax, instead of one tile at a time in front of each P V product (where the wave
+  // would wait for LDS four times with the matrix pipe idle).
+  const int g = lane >> 4, gi = lane & 15;
+  const int r8 = gi >> 1, hh = gi & 1;
+  constexpr bool kEarlyV = DVT <= 4;
+  i32x8 vfe[kEarlyV ? DVT : 1];
+  if constexpr (kEarlyV) {
+#pragma unroll
+    for (int t = 0; t < DVT; ++t) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const int krow = 32 * (p >> 1) + 8 * (2 * (p & 1) + (r8 >> 2)) + 4 * h + (r8 & 3);
+        const int off = v_lds_offset<kVRow>(krow, 2 * t + (g & 1)) + hh * 8;
+        const i32x2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((SDPA_LDS_AS i32x2*)((SDPA_LDS_AS uint8_t*)vb + off));
+        vfe[t][2 * p] = w[0];
+        vfe[t][2 * p + 1] = w[1];
+      }
+    }
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+    for (int t = 0; t < DVT; ++t) asm volatile("" : "+v"(vfe[t]));  // the reads are issued here, not sunk to their use
+#endif
+  }
+
   // scores in units of log2, masks applied
-    float mx = -__builtin_inff();
+  float mx = -__builtin_inff();
   if (!edge && sc2 >= 0.0f) {
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -221,7 +246,11 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
         mx = __builtin_fmaxf(mx, x);
       }
   }
-  mx = __builtin_fmaxf(mx, __shfl_xor(mx, 32, 64));
+  {  // the other half-wave's maximum for the same query row: a swap of register halves, no trip through LDS
+    typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
+    const u32x2v sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+    mx = __builtin_fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+  }
   const float m_new = __builtin_fmaxf(m_run, mx);
   const float m_use = m_new == -__builtin_inff() ? 0.0f : m_new;
   const float alpha = fast_exp2(m_run - m_use);
@@ -248,9 +277,12 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
           psum += p[i];
           if (CLAMP) p[i] = __builtin_elementwise_minimum(p[i], kMax8);
         }
-        // both halves of the word are written: what it held before does not matter, and taking the register's
-        // previous contents as the "old" value saves the move that a zero would cost
-        int w = pf[4 * t + j];
+        // Both halves of the word are written, so what it held before does not matter: the empty statement
+        // makes it "defined" for the compiler at no cost, where a zero would cost a move per word.
+        int w = 0;
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("" : "=v"(w));
+#endif
         if constexpr (FMT == MI355Q_E5M2) {
           w = __builtin_amdgcn_cvt_pk_bf8_f32(p[0], p[1], w, false);
           w = __builtin_amdgcn_cvt_pk_bf8_f32(p[2], p[3], w, true);
@@ -276,10 +308,12 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
   }
 
   // O^T += V^T P^T; k-slot 8 p + r' of half-wave h is key 32 (p / 2) + 8 (2 (p % 2) + r' / 4) + 4 h + r' % 4
-  const int g = lane >> 4, gi = lane & 15;
-  const int r8 = gi >> 1, hh = gi & 1;
 #pragma unroll
   for (int t = 0; t < DVT; ++t) {
+    if constexpr (kEarlyV) {
+      o[t] = sdpa_mfma<FMT>(vfe[t], pf, o[t]);
+      continue;
+    }
     i32x8 vf;
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
