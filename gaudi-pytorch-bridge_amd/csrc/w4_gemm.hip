@@ -505,7 +505,9 @@ __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
 //  * the zero-points are not two more planes: sum_k a (q - z) = sum_k a q - z sum_k a, and the row
 //    sums of the stage's A tile come from one producer wave (one MFMA against a plane of ones, the
 //    producers taking turns), which leaves them in a small ring in LDS for the consumers' fold of
-//    the next stage;
+//    the next stage; in the 32- and 64-row forms another producer leaves -(z x scale) per column
+//    there as fp32, so that the fold is two multiply-adds per element
+//    (total += scale x acc; total += (-z x scale) x row sum);
 //  * with at most 16 rows (M16) the consumers use v_mfma_scale_f32_16x16x128_f8f6f4, half the
 //    matrix work of the 32x32x64 form, which would multiply 16 rows of padding.
 // In the 16x16x128 form with an fp4 first and an fp8 second operand, lane group g = lane / 16 of the
@@ -545,6 +547,8 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
   static_assert(kConsumers * epilogue_stage_floats<MT, 1>() * 4 <= S * kStage, "epilogue area overlays the ring");
   __shared__ __attribute__((aligned(1024))) uint8_t lds[S * kStage];
   __shared__ float row_sums[kW4SumRing][BM];
+  // per stage (two kept) and column: minus the group's zero-point times its scale, fp32 (32- and 64-row forms)
+  __shared__ __attribute__((aligned(16))) float zs_rows[2][(M16 || !HAS_Z) ? 4 : kW4WideBN];
   __shared__ uint32_t ticket_drawn;
 
   GemmArgs g = a.g;
@@ -652,6 +656,22 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         });
       }
     };
+    // -(zero-point) x scale of the stage's group, four columns per lane, for the consumers' fold one stage later:
+    // what every consumer lane would otherwise work out for its sixteen columns in every stage.
+    const uint32_t pflip = a.is_signed ? 0x8888u : 0u, pzmask = a.zp ? 0xffffu : 0u;
+    auto column_rows = [&](int off, int slot) {
+      const uint8_t* st = lds + off;
+      const u32x2 sw = *reinterpret_cast<const u32x2*>(st + kOffScale + 8 * lane);
+      const uint32_t zw = ((uint32_t)*reinterpret_cast<const uint16_t*>(st + kOffZp + 2 * lane) & pzmask) ^ pflip;
+      f32x4 sf, zf;
+      sf[0] = __uint_as_float(sw[0] << 16);
+      sf[1] = __uint_as_float(sw[0] & 0xffff0000u);
+      sf[2] = __uint_as_float(sw[1] << 16);
+      sf[3] = __uint_as_float(sw[1] & 0xffff0000u);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) zf[i] = -(float)((zw >> (4 * i)) & 15u) * sf[i];
+      *reinterpret_cast<f32x4*>(&zs_rows[slot][4 * lane]) = zf;
+    };
 #pragma unroll
     for (int s = 0; s < S - 1; ++s) issue_stage(s * kStage, s);
     int wr_off = (S - 1) * kStage, rd_off = 0;
@@ -660,6 +680,9 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
       wait_for_stage(KT - 1 - kt);
       __syncthreads();
       issue_stage(wr_off, kt + S - 1);
+      if constexpr (!M16 && HAS_Z) {
+        if (((kt + 2) & 3) == wq) column_rows(rd_off, kt & 1);
+      }
       if (HAS_Z && (kt & 3) == wq) sum_rows(rd_off, kt & (kW4SumRing - 1));
       wr_off += kStage;
       if (wr_off == S * kStage) wr_off = 0;
@@ -773,26 +796,30 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         const int row = 32 * j + 16 * th + tr;
         poff[j] = kOffPacked + row * 128 + ((wq ^ ((row >> 1) & 7)) << 4) + (tg & 1) * 8;
       }
-      const int zoff = kOffZp + (wn / 8) * 4;  // the four words of this wave's columns
-      const int zshift = 16 * (lane >> 5);
       const int soff = kOffScale + (wn + 4 * (lane >> 5)) * 2;
       // two sets of partial sums, folded one stage late behind the next stage's MFMAs; with 64 rows there are
       // registers for one set only, folded at the start of the next stage, before its MFMAs overwrite it
       constexpr int NB = MT == 1 ? 2 : 1;
       f32x16 acc[NB][MT];
       float sc[16];
-      u32x4 zprev = {0u, 0u, 0u, 0u};
-      auto fold = [&](auto bc, int sum_slot) {
+      // total += scale x acc - (zero-point x scale) x (row sum of A): the second factor comes ready from a producer
+      const int zsoff = wn + 4 * (lane >> 5);
+      auto fold = [&](auto bc, int stage_no) {
         constexpr int B = decltype(bc)::value % NB;
+        f32x4 zs[4];
+        if constexpr (HAS_Z) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) zs[q] = *reinterpret_cast<const f32x4*>(&zs_rows[stage_no & 1][zsoff + 8 * q]);
+        }
         static_for<MT>([&](auto ic) {
           constexpr int i = decltype(ic)::value;
           float rs = 0.0f;
-          if constexpr (HAS_Z) rs = row_sums[sum_slot][32 * i + (lane & 31)];
+          if constexpr (HAS_Z) rs = row_sums[stage_no & (kW4SumRing - 1)][32 * i + (lane & 31)];
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
-            float v = acc[B][i][e];
-            if constexpr (HAS_Z) v = __builtin_fmaf(-(float)((zprev[e >> 2] >> (4 * (e & 3))) & 15u), rs, v);
-            total[16 * i + e] = __builtin_fmaf(v, sc[e], total[16 * i + e]);
+            float t = __builtin_fmaf(acc[B][i][e], sc[e], total[16 * i + e]);
+            if constexpr (HAS_Z) t = __builtin_fmaf(zs[e >> 2][e & 3], rs, t);
+            total[16 * i + e] = t;
           }
         });
       };
@@ -820,8 +847,6 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         u32x2 snew[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) snew[q] = *reinterpret_cast<const u32x2*>(st + soff + q * 16);
-        u32x4 znew = {0u, 0u, 0u, 0u};
-        if constexpr (HAS_Z) znew = *reinterpret_cast<const u32x4*>(st + zoff);
         if constexpr (HAVE_PREV && NB == 1) fold(std::integral_constant<int, 0>{}, (slot - 1) & (kW4SumRing - 1));
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -853,7 +878,6 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
           sc[4 * q + 1] = __uint_as_float(snew[q][0] & 0xffff0000u);
           sc[4 * q + 2] = __uint_as_float(snew[q][1] << 16);
           sc[4 * q + 3] = __uint_as_float(snew[q][1] & 0xffff0000u);
-          zprev[q] = (((znew[q] & zmask) ^ flip) >> zshift) & 0xffffu;
         }
         rd_off += kStage;
         if (rd_off == S * kStage) rd_off = 0;
