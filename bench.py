@@ -538,7 +538,7 @@ def bench_sdpa(oracle, dev, steps, warmup, cpu):
         nbytes = 2 * B * HK * S * D + B * H * D + 2 * B * H * D
         out.append(hbm_entry(f"fp8_sdpa_decode_B{B}_S{S}", f"fp8_sdpa_recomp_fwd, one query per head, batch {B}, 32 query / 8 kv heads, "
                                                            f"kv_len = {S}, head_dim 128, e4m3fn -> bf16", nbytes, ms, max(steps, 50),
-                             "fp8_sdpa_decode_kernel<2,4,e4m3fn> + fp8_sdpa_decode_merge_kernel"))
+                             "fp8_sdpa_decode_kernel<2,4,e4m3fn>"))
         del ks, vs
     return out
 

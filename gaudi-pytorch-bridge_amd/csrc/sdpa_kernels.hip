@@ -67,6 +67,7 @@ struct SdpaArgs {
   int rows;         // rows of the tile that hold a query
   int nsplit, blocks_per_split;
   float* ws;        // partial results of the key splits when nsplit > 1
+  uint32_t* tickets;  // one arrival counter per group, zero between launches
 };
 
 __device__ __forceinline__ float sdpa_scale(const SdpaArgs& a, int i, float absent) {
@@ -815,7 +816,11 @@ __global__ __launch_bounds__(kSdpaThreads) void fp8_sdpa_decode_kernel(const Sdp
     uint8_t* orow = a.out + (o_off + (int64_t)rin * a.o_bs[2] + (int64_t)rq * a.ldo) * (a.out_fp8 ? 1 : 2);
     sdpa_store_row<DVT>(a, orow, row < a.rows, dvg == 0 ? inv_l : 0.0f, dvg, 8, val);
   } else {
-    // unnormalised: the merged maximum, the merged sum and O for the second kernel
+    // Unnormalised: the merged maximum, the merged sum and O of this split go to the workspace; the workgroup
+    // that draws the group's last ticket merges the splits in their order, whoever came last, and stores the
+    // rows.  The partial results are written and read with device-scope atomic accesses, which go past this
+    // XCD's cache to where the other XCDs see them: no cache has to be written back or invalidated as a whole,
+    // which a fence would do.  The last one returns the counter to zero for the next launch.
     float M = -__builtin_inff();
     for (int w = 0; w < 4; ++w) M = __builtin_fmaxf(M, parts[w * kDecodeTileFloats(DVT) + 32 * DVT * 32 + row]);
     float L = 0.0f, val[DVT * 32 / 8];
@@ -829,56 +834,48 @@ __global__ __launch_bounds__(kSdpaThreads) void fp8_sdpa_decode_kernel(const Sdp
 #pragma unroll
       for (int i = 0; i < DVT * 32 / 8; ++i) val[i] += pw[(dvg + 8 * i) * 32 + row] * wgt;
     }
-    float* out = a.ws + ((int64_t)grp * a.nsplit + split) * kDecodeTileFloats(DVT);
+    float* group_parts = a.ws + (int64_t)grp * a.nsplit * kDecodeTileFloats(DVT);
+    float* out = group_parts + (int64_t)split * kDecodeTileFloats(DVT);
 #pragma unroll
-    for (int i = 0; i < DVT * 32 / 8; ++i) out[(dvg + 8 * i) * 32 + row] = val[i];
+    for (int i = 0; i < DVT * 32 / 8; ++i)
+      __hip_atomic_store(out + (dvg + 8 * i) * 32 + row, val[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (dvg == 0) {
-      out[32 * DVT * 32 + row] = M;
-      out[32 * DVT * 32 + 32 + row] = L;
+      __hip_atomic_store(out + 32 * DVT * 32 + row, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(out + 32 * DVT * 32 + 32 + row, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-  }
-}
-
-// The splits of one group merged, normalised and stored: a workgroup takes eight columns of the
-// group's tile, a thread one (row, column) and all the splits.
-template <int DVT>
-__global__ __launch_bounds__(kSdpaThreads) void fp8_sdpa_decode_merge_kernel(const SdpaArgs a) {
-  const int64_t grp = blockIdx.x;
-  int64_t q_off, k_off, v_off, m_off, o_off;
-  sdpa_group_offsets(a, grp, q_off, k_off, v_off, m_off, o_off);
-  const int tid = threadIdx.x, row = tid & 31, d = blockIdx.y * 8 + (tid >> 5);
-  const bool row_ok = row < a.rows;
-  const float* parts = a.ws + grp * a.nsplit * kDecodeTileFloats(DVT);
-  float M = -__builtin_inff(), L = 0.0f, O = 0.0f;
-  if (row_ok) {
-    for (int w = 0; w < a.nsplit; ++w) M = __builtin_fmaxf(M, parts[(int64_t)w * kDecodeTileFloats(DVT) + 32 * DVT * 32 + row]);
+    __builtin_amdgcn_s_waitcnt(0);  // the stores have been acknowledged before the ticket is drawn
+    __syncthreads();
+    uint32_t* drawn = reinterpret_cast<uint32_t*>(lds);  // the tiles in LDS have been read
+    if (tid == 0) {
+      const uint32_t t = __hip_atomic_fetch_add(a.tickets + grp, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (t == (uint32_t)a.nsplit - 1) __hip_atomic_store(a.tickets + grp, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *drawn = t;
+    }
+    __syncthreads();
+    if (*drawn != (uint32_t)a.nsplit - 1) return;
+    M = -__builtin_inff();
+    for (int w = 0; w < a.nsplit; ++w)
+      M = __builtin_fmaxf(M, __hip_atomic_load(group_parts + (int64_t)w * kDecodeTileFloats(DVT) + 32 * DVT * 32 + row, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT));
+    L = 0.0f;
+#pragma unroll
+    for (int i = 0; i < DVT * 32 / 8; ++i) val[i] = 0.0f;
     for (int w = 0; w < a.nsplit; ++w) {
-      const float* pw = parts + (int64_t)w * kDecodeTileFloats(DVT);
-      const float mw = pw[32 * DVT * 32 + row];
+      const float* pw = group_parts + (int64_t)w * kDecodeTileFloats(DVT);
+      const float mw = __hip_atomic_load(pw + 32 * DVT * 32 + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       const float wgt = mw == -__builtin_inff() ? 0.0f : fast_exp2(mw - M);
-      L += pw[32 * DVT * 32 + 32 + row] * wgt;
-      O += pw[d * 32 + row] * wgt;
+      L += __hip_atomic_load(pw + 32 * DVT * 32 + 32 + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * wgt;
+#pragma unroll
+      for (int i = 0; i < DVT * 32 / 8; ++i)
+        val[i] += __hip_atomic_load(pw + (dvg + 8 * i) * 32 + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * wgt;
     }
-  }
-  const float dv = sdpa_scale(a, 2, 1.0f), qs = sdpa_scale(a, 3, 1.0f), ds = sdpa_scale(a, 5, 1.0f / qs);
-  const float l = L / qs;
-  const float inv_l = l > 0.0f ? 1.0f / l : 0.0f;
-  const float v = O * inv_l * (ds * dv);
-  const bool store = row_ok && d < a.Dv;
-  if (store) {
+    const float l = L / qs;
+    const float inv_l = l > 0.0f ? 1.0f / l : 0.0f;
+#pragma unroll
+    for (int i = 0; i < DVT * 32 / 8; ++i) val[i] *= inv_l;
     const int rin = a.pack ? row / a.L : 0, rq = a.pack ? row - rin * a.L : row;
     uint8_t* orow = a.out + (o_off + (int64_t)rin * a.o_bs[2] + (int64_t)rq * a.ldo) * (a.out_fp8 ? 1 : 2);
-    if (a.out_fp8) orow[d] = (uint8_t)(cvt_fp8x4<MI355Q_E4M3FN>(v * sdpa_scale(a, 4, 1.0f), 0.f, 0.f, 0.f) & 0xffu);
-    else reinterpret_cast<uint16_t*>(orow)[d] = (uint16_t)(pack_bf16x2(v, 0.f) & 0xffffu);
-  }
-  const int lane = tid & 63;
-  if (a.amax_s != nullptr && blockIdx.y == 0) {
-    const uint32_t m = wave_max_u32(__float_as_uint(row_ok && tid < 32 ? inv_l : 0.0f));
-    if (lane == 0 && m != 0u) atomicMax(reinterpret_cast<unsigned int*>(a.amax_s), m);
-  }
-  if (a.amax_o != nullptr) {
-    const uint32_t m = wave_max_u32(__float_as_uint(store ? __builtin_fabsf(v) : 0.0f));
-    if (lane == 0 && m != 0u) atomicMax(reinterpret_cast<unsigned int*>(a.amax_o), m);
+    sdpa_store_row<DVT>(a, orow, row < a.rows, dvg == 0 ? inv_l : 0.0f, dvg, 8, val);
   }
 }
 
@@ -887,17 +884,13 @@ static int sdpa_decode_launch(const SdpaArgs& a, int fmt, int64_t groups, hipStr
   const dim3 grid((unsigned)(groups * a.nsplit));
   if (fmt == MI355Q_E5M2) hipLaunchKernelGGL((fp8_sdpa_decode_kernel<DKC, DVT, MI355Q_E5M2>), grid, dim3(kSdpaThreads), 0, st, a);
   else hipLaunchKernelGGL((fp8_sdpa_decode_kernel<DKC, DVT, MI355Q_E4M3FN>), grid, dim3(kSdpaThreads), 0, st, a);
-  if (hipGetLastError() != hipSuccess) return MI355Q_ERR_LAUNCH;
-  if (a.nsplit > 1) {
-    hipLaunchKernelGGL((fp8_sdpa_decode_merge_kernel<DVT>), dim3((unsigned)groups, DVT * 32 / 8), dim3(kSdpaThreads), 0, st, a);
-    if (hipGetLastError() != hipSuccess) return MI355Q_ERR_LAUNCH;
-  }
-  return MI355Q_OK;
+  return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
 }
 
 static int compute_units_sdpa();
 
 // How the few-queries kernel would run a problem: rows of the tile, groups, splits (0 groups: it does not apply).
+constexpr size_t kSdpaTicketBytes = 1024;  // arrival counters in front of the partial results
 struct SdpaDecodePlan {
   int64_t groups = 0;
   int pack = 0, rows = 0, nsplit = 1, blocks_per_split = 0, dvt = 0;
@@ -920,7 +913,13 @@ static SdpaDecodePlan sdpa_decode_plan(const mi355q_sdpa_desc* d, int cus) {
   want = want < 1 ? 1 : (want > most ? most : want);
   p.blocks_per_split = (int)((nblk + want - 1) / want);
   p.nsplit = (nblk + p.blocks_per_split - 1) / p.blocks_per_split;
-  p.ws_bytes = p.nsplit > 1 ? (size_t)p.groups * p.nsplit * kDecodeTileFloats(p.dvt) * sizeof(float) : 0;
+  // One arrival counter per group in an area of a fixed size, then the splits' partial results: a workspace that
+  // is used for problems of different shapes finds the counters zero whatever the last shape left behind them.
+  if (p.nsplit > 1 && (size_t)p.groups * 4 > kSdpaTicketBytes) {
+    p.nsplit = 1;
+    p.blocks_per_split = nblk;
+  }
+  p.ws_bytes = p.nsplit > 1 ? kSdpaTicketBytes + (size_t)p.groups * p.nsplit * kDecodeTileFloats(p.dvt) * sizeof(float) : 0;
   return p;
 }
 
@@ -1053,7 +1052,8 @@ int mi355q_fp8_sdpa_fwd(const void* q, const void* k, const void* v, int fp8_fmt
     a.rows = plan.rows;
     a.nsplit = plan.nsplit;
     a.blocks_per_split = plan.blocks_per_split;
-    a.ws = static_cast<float*>(workspace);
+    a.tickets = static_cast<uint32_t*>(workspace);
+    a.ws = workspace != nullptr ? reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + kSdpaTicketBytes) : nullptr;
     return plan.dvt == 2 ? sdpa_decode_launch<1, 2>(a, fp8_fmt, plan.groups, st) : sdpa_decode_launch<2, 4>(a, fp8_fmt, plan.groups, st);
   }
   if (dmax <= 64) return sdpa_launch<1, 2>(a, fp8_fmt, blocks, st);

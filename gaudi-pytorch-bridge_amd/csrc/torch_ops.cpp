@@ -22,6 +22,7 @@
 #include <cstdlib>
 #include <iostream>
 #include <map>
+#include <tuple>
 #include <mutex>
 #include <sstream>
 
@@ -735,18 +736,20 @@ Tensor convert_from_uint4(const Tensor& input, const Tensor& scale,
 // fused op; shapes the kernel does not take raise (there is no second route to the same bits).
 //
 // The kernel's split over K keeps arrival counters in its workspace, which have to be zero when a
-// call starts and are left zero by every call: one zero-filled buffer per (device, stream) is kept
-// here and grown on demand, so that a call launches one kernel and nothing else.  Calls on one
-// stream run in order, which is all the sharing the buffer allows.  While a stream is being
-// captured into a graph no buffer is handed out (its memory would belong to the graph's pool, and
-// replays of two graphs could overlap): the kernel then runs without the split.
-Tensor w4a8_workspace(const Tensor& like, size_t bytes) {
+// call starts and are left zero by every call (the key splits of the attention kernel for few
+// queries do the same): one zero-filled buffer per (device, stream, op) is kept here and grown on
+// demand, so that a call launches one kernel and nothing else.  Calls on one stream run in order,
+// which is all the sharing the buffer allows; the two ops lay their counters out differently and
+// do not share.  While a stream is being captured into a graph no buffer is handed out (its memory
+// would belong to the graph's pool, and replays of two graphs could overlap).
+enum TicketWorkspaceOp { kWsW4a8 = 0, kWsSdpa = 1 };
+Tensor ticket_workspace(const Tensor& like, size_t bytes, TicketWorkspaceOp op) {
   if (bytes == 0 || c10::hip::currentStreamCaptureStatusMayInitCtx() != c10::hip::CaptureStatus::None) return Tensor();
   static std::mutex mu;
   // never destroyed: a static Tensor would be freed after the HIP runtime has shut down
-  static auto* cache = new std::map<std::pair<int, void*>, Tensor>();
+  static auto* cache = new std::map<std::tuple<int, void*, int>, Tensor>();
   std::lock_guard<std::mutex> lock(mu);
-  Tensor& t = (*cache)[std::make_pair((int)like.device().index(), current_stream(like))];
+  Tensor& t = (*cache)[std::make_tuple((int)like.device().index(), current_stream(like), (int)op)];
   if (!t.defined() || (size_t)t.numel() < bytes) t = at::zeros({(int64_t)bytes}, like.options().dtype(at::kByte));
   return t;
 }
@@ -799,7 +802,8 @@ Tensor w4a8_gemm(const Tensor& A, const Tensor& packed, const Tensor& scale, con
     b = bias->to(out_dtype).contiguous();
   }
   MI355Q_OP_INFO("w4a8_gemm : A=" << A.sizes() << " packed=" << packed.sizes() << " group=" << group << " signed=" << is_signed);
-  Tensor ws = w4a8_workspace(a, mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, to_mi355q_dtype(s.scalar_type())));
+  // under graph capture: none, and the kernel then runs without the split
+  Tensor ws = ticket_workspace(a, mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, to_mi355q_dtype(s.scalar_type())), kWsW4a8);
   const int st = mi355q_w4a8_gemm(a.data_ptr(), to_mi355q_dtype(a.scalar_type()), K, w.data_ptr<int32_t>(), N / 8, s.data_ptr(),
                                   to_mi355q_dtype(s.scalar_type()), has_zp ? z.data_ptr<int32_t>() : nullptr, is_signed ? 1 : 0,
                                   group, out.data_ptr(), to_mi355q_dtype(out_dtype), N, M, N, K, sa_dev, 1.0f, sa_mode,
@@ -1142,8 +1146,13 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
   }
   // few queries against many keys: the partial results of the key splits pass through a workspace
   const size_t ws_bytes = mi355q_fp8_sdpa_workspace_bytes(&d);
+  // (their arrival counters start from zero and are left zero: the buffer kept per stream, or, while the stream
+  // is being captured into a graph, a zero-filled one of the graph's own)
   Tensor ws;
-  if (ws_bytes > 0) ws = at::empty({(int64_t)ws_bytes}, opts.dtype(at::kByte));
+  if (ws_bytes > 0) {
+    ws = ticket_workspace(qc, ws_bytes, kWsSdpa);
+    if (!ws.defined()) ws = at::zeros({(int64_t)ws_bytes}, opts.dtype(at::kByte));
+  }
   check_status(mi355q_fp8_sdpa_fwd(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), to_mi355q_dtype(dt), has_mask ? mk.data_ptr() : nullptr,
                                    mask_kind, out.data_ptr(), to_mi355q_dtype(out_dt), &d, (float)scale, is_causal ? 1 : 0, sc_dev,
                                    sc_host, is_amax_s ? amax_s.data_ptr<float>() : nullptr,

@@ -993,7 +993,10 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
 struct W4WidePlan {
   int rows, row_blocks, strips, parts;
   int tile_rows() const { return rows == 64 ? 64 : 32; }
-  size_t ticket_bytes() const { return ((size_t)strips * row_blocks * 4 + 255) / 256 * 256; }
+  // The counters sit in front of the partial sums, in an area of a fixed size: a workspace that is used for
+  // problems of different shapes then finds them zero whatever the last shape left in the partial sums.
+  // K is only split for at most 128 strips (256 / groups >= 2 below).
+  static constexpr size_t ticket_bytes() { return 1024; }
   size_t workspace_bytes() const {
     return parts < 2 ? 0 : ticket_bytes() + (size_t)parts * strips * row_blocks * w4_wide_partial_bytes(tile_rows());
   }
@@ -1010,6 +1013,7 @@ inline W4WidePlan w4a8_wide_plan(int64_t M, int64_t N, int64_t K, int64_t group,
   // too few workgroups for the chip even so: the 128-column strips have twice as many
   if (parts < 2) parts = groups >= 100 ? 1 : 0;
   if (p.row_blocks > 65535) parts = 0;
+  if (parts >= 2 && (size_t)groups * 4 > W4WidePlan::ticket_bytes()) parts = 1;  // (cannot happen: 256 / groups >= 2)
   p.parts = (int)parts;
   return p;
 }

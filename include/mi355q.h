@@ -250,13 +250,13 @@ int mi355q_fp8_gemm(const void* A, int fmt_a, int trans_a, int64_t lda,
  * pointers 16-byte aligned; otherwise MI355Q_ERR_UNSUPPORTED, and the caller expands the weights
  * with mi355q_dequant_4bit.
  *
- * workspace: with at most 32 rows of A, groups of 128 and bf16 scales, K is walked in parts by
- * several workgroups per 256 columns, which meet through `workspace`:
+ * workspace: with groups of 128 and bf16 scales, K is walked in parts by several workgroups per
+ * 256 columns where that fills the chip better, which meet through `workspace`:
  * mi355q_w4a8_gemm_workspace_bytes() of device memory, 16-byte aligned (0: the shape is not split
- * and no workspace is read).  Its first (N / 256 rounded up) 32-bit words, rounded up to 256 bytes,
- * are arrival counters: they have to be zero when a call starts and every call leaves them zero, so
- * a workspace is zero-filled once, when it is allocated, and then reused.  Calls that share a
- * workspace must not overlap (one stream, or an order between the streams).  NULL is allowed: the
+ * and no workspace is read).  Its first KiB holds arrival counters (whatever the shape): they have
+ * to be zero when a call starts and every call leaves them zero, so a workspace is zero-filled
+ * once, when it is allocated, and then reused, also for other shapes it is large enough for.  Calls
+ * that share a workspace must not overlap (one stream, or an order between the streams).  NULL is allowed: the
  * call then runs without the split, slower for these shapes.  Too small or misaligned:
  * MI355Q_ERR_WORKSPACE.  The parts are added in a fixed order: a result does not depend on which
  * workgroup finished last.
@@ -365,9 +365,13 @@ typedef struct mi355q_sdpa_desc {
  * Few queries against many keys (decoding: at most 32 rows of (innermost batch index, query) that
  * share a k and v, kv_len >= 512, head dimensions up to 128, 16-byte aligned rows) run on a kernel
  * that splits the keys over workgroups; the splits' partial results pass through `workspace`
- * (device memory, mi355q_fp8_sdpa_workspace_bytes(desc) bytes, 0 when the problem does not split).
- * Without a workspace of that size the call still works, one workgroup per group of rows.
- * Nothing is allocated here.
+ * (device memory, 4-byte aligned, mi355q_fp8_sdpa_workspace_bytes(desc) bytes, 0 when the problem
+ * does not split), and the workgroup of a group that finishes last merges them (one launch).  The
+ * workspace begins with 1 KiB of arrival counters: it has to be zero-filled before its first use,
+ * every call leaves the counters zero, so it can be passed again as it is (to this entry point,
+ * for any problem it is large enough for); calls that may overlap in time need workspaces of
+ * their own.  Without a workspace of that size the call still works, one workgroup per group of
+ * rows.  Nothing is allocated here.
  */
 size_t mi355q_fp8_sdpa_workspace_bytes(const mi355q_sdpa_desc* desc);
 /* How the few-queries kernel would walk the keys of a problem with a workspace of that size:

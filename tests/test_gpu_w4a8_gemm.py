@@ -158,9 +158,9 @@ def test_split_k_workspace_c_abi(oracle, pkg, dev):
     M, K, N, group = 24, 4096, 1312, 128
     need = lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, pkg.BF16)
     strips = (N + 255) // 256
-    assert need == 256 + 4 * strips * 32 * 256 * 4                        # K / 128 / 8 = 4 parts
-    assert lib.mi355q_w4a8_gemm_workspace_bytes(33, N, K, group, pkg.BF16) == 256 + 4 * strips * 64 * 256 * 4    # 64-row tiles
-    assert lib.mi355q_w4a8_gemm_workspace_bytes(130, N, K, group, pkg.BF16) == 256 + 4 * strips * 3 * 64 * 256 * 4  # three row blocks
+    assert need == 1024 + 4 * strips * 32 * 256 * 4                       # 1 KiB of counters; K / 128 / 8 = 4 parts
+    assert lib.mi355q_w4a8_gemm_workspace_bytes(33, N, K, group, pkg.BF16) == 1024 + 4 * strips * 64 * 256 * 4   # 64-row tiles
+    assert lib.mi355q_w4a8_gemm_workspace_bytes(130, N, K, group, pkg.BF16) == 1024 + 4 * strips * 3 * 64 * 256 * 4  # three row blocks
     assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, 256, pkg.BF16) == 0       # groups of two stages
     assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, pkg.F32) == 0      # fp32 scales
     assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, 1024, group, pkg.BF16) == 0  # too few stages to split
@@ -180,7 +180,7 @@ def test_split_k_workspace_c_abi(oracle, pkg, dev):
         assert call(C, Ad, workspace, nbytes) == 0
         torch.cuda.synchronize()
         assert torch.equal(C.cpu().double(), expect)
-        assert int(ws[:256].view(torch.int32).abs().sum()) == 0
+        assert int(ws[:1024].view(torch.int32).abs().sum()) == 0
     C = torch.full((M, N), -5.0, device=dev)
     assert call(C, Ad, ws, need - 1) == 4 and call(C, Ad, ws[1:], need) == 4      # too small, misaligned
     torch.cuda.synchronize()
@@ -209,6 +209,32 @@ def test_split_k_workspace_c_abi(oracle, pkg, dev):
     torch.cuda.synchronize()
     assert torch.equal(C[:, :N].cpu(), (expect[:M2] * sa.double()[:, None] + bias.double()).float().bfloat16())
     assert (C[:, N:] == -5.0).all()
+
+
+def test_one_workspace_for_problems_of_different_shapes(oracle, pkg, dev):
+    """A workspace sized for the largest problem serves a narrow one (one strip) and then a wide one (many strips),
+    and the narrow one again: the counters have a place of their own in front, which no shape's partial sums reach."""
+    lib = pkg.capi()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    gen = torch.Generator().manual_seed(12)
+    K, group = 4096, 128
+    shapes = [(24, 256), (40, 2304), (24, 256), (16, 6400)]
+    need = max(lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, pkg.BF16) for M, N in shapes)
+    assert need > 0
+    ws = torch.zeros(need, dtype=torch.uint8, device=dev)
+    for M, N in shapes:
+        assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, pkg.BF16) > 0
+        q, z, s, pk, pz = weights(oracle, gen, K, N, group, False, True, pow2=True)
+        a = torch.randint(-4, 5, (M, K), generator=gen).float()
+        expect = a.double() @ ((q - z.repeat_interleave(group, 0)).double() * s.double().repeat_interleave(group, 0))
+        Ad, pkd, sd, pzd = a.to(E4).to(dev), pk.to(dev), s.to(dev), pz.to(dev)
+        C = torch.full((M, N), -5.0, device=dev)
+        assert lib.mi355q_w4a8_gemm(Ad.data_ptr(), pkg.E4M3FN, K, pkd.data_ptr(), N // 8, sd.data_ptr(), pkg.BF16, pzd.data_ptr(), 0,
+                                    group, C.data_ptr(), pkg.F32, N, M, N, K, None, 1.0, pkg.GS_NONE, None, ws.data_ptr(), need,
+                                    stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.cpu().double(), expect), (M, N)
+        assert not ws[:1024].any()
 
 
 def test_meta_and_checks(dev):

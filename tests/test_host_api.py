@@ -50,7 +50,7 @@ def test_library_exports_every_declared_symbol(pkg):
     lib = pkg.capi()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.mi355q_abi_version() == 5
+    assert lib.mi355q_abi_version() == 6
     assert lib.mi355q_status_string(0) == b"ok"
     assert b"invalid" in lib.mi355q_status_string(1)
 
