@@ -1069,9 +1069,11 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
   if (q.is_meta())
     return SdpaOut(out, at::empty({1}, opts.dtype(stat_dt)), at::empty({1}, opts.dtype(linv_dt)), at::empty({1}, opts.dtype(at::kInt)),
                    at::empty({1}, opts.dtype(at::kFloat)), at::empty({1}, opts.dtype(at::kFloat)));
-  // the five one-element outputs (placeholders in inference, sdpa_gen.cpp:944-965) share one zeroed
-  // allocation: one fill instead of five
-  Tensor pool = at::zeros({40}, opts.dtype(at::kByte));
+  // The five one-element outputs share one allocation.  In inference m, linv and seed are dummies that the
+  // reference's kernel does not write either (sdpa_gen.cpp:949-965), and so are amax_s / amax_o when not asked
+  // for: they are not filled here (a fill is a launch of its own in front of every call); the amax words that
+  // are asked for are cleared by the C entry point.
+  Tensor pool = at::empty({40}, opts.dtype(at::kByte));
   auto one = [&](int slot, at::ScalarType t) { return pool.slice(0, 8 * slot, 8 * slot + (int64_t)c10::elementSize(t)).view(t); };
   Tensor m = one(0, stat_dt), linv = one(1, linv_dt), seed = one(2, at::kInt), amax_s = one(3, at::kFloat), amax_o = one(4, at::kFloat);
   DeviceGuard guard(q.device());
@@ -1096,11 +1098,16 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
     pr = at::nan_to_num(pr, 0.0);   // a row with every key masked
     out.copy_(at::matmul(pr.to(dt), v));
     if (pr.numel() > 0) amax_s.copy_(pr.max().reshape({1}));
+    else amax_s.zero_();
     if (out.numel() > 0) amax_o.copy_(out.to(at::kFloat).abs().max().reshape({1}));
+    else amax_o.zero_();
     return SdpaOut(out, m, linv, seed, amax_s, amax_o);
   }
 
-  if (out.numel() == 0) return SdpaOut(out, m, linv, seed, amax_s, amax_o);
+  if (out.numel() == 0) {
+    pool.zero_();  // an empty problem has maxima of zero
+    return SdpaOut(out, m, linv, seed, amax_s, amax_o);
+  }
   TORCH_CHECK(Dk <= 256 && Dv <= 256, "fp8_sdpa_recomp_fwd: head dimensions up to 256 are supported, got ", Dk, " and ", Dv);
   Tensor qc = sdpa_unit_rows(q), kc = sdpa_unit_rows(k), vc = sdpa_unit_rows(v);
   mi355q_sdpa_desc d{};
