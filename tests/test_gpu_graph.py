@@ -113,6 +113,53 @@ def test_graph_replays_of_the_reductions(dev):
             assert torch.equal(a.view(torch.uint8) if a.dtype == E4 else a, b.view(torch.uint8) if b.dtype == E4 else b), rep
 
 
+def decode_step(q, k, v, x8, pk, s, z):
+    """Attention for one query per head against a long cache (the keys split over workgroups, which meet through
+    arrival counters in a workspace) and a W4A8 product (without its split while a graph is captured)."""
+    o = ops.fp8_sdpa_recomp_fwd(q, k, v, None, 0.0, 128 ** -0.5, False, False, "None", None, None, None, None, None, None,
+                                False, False, None, "left")[0]
+    y = torch.ops.mi355q.w4a8_gemm(x8, pk, s, z, False, torch.bfloat16, None, None)
+    return o, y
+
+
+def test_graph_replays_of_a_decode_step(dev):
+    """The key split's counters live in a zero-filled tensor of the graph's own while capturing (the fill is a
+    kernel of the graph, so every replay starts from zero) and in the stream's kept workspace in eager runs: same
+    bits either way, replay after replay, with eager calls in between."""
+    g = torch.Generator().manual_seed(14)
+    B, G, HG, S, D = 1, 2, 4, 4096, 128
+    k = torch.randn(B, G, 1, S, D, generator=g).to(E4).to(dev)
+    v = torch.randn(B, G, 1, S, D, generator=g).to(E4).to(dev)
+    K, N = 4096, 512
+    pk = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), generator=g, dtype=torch.int64).to(torch.int32).to(dev)
+    s = (torch.rand(K // 128, N, generator=g) * 0.019 + 0.001).bfloat16().to(dev)
+    z = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 128, N // 8), generator=g, dtype=torch.int64).to(torch.int32).to(dev)
+    static_q = torch.randn(B, G, HG, 1, D, generator=g).to(E4).to(dev)
+    static_x = torch.randn(8, K, generator=g).to(E4).to(dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            decode_step(static_q, k, v, static_x, pk, s, z)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = decode_step(static_q, k, v, static_x, pk, s, z)
+    for rep in range(4):
+        q = (torch.randn(B, G, HG, 1, D, generator=g) * (rep + 1)).to(E4).to(dev)
+        x = torch.randn(8, K, generator=g).to(E4).to(dev)
+        static_q.copy_(q)
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        ref = decode_step(q, k, v, x, pk, s, z)
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], ref[0]), rep
+        # the W4A8 product adds its K parts in another order with the split (eager) than without (captured)
+        assert torch.allclose(got[1].float(), ref[1].float(), rtol=2 ** -6, atol=2 ** -6 * float(ref[1].float().abs().max())), rep
+
+
 def test_ops_follow_the_current_stream(oracle, dev):
     """Work is enqueued on torch's current stream (as the reference uses the current HPUStream,
     habana_eager/eager_exec.cpp:341), not on the default one: results are right when the inputs were
