@@ -259,6 +259,20 @@ def bench_ceilings(pkg, dev, steps, warmup):
                     f"{4 * wps} waves on each of {cus} CUs, register operands", "metric": "TFLOP/s",
                     "value": round(flop / (ms * 1e-3) / 1e12, 1), "unit": "TFLOP/s", "ms_per_call": round(ms, 5), "steps": max(steps, 20),
                     "implied_clock_ghz": round(per_wave * 64 / (ms * 1e-3) / 1e9 * wps, 3)})
+    # MFMAs and vector work side by side (what the attention kernel's softmax can hide under its MFMAs, and how)
+    passes = 4000
+    for name, wps, m0, m1, what in (
+            ("mfma_one_wave", 1, 1, 1, "four MFMAs per pass, one wave per SIMD"),
+            ("exp_one_wave", 1, 2, 2, "32 x (v_exp_f32, v_mul_f32) per pass, one wave per SIMD"),
+            ("mfma_and_exp_in_one_wave", 1, 3, 3, "both dealt out in turns in one wave per SIMD"),
+            ("mfma_two_waves", 2, 1, 1, "four MFMAs per pass and wave, two waves per SIMD"),
+            ("exp_two_waves", 2, 2, 2, "32 x (v_exp_f32, v_mul_f32) per pass and wave, two waves per SIMD"),
+            ("mfma_wave_beside_exp_wave", 2, 1, 2, "one wave per SIMD issues only the MFMAs, the other only the vector work"),
+            ("mfma_and_exp_in_both_waves", 2, 3, 3, "both dealt out in turns in each of two waves per SIMD")):
+        ms = time_gpu(lambda i: lib.mi355q_probe_coexec(wps, passes, m0, m1, cus, sink.data_ptr(), st), max(steps, 20), warmup)
+        out.append({"name": "coexec_" + name, "workload": what + f" ({passes} passes, {cus} workgroups, register operands)",
+                    "metric": "ns per pass", "value": round(ms * 1e6 / passes, 1), "unit": "ns", "ms_per_call": round(ms, 5),
+                    "steps": max(steps, 20)})
     for mib in (32, 128, 2048):
         nbytes = mib << 20
         sets = 1 if nbytes >= (1 << 30) else n_sets(nbytes)

@@ -34,6 +34,59 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(int pairs, float* sink)
   if (s == 123.456f) sink[0] = s;   // keeps the loop alive; practically never true
 }
 
+// MFMAs and vector instructions side by side, on register operands.  Per pass a wave issues four MFMAs (four
+// accumulators), 32 x (v_exp_f32, v_mul_f32) in eight independent chains, or both dealt out in turns (an MFMA, then
+// eight of the pairs), as its mode says: bit 0 the MFMAs, bit 1 the vector work.  Waves 0-3 of a workgroup (the
+// first wave of each SIMD) take mode_first, waves 4-7 (the second) mode_second.
+__global__ __launch_bounds__(512) void probe_coexec_kernel(int passes, int mode_first, int mode_second, float* sink) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int mode = wave >= 4 ? mode_second : mode_first;
+  probe_i32x8 a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = (int)(threadIdx.x * 0x01010101u + i * 0x11u) & 0x37373737;
+    b[i] = (int)(threadIdx.x * 0x03030303u + i * 0x07u) & 0x37373737;
+  }
+  probe_f32x16 acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+  float x[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) x[i] = 0.001f * (float)(threadIdx.x + i);
+  if (mode == 3) {
+    for (int it = 0; it < passes; ++it) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[j], 0, 0, 0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = __builtin_amdgcn_exp2f(x[i]) * 0.5f;
+      }
+    }
+  } else if (mode == 1) {
+    for (int it = 0; it < passes; ++it) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[j], 0, 0, 0, 0, 0, 0);
+    }
+  } else if (mode == 2) {
+    for (int it = 0; it < passes; ++it) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = __builtin_amdgcn_exp2f(x[i]) * 0.5f;
+    }
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += acc[j][r];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s += x[i];
+  if (s == 123.456f) sink[0] = s;   // keeps the loops alive; practically never true
+}
+
 // 16 bytes per lane, read only: the sum keeps the loads alive, one store per workgroup at most.
 __global__ __launch_bounds__(1024) void probe_read_kernel(const u32x4* __restrict__ x, int64_t n16, uint32_t* sink) {
   uint32_t acc = 0;
@@ -86,6 +139,15 @@ int mi355q_probe_mfma(int waves_per_simd, int mfma_per_wave, int workgroups, flo
     return MI355Q_ERR_INVALID_ARGUMENT;
   hipLaunchKernelGGL(probe_mfma_kernel, dim3((unsigned)workgroups), dim3(256u * waves_per_simd), 0, static_cast<hipStream_t>(stream),
                      mfma_per_wave / 2, sink);
+  return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
+}
+
+int mi355q_probe_coexec(int waves_per_simd, int passes, int mode_first, int mode_second, int workgroups, float* sink, void* stream) {
+  if ((waves_per_simd != 1 && waves_per_simd != 2) || passes <= 0 || workgroups <= 0 || sink == nullptr || mode_first < 0 ||
+      mode_first > 3 || mode_second < 0 || mode_second > 3)
+    return MI355Q_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(probe_coexec_kernel, dim3((unsigned)workgroups), dim3(256u * waves_per_simd), 0, static_cast<hipStream_t>(stream),
+                     passes, mode_first, mode_second, sink);
   return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
 }
 

@@ -404,6 +404,13 @@ int mi355q_probe_read(const void* x, int64_t bytes, int workgroups, void* sink, 
 int mi355q_probe_strip_read(const void* x, int64_t pitch, int64_t rows, int strip_bytes, int parts, int nontemporal,
                             void* sink, void* stream);
 
+/* mi355q_probe_coexec: how much of the MFMA time hides under vector work.  Per pass a wave issues four
+ * v_mfma_f32_32x32x64_f8f6f4 (mode bit 0), 32 x (v_exp_f32, v_mul_f32) in eight independent chains (bit 1),
+ * or both dealt out in turns (3); the first wave of each SIMD takes mode_first, the second (waves_per_simd
+ * = 2) mode_second.  Register operands only. */
+int mi355q_probe_coexec(int waves_per_simd, int passes, int mode_first, int mode_second, int workgroups, float* sink,
+                        void* stream);
+
 /* Name of the kernel variant mi355q_fp8_gemm would pick for a problem
  * (for logs and profiles; static string). */
 const char* mi355q_fp8_gemm_variant(int trans_a, int64_t lda, int trans_b, int64_t ldb,
