@@ -173,15 +173,36 @@ __global__ void sdpa_clear_amax_kernel(float* a, float* b) {
 // online-softmax update of (m_run, l_run, o), and O^T += V^T P^T from the V tile at vb.  qpos is the
 // lane's query position (for the causal comparison), mrow its row of the mask; `edge` says that some
 // score of the block may need masking (wave-uniform), otherwise the cheap path runs.
-template <int DKC, int DVT, int FMT>
+template <int DKC, int DVT, int FMT, bool QL = false>
 __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb, const uint8_t* vb, int kv0, bool edge, int qpos,
                                            bool q_ok, const uint8_t* mrow, const i32x8 (&qf)[DKC], float sc2, float lqs, bool clamp_p,
-                                           f32x16 (&o)[DVT], float& m_run, float& l_run) {
+                                           f32x16 (&o)[DVT], float& m_run, float& l_run, const uint8_t* qbase = nullptr) {
   constexpr int KROW = DKC * 64;
   constexpr int kVRow = DVT <= 4 ? 128 : 256;
   constexpr float kMax8 = FMT == MI355Q_E5M2 ? 57344.0f : 448.0f;
   const int lane = threadIdx.x & 63, lq = lane & 31, h = lane >> 5;
   f32x16 s[2];
+  if constexpr (QL) {
+    // the query fragments come from LDS, one depth step at a time (registers for a third wave per SIMD)
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[t][r] = 0.0f;
+#pragma unroll
+    for (int c = 0; c < DKC; ++c) {
+      const u32x4 qlo = *reinterpret_cast<const u32x4*>(qbase + (c * 2) * 1024);
+      const u32x4 qhi = *reinterpret_cast<const u32x4*>(qbase + (c * 2 + 1) * 1024);
+      const i32x8 q = {(int)qlo[0], (int)qlo[1], (int)qlo[2], (int)qlo[3], (int)qhi[0], (int)qhi[1], (int)qhi[2], (int)qhi[3]};
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int row = 32 * t + lq;
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(kb + k_lds_offset<KROW>(row, c * 4 + h * 2));
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(kb + k_lds_offset<KROW>(row, c * 4 + h * 2 + 1));
+        const i32x8 kf = {(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+        s[t] = sdpa_mfma<FMT>(kf, q, s[t]);
+      }
+    }
+  } else {
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
 #pragma unroll
@@ -195,13 +216,14 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
       s[t] = sdpa_mfma<FMT>(kf, qf[c], s[t]);
     }
   }
+  }
 
   // The V fragments do not depend on the scores: for up to four tiles their LDS reads go out here, under the
   // score MFMAs and the softmax, instead of one tile at a time in front of each P V product (where the wave
   // would wait for LDS four times with the matrix pipe idle).
   const int g = lane >> 4, gi = lane & 15;
   const int r8 = gi >> 1, hh = gi & 1;
-  constexpr bool kEarlyV = DVT <= 4;
+  constexpr bool kEarlyV = DVT <= 4 && !QL;
   i32x8 vfe[kEarlyV ? DVT : 1];
   if constexpr (kEarlyV) {
 #pragma unroll
@@ -328,6 +350,13 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
   }
 }
 
+// Head dimension 128 with direct loads: the query fragments live in LDS instead of 16 registers and the ring has
+// two stages instead of four, which brings a workgroup to 161 registers and 48 KB of LDS, so that three
+// workgroups fit a CU (three waves per SIMD).  A wave alone needs about 3500 cycles for a block of 64 keys (a
+// chain of LDS reads, MFMAs, the softmax and MFMAs again) of which 1200 are vector work and 512 MFMA time, so a
+// SIMD is as busy as it has waves to switch between.
+constexpr bool sdpa_q_in_lds(int dkc, int dvt, bool dma) { return dma && dkc == 2 && dvt == 4; }
+
 // DKC: 64-byte steps of the q.k depth (head_dim_qk <= 64 DKC); DVT: 32-column tiles of v
 // (head_dim_v <= 32 DVT).
 // DMA: K and V blocks go from global memory straight into LDS (aligned tensors), a ring of kStages blocks;
@@ -336,7 +365,8 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
 // puts there (vmcnt(0), in front of the first MFMA of every block) also waits for the blocks just requested
 // by the direct route.
 template <int DKC, int DVT, int FMT, bool DMA>
-__global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd_kernel(const SdpaArgs a) {
+__global__ __launch_bounds__(kSdpaThreads, (sdpa_q_in_lds(DKC, DVT, DMA) ? 3 : DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd_kernel(const SdpaArgs a) {
+  constexpr bool kQLds = sdpa_q_in_lds(DKC, DVT, DMA);
   constexpr int KROW = DKC * 64;
   constexpr int kVRow = DVT <= 4 ? 128 : 256;  // bytes of an LDS row of V
   constexpr int KCPR = KROW / 16;           // chunks per K row
@@ -347,9 +377,11 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
   constexpr int VLOADS = kSdpaBN * VCPR / kSdpaThreads;
   static_assert(KLOADS >= 1 && VLOADS >= 1, "block too small for the workgroup");
   // Direct loads run kStages - 1 blocks ahead of the arithmetic (a block's arithmetic takes about a
-  // microsecond, less than a load from HBM under load); the route through registers uses two buffers.
-  constexpr int kStages = 4;
+  // microsecond, less than a load from HBM under load; with the queries in LDS one block ahead, which the
+  // third workgroup on the CU covers); the route through registers uses two buffers.
+  constexpr int kStages = kQLds ? 2 : 4;
   __shared__ __align__(1024) uint8_t lds[kStages * (KBYTES + VBYTES)];
+  __shared__ __align__(16) uint8_t qlds[kQLds ? 4 * 4096 : 16];  // per wave: [depth chunk of 16 bytes][half-wave][row]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in every lane, and known to be
@@ -406,6 +438,16 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
 #pragma unroll
   for (int c = 0; c < DKC; ++c) asm volatile("" : : "v"(qf[c]));
 #endif
+  const uint8_t* qbase = qlds + (kQLds ? wave * 4096 + h * 512 + lq * 16 : 0);
+  if constexpr (kQLds) {
+#pragma unroll
+    for (int c = 0; c < DKC; ++c) {
+      *reinterpret_cast<u32x4*>(qlds + wave * 4096 + (c * 2) * 1024 + h * 512 + lq * 16) =
+          u32x4{(uint32_t)qf[c][0], (uint32_t)qf[c][1], (uint32_t)qf[c][2], (uint32_t)qf[c][3]};
+      *reinterpret_cast<u32x4*>(qlds + wave * 4096 + (c * 2 + 1) * 1024 + h * 512 + lq * 16) =
+          u32x4{(uint32_t)qf[c][4], (uint32_t)qf[c][5], (uint32_t)qf[c][6], (uint32_t)qf[c][7]};
+    }
+  }
 
   int nblk = (a.S + kSdpaBN - 1) / kSdpaBN;
   if (a.causal) {
@@ -522,7 +564,7 @@ __global__ __launch_bounds__(kSdpaThreads, (DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd
     const bool active = !(a.causal && kv0 > wq0 + 31);
     if (active) {
       const bool edge = (a.causal && kv0 + kSdpaBN - 1 > wq0) || kv0 + kSdpaBN > a.S || a.mask_kind != kMaskNone;
-      sdpa_block<DKC, DVT, FMT>(a, kb, vb, kv0, edge, qrow, q_ok, mrow, qf, sc2, lqs, clamp_p, o, m_run, l_run);
+      sdpa_block<DKC, DVT, FMT, kQLds>(a, kb, vb, kv0, edge, qrow, q_ok, mrow, qf, sc2, lqs, clamp_p, o, m_run, l_run, qbase);
     }
 
     if constexpr (DMA) {
