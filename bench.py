@@ -58,8 +58,8 @@ MEASURED_TRAFFIC = {
     "w4a8_gemm_M32": 140.24e6,
     "w4a8_gemm_M64": 159.36e6,
     "w4a8_gemm_M256": 284.69e6,     # four row blocks of 64 stream the weights; the caches catch half of it
-    "fp8_sdpa_B1_L8192": 127.62e6,
-    "fp8_sdpa_B4_L4096": 235.35e6,
+    "fp8_sdpa_B1_L8192": 124.23e6,
+    "fp8_sdpa_B4_L4096": 235.55e6,
     "fp8_sdpa_decode_B64_S4096": 537.35e6,
     "fp8_sdpa_decode_B8_S8192": 143.14e6,   # fp8_sdpa_decode_kernel 138.75 + fp8_sdpa_decode_merge_kernel 4.39
     "softmax_fp8": 1609.30e6,
