@@ -208,9 +208,10 @@ def test_grouped_query_layout(oracle, dev):
     check_bf16(out, ref)
 
 
-def test_e5m2_inputs(oracle, dev):
-    gen = torch.Generator().manual_seed(10)
-    q, k, v = make_qkv(gen, (2, 2, 100, 64), (2, 2, 140, 64), (2, 2, 140, 64), fmt=E5)
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_e5m2_inputs(oracle, dev, D):
+    gen = torch.Generator().manual_seed(10 + D)
+    q, k, v = make_qkv(gen, (2, 2, 100, D), (2, 2, 140, D), (2, 2, 140, D), fmt=E5)
     out = run_op(dev, q, k, v, causal=True, scales=(None, None, None, 1024.0, None, 1 / 1024.0))[0]
     ref, _, _ = oracle.torch_fp8_sdpa(q, k, v, is_causal=True, q_scale_s=1024.0, d_scale_s=1 / 1024.0)
     # e5m2 probabilities have a 2-bit mantissa: one flipped rounding weighs four times an e4m3 one
@@ -218,9 +219,10 @@ def test_e5m2_inputs(oracle, dev):
     assert ((out - ref).abs() <= ref.abs() * 2.0 ** -7 + 1.5e-2 * ref.abs().max()).all()
 
 
-def test_q_scale_s_beyond_the_fp8_range_saturates(oracle, dev):
+@pytest.mark.parametrize("D", [64, 128])
+def test_q_scale_s_beyond_the_fp8_range_saturates(oracle, dev, D):
     gen = torch.Generator().manual_seed(11)
-    q, k, v = make_qkv(gen, (1, 2, 64, 64), (1, 2, 64, 64), (1, 2, 64, 64), spread=3.0)
+    q, k, v = make_qkv(gen, (1, 2, 64, D), (1, 2, 64, D), (1, 2, 64, D), spread=3.0)
     out = run_op(dev, q, k, v, scales=(None, None, None, 1000.0, None, 1e-3))[0]
     ref, _, _ = oracle.torch_fp8_sdpa(q, k, v, q_scale_s=1000.0, d_scale_s=1e-3)
     check_bf16(out, ref)
