@@ -70,6 +70,20 @@ MEASURED_TRAFFIC = {
 
 RAMP_SECONDS = 0.15
 
+# --only tokens: a group name runs the whole group, group_case one workload of it (one profile row per workload)
+GROUPS = ("gemm", "cast", "castlarge", "int4", "decode", "mlp", "reduce", "w4a8", "w4a16", "sdpa", "ceilings")
+DEFAULT_GROUPS = tuple(g for g in GROUPS if g != "ceilings")   # the probes run on request only
+WHICH = set()
+
+
+def want(group, case=None):
+    """True when --only names the group, or this case of it (e.g. w4a8_M256, sdpa_B1, sdpa_decode_B8, decode_M64)."""
+    if group in WHICH:
+        return True
+    if case is None:
+        return any(t.startswith(group + "_") for t in WHICH)
+    return f"{group}_{case}" in WHICH
+
 
 def time_gpu(fn, steps, warmup):
     """Average milliseconds per call of fn(i), HIP events on the current stream.
@@ -118,13 +132,18 @@ def time_cpu(fn, min_seconds=3.0, max_runs=5):
     return ts[len(ts) // 2]
 
 
-def hbm_entry(name, workload, bytes_per_call, ms, steps, kernel, cpu=None, extra=None):
+def hbm_entry(name, workload, bytes_per_call, ms, steps, kernel, cpu=None, extra=None, ceiling=None):
+    """ceiling: GB/s of a plain 16-byte copy moving the same number of bytes in the same run (what a streaming
+    kernel of this size can reach on this machine; reported beside the published peak, never instead of it)."""
     gbs = bytes_per_call / (ms * 1e-3) / 1e9
     e = {"name": name, "workload": workload, "metric": "GB/s", "value": round(gbs, 1), "unit": "GB/s",
          "ms_per_call": round(ms, 5), "steps": steps,
          "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                       "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                       "algorithmic_bytes": bytes_per_call, "traffic": MEASURED_TRAFFIC.get(name)}}
+    if ceiling is not None:
+        e["roofline"]["ceiling_same_size"] = {"what": "plain copy of the same number of bytes (read + written), same run",
+                                              "GB/s": round(ceiling, 1), "frac_of_peak": round(ceiling / HBM_PEAK_GBS, 4)}
     if cpu is not None:
         e["cpu_baseline"] = cpu
     if extra:
@@ -177,6 +196,16 @@ def bench_cast(pkg, oracle, dev, steps, warmup, cpu, c1=True, large=True):
     if not c1:
         del xs, y8, yb
         return out + bench_cast_large(lib, pkg, gen, dev, sd, st, ok, steps)
+
+    def copy_rate(total_bytes):
+        # the library's 16-byte copy kernel moving total_bytes (half read, half written) between the same rotating buffers
+        half = total_bytes // 2
+        t = time_gpu(lambda i: ok(lib.mi355q_cast_to_fp8(xs[i % sets].data_ptr(), pkg.E4M3FN, yb[i % sets].data_ptr(), pkg.E4M3FN,
+                                                         None, 0.0, pkg.SCALE_NONE, half, 1, 1, None, st)), steps, warmup)
+        return total_bytes / (t * 1e-3) / 1e9
+
+    ceil_48 = copy_rate(3 * n)     # the casts move 48 MiB
+    ceil_32 = copy_rate(2 * n)     # the amax pass reads 32 MiB
     ms = time_gpu(lambda i: ok(lib.mi355q_amax(xs[i % sets].data_ptr(), pkg.BF16, n, am.data_ptr(), st)), steps, warmup)
     assert am.cpu() == amax
     c = None
@@ -184,7 +213,7 @@ def bench_cast(pkg, oracle, dev, steps, warmup, cpu, c1=True, large=True):
         t = time_cpu(lambda: x.abs().max().float())
         c = {"value": round(2 * n / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
              "sample": "full 4096x4096 bf16 tensor, x.abs().max()"}
-    out.append(hbm_entry("amax", "C1a amax of bf16 [4096,4096]", 2 * n, ms, steps, "fill_u32 + amax_vec<bf16>", c))
+    out.append(hbm_entry("amax", "C1a amax of bf16 [4096,4096]", 2 * n, ms, steps, "amax_vec<bf16>", c, ceiling=ceil_32))
 
     def cast_to(i, with_amax):
         j = i % sets
@@ -198,11 +227,11 @@ def bench_cast(pkg, oracle, dev, steps, warmup, cpu, c1=True, large=True):
         c = {"value": round(3 * n / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
              "sample": "full 4096x4096 bf16 tensor, (x*s.to(bf16)).clamp(-448,448).to(float8_e4m3fn)"}
     out.append(hbm_entry("cast_to_fp8_v2", "C1b cast_to_fp8_v2 bf16 [4096,4096] -> e4m3fn, per-tensor scale",
-                         3 * n, ms, steps, "cast_to_fp8_vec8<bf16,e4m3fn,scalar>", c))
+                         3 * n, ms, steps, "cast_to_fp8_vec8<bf16,e4m3fn,scalar>", c, ceiling=ceil_48))
 
     ms = time_gpu(lambda i: cast_to(i, True), steps, warmup)
     out.append(hbm_entry("cast_to_fp8_v2+amax", "C1 cast_to_fp8_v2 with is_amax=True (one pass)", 3 * n + 4, ms, steps,
-                         "fill_u32 + cast_to_fp8_vec8<bf16,e4m3fn,scalar,amax>"))
+                         "cast_to_fp8_vec8<bf16,e4m3fn,scalar,amax>", ceiling=ceil_48))
 
     ms = time_gpu(lambda i: ok(lib.mi355q_cast_from_fp8(y8[i % sets].data_ptr(), pkg.E4M3FN, yb[i % sets].data_ptr(),
                                                         pkg.BF16, sinv.data_ptr(), 0.0, pkg.SCALE_DEV, n, 1, 1, st)),
@@ -214,7 +243,7 @@ def bench_cast(pkg, oracle, dev, steps, warmup, cpu, c1=True, large=True):
         c = {"value": round(3 * n / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
              "sample": "full 4096x4096 e4m3fn tensor, x8.to(bf16) * s_inv.to(bf16)"}
     out.append(hbm_entry("cast_from_fp8", "C1c cast_from_fp8 e4m3fn [4096,4096] -> bf16", 3 * n, ms, steps,
-                         "cast_from_fp8_vec<e4m3fn,bf16,scalar>", c))
+                         "cast_from_fp8_vec<e4m3fn,bf16,scalar>", c, ceiling=ceil_48))
     # fp8 -> fp8 is a plain copy (the reference forwards an fp8 input unchanged): the copy
     # kernel of known size that hardware byte counters are calibrated against
     ms = time_gpu(lambda i: ok(lib.mi355q_cast_to_fp8(y8[i % sets].data_ptr(), pkg.E4M3FN, yb[i % sets].data_ptr(),
@@ -247,13 +276,14 @@ def bench_ceilings(pkg, dev, steps, warmup):
     buffers to exceed the Infinity Cache).  Reference points for the roofline fractions, not workloads."""
     import ctypes
     lib = pkg.capi()
+    probe = pkg.probes()     # libmi355q_probe.so: measurement kernels, not part of the product library
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     sink = torch.zeros(16, device=dev)
     out = []
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     for wps in (1, 2):
         per_wave = 4000
-        ms = time_gpu(lambda i: lib.mi355q_probe_mfma(wps, per_wave, cus, sink.data_ptr(), st), max(steps, 20), warmup)
+        ms = time_gpu(lambda i: probe.mi355q_probe_mfma(wps, per_wave, cus, sink.data_ptr(), st), max(steps, 20), warmup)
         flop = 131072.0 * per_wave * 4 * wps * cus
         out.append({"name": f"ceiling_mfma_fp8_{wps}_wave_per_simd", "workload": f"{per_wave} back-to-back v_mfma_f32_32x32x64_f8f6f4 per wave, "
                     f"{4 * wps} waves on each of {cus} CUs, register operands", "metric": "TFLOP/s",
@@ -269,7 +299,7 @@ def bench_ceilings(pkg, dev, steps, warmup):
             ("exp_two_waves", 2, 2, 2, "32 x (v_exp_f32, v_mul_f32) per pass and wave, two waves per SIMD"),
             ("mfma_wave_beside_exp_wave", 2, 1, 2, "one wave per SIMD issues only the MFMAs, the other only the vector work"),
             ("mfma_and_exp_in_both_waves", 2, 3, 3, "both dealt out in turns in each of two waves per SIMD")):
-        ms = time_gpu(lambda i: lib.mi355q_probe_coexec(wps, passes, m0, m1, cus, sink.data_ptr(), st), max(steps, 20), warmup)
+        ms = time_gpu(lambda i: probe.mi355q_probe_coexec(wps, passes, m0, m1, cus, sink.data_ptr(), st), max(steps, 20), warmup)
         out.append({"name": "coexec_" + name, "workload": what + f" ({passes} passes, {cus} workgroups, register operands)",
                     "metric": "ns per pass", "value": round(ms * 1e6 / passes, 1), "unit": "ns", "ms_per_call": round(ms, 5),
                     "steps": max(steps, 20)})
@@ -278,7 +308,7 @@ def bench_ceilings(pkg, dev, steps, warmup):
         sets = 1 if nbytes >= (1 << 30) else n_sets(nbytes)
         bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev).view(E4) for _ in range(sets)]
         k = max(steps, 20) if mib < 2048 else 5
-        ms = time_gpu(lambda i: lib.mi355q_probe_read(bufs[i % sets].data_ptr(), nbytes, 2 * cus, sink.data_ptr(), st), k, warmup)
+        ms = time_gpu(lambda i: probe.mi355q_probe_read(bufs[i % sets].data_ptr(), nbytes, 2 * cus, sink.data_ptr(), st), k, warmup)
         out.append(hbm_entry(f"ceiling_read_{mib}MiB", f"read-only stream over {mib} MiB, 16-byte loads, nothing stored", nbytes, ms, k, "probe_read_kernel"))
         half = nbytes // 2
         dst = [torch.empty(half, dtype=E4, device=dev) for _ in range(min(sets, 4))]
@@ -293,7 +323,7 @@ def bench_ceilings(pkg, dev, steps, warmup):
     bufs = [torch.randint(0, 255, (rows * pitch,), dtype=torch.uint8, device=dev) for _ in range(sets)]
     for strip, parts, nt in ((64, 1, 1), (128, 1, 0), (128, 1, 1), (256, 2, 1)):
         k = max(steps, 20)
-        ms = time_gpu(lambda i: lib.mi355q_probe_strip_read(bufs[i % sets].data_ptr(), pitch, rows, strip, parts, nt, sink.data_ptr(), st), k, warmup)
+        ms = time_gpu(lambda i: probe.mi355q_probe_strip_read(bufs[i % sets].data_ptr(), pitch, rows, strip, parts, nt, sink.data_ptr(), st), k, warmup)
         out.append(hbm_entry(f"ceiling_strip_read_{strip}B" + ("_nt" if nt else "") + (f"_K{parts}" if parts > 1 else ""),
                              f"[{rows}, {pitch}] bytes read in strips of {strip} bytes per row, {pitch // strip * parts} workgroups"
                              + (f", the rows in {parts} ranges" if parts > 1 else "") + (", nontemporal loads" if nt else ""),
@@ -454,6 +484,8 @@ def bench_gemm_decode(ops, oracle, dev, steps, warmup):
     for M in (16, 64, 256):
         x = torch.randn(M, K, generator=gen)
         x[:, cols] *= 20
+        if not want("decode", f"M{M}"):
+            continue
         x = x.bfloat16().to(dev)
         x8, sx_inv = torch.ops.mi355q.quantize_rows(x, E4)   # per-token amax, scale = 448 / amax, cast
         ms = time_gpu(lambda i: ops.fp8_gemm_v2(x8, False, w8s[i % 2], False, None, torch.bfloat16, sx_inv, sw_inv,
@@ -491,6 +523,8 @@ def bench_w4a8(oracle, dev, steps, warmup, cpu):
     for M in (16, 32, 64, 256):
         x = torch.randn(M, K, generator=gen)
         x[:, cols] *= 20
+        if not want("w4a8", f"M{M}"):
+            continue
         x8, sx_inv = torch.ops.mi355q.quantize_rows(x.bfloat16().to(dev), E4)
         ms = time_gpu(lambda i: torch.ops.mi355q.w4a8_gemm(x8, packs[i % 3], scale, zp, False, torch.bfloat16, sx_inv, None),
                       steps, warmup)
@@ -519,6 +553,8 @@ def bench_sdpa(oracle, dev, steps, warmup, cpu):
     H, HK, D = 32, 8, 128
     sc = 1.0 / math.sqrt(D)
     for B, L in ((1, 8192), (4, 4096)):
+        if not want("sdpa", f"B{B}"):
+            continue
         q = torch.randn(B, HK, H // HK, L, D, generator=gen).to(E4).to(dev)     # the grouped-query view of [B, H, L, D]
         k = torch.randn(B, HK, 1, L, D, generator=gen).to(E4).to(dev)
         v = torch.randn(B, HK, 1, L, D, generator=gen).to(E4).to(dev)
@@ -542,6 +578,8 @@ def bench_sdpa(oracle, dev, steps, warmup, cpu):
         out.append(e)
     # decoding: one query per head against a long cache; bound by reading k and v once
     for B, S in ((64, 4096), (8, 8192)):
+        if not want("sdpa", f"decode_B{B}"):
+            continue
         q = torch.randn(B, HK, H // HK, 1, D, generator=gen).to(E4).to(dev)
         sets = n_sets(2 * B * HK * S * D)
         ks = [torch.randn(B, HK, 1, S, D, generator=gen).to(E4).to(dev) for _ in range(sets)]
@@ -626,7 +664,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,cast,castlarge,int4,decode,mlp,reduce,w4a8,sdpa,ceilings")
+    ap.add_argument("--only", type=str, default="",
+                    help="comma list of groups (gemm,cast,castlarge,int4,decode,mlp,reduce,w4a8,w4a16,sdpa,ceilings) or single workloads "
+                         "(decode_M16|M64|M256, w4a8_M16|M32|M64|M256, w4a16_M16|M64|M256, sdpa_B1|B4|decode_B64|decode_B8); "
+                         "default: every group but ceilings (the measurement probes)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -643,28 +684,36 @@ def main():
     ops = torch.ops.hpu
     dev = torch.device("cuda:0")
     torch.set_num_threads(min(os.cpu_count() or 1, 16))
-    which = set(args.only.split(",")) if args.only else {"gemm", "cast", "castlarge", "int4", "decode", "mlp", "reduce", "w4a8", "sdpa", "ceilings"}
+    WHICH.update(args.only.split(",") if args.only else DEFAULT_GROUPS)
+    for t in WHICH:
+        if t.split("_")[0] not in GROUPS:
+            ap.error(f"--only: unknown workload {t!r}")
+    which = {g for g in GROUPS if want(g)}
     cpu = not args.no_cpu
     k_stream = max(args.steps, 50)      # the microsecond-scale kernels need more calls for a stable mean
     w_stream = max(args.warmup, 10)
 
+    # Rows beyond the five benchmark configurations come first and C5, C4, C2, C1 last: a log that keeps
+    # only the end of this long line keeps the configurations.
     ops_out = []
-    if "cast" in which or "castlarge" in which:
-        ops_out += bench_cast(pkg, oracle, dev, k_stream, w_stream, cpu, c1="cast" in which, large="castlarge" in which)
-    if "int4" in which:
-        ops_out += bench_int4(pkg, oracle, dev, k_stream, w_stream, cpu)
-    if "decode" in which:
-        ops_out += bench_gemm_decode(ops, oracle, dev, args.steps, args.warmup)
-    if "mlp" in which:
-        ops_out.append(bench_mlp(ops, dev, max(args.steps // 2, 5), args.warmup))
-    if "reduce" in which:
-        ops_out += bench_reductions(pkg, oracle, dev, args.steps, args.warmup, cpu)
-    if "w4a8" in which:
-        ops_out += bench_w4a8(oracle, dev, args.steps, args.warmup, cpu)
-    if "sdpa" in which:
-        ops_out += bench_sdpa(oracle, dev, args.steps, args.warmup, cpu)
     if "ceilings" in which:
         ops_out += bench_ceilings(pkg, dev, args.steps, args.warmup)
+    if "reduce" in which:
+        ops_out += bench_reductions(pkg, oracle, dev, args.steps, args.warmup, cpu)
+    if "sdpa" in which:
+        ops_out += bench_sdpa(oracle, dev, args.steps, args.warmup, cpu)
+    if "w4a16" in which:
+        ops_out += bench_w4a16(oracle, dev, args.steps, args.warmup, cpu)
+    if "w4a8" in which:
+        ops_out += bench_w4a8(oracle, dev, args.steps, args.warmup, cpu)
+    if "mlp" in which:
+        ops_out.append(bench_mlp(ops, dev, max(args.steps // 2, 5), args.warmup))
+    if "decode" in which:
+        ops_out += bench_gemm_decode(ops, oracle, dev, args.steps, args.warmup)
+    if "int4" in which:
+        ops_out += bench_int4(pkg, oracle, dev, k_stream, w_stream, cpu)
+    if "cast" in which or "castlarge" in which:
+        ops_out += bench_cast(pkg, oracle, dev, k_stream, w_stream, cpu, c1="cast" in which, large="castlarge" in which)
 
     line = {"metric": "cast/dequant GB/s (% HBM peak); fp8_gemm_v2 TFLOP/s (% fp8 MFMA peak)",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True,
@@ -696,6 +745,8 @@ def main():
         if "cpu_baseline" in first:
             line["cpu_baseline"] = first["cpu_baseline"]
     line["ops"] = ops_out
+    # every entry once more in short form, last in the line: name -> [value, unit, fraction of the published peak]
+    line["summary"] = {e["name"]: [e["value"], e["unit"], e.get("roofline", {}).get("frac")] for e in ops_out}
     print(json.dumps(line))
 
 

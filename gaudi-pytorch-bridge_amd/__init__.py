@@ -81,16 +81,30 @@ def capi():
     L.mi355q_fp8_sdpa_workspace_bytes.restype = c.c_size_t
     L.mi355q_fp8_sdpa_key_splits.argtypes = [vp, vp]
     L.mi355q_fp8_sdpa_key_splits.restype = i32
-    L.mi355q_probe_mfma.argtypes = [i32, i32, i32, vp, vp]
-    L.mi355q_probe_read.argtypes = [vp, i64, i32, vp, vp]
-    L.mi355q_probe_coexec.argtypes = [i32, i32, i32, i32, i32, vp, vp]
-    L.mi355q_probe_strip_read.argtypes = [vp, i64, i64, i32, i32, i32, vp, vp]
     L.mi355q_fp8_gemm_variant.restype = c.c_char_p
     for name in ("mi355q_amax", "mi355q_rowwise_amax", "mi355q_quantize_rows", "mi355q_silu_mul_quantize_rows", "mi355q_cast_to_fp8", "mi355q_cast_to_fp8_sr", "mi355q_cast_to_fp8_hybrid", "mi355q_cast_from_fp8",
-                 "mi355q_dequant_4bit", "mi355q_fp8_gemm", "mi355q_w4a8_gemm", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8", "mi355q_fp8_sdpa_fwd", "mi355q_probe_mfma", "mi355q_probe_read", "mi355q_probe_strip_read", "mi355q_probe_coexec"):
+                 "mi355q_dequant_4bit", "mi355q_fp8_gemm", "mi355q_w4a8_gemm", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8", "mi355q_fp8_sdpa_fwd"):
         getattr(L, name).restype = i32
     L._typed = True
     return L
+
+
+def probes():
+    """ctypes handle of libmi355q_probe.so: measurement kernels for ``bench.py --only ceilings``
+    (csrc/bench/probe_kernels.hip); not part of the product ABI, loaded on request only."""
+    path = os.path.join(_HERE, "libmi355q_probe.so")
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: build it with `python {os.path.join(_HERE, 'build.py')}`")
+    c = ctypes
+    i64, vp, i32 = c.c_int64, c.c_void_p, c.c_int
+    P = c.CDLL(path)
+    P.mi355q_probe_mfma.argtypes = [i32, i32, i32, vp, vp]
+    P.mi355q_probe_read.argtypes = [vp, i64, i32, vp, vp]
+    P.mi355q_probe_coexec.argtypes = [i32, i32, i32, i32, i32, vp, vp]
+    P.mi355q_probe_strip_read.argtypes = [vp, i64, i64, i32, i32, i32, vp, vp]
+    for name in ("mi355q_probe_mfma", "mi355q_probe_read", "mi355q_probe_strip_read", "mi355q_probe_coexec"):
+        getattr(P, name).restype = i32
+    return P
 
 
 # enums of include/mi355q.h
@@ -104,7 +118,7 @@ SDPA_MASK_NONE, SDPA_MASK_BOOL, SDPA_MASK_BF16, SDPA_MASK_F32 = 0, 1, 2, 3
 EXPORTED_SYMBOLS = (
     "mi355q_abi_version", "mi355q_status_string", "mi355q_amax", "mi355q_rowwise_amax",
     "mi355q_quantize_rows", "mi355q_silu_mul_quantize_rows", "mi355q_cast_to_fp8", "mi355q_cast_to_fp8_sr", "mi355q_cast_to_fp8_hybrid", "mi355q_cast_from_fp8", "mi355q_dequant_4bit", "mi355q_fp8_gemm",
-    "mi355q_w4a8_gemm", "mi355q_w4a8_gemm_workspace_bytes", "mi355q_fp8_gemm_variant", "mi355q_sum_fp8_workspace_bytes", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8", "mi355q_fp8_sdpa_fwd", "mi355q_fp8_sdpa_workspace_bytes", "mi355q_fp8_sdpa_key_splits", "mi355q_probe_mfma", "mi355q_probe_read", "mi355q_probe_strip_read", "mi355q_probe_coexec",
+    "mi355q_w4a8_gemm", "mi355q_w4a8_gemm_workspace_bytes", "mi355q_fp8_gemm_variant", "mi355q_sum_fp8_workspace_bytes", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8", "mi355q_fp8_sdpa_fwd", "mi355q_fp8_sdpa_workspace_bytes", "mi355q_fp8_sdpa_key_splits",
 )
 
 _load()

@@ -4,6 +4,8 @@
                    (hipcc, no torch dependency)
   mi355q_torch.so  TORCH_LIBRARY(hpu) host layer that calls the C ABI
                    (g++ against the installed PyTorch-ROCm)
+  libmi355q_probe.so  measurement probes (csrc/bench/), loaded by
+                   ``bench.py --only ceilings`` alone; not part of the product ABI
 
 Run as ``python gaudi-pytorch-bridge_amd/build.py`` or call ``build()``.
 """
@@ -17,8 +19,9 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB_KERNELS = os.path.join(HERE, "libmi355q.so")
 LIB_TORCH = os.path.join(HERE, "mi355q_torch.so")
+LIB_PROBE = os.path.join(HERE, "libmi355q_probe.so")
 
-HIP_SOURCES = ["cast_kernels.hip", "int4_kernels.hip", "reduce_kernels.hip", "gemm_api.hip", "gemm_inst_kk.hip", "gemm_inst_km.hip", "gemm_inst_mk.hip", "gemm_inst_mm.hip", "w4_gemm.hip", "sdpa_kernels.hip", "probe_kernels.hip", "api.cpp"]
+HIP_SOURCES = ["cast_kernels.hip", "int4_kernels.hip", "reduce_kernels.hip", "gemm_api.hip", "gemm_inst_kk.hip", "gemm_inst_km.hip", "gemm_inst_mk.hip", "gemm_inst_mm.hip", "w4_gemm.hip", "sdpa_kernels.hip", "api.cpp"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -56,6 +59,12 @@ def build_kernels(verbose=False, jobs=8):
     return LIB_KERNELS
 
 
+def build_probes(verbose=False):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    _run([hipcc] + HIPCC_FLAGS + ["-shared", "-x", "hip", os.path.join(CSRC, "bench", "probe_kernels.hip"), "-o", LIB_PROBE], verbose)
+    return LIB_PROBE
+
+
 def build_torch_ext(verbose=False):
     import torch
     from torch.utils import cpp_extension as ce
@@ -79,7 +88,9 @@ def build_torch_ext(verbose=False):
 def build(verbose=False, jobs=8):
     with ThreadPoolExecutor(max_workers=2) as ex:
         k = ex.submit(build_kernels, verbose, jobs)
+        p = ex.submit(build_probes, verbose)
         k.result()
+        p.result()
     build_torch_ext(verbose)
     return LIB_KERNELS, LIB_TORCH
 

@@ -3,7 +3,7 @@
 
 extern "C" {
 
-int mi355q_abi_version(void) { return 6; }
+int mi355q_abi_version(void) { return 7; }
 
 const char* mi355q_status_string(int status) {
   switch (status) {

@@ -1,8 +1,23 @@
-// Measurement aids: what this GPU sustains with nothing in the way.  bench.py times them in the
-// same run as the kernels they bound, so that a roofline fraction can be read against the
-// machine's real ceiling (clocks under load, HBM rate at a given size) as well as against the
-// published peak.  No part of the product path calls these.
-#include "device_common.h"
+// Measurement aids: what this GPU sustains with nothing in the way.  They are built into a library
+// of their own (libmi355q_probe.so), which only `bench.py --only ceilings` loads: the product library
+// and its header export none of this.  Timed in the same run as the kernels they bound, they let a
+// roofline fraction be read against the machine's real ceiling (clocks under load, HBM rate at a given
+// size) as well as against the published peak.
+//
+//   mi355q_probe_mfma        `workgroups` workgroups of 4 * waves_per_simd waves (1 or 2 per SIMD), each wave
+//                            issuing mfma_per_wave back-to-back v_mfma_f32_32x32x64_f8f6f4 (131072 flop each)
+//                            on register operands: the fp8 MFMA rate at the clock the GPU holds under load
+//   mi355q_probe_read        reads `bytes` bytes (a multiple of 16, 16-byte aligned) with 16-byte loads and
+//                            stores nothing: the HBM read rate at that size
+//   mi355q_probe_strip_read  reads a row-major byte matrix [rows, pitch] the way the decode-shaped GEMMs read
+//                            their weights: pitch / strip_bytes strips (64, 128 or 256 bytes of every row), the
+//                            rows of a strip cut into `parts` ranges, one workgroup per strip and range
+//   mi355q_probe_coexec      how much of the MFMA time hides under vector work: per pass a wave issues four
+//                            MFMAs (mode bit 0), 32 x (v_exp_f32, v_mul_f32) in eight chains (bit 1), or both
+//                            dealt out in turns (3); the first wave of each SIMD takes mode_first, the second
+//                            mode_second
+// sink: a few bytes of device memory that are practically never written.
+#include "../device_common.h"
 
 namespace mi355q {
 

@@ -68,6 +68,10 @@ struct SdpaArgs {
   int nsplit, blocks_per_split;
   float* ws;        // partial results of the key splits when nsplit > 1
   uint32_t* tickets;  // one arrival counter per group, zero between launches
+  // keys a batch entry may attend to: valid_len[b] of them, the last ones (left padding) or the first ones
+  // (right padding), b the index along batch dimension valid_dim; null = all S keys
+  const int32_t* valid_len;
+  int valid_dim, pad_left;
 };
 
 __device__ __forceinline__ float sdpa_scale(const SdpaArgs& a, int i, float absent) {
@@ -176,7 +180,8 @@ __global__ void sdpa_clear_amax_kernel(float* a, float* b) {
 template <int DKC, int DVT, int FMT, bool QL = false>
 __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb, const uint8_t* vb, int kv0, bool edge, int qpos,
                                            bool q_ok, const uint8_t* mrow, const i32x8 (&qf)[DKC], float sc2, float lqs, bool clamp_p,
-                                           f32x16 (&o)[DVT], float& m_run, float& l_run, const uint8_t* qbase = nullptr) {
+                                           f32x16 (&o)[DVT], float& m_run, float& l_run, const uint8_t* qbase = nullptr,
+                                           int klo = 0, int khi = 0x7fffffff) {
   constexpr int KROW = DKC * 64;
   constexpr int kVRow = DVT <= 4 ? 128 : 256;
   constexpr float kMax8 = FMT == MI355Q_E5M2 ? 57344.0f : 448.0f;
@@ -258,7 +263,7 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
       for (int r = 0; r < 16; ++r) {
         const int kv = kv0 + 32 * t + 8 * (r >> 2) + 4 * h + (r & 3);
         float x = s[t][r] * sc2;
-        bool dead = kv >= a.S || (a.causal && kv > qpos);
+        bool dead = kv >= a.S || kv >= khi || kv < klo || (a.causal && kv > qpos);
         if (a.mask_kind != kMaskNone && q_ok && kv < a.S) {
           if (a.mask_kind == kMaskBool) dead = dead || mrow[kv] == 0;
           else if (a.mask_kind == kMaskBf16) x += bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(mrow)[kv]) * kLog2e;
@@ -395,6 +400,7 @@ __global__ __launch_bounds__(kSdpaThreads, (sdpa_q_in_lds(DKC, DVT, DMA) ? 3 : D
   int64_t bi = id / a.nqb;
   const int qb = a.nqb - 1 - (id - (int)bi * a.nqb);  // under a causal mask the long rows start first
   int64_t q_off = 0, k_off = 0, v_off = 0, m_off = 0, o_off = 0;
+  int64_t b_valid = 0;
 #pragma unroll
   for (int d = 2; d >= 0; --d) {
     const int64_t b = bi % a.bdim[d];
@@ -404,10 +410,20 @@ __global__ __launch_bounds__(kSdpaThreads, (sdpa_q_in_lds(DKC, DVT, DMA) ? 3 : D
     v_off += b * a.v_bs[d];
     m_off += b * a.m_bs[d];
     o_off += b * a.o_bs[d];
+    if (d == a.valid_dim) b_valid = b;
   }
   const uint8_t* qp = a.q + q_off;
   const uint8_t* kp = a.k + k_off;
   const uint8_t* vp = a.v + v_off;
+  // the window of keys this batch entry may attend to
+  int klo = 0, khi = a.S;
+  if (a.valid_len != nullptr) {
+    int n = a.valid_len[b_valid];
+    n = n < 0 ? 0 : (n > a.S ? a.S : n);
+    n = __builtin_amdgcn_readfirstlane(n);
+    if (a.pad_left) klo = a.S - n;
+    else khi = n;
+  }
 
   const int q0 = qb * kSdpaBM;
   const int wq0 = q0 + wave * 32;  // first query row of this wave
@@ -449,12 +465,14 @@ __global__ __launch_bounds__(kSdpaThreads, (sdpa_q_in_lds(DKC, DVT, DMA) ? 3 : D
     }
   }
 
-  int nblk = (a.S + kSdpaBN - 1) / kSdpaBN;
+  // blocks blk0 .. nblk - 1 hold the keys of the window
+  int nblk = (khi + kSdpaBN - 1) / kSdpaBN;
   if (a.causal) {
     const int last_q = (q0 + kSdpaBM < a.L ? q0 + kSdpaBM : a.L) - 1;
     const int lim = last_q / kSdpaBN + 1;  // blocks that hold a key <= the last query row
     nblk = nblk < lim ? nblk : lim;
   }
+  const int blk0 = klo / kSdpaBN < nblk ? klo / kSdpaBN : nblk;
 
   u32x4 kreg[KLOADS], vreg[VLOADS];
   auto fetch = [&](int blk) {
@@ -495,8 +513,10 @@ __global__ __launch_bounds__(kSdpaThreads, (sdpa_q_in_lds(DKC, DVT, DMA) ? 3 : D
   int kvoff[KREG], vvoff[VREG];
   SdpaWalker wk{reinterpret_cast<uint64_t>(kp), 0}, wv{reinterpret_cast<uint64_t>(vp), 0};
   if constexpr (DMA) {
-    wk.left = (int64_t)(a.S - 1) * a.ldk + a.Dk;
-    wv.left = (int64_t)(a.S - 1) * a.ldv + a.Dv;
+    wk.base += (uint64_t)blk0 * kSdpaBN * a.ldk;
+    wv.base += (uint64_t)blk0 * kSdpaBN * a.ldv;
+    wk.left = (int64_t)(a.S - 1 - blk0 * kSdpaBN) * a.ldk + a.Dk;
+    wv.left = (int64_t)(a.S - 1 - blk0 * kSdpaBN) * a.ldv + a.Dv;
 #pragma unroll
     for (int n = 0; n < KREG; ++n) {
       const int pos = (wave * KREG + n) * 64 + lane;  // 16-byte slot of the tile this lane fills
@@ -534,37 +554,39 @@ __global__ __launch_bounds__(kSdpaThreads, (sdpa_q_in_lds(DKC, DVT, DMA) ? 3 : D
   float l_run = 0.0f;               // this half-wave's share of the running sum (times q_scale_s)
 
   const uint8_t* mrow = a.mask + (m_off + (int64_t)qrow * a.ldm) * (a.mask_kind == kMaskBool ? 1 : a.mask_kind == kMaskBf16 ? 2 : 4);
-  if (nblk > 0) {
+  // ring positions count from the window's first block
+  if (nblk > blk0) {
     if constexpr (DMA) {
-      for (int b = 0; b < kStages - 1 && b < nblk; ++b) issue_block(b);
-      if (nblk >= kStages - 1 && (kStages - 1) * kSdpaBN <= a.S) {
+      for (int b = 0; b < kStages - 1 && blk0 + b < nblk; ++b) issue_block(b);
+      if (nblk - blk0 >= kStages - 1 && (blk0 + kStages - 1) * kSdpaBN <= a.S) {
         constexpr int cnt = (kStages - 2) * (KREG + VREG);
-        __builtin_amdgcn_s_waitcnt((cnt & 15) | ((cnt >> 4) << 14) | 0x0f70);  // block 0 has landed
+        __builtin_amdgcn_s_waitcnt((cnt & 15) | ((cnt >> 4) << 14) | 0x0f70);  // the first block has landed
       } else {
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
       }
     } else {
-      fetch(0);
+      fetch(blk0);
       commit(0);
     }
   }
   __syncthreads();
 
-  for (int blk = 0; blk < nblk; ++blk) {
+  for (int blk = blk0; blk < nblk; ++blk) {
     const int kv0 = blk * kSdpaBN;
+    const int pos = blk - blk0;
     if constexpr (DMA) {
-      if (blk + kStages - 1 < nblk) issue_block((blk + kStages - 1) % kStages);
+      if (blk + kStages - 1 < nblk) issue_block((pos + kStages - 1) % kStages);
     } else {
       if (blk + 1 < nblk) fetch(blk + 1);
     }
-    const uint8_t* kb = lds + (DMA ? blk % kStages : blk & 1) * (KBYTES + VBYTES);
+    const uint8_t* kb = lds + (DMA ? pos % kStages : pos & 1) * (KBYTES + VBYTES);
     const uint8_t* vb = kb + KBYTES;
 
     // a wave whose 32 rows all lie above this block's first key has nothing to add
     const bool active = !(a.causal && kv0 > wq0 + 31);
     if (active) {
-      const bool edge = (a.causal && kv0 + kSdpaBN - 1 > wq0) || kv0 + kSdpaBN > a.S || a.mask_kind != kMaskNone;
-      sdpa_block<DKC, DVT, FMT, kQLds>(a, kb, vb, kv0, edge, qrow, q_ok, mrow, qf, sc2, lqs, clamp_p, o, m_run, l_run, qbase);
+      const bool edge = (a.causal && kv0 + kSdpaBN - 1 > wq0) || kv0 + kSdpaBN > khi || kv0 < klo || a.mask_kind != kMaskNone;
+      sdpa_block<DKC, DVT, FMT, kQLds>(a, kb, vb, kv0, edge, qrow, q_ok, mrow, qf, sc2, lqs, clamp_p, o, m_run, l_run, qbase, klo, khi);
     }
 
     if constexpr (DMA) {
@@ -579,7 +601,7 @@ __global__ __launch_bounds__(kSdpaThreads, (sdpa_q_in_lds(DKC, DVT, DMA) ? 3 : D
         __builtin_amdgcn_s_waitcnt(0x0f70);
       }
     } else {
-      if (blk + 1 < nblk) commit((blk + 1) & 1);
+      if (blk + 1 < nblk) commit((pos + 1) & 1);
     }
     __syncthreads();
   }
@@ -942,6 +964,7 @@ static SdpaDecodePlan sdpa_decode_plan(const mi355q_sdpa_desc* d, int cus) {
   SdpaDecodePlan p;
   const bool shared = d->batch[2] > 1 && d->k_bstride[2] == 0 && d->v_bstride[2] == 0;
   const int64_t inner = shared ? d->batch[2] : 1;
+  if (d->valid_seq_len != nullptr) return p;  // a per-batch key window runs on the kernel for many queries
   if (inner * d->q_len > 32 || d->kv_len < 512 || d->head_dim_qk > 128 || d->head_dim_v > 128) return p;
   p.pack = shared;
   p.rows = (int)(inner * d->q_len);
@@ -1081,9 +1104,14 @@ int mi355q_fp8_sdpa_fwd(const void* q, const void* k, const void* v, int fp8_fmt
   }
   a.amax_s = amax_s;
   a.amax_o = amax_o;
+  a.valid_len = d->valid_seq_len;
+  a.valid_dim = d->valid_seq_len != nullptr ? d->valid_seq_dim : -1;
+  a.pad_left = d->seq_padding_left != 0;
+  if (d->valid_seq_len != nullptr && (d->valid_seq_dim < 0 || d->valid_seq_dim > 2)) return MI355Q_ERR_INVALID_ARGUMENT;
 
   const int64_t dmax = d->head_dim_qk > d->head_dim_v ? d->head_dim_qk : d->head_dim_v;
   // a few queries against many keys: the kernel that splits the keys (direct loads only)
+  // (a per-batch key window is served by the other kernel alone)
   SdpaDecodePlan plan = sdpa_decode_plan(d, compute_units_sdpa());
   if (plan.groups > 0 && a.dma && plan.groups * (int64_t)plan.nsplit <= 0x7fffffff) {
     if (plan.nsplit > 1 && (workspace == nullptr || workspace_bytes < plan.ws_bytes || !aligned_to(workspace, 4))) {

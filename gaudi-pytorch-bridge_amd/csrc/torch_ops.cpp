@@ -1031,6 +1031,60 @@ void sdpa_batch_strides(const Tensor& t, const std::vector<int64_t>& bshape, int
 
 Tensor sdpa_unit_rows(const Tensor& t) { return (t.dim() >= 1 && t.stride(-1) != 1 && t.size(-1) > 1) ? t.contiguous() : t; }
 
+// seq_padding_type of the ops: "left" or "right" (the wrapper lower-cases it, Fp8FusedSDPA.py:112); it only
+// matters when valid_seq_len is given (flags SEQ_PADDING_LEFT / RIGHT, sdpa_gen.cpp:850-851).
+bool sdpa_padding_left(c10::string_view seq_padding_type, bool has_valid) {
+  const bool left = seq_padding_type == "left" || seq_padding_type == "Left" || seq_padding_type == "LEFT";
+  const bool right = seq_padding_type == "right" || seq_padding_type == "Right" || seq_padding_type == "RIGHT";
+  TORCH_CHECK(!has_valid || left || right, "seq_padding_type must be \"left\" or \"right\", got \"", std::string(seq_padding_type), "\"");
+  return !right;
+}
+
+// valid_seq_len: one count of valid (unpadded) keys per entry of the outermost batch dimension -> int32 on q's device
+Tensor sdpa_valid_seq_len(const Tensor& t, const Tensor& q, const std::vector<int64_t>& bshape, const char* op) {
+  const int64_t nbatch = bshape.empty() ? 1 : bshape[0];
+  TORCH_CHECK(at::isIntegralType(t.scalar_type(), false), op, ": valid_seq_len must be an integer tensor, got ", t.scalar_type());
+  TORCH_CHECK(t.numel() == nbatch, op, ": valid_seq_len must hold one value per batch entry (", nbatch, "), got ", t.sizes());
+  if (q.is_meta()) return t;
+  TORCH_CHECK(t.device() == q.device(), op, ": valid_seq_len must be on the same device as q");
+  return t.reshape({nbatch}).to(at::kInt).contiguous();
+}
+
+// Keys a query may attend to, as a boolean tensor that broadcasts against the scores [batch..., L, S]
+// (undefined: all of them): the triangular mask and the per-batch key window.
+Tensor sdpa_keep_mask(const Tensor& like, int64_t L, int64_t S, bool is_causal, const Tensor& valid, bool pad_left, int64_t batch_rank) {
+  Tensor keep;
+  auto bopts = like.options().dtype(at::kBool);
+  if (is_causal) keep = at::ones({L, S}, bopts).tril(0);
+  if (valid.defined()) {
+    Tensor j = at::arange(S, like.options().dtype(at::kInt)).reshape({1, S});
+    Tensor n = valid.reshape({-1, 1});
+    Tensor w = pad_left ? j.ge(S - n) : j.lt(n);   // [B, S]
+    std::vector<int64_t> shp(batch_rank + 2, 1);
+    shp[0] = batch_rank > 0 ? w.size(0) : 1;
+    shp.back() = S;
+    if (batch_rank == 0) w = w.reshape({1, S});
+    else w = w.reshape(shp);
+    keep = keep.defined() ? keep.logical_and(w) : w;
+  }
+  return keep;
+}
+
+// softmax(q k^T scale + masks) in fp32 on the device's own matmul and softmax: the route of the bf16 / fp32
+// measurement pass, where nothing is fp8.  A row with every key masked gives zeros.
+Tensor sdpa_probabilities_unfused(const Tensor& q, const Tensor& k, const c10::optional<Tensor>& attention_mask, double scale,
+                                  bool is_causal, const Tensor& valid, bool pad_left, int64_t batch_rank) {
+  const float ninf = -std::numeric_limits<float>::infinity();
+  Tensor s = at::matmul(q, k.transpose(-2, -1)).to(at::kFloat) * scale;
+  if (attention_mask.has_value() && attention_mask->defined()) {
+    if (attention_mask->scalar_type() == at::kBool) s = s.masked_fill(attention_mask->logical_not(), ninf);
+    else s = s + attention_mask->to(at::kFloat);
+  }
+  Tensor keep = sdpa_keep_mask(q, q.size(-2), k.size(-2), is_causal, valid, pad_left, batch_rank);
+  if (keep.defined()) s = s.masked_fill(keep.logical_not(), ninf);
+  return at::nan_to_num(at::softmax(s, -1), 0.0);
+}
+
 // Fp8SDPARecompFwd::AddNode, hpu_ops/backend/sdpa_gen.cpp:806-1000 (inputs, flags, output types);
 // output shapes SDPARecompFwdOutputShapeCommon / Fp8SDPARecompFwdOutputShape, :597-706.
 SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tensor& v, const c10::optional<Tensor>& attention_mask,
@@ -1041,13 +1095,17 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
                                    c10::string_view seq_padding_type) {
   TORCH_CHECK(!requires_backward, "fp8_sdpa_recomp_fwd: only the inference forward (requires_backward=False) is implemented");
   TORCH_CHECK(p == 0.0, "fp8_sdpa_recomp_fwd: dropout is not implemented (p must be 0)");
-  TORCH_CHECK(!(valid_seq_len.has_value() && valid_seq_len->defined()), "fp8_sdpa_recomp_fwd: valid_seq_len is not implemented");
   TORCH_CHECK(softmax_mode == "none" || softmax_mode == "None" || softmax_mode == "fast", "fp8_sdpa_recomp_fwd: softmax_mode must be \"none\" or \"fast\"");
   const int64_t rank = q.dim();
   TORCH_CHECK(rank >= 2 && rank <= 5 && k.dim() == rank && v.dim() == rank,
               "fp8_sdpa_recomp_fwd: q, k and v must have the same rank, between 2 and 5");
   const bool has_mask = attention_mask.has_value() && attention_mask->defined();
   TORCH_CHECK(!(has_mask && is_causal), "fp8_sdpa_recomp_fwd: attention_mask and is_causal exclude each other");
+  const bool has_valid = valid_seq_len.has_value() && valid_seq_len->defined();
+  const bool pad_left = sdpa_padding_left(seq_padding_type, has_valid);
+  // the wrapper's contract (Fp8FusedSDPA.py:123-126): only in inference with the triangular mask
+  TORCH_CHECK(!has_valid || (is_causal && !has_mask),
+              "fp8_sdpa_recomp_fwd: valid_seq_len is supported only in inference with is_causal and no attention_mask");
   const int64_t L = q.size(-2), S = k.size(-2), Dk = q.size(-1), Dv = v.size(-1);
   TORCH_CHECK(k.size(-1) == Dk, "fp8_sdpa_recomp_fwd: q and k must have the same head dimension");
   TORCH_CHECK(v.size(-2) == S, "fp8_sdpa_recomp_fwd: k and v must have the same sequence length");
@@ -1065,7 +1123,9 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
   const at::ScalarType stat_dt = fp8_in ? at::kBFloat16 : dt;
   auto opts = q.options();
   Tensor out = at::empty(out_shape, opts.dtype(out_dt));
-  const at::ScalarType linv_dt = fp8_in || softmax_mode == "fast" ? at::kBFloat16 : at::kFloat;
+  // Float; BFloat16 for fp8 q and for bf16 q with softmax_mode "fast" (eager_custom_op_register.cpp:1795-1803)
+  const at::ScalarType linv_dt = fp8_in || (softmax_mode == "fast" && dt == at::kBFloat16) ? at::kBFloat16 : at::kFloat;
+  Tensor valid = has_valid ? sdpa_valid_seq_len(*valid_seq_len, q, bshape, "fp8_sdpa_recomp_fwd") : Tensor();
   if (q.is_meta())
     return SdpaOut(out, at::empty({1}, opts.dtype(stat_dt)), at::empty({1}, opts.dtype(linv_dt)), at::empty({1}, opts.dtype(at::kInt)),
                    at::empty({1}, opts.dtype(at::kFloat)), at::empty({1}, opts.dtype(at::kFloat)));
@@ -1085,17 +1145,7 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
     // The measurement pass of the reference's flow: bf16 / fp32 q, k, v, no fp8 anywhere; only amax_s
     // (and amax_o) are wanted from it.  It runs on the device's own matmul and softmax.
     TORCH_CHECK(dt == at::kBFloat16 || dt == at::kFloat, "fp8_sdpa_recomp_fwd: q, k and v must be fp8, bfloat16 or float");
-    Tensor s = at::matmul(q, k.transpose(-2, -1)).to(at::kFloat) * scale;
-    if (has_mask) {
-      if (attention_mask->scalar_type() == at::kBool) s = s.masked_fill(attention_mask->logical_not(), -std::numeric_limits<float>::infinity());
-      else s = s + attention_mask->to(at::kFloat);
-    }
-    if (is_causal) {
-      Tensor keep = at::ones({L, S}, opts.dtype(at::kBool)).tril(0);
-      s = s.masked_fill(keep.logical_not(), -std::numeric_limits<float>::infinity());
-    }
-    Tensor pr = at::softmax(s, -1);
-    pr = at::nan_to_num(pr, 0.0);   // a row with every key masked
+    Tensor pr = sdpa_probabilities_unfused(q, k, attention_mask, scale, is_causal, valid, pad_left, (int64_t)bshape.size());
     out.copy_(at::matmul(pr.to(dt), v));
     if (pr.numel() > 0) amax_s.copy_(pr.max().reshape({1}));
     else amax_s.zero_();
@@ -1120,6 +1170,11 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
   sdpa_batch_strides(out, bshape, d.out_bstride, "out");
   d.q_len = L; d.kv_len = S; d.head_dim_qk = Dk; d.head_dim_v = Dv;
   d.ldq = qc.stride(-2); d.ldk = kc.stride(-2); d.ldv = vc.stride(-2); d.ldo = out.stride(-2);
+  if (has_valid) {
+    d.valid_seq_len = valid.data_ptr<int32_t>();
+    d.valid_seq_dim = nb == 0 ? 2 : (int32_t)(3 - nb);   // the outermost batch dimension
+    d.seq_padding_left = pad_left ? 1 : 0;
+  }
   Tensor mk;
   int mask_kind = MI355Q_SDPA_MASK_NONE;
   if (has_mask) {
@@ -1191,6 +1246,148 @@ SdpaOut fp8_sdpa_recomp_fwd_scalar(const Tensor& q, const Tensor& k, const Tenso
                                     sdpa_scale(d_scale_q), sdpa_scale(d_scale_k), sdpa_scale(d_scale_v), sdpa_scale(q_scale_s),
                                     sdpa_scale(q_scale_o), sdpa_scale(d_scale_s), is_amax_s, is_amax_o, valid_seq_len,
                                     seq_padding_type);
+}
+
+// --------------------------------------------------------------- fp8_sdpa_fwd
+//
+// The forward without recomputation (Fp8SDPAFwd::AddNode, hpu_ops/backend/sdpa_gen.cpp:340-437; output shapes
+// SDPAFwdOutputShapeCommon :103-150 and Fp8SDPAFwdOutputShape :267-272; eager wrapper
+// habana_eager/eager_custom_op_register.cpp:1544-1660), which the reference's module calls whenever
+// recomputation is switched off, inference included (Fp8FusedSDPA.py:163-182).  It returns the attention
+// output, the probability matrix P [batch..., L, S] in q's dtype (what a backward pass would read instead of
+// recomputing it), the dropout mask (a one-element Char placeholder without dropout) and amax_s.  Materialising
+// P is the point of the op, so it runs unfused on this library's own kernels: the scores are one batched fp8 GEMM
+// (q k^T, d_scale_q and d_scale_k in its epilogue), softmax_fp8 scales them, adds the mask and writes
+// P = fp8(softmax q_scale_s), and out = (P v) d_scale_s d_scale_v is a second fp8 GEMM.  Here the
+// probabilities are normalised before they are rounded to fp8 (in the recompute op they are rounded per block
+// of keys against the running maximum); the reference's kernel is closed on this point.  A row whose keys are
+// all masked holds equal scores and attends to all keys evenly (the recompute op gives zeros there).
+using SdpaFwdOut = std::tuple<Tensor, Tensor, Tensor, Tensor>;
+
+SdpaFwdOut fp8_sdpa_fwd(const Tensor& q, const Tensor& k, const Tensor& v, const c10::optional<Tensor>& attention_mask, double p,
+                        double scale, bool is_causal, c10::string_view softmax_mode, const c10::optional<Tensor>& d_scale_q,
+                        const c10::optional<Tensor>& d_scale_k, const c10::optional<Tensor>& d_scale_v,
+                        const c10::optional<Tensor>& q_scale_s, const c10::optional<Tensor>& q_scale_o,
+                        const c10::optional<Tensor>& d_scale_s, bool is_amax_s, const c10::optional<Tensor>& valid_seq_len,
+                        c10::string_view seq_padding_type) {
+  TORCH_CHECK(p == 0.0, "fp8_sdpa_fwd: dropout is not implemented (p must be 0)");
+  TORCH_CHECK(softmax_mode == "none" || softmax_mode == "None" || softmax_mode == "fast", "fp8_sdpa_fwd: softmax_mode must be \"none\" or \"fast\"");
+  const int64_t rank = q.dim();
+  TORCH_CHECK(rank >= 2 && rank <= 5 && k.dim() == rank && v.dim() == rank, "fp8_sdpa_fwd: q, k and v must have the same rank, between 2 and 5");
+  const bool has_mask = attention_mask.has_value() && attention_mask->defined();
+  TORCH_CHECK(!(has_mask && is_causal), "fp8_sdpa_fwd: attention_mask and is_causal exclude each other");
+  const bool has_valid = valid_seq_len.has_value() && valid_seq_len->defined();
+  const bool pad_left = sdpa_padding_left(seq_padding_type, has_valid);
+  TORCH_CHECK(!has_valid || (is_causal && !has_mask), "fp8_sdpa_fwd: valid_seq_len is supported only with is_causal and no attention_mask");
+  const int64_t L = q.size(-2), S = k.size(-2), Dk = q.size(-1), Dv = v.size(-1);
+  TORCH_CHECK(k.size(-1) == Dk, "fp8_sdpa_fwd: q and k must have the same head dimension");
+  TORCH_CHECK(v.size(-2) == S, "fp8_sdpa_fwd: k and v must have the same sequence length");
+  const at::ScalarType dt = q.scalar_type();
+  TORCH_CHECK(k.scalar_type() == dt && v.scalar_type() == dt, "fp8_sdpa_fwd: q, k and v must have the same dtype");
+  std::vector<int64_t> qb(q.sizes().begin(), q.sizes().end() - 2), kb(k.sizes().begin(), k.sizes().end() - 2),
+      vb(v.sizes().begin(), v.sizes().end() - 2);
+  std::vector<int64_t> pshape = at::infer_size(qb, kb);          // batch dims of q k^T
+  std::vector<int64_t> oshape = at::infer_size(pshape, vb);
+  const int64_t nb = (int64_t)oshape.size();
+  pshape.push_back(L);
+  pshape.push_back(S);
+  oshape.push_back(L);
+  oshape.push_back(Dv);
+  const bool fp8_in = is_fp8(dt);
+  const bool has_qo = q_scale_o.has_value() && q_scale_o->defined() && q_scale_o->numel() > 0;
+  // out: q's dtype, or bf16 for fp8 q without q_scale_o (sdpa_gen.cpp:412-424); P: q's dtype; amax_s: Float
+  const at::ScalarType out_dt = fp8_in ? (has_qo ? dt : at::kBFloat16) : dt;
+  auto opts = q.options();
+  if (q.is_meta())
+    return SdpaFwdOut(at::empty(oshape, opts.dtype(out_dt)), at::empty(pshape, opts.dtype(dt)), at::empty({1}, opts.dtype(at::kChar)),
+                      at::empty({1}, opts.dtype(at::kFloat)));
+  DeviceGuard guard(q.device());
+  TORCH_CHECK(k.device() == q.device() && v.device() == q.device(), "fp8_sdpa_fwd: q, k and v must be on one device");
+  Tensor dm = at::zeros({1}, opts.dtype(at::kChar));
+  Tensor amax_s = at::zeros({1}, opts.dtype(at::kFloat));
+  std::vector<int64_t> bshape(oshape.begin(), oshape.end() - 2);
+  Tensor valid = has_valid ? sdpa_valid_seq_len(*valid_seq_len, q, bshape, "fp8_sdpa_fwd") : Tensor();
+  MI355Q_OP_INFO("fp8_sdpa_fwd : q=" << q.sizes() << " k=" << k.sizes() << " v=" << v.sizes() << " " << dt << " -> " << out_dt
+                                      << (is_causal ? " causal" : "") << (has_mask ? " mask" : ""));
+  if (!fp8_in) {
+    // bf16 / fp32 q, k, v (the measurement pass): nothing is fp8, the device's own matmul and softmax
+    TORCH_CHECK(dt == at::kBFloat16 || dt == at::kFloat, "fp8_sdpa_fwd: q, k and v must be fp8, bfloat16 or float");
+    Tensor pr = sdpa_probabilities_unfused(q, k, attention_mask, scale, is_causal, valid, pad_left, nb);
+    Tensor P = pr.to(dt);
+    Tensor out = at::matmul(P, v);
+    if (is_amax_s && pr.numel() > 0) amax_s.copy_(pr.max().reshape({1}));
+    return SdpaFwdOut(out, P, dm, amax_s);
+  }
+  if (L == 0 || S == 0 || c10::multiply_integers(oshape) == 0 || Dk == 0) {
+    return SdpaFwdOut(at::zeros(oshape, opts.dtype(out_dt)), at::zeros(pshape, opts.dtype(dt)), dm, amax_s);
+  }
+  // scores = (q d_scale_q)(k d_scale_k)^T, bf16
+  Tensor scores = fp8_gemm_v2_impl(q, false, k, true, c10::nullopt, at::kBFloat16, opt_tensor_iv(d_scale_q), opt_tensor_iv(d_scale_k),
+                                   c10::nullopt, false, c10::nullopt);
+  // the masks as one additive bf16 tensor of the rank of the scores (first and last extent as theirs, 1 or
+  // theirs in between: the form softmax_fp8 takes).  Masked entries get the most negative finite value.
+  Tensor add;
+  {
+    const float kMasked = -3.0e38f;
+    Tensor m;
+    if (has_mask) {
+      TORCH_CHECK(attention_mask->device() == q.device(), "fp8_sdpa_fwd: attention_mask must be on the same device as q");
+      if (attention_mask->scalar_type() == at::kBool)
+        m = at::zeros({1}, opts.dtype(at::kBFloat16)).masked_fill(attention_mask->logical_not(), kMasked);
+      else m = attention_mask->to(at::kBFloat16).clamp_min(kMasked);
+    } else {
+      Tensor keep = sdpa_keep_mask(q, L, S, is_causal, valid, pad_left, nb);
+      if (keep.defined()) m = at::zeros({1}, opts.dtype(at::kBFloat16)).masked_fill(keep.logical_not(), kMasked);
+    }
+    if (m.defined()) {
+      TORCH_CHECK(m.dim() <= scores.dim(), "fp8_sdpa_fwd: attention_mask has more dimensions than the scores");
+      while (m.dim() < scores.dim()) m = m.unsqueeze(0);
+      std::vector<int64_t> shp(m.sizes().begin(), m.sizes().end());
+      for (int64_t i = 0; i < (int64_t)shp.size(); ++i)
+        TORCH_CHECK(shp[i] == 1 || shp[i] == scores.size(i), "fp8_sdpa_fwd: attention_mask ", attention_mask.has_value() ? attention_mask->sizes() : m.sizes(),
+                    " does not broadcast to the scores ", scores.sizes());
+      shp.front() = scores.size(0);
+      shp.back() = S;
+      add = m.expand(shp).contiguous();
+    }
+  }
+  // P = fp8(softmax(scores scale + mask) q_scale_s); an e5m2 q takes bf16 probabilities and the cast kernel
+  const bool has_qs = q_scale_s.has_value() && q_scale_s->defined() && q_scale_s->numel() > 0;
+  SoftmaxScale in_s = softmax_scale(scale);
+  SoftmaxScale out_s = softmax_scale(1.0);
+  Tensor qs_holder;
+  if (has_qs) {
+    TORCH_CHECK(q_scale_s->numel() == 1, "fp8_sdpa_fwd: q_scale_s must have one element, got ", q_scale_s->sizes());
+    qs_holder = q_scale_s->to(q.device(), at::kFloat).reshape({1});
+    out_s.dev = qs_holder.data_ptr<float>();
+  }
+  Tensor P;
+  if (dt == at::kFloat8_e4m3fn && !is_amax_s) {
+    P = softmax_fp8_common(scores, -1, in_s, out_s, SoftmaxScale(), add.defined() ? c10::optional<Tensor>(add) : c10::nullopt);
+  } else {
+    // bf16 probabilities first (their maximum is amax_s), then the scaled cast to q's format
+    Tensor x = scores.to(at::kFloat) * scale;
+    if (add.defined()) x = x + add.to(at::kFloat);
+    Tensor pb = softmax_fp8_common(x.to(at::kBFloat16), -1, SoftmaxScale(), SoftmaxScale(), SoftmaxScale(), c10::nullopt);
+    if (is_amax_s) {
+      check_status(mi355q_amax(pb.data_ptr(), MI355Q_BF16, pb.numel(), amax_s.data_ptr<float>(), current_stream(pb)), "mi355q_amax");
+    }
+    P = at::empty(pb.sizes(), opts.dtype(dt));
+    CastScale cs = resolve_cast_scale(has_qs ? IValue(qs_holder) : IValue(), c10::nullopt, pb);
+    check_status(launch_cast_to(pb, P, cs, nullptr, false), "mi355q_cast_to_fp8");
+  }
+  // out = (P d_scale_s)(v d_scale_v); d_scale_s defaults to 1 / q_scale_s
+  const bool has_ds = d_scale_s.has_value() && d_scale_s->defined() && d_scale_s->numel() > 0;
+  IValue ds_iv = has_ds ? IValue(*d_scale_s) : (has_qs ? IValue(qs_holder.reciprocal()) : IValue());
+  Tensor out = fp8_gemm_v2_impl(P, false, v, false, c10::nullopt, at::kBFloat16, ds_iv, opt_tensor_iv(d_scale_v), c10::nullopt, false,
+                                c10::nullopt);
+  if (out_dt != at::kBFloat16) {
+    Tensor o8 = at::empty(out.sizes(), opts.dtype(out_dt));
+    CastScale cs = resolve_cast_scale(IValue(q_scale_o->to(q.device(), at::kFloat)), c10::nullopt, out);
+    check_status(launch_cast_to(out, o8, cs, nullptr, false), "mi355q_cast_to_fp8");
+    out = o8;
+  }
+  return SdpaFwdOut(out, P, dm, amax_s);
 }
 
 // ------------------------------------------------------------- amax helpers
@@ -1381,6 +1578,10 @@ TORCH_LIBRARY(hpu, m) {
   m.def("hpu::softmax_fp8.Scalar(Tensor input, int dim, float input_scale, float output_scale, float inv_attn_heads, Tensor? fused_add=None) -> Tensor");
   m.def("hpu::sum_fp8(Tensor self, int[1]? dim=None, bool keepdim=False, ScalarType? out_dtype=None) -> Tensor");
   m.def("hpu::fp8_sdpa_recomp_fwd(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, bool requires_backward, str softmax_mode, Tensor? d_scale_q, Tensor? d_scale_k, Tensor? d_scale_v, Tensor? q_scale_s, Tensor? q_scale_o, Tensor? d_scale_s, bool is_amax_s, bool is_amax_0, Tensor? valid_seq_len, str seq_padding_type ) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)");
+  m.def("hpu::fp8_sdpa_recomp_fwd_non_dropout(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, bool requires_backward, str softmax_mode, Tensor? d_scale_q, Tensor? d_scale_k, Tensor? d_scale_v, Tensor? q_scale_s, Tensor? q_scale_o, Tensor? d_scale_s, bool is_amax_s, bool is_amax_0, Tensor? valid_seq_len, str seq_padding_type ) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)");
+  m.def("hpu::fp8_sdpa_recomp_fwd_non_dropout.scalar(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, bool requires_backward, str softmax_mode, float d_scale_q, float d_scale_k, float d_scale_v, float q_scale_s, float q_scale_o, float d_scale_s, bool is_amax_s, bool is_amax_0,  Tensor? valid_seq_len, str seq_padding_type ) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)");
+  m.def("hpu::fp8_sdpa_fwd(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, str softmax_mode, Tensor? d_scale_q, Tensor? d_scale_k, Tensor? d_scale_v, Tensor? q_scale_s, Tensor? q_scale_o, Tensor? d_scale_s, bool is_amax_s, Tensor? valid_seq_len, str seq_padding_type) -> (Tensor, Tensor, Tensor, Tensor)");
+  m.def("hpu::fp8_sdpa_fwd_non_dropout(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, str softmax_mode, Tensor? d_scale_q, Tensor? d_scale_k, Tensor? d_scale_v, Tensor? q_scale_s, Tensor? q_scale_o, Tensor? d_scale_s, bool is_amax_s, Tensor? valid_seq_len, str seq_padding_type) -> (Tensor, Tensor, Tensor, Tensor)");
   m.def("hpu::fp8_sdpa_recomp_fwd.scalar(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, bool requires_backward, str softmax_mode, float d_scale_q, float d_scale_k, float d_scale_v, float q_scale_s, float q_scale_o, float d_scale_s, bool is_amax_s, bool is_amax_0, Tensor? valid_seq_len, str seq_padding_type ) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)");
 }
 
@@ -1414,7 +1615,11 @@ TORCH_LIBRARY(mi355q, m) {
   m.impl("softmax_fp8.Scalar", softmax_fp8_scalar);                                            \
   m.impl("sum_fp8", sum_fp8);                                                                  \
   m.impl("fp8_sdpa_recomp_fwd", fp8_sdpa_recomp_fwd);                                          \
-  m.impl("fp8_sdpa_recomp_fwd.scalar", fp8_sdpa_recomp_fwd_scalar);
+  m.impl("fp8_sdpa_recomp_fwd.scalar", fp8_sdpa_recomp_fwd_scalar);                            \
+  m.impl("fp8_sdpa_recomp_fwd_non_dropout", fp8_sdpa_recomp_fwd);                              \
+  m.impl("fp8_sdpa_recomp_fwd_non_dropout.scalar", fp8_sdpa_recomp_fwd_scalar);                \
+  m.impl("fp8_sdpa_fwd", fp8_sdpa_fwd);                                                        \
+  m.impl("fp8_sdpa_fwd_non_dropout", fp8_sdpa_fwd);
 
 TORCH_LIBRARY_IMPL(hpu, CUDA, m) { MI355Q_REGISTER_HPU(m) }
 TORCH_LIBRARY_IMPL(hpu, Meta, m) { MI355Q_REGISTER_HPU(m) }

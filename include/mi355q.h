@@ -332,7 +332,7 @@ int mi355q_softmax_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols,
  * by -inf gives zeros.  Replaces the "sdpa_recomp_fwd" node that hpu::fp8_sdpa_recomp_fwd
  * builds with requires_backward false and dropout 0 (Fp8SDPARecompFwd::AddNode,
  * hpu_ops/backend/sdpa_gen.cpp:806-1000; schema habana_eager/eager_custom_op_register.cpp:
- * 2286-2296; the flags for valid_seq_len and dropout have no counterpart here).
+ * 2286-2296; the dropout flags have no counterpart here).
  *
  * q is [batch..., q_len, head_dim_qk], k [batch..., kv_len, head_dim_qk], v [batch..., kv_len,
  * head_dim_v], out [batch..., q_len, head_dim_v], the mask [batch..., q_len, kv_len] with unit
@@ -359,6 +359,15 @@ typedef struct mi355q_sdpa_desc {
   int64_t q_bstride[3], k_bstride[3], v_bstride[3], mask_bstride[3], out_bstride[3];
   int64_t q_len, kv_len, head_dim_qk, head_dim_v;
   int64_t ldq, ldk, ldv, ldmask, ldo;
+  /* Per-batch key window (the op's valid_seq_len / seq_padding_type, flags VALID_SEQ_LEN_PRESENT,
+   * SEQ_PADDING_LEFT / RIGHT of sdpa_gen.cpp:849-851, 902-904): valid_seq_len, where not NULL, holds
+   * batch[valid_seq_dim] int32 values on the device; entry b of that batch dimension attends to its
+   * last valid_seq_len[b] keys (seq_padding_left != 0: the padding sits in front) or its first
+   * (seq_padding_left == 0), on top of the causal mask.  Values are clamped to [0, kv_len]; a query
+   * row left with no key gives zeros. */
+  const int32_t* valid_seq_len;
+  int32_t valid_seq_dim;
+  int32_t seq_padding_left;
 } mi355q_sdpa_desc;
 
 /*
@@ -385,31 +394,6 @@ int mi355q_fp8_sdpa_fwd(const void* q, const void* k, const void* v, int fp8_fmt
                         float softmax_scale, int is_causal, const float* const* scale_dev,
                         const float* scale_host, float* amax_s, float* amax_o, void* workspace,
                         size_t workspace_bytes, void* stream);
-
-/*
- * Measurement aids without a counterpart in the reference; the product path never calls them.
- * mi355q_probe_mfma runs `workgroups` workgroups of 4 * waves_per_simd waves (1 or 2 per SIMD),
- * each wave issuing mfma_per_wave back-to-back v_mfma_f32_32x32x64_f8f6f4 (131072 flop each) on
- * register operands: timed, it gives the fp8 MFMA rate this GPU sustains at its clock under load.
- * mi355q_probe_read reads `bytes` bytes (a multiple of 16, 16-byte aligned) with 16-byte loads
- * and stores nothing: timed, the HBM read rate at that size.  sink: a few bytes of device memory
- * that are practically never written.
- */
-int mi355q_probe_mfma(int waves_per_simd, int mfma_per_wave, int workgroups, float* sink, void* stream);
-int mi355q_probe_read(const void* x, int64_t bytes, int workgroups, void* sink, void* stream);
-/* mi355q_probe_strip_read reads a row-major byte matrix [rows, pitch] the way the decode-shaped GEMMs read
- * their weights: pitch / strip_bytes strips (64, 128 or 256 bytes of every row), the rows of a strip cut
- * into `parts` ranges, one workgroup per strip and range, 16-byte loads with or without the nontemporal
- * hint, nothing stored. */
-int mi355q_probe_strip_read(const void* x, int64_t pitch, int64_t rows, int strip_bytes, int parts, int nontemporal,
-                            void* sink, void* stream);
-
-/* mi355q_probe_coexec: how much of the MFMA time hides under vector work.  Per pass a wave issues four
- * v_mfma_f32_32x32x64_f8f6f4 (mode bit 0), 32 x (v_exp_f32, v_mul_f32) in eight independent chains (bit 1),
- * or both dealt out in turns (3); the first wave of each SIMD takes mode_first, the second (waves_per_simd
- * = 2) mode_second.  Register operands only. */
-int mi355q_probe_coexec(int waves_per_simd, int passes, int mode_first, int mode_second, int workgroups, float* sink,
-                        void* stream);
 
 /* Name of the kernel variant mi355q_fp8_gemm would pick for a problem
  * (for logs and profiles; static string). */

@@ -430,9 +430,68 @@ def _sdpa_scale(s, default):
     return float(s) if float(s) != 0.0 else default
 
 
+def key_window(valid_seq_len, seq_padding_type, S, batch_rank):
+    """bool [B, 1, ..., 1, S] (batch_rank + 2 dimensions): the keys entry b of the outermost batch dimension may
+    attend to, valid_seq_len[b] of them, the last ones for left padding and the first ones for right padding."""
+    n = torch.as_tensor(valid_seq_len).detach().cpu().to(torch.int64).reshape(-1, 1).clamp(0, S)
+    j = torch.arange(S).reshape(1, S)
+    pad = seq_padding_type.lower()
+    assert pad in ("left", "right")
+    w = (j >= S - n) if pad == "left" else (j < n)
+    if batch_rank == 0:
+        return w.reshape(1, S)
+    return w.reshape(w.shape[0], *([1] * batch_rank), S)
+
+
+def torch_fp8_sdpa_unfused(q, k, v, attn_mask=None, scale=None, is_causal=False, d_scale_q=None, d_scale_k=None, d_scale_v=None,
+                           q_scale_s=None, q_scale_o=None, d_scale_s=None, valid_seq_len=None, seq_padding_type="left"):
+    """hpu::fp8_sdpa_fwd without dropout, fp8 q / k / v: the forward that keeps the probability matrix
+    (Fp8SDPAFwd::AddNode, hpu_ops/backend/sdpa_gen.cpp:340-437; outputs :103-150).  The kernel behind the
+    reference's node is closed; this restates the op as the three steps its outputs imply, each step one of
+    the family's own ops: scores = bf16((q d_scale_q)(k d_scale_k)^T) (fp8_gemm_v2, fp32 accumulation),
+    P = fp8(bf16(softmax(scores scale + mask)) q_scale_s) (softmax_fp8), out = bf16((P d_scale_s)(v d_scale_v))
+    (fp8_gemm_v2), or fp8(out q_scale_o).  Masked scores take the most negative finite bf16-representable value
+    -3e38 instead of -inf, so a row with every key masked attends to all keys evenly.  Returns (out, P, amax_s),
+    amax_s the largest bf16 probability."""
+    f8 = q.dtype
+    dq, dk, dv = _sdpa_scale(d_scale_q, 1.0), _sdpa_scale(d_scale_k, 1.0), _sdpa_scale(d_scale_v, 1.0)
+    qs = _sdpa_scale(q_scale_s, 1.0)
+    ds = _sdpa_scale(d_scale_s, float(torch.tensor(qs, dtype=torch.float32).reciprocal()))
+    qo = _sdpa_scale(q_scale_o, None)
+    L, S = q.shape[-2], k.shape[-2]
+    if scale is None:
+        scale = 1.0 / (q.shape[-1] ** 0.5)
+    f32 = lambda x: torch.tensor(float(x), dtype=torch.float32)
+    sc = (torch.matmul(q.detach().cpu().float(), k.detach().cpu().float().transpose(-2, -1)) * f32(dq) * f32(dk)).to(torch.bfloat16)
+    x = sc.float() * f32(scale)
+    masked = torch.tensor(-3.0e38).to(torch.bfloat16).float()
+    if attn_mask is not None:
+        m_ = attn_mask.detach().cpu()
+        x = x + (torch.where(m_, 0.0, masked) if m_.dtype == torch.bool else m_.to(torch.bfloat16).float().clamp_min(masked))
+    else:
+        keep = None
+        if is_causal:
+            keep = torch.ones(L, S, dtype=torch.bool).tril(0)
+        if valid_seq_len is not None:
+            w = key_window(valid_seq_len, seq_padding_type, S, sc.dim() - 2)
+            keep = w if keep is None else keep & w
+        if keep is not None:
+            x = x + torch.where(keep, 0.0, masked)
+    pb = torch.softmax(x, -1).to(torch.bfloat16)
+    amax_s = pb.float().max() if pb.numel() else torch.tensor(0.0)
+    mx8 = FP8_MAX[f8]
+    P = (pb.float() * f32(qs)).clamp(-mx8, mx8).to(f8)
+    out = (torch.matmul(P.float(), v.detach().cpu().float()) * f32(ds) * f32(dv))
+    if qo is not None:
+        res = (out.to(torch.bfloat16).float() * f32(qo)).clamp(-mx8, mx8).to(f8)
+    else:
+        res = out.to(torch.bfloat16)
+    return res, P, amax_s
+
+
 def torch_fp8_sdpa(q, k, v, attn_mask=None, scale=None, is_causal=False, d_scale_q=None, d_scale_k=None,
                    d_scale_v=None, q_scale_s=None, q_scale_o=None, d_scale_s=None, block=64, quantize_p=True,
-                   key_streams=None):
+                   key_streams=None, valid_seq_len=None, seq_padding_type="left"):
     """hpu::fp8_sdpa_recomp_fwd in inference (requires_backward False, dropout 0), fp8 q/k/v.
 
     The arithmetic of that op lives in a closed device-kernel library (GUID "sdpa_recomp_fwd",
@@ -458,6 +517,12 @@ def torch_fp8_sdpa(q, k, v, attn_mask=None, scale=None, is_causal=False, d_scale
     them -- `splits` ranges of `blocks_per_split` blocks, inside a range `waves` streams that take every
     waves-th block, each stream with its own running maximum (which is what p is rounded against), the
     streams' (m, l, O) merged exactly at the end.  Without rounding the result does not depend on it.
+    valid_seq_len (one integer per entry of the outermost batch dimension; flags VALID_SEQ_LEN_PRESENT,
+    SEQ_PADDING_LEFT / RIGHT, sdpa_gen.cpp:849-851; the wrapper allows it only with is_causal and no mask,
+    Fp8FusedSDPA.py:123-126): entry b attends to its last valid_seq_len[b] keys when the padding is on the
+    left and to its first when it is on the right, on top of the triangular mask.  (Nothing in the
+    reference's tree runs the op with it; this is the reading of the argument names and of the wrapper's
+    contract, pinned in tests/test_oracle_sdpa.py as plain attention on the valid slice.)
     Returns (out, amax_s, amax_o): amax_s = max softmax probability = max_i 1 / l_i, amax_o = max |out|
     before q_scale_o.  Batch dimensions broadcast as torch.matmul's do."""
     f8 = v.dtype
@@ -484,6 +549,8 @@ def torch_fp8_sdpa(q, k, v, attn_mask=None, scale=None, is_causal=False, d_scale
         s = s.masked_fill(~keep, float("-inf"))
     bshape = torch.broadcast_shapes(s.shape[:-2], V.shape[:-2])
     s = s.expand(*bshape, L, S)
+    if valid_seq_len is not None:
+        s = s.masked_fill(~key_window(valid_seq_len, seq_padding_type, S, len(bshape)), float("-inf"))
     V = V.expand(*bshape, S, V.shape[-1])
     step = S if block is None else block
 

@@ -54,7 +54,7 @@ def key_walk(pkg, q, k, v, workspace=True):
     def strides(t):
         st = [0] * (3 - nb) + [0 if t.shape[i] == 1 else t.stride(i) for i in range(nb)]
         return st
-    desc = (ctypes.c_int64 * 27)(*batch, *strides(q), *strides(k), *strides(v), 0, 0, 0, 0, 0, 0,
+    desc = (ctypes.c_int64 * 29)(*batch, *strides(q), *strides(k), *strides(v), 0, 0, 0, 0, 0, 0,
                                  q.shape[-2], k.shape[-2], q.shape[-1], v.shape[-1],
                                  q.stride(-2), k.stride(-2), v.stride(-2), 0, v.shape[-1])
     per = ctypes.c_int64(0)
@@ -306,7 +306,7 @@ def test_few_queries_without_a_workspace(oracle, pkg, dev):
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     out = torch.empty(B, G, HG, 1, D, dtype=torch.bfloat16, device=dev)
     lib = pkg.capi()
-    desc = (ctypes.c_int64 * 27)(B, G, HG, 0, HG * D, D, 0, S * D, 0, 0, S * D, 0, 0, 0, 0, 0, HG * D, D, 1, S, D, D, D, D, D, 0, D)
+    desc = (ctypes.c_int64 * 29)(B, G, HG, 0, HG * D, D, 0, S * D, 0, 0, S * D, 0, 0, 0, 0, 0, HG * D, D, 1, S, D, D, D, D, D, 0, D)
     assert lib.mi355q_fp8_sdpa_workspace_bytes(desc) > 0
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     assert lib.mi355q_fp8_sdpa_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), pkg.E4M3FN, None, 0, out.data_ptr(), pkg.BF16, desc,
@@ -323,7 +323,7 @@ def test_few_queries_with_the_callers_workspace(oracle, pkg, dev):
     gen = torch.Generator().manual_seed(22)
     B, G, HG, S, D = 1, 2, 4, 3000, 128
     lib = pkg.capi()
-    desc = (ctypes.c_int64 * 27)(B, G, HG, 0, HG * D, D, 0, S * D, 0, 0, S * D, 0, 0, 0, 0, 0, HG * D, D, 1, S, D, D, D, D, D, 0, D)
+    desc = (ctypes.c_int64 * 29)(B, G, HG, 0, HG * D, D, 0, S * D, 0, 0, S * D, 0, 0, 0, 0, 0, HG * D, D, 1, S, D, D, D, D, D, 0, D)
     nbytes = lib.mi355q_fp8_sdpa_workspace_bytes(desc)
     assert nbytes > 0 and lib.mi355q_fp8_sdpa_key_splits(desc, None) > 1
     ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
@@ -383,7 +383,7 @@ def test_c_entry_point_rejects_bad_arguments(pkg, dev):
     lib = pkg.capi()
     q = torch.zeros(16, 64, device=dev).to(E4)
     out = torch.zeros(16, 64, device=dev, dtype=torch.bfloat16)
-    desc = (ctypes.c_int64 * 27)(*([1, 1, 1] + [0] * 15 + [16, 16, 64, 64] + [64, 64, 64, 0, 64]))
+    desc = (ctypes.c_int64 * 29)(*([1, 1, 1] + [0] * 15 + [16, 16, 64, 64] + [64, 64, 64, 0, 64]))
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     ok = lib.mi355q_fp8_sdpa_fwd(q.data_ptr(), q.data_ptr(), q.data_ptr(), pkg.E4M3FN, None, 0, out.data_ptr(), pkg.BF16,
                                  desc, 0.125, 0, None, None, None, None, None, 0, st)
@@ -397,3 +397,146 @@ def test_c_entry_point_rejects_bad_arguments(pkg, dev):
     desc[20] = 300                   # head_dim_qk
     assert lib.mi355q_fp8_sdpa_fwd(q.data_ptr(), q.data_ptr(), q.data_ptr(), pkg.E4M3FN, None, 0, out.data_ptr(), pkg.BF16,
                                    desc, 0.125, 0, None, None, None, None, None, 0, st) == 2
+
+
+# ------------------------------------------------------------------ valid_seq_len / seq_padding_type
+
+def run_valid(dev, op, q, k, v, valid, pad, scales=(None, None, None, 128.0, None, 1.0 / 128.0), scalar=False):
+    scale = 1.0 / math.sqrt(q.shape[-1])
+    sc = [0.0 if s is None else float(s) for s in scales] if scalar else [None if s is None else torch.tensor([float(s)], device=dev) for s in scales]
+    return op(q.to(dev), k.to(dev), v.to(dev), None, 0.0, scale, True, False, "None", *sc, False, False, valid.to(dev), pad)
+
+
+@pytest.mark.parametrize("pad", ["left", "right"])
+@pytest.mark.parametrize("layout", ["bhld", "gqa5d", "bld"])
+@pytest.mark.parametrize("S,D", [(200, 64), (333, 128), (130, 256)])
+def test_valid_seq_len(oracle, dev, pad, layout, S, D):
+    """The per-batch key window of the inference forward (sdpa_gen.cpp:849-851, 902-904; Fp8FusedSDPA.py:123-126),
+    incl. the wrapper's 5-d grouped-query layout; counts of 0, 1, kv_len, beyond kv_len, and off the 64-key blocks."""
+    gen = torch.Generator().manual_seed(S + D)
+    B = 6
+    if layout == "bhld":
+        q, k, v = make_qkv(gen, (B, 2, S, D), (B, 2, S, D), (B, 2, S, D))
+    elif layout == "gqa5d":
+        q, k, v = make_qkv(gen, (B, 2, 2, S, D), (B, 2, 1, S, D), (B, 2, 1, S, D))
+    else:
+        q, k, v = make_qkv(gen, (B, S, D), (B, S, D), (B, S, D))
+    valid = torch.tensor([S, 0, 1, S + 50, 64, S - 71], dtype=torch.int32)
+    out = run_valid(dev, torch.ops.hpu.fp8_sdpa_recomp_fwd, q, k, v, valid, pad)[0]
+    ref, _, _ = oracle.torch_fp8_sdpa(q, k, v, is_causal=True, q_scale_s=128.0, d_scale_s=1 / 128.0, valid_seq_len=valid,
+                                      seq_padding_type=pad)
+    check_bf16(out, ref, f"{pad} {layout} {S} {D}", vmax=float(v.float().abs().max()))
+    # rows that see no key are exactly zero; an int64 tensor is taken as well, and so is the alias with .scalar
+    o = out.cpu().float()
+    assert torch.count_nonzero(o[1]) == 0
+    if pad == "left":
+        assert torch.count_nonzero(o[2][..., : S - 1, :]) == 0
+    out2 = run_valid(dev, torch.ops.hpu.fp8_sdpa_recomp_fwd_non_dropout.scalar, q, k, v, valid.long(), pad, scalar=True)[0]
+    assert torch.equal(out2.cpu().view(torch.int16), out.cpu().view(torch.int16))
+
+
+def test_valid_seq_len_through_the_c_abi(oracle, pkg, dev):
+    lib = pkg.capi()
+    gen = torch.Generator().manual_seed(77)
+    B, H, S, D = 3, 2, 300, 128
+    q, k, v = make_qkv(gen, (B, H, S, D), (B, H, S, D), (B, H, S, D))
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    valid = torch.tensor([300, 129, 7], dtype=torch.int32)
+    vd_len = valid.to(dev)
+    out = torch.empty(B, H, S, D, dtype=torch.bfloat16, device=dev)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    host = (ctypes.c_float * 6)(0, 0, 0, 128.0, 0, 1 / 128.0)
+    for pad_left in (1, 0):
+        desc = (ctypes.c_int64 * 29)(1, B, H, 0, H * S * D, S * D, 0, H * S * D, S * D, 0, H * S * D, S * D, 0, 0, 0, 0, H * S * D, S * D,
+                                     S, S, D, D, D, D, D, 0, D, vd_len.data_ptr(), 1 | (pad_left << 32))
+        assert lib.mi355q_fp8_sdpa_workspace_bytes(desc) == 0
+        assert lib.mi355q_fp8_sdpa_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), pkg.E4M3FN, None, 0, out.data_ptr(), pkg.BF16, desc,
+                                       1.0 / math.sqrt(D), 1, None, host, None, None, None, 0, st) == 0
+        ref, _, _ = oracle.torch_fp8_sdpa(q, k, v, is_causal=True, q_scale_s=128.0, d_scale_s=1 / 128.0, valid_seq_len=valid,
+                                          seq_padding_type="left" if pad_left else "right")
+        check_bf16(out, ref, f"c abi pad_left={pad_left}", vmax=float(v.float().abs().max()))
+    desc[28] = 3      # a batch dimension that does not exist
+    assert lib.mi355q_fp8_sdpa_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), pkg.E4M3FN, None, 0, out.data_ptr(), pkg.BF16, desc,
+                                   0.1, 1, None, host, None, None, None, 0, st) == 1
+
+
+def test_valid_seq_len_needs_the_causal_mask(dev):
+    q = torch.zeros(2, 2, 8, 16, device=dev).to(E4)
+    valid = torch.tensor([8, 4], dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError, match="valid_seq_len is supported only"):
+        torch.ops.hpu.fp8_sdpa_recomp_fwd(q, q, q, None, 0.0, 0.25, False, False, "None", *NONE6, False, False, valid, "left")
+    with pytest.raises(RuntimeError, match="one value per batch entry"):
+        torch.ops.hpu.fp8_sdpa_recomp_fwd(q, q, q, None, 0.0, 0.25, True, False, "None", *NONE6, False, False, valid[:1], "left")
+    with pytest.raises(RuntimeError, match="seq_padding_type"):
+        torch.ops.hpu.fp8_sdpa_recomp_fwd(q, q, q, None, 0.0, 0.25, True, False, "None", *NONE6, False, False, valid, "middle")
+
+
+def test_valid_seq_len_measurement_pass_in_bf16(oracle, dev):
+    """bf16 q, k, v (the pass that measures amax_s): the same window."""
+    gen = torch.Generator().manual_seed(3)
+    q, k, v = (torch.randn(2, 2, 70, 32, generator=gen).bfloat16() for _ in range(3))
+    valid = torch.tensor([70, 20], dtype=torch.int32)
+    out = torch.ops.hpu.fp8_sdpa_recomp_fwd(q.to(dev), k.to(dev), v.to(dev), None, 0.0, 0.2, True, False, "None", *NONE6, True, False,
+                                            valid.to(dev), "right")[0]
+    for b, n in enumerate([70, 20]):
+        ref = torch.nn.functional.scaled_dot_product_attention(q[b, :, :n].float(), k[b, :, :n].float(), v[b, :, :n].float(), is_causal=True, scale=0.2)
+        assert torch.allclose(out[b, :, :n].cpu().float(), ref, atol=2e-2, rtol=2e-2)
+
+
+# ------------------------------------------------------------------ fp8_sdpa_fwd: the forward that keeps P
+
+@pytest.mark.parametrize("op_name", ["fp8_sdpa_fwd", "fp8_sdpa_fwd_non_dropout"])
+@pytest.mark.parametrize("case", ["plain", "causal", "bool_mask", "float_mask", "gqa5d", "window_left", "fp8_out", "e5m2"])
+def test_fp8_sdpa_fwd(oracle, dev, op_name, case):
+    """out, P, the dropout-mask placeholder and amax_s of the forward without recomputation against
+    oracle.torch_fp8_sdpa_unfused (Fp8SDPAFwd::AddNode, sdpa_gen.cpp:340-437).  P's codes are compared bit for bit
+    apart from the few entries where the device's exp and the CPU's put a bf16 probability on the other side of a
+    rounding step; out within the GEMM bar of 1e-2 of max |ref| plus what those entries can move."""
+    gen = torch.Generator().manual_seed(len(case))
+    fmt = E5 if case == "e5m2" else E4
+    B, H, L, S, D = 2, 4, 96, 160, 64
+    if case == "gqa5d":
+        q, k, v = make_qkv(gen, (B, 2, 2, L, D), (B, 2, 1, S, D), (B, 2, 1, S, D), fmt)
+    else:
+        q, k, v = make_qkv(gen, (B, H, L, D), (B, H, S, D), (B, H, S, D), fmt)
+    if case == "window_left":
+        q = q[..., :S, :] if L >= S else torch.cat([q, q], -2)[..., :S, :].contiguous()
+    mask, valid, causal = None, None, case in ("causal", "window_left", "gqa5d")
+    if case == "bool_mask":
+        mask = torch.rand(B, 1, L, S, generator=gen) > 0.3
+        mask[..., 0] = True
+    if case == "float_mask":
+        mask = (torch.randn(1, 1, L, S, generator=gen)).bfloat16()
+    if case == "window_left":
+        valid = torch.tensor([S, 45], dtype=torch.int32)
+    qo = 32.0 if case == "fp8_out" else None
+    t = lambda x: None if x is None else torch.tensor([float(x)], device=dev)
+    op = getattr(torch.ops.hpu, op_name)
+    out, P, dm, amax_s = op(q.to(dev), k.to(dev), v.to(dev), None if mask is None else mask.to(dev), 0.0, 0.125, causal, "None",
+                            t(0.5), t(2.0), t(0.25), t(128.0), t(qo), t(1 / 128.0), case == "plain",
+                            None if valid is None else valid.to(dev), "left")
+    ref, Pref, ref_as = oracle.torch_fp8_sdpa_unfused(q, k, v, attn_mask=mask, scale=0.125, is_causal=causal, d_scale_q=0.5, d_scale_k=2.0,
+                                                      d_scale_v=0.25, q_scale_s=128.0, q_scale_o=qo, d_scale_s=1 / 128.0,
+                                                      valid_seq_len=valid, seq_padding_type="left")
+    assert P.dtype == fmt and tuple(P.shape) == tuple(Pref.shape) and tuple(dm.shape) == (1,) and dm.dtype == torch.int8
+    assert amax_s.dtype == torch.float32 and tuple(amax_s.shape) == (1,)
+    assert out.dtype == (fmt if qo is not None else torch.bfloat16) and tuple(out.shape) == tuple(ref.shape)
+    same = P.cpu().view(torch.uint8) == Pref.view(torch.uint8)
+    assert float(same.float().mean()) >= 0.98, f"{case}: only {float(same.float().mean()):.4f} of the probability codes agree"
+    step = Pref.float().abs() * (2.0 ** -2 if fmt == E5 else 2.0 ** -3) + 2.0 ** -6
+    assert ((P.cpu().float() - Pref.float()).abs() <= step).all()
+    err = (out.cpu().float() - ref.float()).abs().max() / ref.float().abs().max()
+    assert float(err) <= (0.13 if qo is not None or fmt == E5 else 2e-2), f"{case}: {float(err)}"
+    if case == "plain":
+        assert abs(float(amax_s.cpu()) - float(ref_as)) <= 2.0 ** -7 * float(ref_as)
+
+
+def test_fp8_sdpa_fwd_measurement_pass_and_checks(dev):
+    gen = torch.Generator().manual_seed(9)
+    q, k, v = (torch.randn(2, 2, 40, 32, generator=gen).bfloat16().to(dev) for _ in range(3))
+    out, P, dm, amax_s = torch.ops.hpu.fp8_sdpa_fwd(q, k, v, None, 0.0, 0.2, True, "None", *NONE6, True, None, "left")
+    w = torch.softmax((q.float() @ k.float().transpose(-2, -1) * 0.2).masked_fill(~torch.ones(40, 40, dtype=torch.bool, device=dev).tril(), float("-inf")), -1)
+    assert P.dtype == torch.bfloat16 and torch.allclose(P.float(), w, atol=1e-2)
+    assert torch.allclose(out.float(), w @ v.float(), atol=3e-2) and abs(float(amax_s) - float(w.max())) < 1e-3
+    with pytest.raises(RuntimeError, match="dropout is not implemented"):
+        torch.ops.hpu.fp8_sdpa_fwd(q, k, v, None, 0.1, 0.2, True, "None", *NONE6, False, None, "left")

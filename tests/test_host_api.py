@@ -50,7 +50,7 @@ def test_library_exports_every_declared_symbol(pkg):
     lib = pkg.capi()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.mi355q_abi_version() == 6
+    assert lib.mi355q_abi_version() == 7
     assert lib.mi355q_status_string(0) == b"ok"
     assert b"invalid" in lib.mi355q_status_string(1)
 
@@ -317,3 +317,63 @@ def test_softmax_fp8_meta_and_errors(pkg):
                       ((x, 4), "[Dd]imension out of range")):
         with pytest.raises((RuntimeError, IndexError), match=msg):
             f(*args)
+
+
+# ------------------------------------------------------------------ the attention ops' boundary
+
+# habana_eager/eager_custom_op_register.cpp:2274, 2278, 2284-2296
+SDPA_SCHEMAS = {
+    ("fp8_sdpa_fwd", ""): "hpu::fp8_sdpa_fwd(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, str softmax_mode, Tensor? d_scale_q, Tensor? d_scale_k, Tensor? d_scale_v, Tensor? q_scale_s, Tensor? q_scale_o, Tensor? d_scale_s, bool is_amax_s, Tensor? valid_seq_len, str seq_padding_type) -> (Tensor, Tensor, Tensor, Tensor)",
+    ("fp8_sdpa_fwd_non_dropout", ""): "hpu::fp8_sdpa_fwd_non_dropout(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, str softmax_mode, Tensor? d_scale_q, Tensor? d_scale_k, Tensor? d_scale_v, Tensor? q_scale_s, Tensor? q_scale_o, Tensor? d_scale_s, bool is_amax_s, Tensor? valid_seq_len, str seq_padding_type) -> (Tensor, Tensor, Tensor, Tensor)",
+    ("fp8_sdpa_recomp_fwd", ""): "hpu::fp8_sdpa_recomp_fwd(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, bool requires_backward, str softmax_mode, Tensor? d_scale_q, Tensor? d_scale_k, Tensor? d_scale_v, Tensor? q_scale_s, Tensor? q_scale_o, Tensor? d_scale_s, bool is_amax_s, bool is_amax_0, Tensor? valid_seq_len, str seq_padding_type) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)",
+    ("fp8_sdpa_recomp_fwd_non_dropout", ""): "hpu::fp8_sdpa_recomp_fwd_non_dropout(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, bool requires_backward, str softmax_mode, Tensor? d_scale_q, Tensor? d_scale_k, Tensor? d_scale_v, Tensor? q_scale_s, Tensor? q_scale_o, Tensor? d_scale_s, bool is_amax_s, bool is_amax_0, Tensor? valid_seq_len, str seq_padding_type) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)",
+    ("fp8_sdpa_recomp_fwd", "scalar"): "hpu::fp8_sdpa_recomp_fwd.scalar(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, bool requires_backward, str softmax_mode, float d_scale_q, float d_scale_k, float d_scale_v, float q_scale_s, float q_scale_o, float d_scale_s, bool is_amax_s, bool is_amax_0, Tensor? valid_seq_len, str seq_padding_type) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)",
+    ("fp8_sdpa_recomp_fwd_non_dropout", "scalar"): "hpu::fp8_sdpa_recomp_fwd_non_dropout.scalar(Tensor q, Tensor k, Tensor v, Tensor? attention_mask, float p, float scale, bool is_causal, bool requires_backward, str softmax_mode, float d_scale_q, float d_scale_k, float d_scale_v, float q_scale_s, float q_scale_o, float d_scale_s, bool is_amax_s, bool is_amax_0, Tensor? valid_seq_len, str seq_padding_type) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)",
+}
+
+
+@pytest.mark.parametrize("key", sorted(SDPA_SCHEMAS))
+def test_attention_schemas_are_the_references(pkg, key):
+    name, overload = key
+    op = getattr(torch.ops.hpu, name)
+    got = str(getattr(op, overload or "default")._schema)
+    assert got == SDPA_SCHEMAS[key]
+
+
+@pytest.mark.parametrize("qdt,fast,qo,expect", [
+    # out, m, linv dtypes of the recompute forward (sdpa_gen.cpp:917-947, eager_custom_op_register.cpp:1795-1808)
+    (E4, False, False, (torch.bfloat16, torch.bfloat16, torch.bfloat16)),
+    (E4, False, True, (E4, torch.bfloat16, torch.bfloat16)),
+    (torch.bfloat16, False, False, (torch.bfloat16, torch.bfloat16, torch.float32)),
+    (torch.bfloat16, True, False, (torch.bfloat16, torch.bfloat16, torch.bfloat16)),
+    (torch.float32, True, False, (torch.float32, torch.float32, torch.float32)),
+    # e5m2 q: treated like e4m3fn here (the reference would give an e5m2 output and Float linv; stated as a deviation)
+    (E5, False, False, (torch.bfloat16, torch.bfloat16, torch.bfloat16)),
+])
+def test_fp8_sdpa_recomp_fwd_meta_dtypes(pkg, qdt, fast, qo, expect):
+    q, k, v = meta((2, 4, 33, 64), qdt), meta((2, 4, 50, 64), qdt), meta((2, 4, 50, 48), qdt)
+    outs = torch.ops.hpu.fp8_sdpa_recomp_fwd.scalar(q, k, v, None, 0.0, 0.125, True, False, "fast" if fast else "None",
+                                                    1.0, 1.0, 1.0, 128.0, 16.0 if qo else 0.0, 0.0, True, True, None, "left")
+    out, m, linv, seed, amax_s, amax_o = outs
+    assert tuple(out.shape) == (2, 4, 33, 48)
+    assert (out.dtype, m.dtype, linv.dtype) == expect
+    assert seed.dtype == torch.int32 and amax_s.dtype == torch.float32 and amax_o.dtype == torch.float32
+    assert all(tuple(t.shape) == (1,) for t in (m, linv, seed, amax_s, amax_o))
+
+
+def test_fp8_sdpa_fwd_meta(pkg):
+    """out, P [batch..., L, S] in q's dtype, the one-element Char dropout mask, Float amax_s
+    (SDPAFwdOutputShapeCommon, sdpa_gen.cpp:103-150; types :412-436)."""
+    q, k, v = meta((2, 2, 2, 33, 64), E4), meta((2, 2, 1, 50, 64), E4), meta((2, 2, 1, 50, 48), E4)
+    sc = meta((1,), torch.float32)
+    out, P, dm, amax_s = torch.ops.hpu.fp8_sdpa_fwd(q, k, v, None, 0.0, 0.125, True, "None", None, None, None, sc, None, None, False, None, "left")
+    assert tuple(out.shape) == (2, 2, 2, 33, 48) and out.dtype == torch.bfloat16
+    assert tuple(P.shape) == (2, 2, 2, 33, 50) and P.dtype == E4
+    assert tuple(dm.shape) == (1,) and dm.dtype == torch.int8 and tuple(amax_s.shape) == (1,) and amax_s.dtype == torch.float32
+    out = torch.ops.hpu.fp8_sdpa_fwd_non_dropout(q, k, v, None, 0.0, 0.125, True, "None", None, None, None, sc, sc, None, False, None, "left")[0]
+    assert out.dtype == E4
+    with pytest.raises(RuntimeError, match="valid_seq_len is supported only"):
+        torch.ops.hpu.fp8_sdpa_fwd(q, k, v, None, 0.0, 0.125, False, "None", None, None, None, None, None, None, False,
+                                   meta((2,), torch.int32), "left")
+    with pytest.raises(RuntimeError, match="dropout is not implemented"):
+        torch.ops.hpu.fp8_sdpa_fwd(q, k, v, None, 0.5, 0.125, True, "None", None, None, None, None, None, None, False, None, "left")

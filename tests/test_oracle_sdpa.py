@@ -182,3 +182,87 @@ def test_reference_test_case_within_its_tolerances(oracle, causal, use_mask, out
     got = out.float() / so if out8 else out.float()
     assert torch.allclose(got, ref.float(), atol=0.4, rtol=1e-3)
     assert (got - ref.float()).abs().max() < 0.2        # in fact far inside the reference's bound
+
+
+# ------------------------------------------------------------------ valid_seq_len / seq_padding_type
+
+@pytest.mark.parametrize("pad", ["left", "right"])
+@pytest.mark.parametrize("gqa", [False, True])
+def test_a_key_window_is_plain_causal_attention_on_the_valid_slice(oracle, pad, gqa):
+    """Entry b attends to valid_seq_len[b] keys (the last ones for left padding, the first ones for right
+    padding) under the triangular mask: its valid rows equal causal attention on the slice that holds only
+    the valid positions.  Exactly so with the whole row taken at once (block=None), where the rounding of the
+    probabilities does not depend on where the blocks fall."""
+    gen = torch.Generator().manual_seed(11)
+    S = 90
+    if gqa:   # the wrapper's grouped-query view [B, G, H / G, L, D] against [B, G, 1, S, D]
+        q = torch.randn(3, 2, 2, S, 16, generator=gen).to(E4)
+        k = torch.randn(3, 2, 1, S, 16, generator=gen).to(E4)
+        v = torch.randn(3, 2, 1, S, 24, generator=gen).to(E4)
+    else:
+        q = torch.randn(3, 2, S, 16, generator=gen).to(E4)
+        k = torch.randn(3, 2, S, 16, generator=gen).to(E4)
+        v = torch.randn(3, 2, S, 24, generator=gen).to(E4)
+    valid = torch.tensor([90, 37, 1], dtype=torch.int32)
+    out, _, _ = oracle.torch_fp8_sdpa(q, k, v, is_causal=True, q_scale_s=128.0, d_scale_s=1 / 128.0, block=None,
+                                      valid_seq_len=valid, seq_padding_type=pad)
+    for b, n in enumerate(valid.tolist()):
+        sl = slice(S - n, S) if pad == "left" else slice(0, n)
+        part, _, _ = oracle.torch_fp8_sdpa(q[b][..., sl, :], k[b][..., sl, :], v[b][..., sl, :], is_causal=True, q_scale_s=128.0,
+                                           d_scale_s=1 / 128.0, block=None)
+        assert torch.equal(out[b][..., sl, :].view(torch.int16), part.view(torch.int16)), (pad, b)
+        # and against float64 attention with the rounding of the probabilities switched off
+        exact, _, _ = oracle.torch_fp8_sdpa(q, k, v, is_causal=True, quantize_p=False, valid_seq_len=valid, seq_padding_type=pad)
+        ref, _ = plain(q[b][..., sl, :].float(), k[b][..., sl, :].float(), v[b][..., sl, :].float(), causal=True)
+        assert torch.equal(exact[b][..., sl, :].view(torch.int16), ref.float().to(torch.bfloat16).expand_as(exact[b][..., sl, :]).contiguous().view(torch.int16))
+
+
+def test_rows_in_front_of_a_left_padded_window_are_zero_and_counts_are_clamped(oracle):
+    gen = torch.Generator().manual_seed(12)
+    q, k, v = (torch.randn(2, 1, 40, 16, generator=gen).to(E4) for _ in range(3))
+    out, _, _ = oracle.torch_fp8_sdpa(q, k, v, is_causal=True, valid_seq_len=torch.tensor([10, 1000]), seq_padding_type="left")
+    assert torch.count_nonzero(out[0, :, :30].float()) == 0 and torch.count_nonzero(out[0, :, 30:].float()) > 0
+    full, _, _ = oracle.torch_fp8_sdpa(q[1:], k[1:], v[1:], is_causal=True)
+    assert torch.equal(out[1:].view(torch.int16), full.view(torch.int16))          # a count beyond kv_len means all keys
+    none, _, _ = oracle.torch_fp8_sdpa(q, k, v, is_causal=True, valid_seq_len=torch.tensor([0, 0]), seq_padding_type="right")
+    assert torch.count_nonzero(none.float()) == 0
+
+
+# ------------------------------------------------------------------ the forward that keeps P (fp8_sdpa_fwd)
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_unfused_forward_is_plain_attention_within_its_roundings(oracle, causal):
+    """out and P of oracle.torch_fp8_sdpa_unfused against float64 attention: P / q_scale_s is the softmax to
+    one e4m3 step (2^-4 relative, plus bf16's 2^-9), rows of P sum to q_scale_s within that, and out is within
+    the bound those steps allow (max |v| 2^-4 plus the bf16 steps of scores and output)."""
+    gen = torch.Generator().manual_seed(21)
+    q = torch.randn(2, 3, 48, 32, generator=gen).to(E4)
+    k = torch.randn(2, 3, 80, 32, generator=gen).to(E4)
+    v = torch.randn(2, 3, 80, 16, generator=gen).to(E4)
+    out, P, amax_s = oracle.torch_fp8_sdpa_unfused(q, k, v, is_causal=causal, d_scale_q=0.5, d_scale_k=2.0, d_scale_v=0.25,
+                                                   q_scale_s=128.0, d_scale_s=1 / 128.0)
+    ref, w = plain(q.float() * 0.5, k.float() * 2.0, v.float() * 0.25, causal=causal)
+    assert P.dtype == E4 and P.shape == (2, 3, 48, 80) and out.dtype == torch.bfloat16
+    p = P.double() / 128.0
+    # bf16 scores move a probability by up to exp(2^-9 |s|) - 1; the test's scores stay below 16 in magnitude
+    assert ((p - w).abs() <= w * 2.0 ** -3 + 1e-3).all()
+    assert ((p.sum(-1) - 1).abs() <= 0.08).all()
+    assert ((out.double() - ref).abs() <= 0.13 * v.float().abs().max() * 0.25 + 1e-2).all()
+    assert abs(float(amax_s) - float(w.max())) <= 0.07 * float(w.max()) + 1e-3
+    if causal:
+        assert torch.count_nonzero(P.float().triu(1)) == 0        # masked entries are exactly zero
+
+
+def test_unfused_forward_is_composed_of_the_family_ops(oracle):
+    """The same numbers out of the oracles of fp8_gemm_v2, softmax_fp8 and fp8_gemm_v2 chained by hand."""
+    gen = torch.Generator().manual_seed(22)
+    q = torch.randn(2, 40, 32, generator=gen).to(E4)
+    k = torch.randn(2, 56, 32, generator=gen).to(E4)
+    v = torch.randn(2, 56, 16, generator=gen).to(E4)
+    out, P, _ = oracle.torch_fp8_sdpa_unfused(q, k, v, scale=0.2, d_scale_q=0.5, d_scale_k=2.0, d_scale_v=0.25, q_scale_s=64.0)
+    for b in range(2):
+        sc = oracle.torch_fp8_gemm(q[b], False, k[b], True, torch.bfloat16, 0.5, 2.0)
+        Pb = oracle.torch_softmax_fp8(sc, -1, 0.2, 64.0)
+        ob = oracle.torch_fp8_gemm(Pb, False, v[b], False, torch.bfloat16, 1.0 / 64.0, 0.25)
+        assert torch.equal(P[b].view(torch.uint8), Pb.view(torch.uint8))
+        assert torch.equal(out[b].view(torch.int16), ob.view(torch.int16))
