@@ -59,7 +59,7 @@ def capi():
     L.mi355q_quantize_rows.argtypes = [vp, i32, i64, i64, vp, i32, f32, vp, vp, vp]
     L.mi355q_silu_mul_quantize_rows.argtypes = [vp, i64, vp, i64, i64, i64, vp, i32, f32, vp, vp, vp, vp]
     L.mi355q_cast_to_fp8.argtypes = [vp, i32, vp, i32, vp, f32, i32, i64, i64, i64, vp, vp]
-    L.mi355q_cast_to_fp8_sr.argtypes = [vp, i32, vp, i32, vp, f32, i32, i64, i64, i64, vp, c.c_uint64, c.c_uint64, vp]
+    L.mi355q_cast_to_fp8_sr.argtypes = [vp, i32, vp, i32, vp, f32, i32, i64, i64, i64, vp, c.c_uint64, c.c_uint64, i32, vp]
     L.mi355q_cast_to_fp8_hybrid.argtypes = [vp, i32, i64, vp, vp, vp, vp, i32, c.c_uint64, c.c_uint64, vp, vp]
     L.mi355q_cast_from_fp8.argtypes = [vp, i32, vp, i32, vp, f32, i32, i64, i64, i64, vp]
     L.mi355q_dequant_4bit.argtypes = [vp, vp, vp, i32, i32, i32, i64, i64, i64, vp, vp]

@@ -189,6 +189,15 @@ __global__ __launch_bounds__(kThreads) void cast_to_fp8_generic(
   if (amax != nullptr) block_amax_commit(am, amax);
 }
 
+// Stochastic rounding with flush to zero (round mode CAST_ROUND_SFTZ of GetCastParams,
+// hpu_ops/backend/fp8_ops.cpp:105-119): a scaled value below the format's smallest normal number
+// becomes a zero of its sign instead of being rounded stochastically among the subnormals.
+template <int FMT>
+__device__ __forceinline__ float flush_below_min_normal(float p) {
+  constexpr float kMinNormal = FMT == MI355Q_E5M2 ? 6.103515625e-05f : 0.015625f;  // 2^-14, 2^-6
+  return __builtin_fabsf(p) < kMinNormal ? __builtin_copysignf(0.0f, p) : p;
+}
+
 // Stochastic-rounding cast: four consecutive elements per thread, any scale
 // broadcast, optional amax.  Not a bandwidth-tuned path (training-side casts of
 // optimizer state use it, the inference path rounds to nearest).
@@ -196,7 +205,7 @@ template <bool BF16_IN, int FMT>
 __global__ __launch_bounds__(kThreads) void cast_to_fp8_sr_kernel(
     const uint8_t* __restrict__ x, uint8_t* __restrict__ y, const float* __restrict__ scale,
     float scale_host, int mode, int64_t n, int64_t mid, int64_t inner, uint64_t seed, uint64_t offset,
-    uint32_t* __restrict__ amax) {
+    int flush_subnormals, uint32_t* __restrict__ amax) {
   const int64_t q = (int64_t)blockIdx.x * kThreads + threadIdx.x;  // index of this thread's quad
   const int64_t i0 = q * 4;
   uint32_t am = 0;
@@ -220,6 +229,7 @@ __global__ __launch_bounds__(kThreads) void cast_to_fp8_sr_kernel(
       }
       const uint32_t a = __float_as_uint(v) & 0x7fffffffu;
       am = am > a ? am : a;
+      if (flush_subnormals) p[e] = flush_below_min_normal<FMT>(p[e]);
     }
     const uint64_t ra = counter_random64(seed, offset + 2 * (uint64_t)q);
     const uint64_t rb = counter_random64(seed, offset + 2 * (uint64_t)q + 1);
@@ -285,6 +295,7 @@ __global__ __launch_bounds__(kAmaxThreads) void cast_to_fp8_hybrid_kernel(
       am = am > a ? am : a;
       p5[i] = BF16_IN ? round_to_bf16(v[i] * s5) : v[i] * s5;
       p4[i] = BF16_IN ? round_to_bf16(v[i] * s4) : v[i] * s4;
+      if (stochastic == 2) p5[i] = flush_below_min_normal<MI355Q_E5M2>(p5[i]);
     }
     if constexpr (VEC == 8) {
       u32x2 o5, o4;
@@ -1105,7 +1116,7 @@ int mi355q_rowwise_amax(const void* x, int x_dtype, int64_t rows, int64_t cols, 
 
 int mi355q_cast_to_fp8_sr(const void* x, int x_dtype, void* y, int fp8_fmt, const float* scale_dev,
                           float scale_host, int scale_mode, int64_t outer, int64_t mid, int64_t inner,
-                          float* amax_out, uint64_t seed, uint64_t offset, void* stream) {
+                          float* amax_out, uint64_t seed, uint64_t offset, int flush_subnormals, void* stream) {
   if (fp8_fmt != MI355Q_E4M3FN && fp8_fmt != MI355Q_E5M2) return MI355Q_ERR_INVALID_ARGUMENT;
   if (x_dtype != MI355Q_F32 && x_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
   if (!scale_args_ok(scale_dev, scale_mode, outer, mid, inner)) return MI355Q_ERR_INVALID_ARGUMENT;
@@ -1121,11 +1132,11 @@ int mi355q_cast_to_fp8_sr(const void* x, int x_dtype, void* y, int fp8_fmt, cons
   uint8_t* yb = static_cast<uint8_t*>(y);
   const unsigned g = (unsigned)grid;
   if (x_dtype == MI355Q_BF16) {
-    if (fp8_fmt == MI355Q_E4M3FN) cast_to_fp8_sr_kernel<true, MI355Q_E4M3FN><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, am);
-    else cast_to_fp8_sr_kernel<true, MI355Q_E5M2><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, am);
+    if (fp8_fmt == MI355Q_E4M3FN) cast_to_fp8_sr_kernel<true, MI355Q_E4M3FN><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, flush_subnormals, am);
+    else cast_to_fp8_sr_kernel<true, MI355Q_E5M2><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, flush_subnormals, am);
   } else {
-    if (fp8_fmt == MI355Q_E4M3FN) cast_to_fp8_sr_kernel<false, MI355Q_E4M3FN><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, am);
-    else cast_to_fp8_sr_kernel<false, MI355Q_E5M2><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, am);
+    if (fp8_fmt == MI355Q_E4M3FN) cast_to_fp8_sr_kernel<false, MI355Q_E4M3FN><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, flush_subnormals, am);
+    else cast_to_fp8_sr_kernel<false, MI355Q_E5M2><<<g, kThreads, 0, st>>>(xb, yb, scale_dev, scale_host, scale_mode, n, mid, inner, seed, offset, flush_subnormals, am);
   }
   return launch_status();
 }

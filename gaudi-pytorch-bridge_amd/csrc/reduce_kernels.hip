@@ -506,11 +506,19 @@ static std::mutex sum_scratch_mutex;
 static void* sum_scratch_ptr[kMaxDevices];  // device address of sum_scratch, per device
 
 // Address of the current device's copy of sum_scratch (looked up on the first call per device).
-inline int sum_scratch_of_current_device(float** out) {
+// The lookup is a runtime call that a stream under capture must not see: a first call on a device
+// whose `stream` is being captured is refused (make one call outside the capture first).
+inline int sum_scratch_of_current_device(float** out, hipStream_t stream) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MI355Q_ERR_LAUNCH;
   std::lock_guard<std::mutex> lock(sum_scratch_mutex);
   if (sum_scratch_ptr[dev] == nullptr) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+      (void)hipGetLastError();
+      return MI355Q_ERR_LAUNCH;
+    }
+    if (cap != hipStreamCaptureStatusNone) return MI355Q_ERR_UNSUPPORTED;
     void* p = nullptr;
     if (hipGetSymbolAddress(&p, HIP_SYMBOL(sum_scratch)) != hipSuccess || p == nullptr) {
       (void)hipGetLastError();
@@ -564,7 +572,7 @@ int mi355q_sum_fp8_static(const void* x, int fp8_fmt, int64_t outer, int64_t red
   if (mi355q_sum_fp8_workspace_bytes(outer, reduce, inner) > (size_t)MI355Q_SUM_FP8_STATIC_SCRATCH_BYTES)
     return MI355Q_ERR_TOO_LARGE;
   float* ws = nullptr;
-  const int got = sum_scratch_of_current_device(&ws);
+  const int got = sum_scratch_of_current_device(&ws, static_cast<hipStream_t>(stream));
   if (got != MI355Q_OK) return got;
   // Nothing has to be cleared between calls: every slice writes its partial sum of every
   // output before sum_finish_kernel, ordered behind it on the stream, reads them.

@@ -190,6 +190,17 @@ std::pair<uint64_t, uint64_t> reserve_random(const Tensor& t, int64_t numel) {
   return gen->philox_engine_inputs((uint64_t)((numel + 1) / 2));
 }
 
+// PT_HPU_STOCHASTIC_ROUNDING_MODE (scripts/env_flags.yaml:753-758, default 1): 1 makes the stochastic casts
+// from bfloat16 to e5m2 flush to zero below the smallest normal number (is_sr_sftz, hpu_ops/fp8_ops.h:52),
+// 0 leaves them plain stochastic rounding.  Read once, as the reference does.
+bool sr_flush_to_zero_mode() {
+  static const bool on = [] {
+    const char* v = std::getenv("PT_HPU_STOCHASTIC_ROUNDING_MODE");
+    return v == nullptr || std::atoi(v) == 1;
+  }();
+  return on;
+}
+
 // One call for both rounding modes.
 int launch_cast_to(const Tensor& x, Tensor& out, const CastScale& cs, float* amax, bool stochastic) {
   const int xd = to_mi355q_dtype(x.scalar_type()), od = to_mi355q_dtype(out.scalar_type());
@@ -197,8 +208,10 @@ int launch_cast_to(const Tensor& x, Tensor& out, const CastScale& cs, float* ama
     return mi355q_cast_to_fp8(x.data_ptr(), xd, out.data_ptr(), od, cs.dev, cs.host, cs.mode, cs.outer, cs.mid,
                               cs.inner, amax, current_stream(x));
   const auto r = reserve_random(x, x.numel());
+  // GetCastParams, fp8_ops.cpp:105-119: SFTZ only from bfloat16 to e5m2
+  const bool sftz = sr_flush_to_zero_mode() && x.scalar_type() == at::kBFloat16 && out.scalar_type() == at::kFloat8_e5m2;
   return mi355q_cast_to_fp8_sr(x.data_ptr(), xd, out.data_ptr(), od, cs.dev, cs.host, cs.mode, cs.outer, cs.mid,
-                               cs.inner, amax, r.first, r.second, current_stream(x));
+                               cs.inner, amax, r.first, r.second, sftz ? 1 : 0, current_stream(x));
 }
 
 // ------------------------------------------------------------ cast_to_fp8_v2
@@ -646,7 +659,9 @@ std::tuple<Tensor, Tensor, Tensor> cast_to_fp8_hybrid(const Tensor& input, const
   if (stochastic_rounding) r = reserve_random(x, x.numel());
   check_status(mi355q_cast_to_fp8_hybrid(x.data_ptr(), to_mi355q_dtype(src), x.numel(), y5.data_ptr(), y4.data_ptr(),
                                          s5.defined() ? s5.data_ptr<float>() : nullptr,
-                                         s4.defined() ? s4.data_ptr<float>() : nullptr, stochastic_rounding ? 1 : 0,
+                                         s4.defined() ? s4.data_ptr<float>() : nullptr,
+                                         // CastToFp8HybridParams, cast_to_fp8_hybrid_gen.cpp:26-35: SFTZ for a bfloat16 input
+                                         !stochastic_rounding ? 0 : (sr_flush_to_zero_mode() && src == at::kBFloat16 ? 2 : 1),
                                          r.first, r.second, is_amax ? amax.data_ptr<float>() : nullptr,
                                          current_stream(x)),
                "mi355q_cast_to_fp8_hybrid");
@@ -743,15 +758,33 @@ Tensor convert_from_uint4(const Tensor& input, const Tensor& scale,
 // do not share.  While a stream is being captured into a graph no buffer is handed out (its memory
 // would belong to the graph's pool, and replays of two graphs could overlap).
 enum TicketWorkspaceOp { kWsW4a8 = 0, kWsSdpa = 1 };
+struct TicketWorkspaceCache {
+  std::mutex mu;
+  std::map<std::tuple<int, void*, int>, Tensor> map;
+};
+TicketWorkspaceCache& ticket_workspace_cache() {
+  // never destroyed: a static Tensor would be freed after the HIP runtime has shut down
+  static auto* cache = new TicketWorkspaceCache();
+  return *cache;
+}
+void ticket_workspace_cache_erase(int device, void* stream, int op) {
+  TicketWorkspaceCache& c = ticket_workspace_cache();
+  std::lock_guard<std::mutex> lock(c.mu);
+  c.map.erase(std::make_tuple(device, stream, op));
+}
 Tensor ticket_workspace(const Tensor& like, size_t bytes, TicketWorkspaceOp op) {
   if (bytes == 0 || c10::hip::currentStreamCaptureStatusMayInitCtx() != c10::hip::CaptureStatus::None) return Tensor();
-  static std::mutex mu;
-  // never destroyed: a static Tensor would be freed after the HIP runtime has shut down
-  static auto* cache = new std::map<std::tuple<int, void*, int>, Tensor>();
-  std::lock_guard<std::mutex> lock(mu);
-  Tensor& t = (*cache)[std::make_tuple((int)like.device().index(), current_stream(like), (int)op)];
+  TicketWorkspaceCache& c = ticket_workspace_cache();
+  std::lock_guard<std::mutex> lock(c.mu);
+  Tensor& t = c.map[std::make_tuple((int)like.device().index(), current_stream(like), (int)op)];
   if (!t.defined() || (size_t)t.numel() < bytes) t = at::zeros({(int64_t)bytes}, like.options().dtype(at::kByte));
   return t;
+}
+// After a call that used the buffer has failed: its counters may be left non-zero (no workgroup then draws a
+// group's last ticket and the output stays unwritten), so the buffer is dropped and the next call starts from a
+// zero-filled one.
+void drop_ticket_workspace(const Tensor& like, TicketWorkspaceOp op) {
+  ticket_workspace_cache_erase((int)like.device().index(), current_stream(like), (int)op);
 }
 
 Tensor w4a8_gemm(const Tensor& A, const Tensor& packed, const Tensor& scale, const c10::optional<Tensor>& zero_point,
@@ -775,6 +808,12 @@ Tensor w4a8_gemm(const Tensor& A, const Tensor& packed, const Tensor& scale, con
                 zero_point->sizes());
   std::vector<int64_t> out_shape(A.sizes().begin(), A.sizes().end());
   out_shape.back() = N;
+  // every pointer the kernel dereferences: a host (or other GPU's) zero_point or bias would be a memory fault on the device
+  TORCH_CHECK(!has_zp || zero_point->device() == A.device(), "mi355q::w4a8_gemm zero_point must be on the same device as A, got ",
+              has_zp ? zero_point->device() : A.device(), " and ", A.device());
+  TORCH_CHECK(!(bias.has_value() && bias->defined()) || bias->device() == A.device(),
+              "mi355q::w4a8_gemm bias must be on the same device as A, got ", (bias.has_value() && bias->defined()) ? bias->device() : A.device(),
+              " and ", A.device());
   if (A.is_meta()) return at::empty(out_shape, A.options().dtype(out_dtype));
   TORCH_CHECK(A.device() == packed.device() && A.device() == scale.device(), "mi355q::w4a8_gemm operands must be on the same device");
   DeviceGuard guard(A.device());
@@ -809,6 +848,7 @@ Tensor w4a8_gemm(const Tensor& A, const Tensor& packed, const Tensor& scale, con
                                   group, out.data_ptr(), to_mi355q_dtype(out_dtype), N, M, N, K, sa_dev, 1.0f, sa_mode,
                                   b.defined() ? b.data_ptr() : nullptr, ws.defined() ? ws.data_ptr() : nullptr,
                                   ws.defined() ? (size_t)ws.numel() : 0, current_stream(a));
+  if (st != MI355Q_OK && ws.defined()) drop_ticket_workspace(a, kWsW4a8);
   TORCH_CHECK(st != MI355Q_ERR_UNSUPPORTED,
               "mi355q::w4a8_gemm takes groups that are multiples of 128, N a multiple of 32 and K a multiple of 16 (got group ",
               group, ", N ", N, ", K ", K, "); expand the weights with hpu::convert_from_", is_signed ? "int4" : "uint4", " for other shapes");
@@ -1215,12 +1255,13 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
     ws = ticket_workspace(qc, ws_bytes, kWsSdpa);
     if (!ws.defined()) ws = at::zeros({(int64_t)ws_bytes}, opts.dtype(at::kByte));
   }
-  check_status(mi355q_fp8_sdpa_fwd(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), to_mi355q_dtype(dt), has_mask ? mk.data_ptr() : nullptr,
-                                   mask_kind, out.data_ptr(), to_mi355q_dtype(out_dt), &d, (float)scale, is_causal ? 1 : 0, sc_dev,
-                                   sc_host, is_amax_s ? amax_s.data_ptr<float>() : nullptr,
-                                   is_amax_o ? amax_o.data_ptr<float>() : nullptr, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes,
-                                   current_stream(q)),
-               "mi355q_fp8_sdpa_fwd");
+  const int st = mi355q_fp8_sdpa_fwd(qc.data_ptr(), kc.data_ptr(), vc.data_ptr(), to_mi355q_dtype(dt), has_mask ? mk.data_ptr() : nullptr,
+                                     mask_kind, out.data_ptr(), to_mi355q_dtype(out_dt), &d, (float)scale, is_causal ? 1 : 0, sc_dev,
+                                     sc_host, is_amax_s ? amax_s.data_ptr<float>() : nullptr,
+                                     is_amax_o ? amax_o.data_ptr<float>() : nullptr, ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes,
+                                     current_stream(q));
+  if (st != MI355Q_OK && ws_bytes > 0) drop_ticket_workspace(qc, kWsSdpa);
+  check_status(st, "mi355q_fp8_sdpa_fwd");
   return SdpaOut(out, m, linv, seed, amax_s, amax_o);
 }
 

@@ -158,19 +158,25 @@ int mi355q_cast_to_fp8(const void* x, int x_dtype, void* y, int fp8_fmt,
  * from the two neighbouring fp8 values.  Element i takes its random bits from a
  * counter-based generator keyed by (seed, offset + i / 2): the same seed and
  * offset give the same output.  x must be fp32 or bf16.
+ * flush_subnormals != 0 is round mode CAST_ROUND_SFTZ ("stochastic flush to zero", the
+ * reference's default for bf16 -> e5m2, flag is_sr_sftz, hpu_ops/fp8_ops.h:52): a scaled value
+ * below the format's smallest normal number (2^-14 for e5m2, 2^-6 for e4m3fn) gives a zero of
+ * its sign; everything else rounds stochastically as above.
  */
 int mi355q_cast_to_fp8_sr(const void* x, int x_dtype, void* y, int fp8_fmt,
                           const float* scale_dev, float scale_host, int scale_mode,
                           int64_t outer, int64_t mid, int64_t inner,
-                          float* amax_out, uint64_t seed, uint64_t offset, void* stream);
+                          float* amax_out, uint64_t seed, uint64_t offset, int flush_subnormals,
+                          void* stream);
 
 /*
  * One read of x (fp32 or bf16, n elements), two casts: y_e5m2 = fp8_e5m2(x * scale_e5m2) and
  * y_e4m3fn = fp8_e4m3fn(x * scale_e4m3fn), plus optionally amax = max|x|.  Replaces the
  * convert_to_fp8_hybrid node of CastToFp8Hybrid::AddNode
  * (hpu_ops/backend/cast_to_fp8_hybrid_gen.cpp:66-100).  Scales are one fp32 value in device
- * memory each, or NULL for 1.  stochastic != 0 rounds the e5m2 output stochastically (random bits
- * as in mi355q_cast_to_fp8_sr); the e4m3fn output always rounds to nearest even.
+ * memory each, or NULL for 1.  stochastic = 1 rounds the e5m2 output stochastically (random bits
+ * as in mi355q_cast_to_fp8_sr), stochastic = 2 does so with flush to zero below 2^-14 (CAST_ROUND_SFTZ,
+ * cast_to_fp8_hybrid_gen.cpp:26-35); the e4m3fn output always rounds to nearest even.
  */
 int mi355q_cast_to_fp8_hybrid(const void* x, int x_dtype, int64_t n, void* y_e5m2, void* y_e4m3fn,
                               const float* scale_e5m2, const float* scale_e4m3fn, int stochastic,
@@ -293,7 +299,8 @@ int mi355q_sum_fp8(const void* x, int fp8_fmt, int64_t outer, int64_t reduce, in
  * nothing.  The stream's device must be the current device.  All calls on one GPU share the
  * buffer: calls that may overlap on one GPU (different streams) race; calls on one stream,
  * or ordered by events, do not.  The first call on a device looks the buffer's address up
- * (hipGetSymbolAddress, once per device): make it before a graph capture starts.
+ * (hipGetSymbolAddress, once per device): make it before a graph capture starts; a first call
+ * on a device whose stream is being captured returns MI355Q_ERR_UNSUPPORTED and launches nothing.
  */
 #define MI355Q_SUM_FP8_STATIC_SCRATCH_BYTES (2u << 20)
 int mi355q_sum_fp8_static(const void* x, int fp8_fmt, int64_t outer, int64_t reduce, int64_t inner,

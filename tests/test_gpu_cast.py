@@ -398,6 +398,38 @@ def test_stochastic_rounding_is_unbiased(dev, dtype, fmt, lo, hi, max_diff):
     assert zz.tolist() == [448.0, -448.0, 448.0, -448.0, 0.0, 0.5]
 
 
+def test_stochastic_flush_to_zero(pkg, dev):
+    """Round mode SFTZ (GetCastParams, hpu_ops/backend/fp8_ops.cpp:105-119; flag is_sr_sftz, default on:
+    scripts/env_flags.yaml:753-758): from bfloat16 to e5m2 a scaled value below 2^-14, the smallest normal e5m2,
+    gives a zero of its sign; at and above it the cast rounds stochastically as before.  Other type pairs keep plain
+    stochastic rounding (subnormal results occur).  The C entry point takes the mode as an argument."""
+    import ctypes
+    tiny = torch.tensor([3e-5, -3e-5, 6.0e-5, -1.5e-5, 2.0 ** -14, -(2.0 ** -14), 7.0e-5, 1.0], dtype=torch.bfloat16)
+    x = tiny.repeat(4096).to(dev)
+    torch.manual_seed(5)
+    y = ops.cast_to_fp8_v2(x, None, True, False, E5)[0].cpu().view(-1, 8)
+    yf = y.float()
+    assert (yf[:, :4] == 0).all() and (y.view(torch.uint8)[:, 1] == 0x80).all() and (y.view(torch.uint8)[:, 0] == 0).all()
+    assert (yf[:, 4] == 2.0 ** -14).all() and (yf[:, 5] == -(2.0 ** -14)).all() and (yf[:, 7] == 1.0).all()
+    assert set(yf[:, 6].unique().tolist()) == {2.0 ** -14, 2.0 ** -14 * 1.25}      # 7e-5 lies between two normal values
+    # fp32 input (and an e4m3fn output) stay plain stochastic rounding: 3e-5 lands on the subnormals 1.5e-5 * {1, 2} ... or 0
+    y32 = ops.cast_to_fp8_v2(x.float(), None, True, False, E5)[0].cpu().float().view(-1, 8)
+    assert set(y32[:, 0].unique().tolist()) == {2.0 ** -15, 2.0 ** -16 * 3} or set(y32[:, 0].unique().tolist()) <= {2.0 ** -16, 2.0 ** -15, 2.0 ** -16 * 3}
+    assert (y32[:, 0] != 0).any()
+    # the C entry point: the same input with the mode switched off rounds among the subnormals
+    lib = pkg.capi()
+    out = torch.empty(x.shape, dtype=E5, device=dev)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for flush, expect_zero in ((1, True), (0, False)):
+        assert lib.mi355q_cast_to_fp8_sr(x.data_ptr(), pkg.BF16, out.data_ptr(), pkg.E5M2, None, 1.0, pkg.SCALE_NONE, x.numel(), 1, 1,
+                                         None, 11, 0, flush, st) == 0
+        first = out.cpu().float().view(-1, 8)[:, 0]
+        assert bool((first == 0).all()) == expect_zero
+    # the hybrid cast's e5m2 output follows the same rule for a bfloat16 input
+    y5 = ops.cast_to_fp8_hybrid(x, None, None, True, False)[0].cpu().float().view(-1, 8)
+    assert (y5[:, :4] == 0).all() and (y5[:, 4] == 2.0 ** -14).all()
+
+
 def test_cast_more_than_2_31_elements(dev):
     """2^31 + 4104 bf16 elements in one call: indices are 64-bit throughout.  The whole-tensor
     result equals the results of two half-size calls, amax equals torch's, and the cast back

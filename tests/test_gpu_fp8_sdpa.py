@@ -262,6 +262,27 @@ def test_long_sequence_properties(oracle, dev):
     assert (o1 - 1.0).abs().max() <= 2.0 ** -4
 
 
+def test_prefill_at_the_benchmark_shape(oracle, dev):
+    """32 query / 8 kv heads, q_len = kv_len = 8192, head_dim 128, causal, in the wrapper's grouped layout (what
+    bench.py times as fp8_sdpa_B1_L8192: 64 query blocks x 32 heads, kv broadcast along the heads of a group):
+    sampled rows of sampled heads against the oracle, every row of one head against the property that v = 1 gives 1."""
+    G, HG, L, D = 8, 4, 8192, 128
+    gen = torch.Generator().manual_seed(8192)
+    q, k, v = make_qkv(gen, (1, G, HG, L, D), (1, G, 1, L, D), (1, G, 1, L, D))
+    sc = (None, None, None, 128.0, None, 1 / 128.0)
+    out = run_op(dev, q, k, v, causal=True, scales=sc)[0].cpu()
+    assert out.shape == (1, G, HG, L, D)
+    rows = [0, 1, 63, 64, 127, 128, 4095, 4096, 5000, 8063, 8064, 8191]
+    for g, h in ((0, 0), (3, 2), (7, 3)):
+        for i in rows:
+            ref, _, _ = oracle.torch_fp8_sdpa(q[0, g, h, i:i + 1], k[0, g, 0, :i + 1], v[0, g, 0, :i + 1], q_scale_s=128.0, d_scale_s=1 / 128.0)
+            check_bf16(out[0, g, h, i:i + 1], ref, f"group {g} head {h} row {i}", vmax=float(v.float().abs().max()))
+    # heads of one group differ (their queries do), groups read their own k / v
+    assert not torch.equal(out[0, 0, 0], out[0, 0, 1]) and not torch.equal(out[0, 0, 0], out[0, 1, 0])
+    o1 = run_op(dev, q, k, torch.ones_like(v.float()).to(E4), causal=True, scales=sc)[0].cpu().float()
+    assert (o1 - 1.0).abs().max() <= 2.0 ** -4
+
+
 @pytest.mark.parametrize("case", [
     # (batch, kv heads, query heads per kv head, q_len, kv_len, head_dim, causal, mask)
     (2, 2, 4, 1, 1000, 128, False, None),        # grouped-query decoding, keys split over workgroups

@@ -247,3 +247,25 @@ def test_meta_and_checks(dev):
         torch.ops.mi355q.w4a8_gemm(torch.empty(4, 128, device="meta", dtype=E4), pk, s, None, True, torch.bfloat16, None, None)
     with pytest.raises(RuntimeError, match="scale must be"):
         torch.ops.mi355q.w4a8_gemm(a, pk, torch.empty(3, 128, device="meta"), None, True, torch.bfloat16, None, None)
+
+
+@pytest.mark.parametrize("M", [16, 64, 256])
+def test_exact_at_the_benchmark_shape(oracle, dev, M):
+    """K = 8192, N = 28672 (the shape bench.py times: 112 strips of 256 columns, K in two parts, one to four row
+    blocks): small-integer activations, power-of-two group scales and zero-points make every partial sum exact, so
+    the whole [M, N] output is compared bit for bit with an integer matmul."""
+    K, N, group = 8192, 28672, 128
+    gen = torch.Generator().manual_seed(8192 + M)
+    q, z, s, pk, pz = weights(oracle, gen, K, N, group, False, True, pow2=True)
+    a = torch.randint(-2, 3, (M, K), generator=gen).float()
+    sa = torch.exp2(torch.randint(-2, 3, (M, 1), generator=gen).float())
+    # (q - z) s group by group on the GPU in float64 (exact: integers below 2^5 times powers of two)
+    qd, zd, sd = q.to(dev).double(), z.to(dev).double(), s.to(dev).double()
+    w = (qd - zd.repeat_interleave(group, 0)) * sd.repeat_interleave(group, 0)
+    expect = ((a.to(dev).double() @ w) * sa.to(dev).double()).cpu()
+    assert expect.abs().max() < 2 ** 24
+    del w, qd, zd, sd
+    out = torch.ops.mi355q.w4a8_gemm(a.to(E4).to(dev), pk.to(dev), s.to(dev), pz.to(dev), False, torch.float32, sa.to(dev), None)
+    assert torch.equal(out.cpu().double(), expect)
+    out2 = torch.ops.mi355q.w4a8_gemm(a.to(E4).to(dev), pk.to(dev), s.to(dev), pz.to(dev), False, torch.float32, sa.to(dev), None)
+    assert torch.equal(out2, out)

@@ -377,3 +377,15 @@ def test_fp8_sdpa_fwd_meta(pkg):
                                    meta((2,), torch.int32), "left")
     with pytest.raises(RuntimeError, match="dropout is not implemented"):
         torch.ops.hpu.fp8_sdpa_fwd(q, k, v, None, 0.5, 0.125, True, "None", None, None, None, None, None, None, False, None, "left")
+
+
+def test_w4a8_gemm_rejects_a_zero_point_or_bias_on_another_device(pkg):
+    """Every pointer the kernel dereferences is checked against A's device before anything is launched (a host
+    pointer read on the GPU is a memory fault); exercised on meta tensors, where nothing can be launched."""
+    A, packed, scale = meta((16, 256), E4), meta((256, 32), torch.int32), meta((2, 256), torch.bfloat16)
+    out = torch.ops.mi355q.w4a8_gemm(A, packed, scale, meta((2, 32), torch.int32), False, torch.bfloat16, None, meta((256,), torch.bfloat16))
+    assert tuple(out.shape) == (16, 256)
+    with pytest.raises(RuntimeError, match="zero_point must be on the same device as A"):
+        torch.ops.mi355q.w4a8_gemm(A, packed, scale, torch.zeros(2, 32, dtype=torch.int32), False, torch.bfloat16, None, None)
+    with pytest.raises(RuntimeError, match="bias must be on the same device as A"):
+        torch.ops.mi355q.w4a8_gemm(A, packed, scale, None, False, torch.bfloat16, None, torch.zeros(256, dtype=torch.bfloat16))
