@@ -544,6 +544,38 @@ def bench_w4a8(oracle, dev, steps, warmup, cpu):
     return out
 
 
+def bench_w4a16(oracle, dev, steps, warmup, cpu):
+    """The same weights against bf16 activations (mi355q::w4a16_gemm): what a GPTQ model with bf16 activations runs in
+    place of convert_from_uint4 -> bf16 [K, N] -> matmul.  Algorithmic bytes: packed weights, scales, zero points, A (bf16)
+    and C; the reference's route would write and read 470 MB of bf16 weights on top."""
+    out = []
+    gen = torch.Generator().manual_seed(SEED)
+    K, N, G = 8192, 28672, 128
+    packs = [torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), generator=gen, dtype=torch.int64).to(torch.int32).to(dev) for _ in range(3)]
+    scale = (torch.rand(K // G, N, generator=gen) * 0.019 + 0.001).bfloat16().to(dev)
+    zp = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // G, N // 8), generator=gen, dtype=torch.int64).to(torch.int32).to(dev)
+    cols = torch.randperm(K, generator=gen)[:82]
+    for M in (16, 64, 256):
+        x = torch.randn(M, K, generator=gen)
+        x[:, cols] *= 20
+        if not want("w4a16", f"M{M}"):
+            continue
+        xb = x.bfloat16().to(dev)
+        ms = time_gpu(lambda i: torch.ops.mi355q.w4a16_gemm(xb, packs[i % 3], scale, zp, False, torch.bfloat16, None), steps, warmup)
+        nbytes = K * N // 2 + (K // G) * N * 2 + (K // G) * N // 2 + 2 * M * K + 2 * M * N
+        c = None
+        if cpu and M == 16:
+            cols_n = 1024
+            pk, sc_c, zp_c, xc = packs[0][:, :cols_n // 8].cpu(), scale[:, :cols_n].cpu(), zp[:, :cols_n // 8].cpu(), xb.cpu()
+            t = time_cpu(lambda: oracle.torch_w4a16_gemm(xc, pk, sc_c, zp_c, False, torch.bfloat16), min_seconds=3.0)
+            c = {"value": round((K * cols_n // 2) / t / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                 "sample": f"M=16, {cols_n} of the 28672 output columns: unpack, (q - z) * s in float64, matmul"}
+        out.append(hbm_entry(f"w4a16_gemm_M{M}", f"w4a16_gemm M={M} K=8192 N=28672: uint4 weights (group 128, bf16 scales, packed zero points) "
+                                                 "x bf16 activations -> bf16", nbytes, ms, steps, "split_rows_kernel + w4a8_wide_kernel<two planes>", c,
+                             extra={"tflops": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 2)}))
+    return out
+
+
 def bench_sdpa(oracle, dev, steps, warmup, cpu):
     """hpu::fp8_sdpa_recomp_fwd, Llama-3-8B attention shapes (32 query heads, 8 key/value heads, head dimension 128),
     causal, e4m3fn q / k / v, q_scale_s = 128, bf16 output.  MFMA-bound: 4 L S D flop per head, halved by the mask."""

@@ -68,6 +68,10 @@ def capi():
                                   vp, i32, i64, vp, i64, i64, i64, i64, i64, i64, i64, vp]
     L.mi355q_w4a8_gemm.argtypes = [vp, i32, i64, vp, i64, vp, i32, vp, i32, i64, vp, i32, i64, i64, i64, i64,
                                    vp, f32, i32, vp, vp, c.c_size_t, vp]
+    L.mi355q_w4a16_gemm.argtypes = [vp, i32, i64, vp, i64, vp, i32, vp, i32, i64, vp, i32, i64, i64, i64, i64, vp, vp, c.c_size_t, i32, vp]
+    L.mi355q_w4a16_gemm_workspace_bytes.argtypes = [i64, i64, i64, i64, i32]
+    L.mi355q_w4a16_gemm_workspace_bytes.restype = c.c_size_t
+    L.mi355q_split_rows_fp8x2.argtypes = [vp, i32, i64, i64, i64, vp, vp, i64, vp, vp]
     L.mi355q_w4a8_gemm_workspace_bytes.argtypes = [i64, i64, i64, i64, i32]
     L.mi355q_w4a8_gemm_workspace_bytes.restype = c.c_size_t
     L.mi355q_fp8_gemm_variant.argtypes = [i32, i64, i32, i64, i64, i64, i64]
@@ -83,7 +87,7 @@ def capi():
     L.mi355q_fp8_sdpa_key_splits.restype = i32
     L.mi355q_fp8_gemm_variant.restype = c.c_char_p
     for name in ("mi355q_amax", "mi355q_rowwise_amax", "mi355q_quantize_rows", "mi355q_silu_mul_quantize_rows", "mi355q_cast_to_fp8", "mi355q_cast_to_fp8_sr", "mi355q_cast_to_fp8_hybrid", "mi355q_cast_from_fp8",
-                 "mi355q_dequant_4bit", "mi355q_fp8_gemm", "mi355q_w4a8_gemm", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8", "mi355q_fp8_sdpa_fwd"):
+                 "mi355q_dequant_4bit", "mi355q_fp8_gemm", "mi355q_w4a8_gemm", "mi355q_w4a16_gemm", "mi355q_split_rows_fp8x2", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8", "mi355q_fp8_sdpa_fwd"):
         getattr(L, name).restype = i32
     L._typed = True
     return L
@@ -118,7 +122,7 @@ SDPA_MASK_NONE, SDPA_MASK_BOOL, SDPA_MASK_BF16, SDPA_MASK_F32 = 0, 1, 2, 3
 EXPORTED_SYMBOLS = (
     "mi355q_abi_version", "mi355q_status_string", "mi355q_amax", "mi355q_rowwise_amax",
     "mi355q_quantize_rows", "mi355q_silu_mul_quantize_rows", "mi355q_cast_to_fp8", "mi355q_cast_to_fp8_sr", "mi355q_cast_to_fp8_hybrid", "mi355q_cast_from_fp8", "mi355q_dequant_4bit", "mi355q_fp8_gemm",
-    "mi355q_w4a8_gemm", "mi355q_w4a8_gemm_workspace_bytes", "mi355q_fp8_gemm_variant", "mi355q_sum_fp8_workspace_bytes", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8", "mi355q_fp8_sdpa_fwd", "mi355q_fp8_sdpa_workspace_bytes", "mi355q_fp8_sdpa_key_splits",
+    "mi355q_w4a8_gemm", "mi355q_w4a8_gemm_workspace_bytes", "mi355q_w4a16_gemm", "mi355q_w4a16_gemm_workspace_bytes", "mi355q_split_rows_fp8x2", "mi355q_fp8_gemm_variant", "mi355q_sum_fp8_workspace_bytes", "mi355q_sum_fp8", "mi355q_sum_fp8_static", "mi355q_softmax_fp8", "mi355q_fp8_sdpa_fwd", "mi355q_fp8_sdpa_workspace_bytes", "mi355q_fp8_sdpa_key_splits",
 )
 
 _load()

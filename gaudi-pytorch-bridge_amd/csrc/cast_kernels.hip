@@ -430,6 +430,59 @@ __global__ __launch_bounds__(kThreads) void rowwise_amax_kernel(const uint8_t* _
   }
 }
 
+// ------------------------------------------------- bf16 rows as two fp8 planes
+//
+// For the int4-weight GEMM on 16-bit activations (mi355q_w4a16_gemm): a bf16 value has 8 significant
+// bits, an e4m3 value 4, so with a power-of-two row scale s (the largest with max |a| s <= 448)
+//   hi = e4m3(a s)  (round to nearest even)      lo = e4m3((a s - hi) 16)
+// give a s = hi + lo / 16 exactly for every element whose hi is a normal number (the remainder then has
+// at most 4 significant bits), and to within 2^-14 (3e-8 of the row's 448) for the small elements whose
+// remainder falls below e4m3's subnormal spacing.  The matrix unit multiplies the two planes at the fp8
+// rate; 1 / s goes to the GEMM's per-row factor.  One workgroup per row, two passes over it (the second
+// out of the cache).  A row of zeros takes s = 1.
+__global__ __launch_bounds__(kThreads) void split_rows_kernel(const uint16_t* __restrict__ x, int64_t ldx, int64_t cols,
+                                                              uint8_t* __restrict__ hi, uint8_t* __restrict__ lo, int64_t ld,
+                                                              float* __restrict__ scale_inv) {
+  __shared__ uint32_t wave_part[kThreads / 64];
+  const int64_t row = blockIdx.x;
+  const uint16_t* xr = x + row * ldx;
+  uint32_t am = 0;
+  for (int64_t c = threadIdx.x; c < cols; c += kThreads) {
+    const uint32_t a = ((uint32_t)xr[c] & 0x7fffu) << 16;
+    am = am > a ? am : a;
+  }
+  am = wave_max_u32(am);
+  if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = am;
+  __syncthreads();
+  uint32_t r = wave_part[0];
+#pragma unroll
+  for (int w = 1; w < kThreads / 64; ++w) r = r > wave_part[w] ? r : wave_part[w];
+  // amax = m 2^ea with 1 <= m < 2; 448 = 1.75 2^8: s = 2^(8 - ea) when m <= 1.75, else 2^(7 - ea)
+  int e = 0;
+  if (r != 0u && r < 0x7f800000u) {
+    const int ea = (int)(r >> 23) - 127;
+    e = ((r & 0x007fffffu) <= 0x00600000u ? 8 : 7) - (r >= 0x00800000u ? ea : -126);
+    e = e > 126 ? 126 : (e < -126 ? -126 : e);
+  }
+  const float s = __uint_as_float((uint32_t)(e + 127) << 23);
+  if (threadIdx.x == 0) scale_inv[row] = __uint_as_float((uint32_t)(127 - e) << 23);
+  uint8_t* hr = hi + row * ld;
+  uint8_t* lr = lo + row * ld;
+  // four columns per step; ld is a multiple of 16, columns from `cols` to ld are written as zeros
+  for (int64_t c = (int64_t)threadIdx.x * 4; c < ld; c += (int64_t)kThreads * 4) {
+    float p[4], q[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) p[i] = c + i < cols ? __uint_as_float((uint32_t)xr[c + i] << 16) * s : 0.0f;
+    const uint32_t h = cvt_fp8x4<MI355Q_E4M3FN>(p[0], p[1], p[2], p[3]);
+    cvt_f32x4<MI355Q_E4M3FN>(h, q[0], q[1], q[2], q[3]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = (p[i] - q[i]) * 16.0f;   // exact: p and hi agree in their leading bits
+    const uint32_t l = cvt_fp8x4<MI355Q_E4M3FN>(q[0], q[1], q[2], q[3]);
+    *reinterpret_cast<uint32_t*>(hr + c) = h;
+    *reinterpret_cast<uint32_t*>(lr + c) = l;
+  }
+}
+
 // ------------------------------------------------- dynamic per-row quantisation
 //
 // One pass of "per-row amax -> scale = target / amax -> cast with that scale":
@@ -1170,6 +1223,18 @@ int mi355q_cast_to_fp8_hybrid(const void* x, int x_dtype, int64_t n, void* y_e5m
     if (x_dtype == MI355Q_BF16) cast_to_fp8_hybrid_kernel<true, 1><<<grid_for(rest), kAmaxThreads, 0, st>>>(xb, y5, y4, scale_e5m2, scale_e4m3fn, done, rest, stochastic, seed, offset, am);
     else cast_to_fp8_hybrid_kernel<false, 1><<<grid_for(rest), kAmaxThreads, 0, st>>>(xb, y5, y4, scale_e5m2, scale_e4m3fn, done, rest, stochastic, seed, offset, am);
   }
+  return launch_status();
+}
+
+int mi355q_split_rows_fp8x2(const void* x, int x_dtype, int64_t ldx, int64_t rows, int64_t cols, void* hi, void* lo,
+                            int64_t ld, float* scale_inv, void* stream) {
+  if (x_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (rows < 0 || cols < 0 || ldx < cols || ld < cols) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (rows == 0) return MI355Q_OK;
+  if (x == nullptr || hi == nullptr || lo == nullptr || scale_inv == nullptr) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (ld % 16 != 0 || !aligned(hi, 16) || !aligned(lo, 16) || rows > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
+  split_rows_kernel<<<(unsigned)rows, kThreads, 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const uint16_t*>(x), ldx, cols, static_cast<uint8_t*>(hi), static_cast<uint8_t*>(lo), ld, scale_inv);
   return launch_status();
 }
 

@@ -757,7 +757,7 @@ Tensor convert_from_uint4(const Tensor& input, const Tensor& scale,
 // which is all the sharing the buffer allows; the two ops lay their counters out differently and
 // do not share.  While a stream is being captured into a graph no buffer is handed out (its memory
 // would belong to the graph's pool, and replays of two graphs could overlap).
-enum TicketWorkspaceOp { kWsW4a8 = 0, kWsSdpa = 1 };
+enum TicketWorkspaceOp { kWsW4a8 = 0, kWsSdpa = 1, kWsW4a16 = 2 };
 struct TicketWorkspaceCache {
   std::mutex mu;
   std::map<std::tuple<int, void*, int>, Tensor> map;
@@ -853,6 +853,63 @@ Tensor w4a8_gemm(const Tensor& A, const Tensor& packed, const Tensor& scale, con
               "mi355q::w4a8_gemm takes groups that are multiples of 128, N a multiple of 32 and K a multiple of 16 (got group ",
               group, ", N ", N, ", K ", K, "); expand the weights with hpu::convert_from_", is_signed ? "int4" : "uint4", " for other shapes");
   check_status(st, "mi355q_w4a8_gemm");
+  return out;
+}
+
+// mi355q::w4a16_gemm: the same weights against bf16 activations (what the reference gets from
+// convert_from_[u]int4 to bf16 followed by a bf16 matmul, hpu_ops/backend/int4_ops.cpp:40-56), without the
+// bf16 [K, N] matrix: the activations go through the matrix unit as two fp8 planes (mi355q_w4a16_gemm).
+Tensor w4a16_gemm(const Tensor& A, const Tensor& packed, const Tensor& scale, const c10::optional<Tensor>& zero_point,
+                  bool is_signed, at::ScalarType out_dtype, const c10::optional<Tensor>& bias) {
+  TORCH_CHECK(A.scalar_type() == at::kBFloat16, "mi355q::w4a16_gemm A must be bfloat16, got ", A.scalar_type());
+  TORCH_CHECK(packed.scalar_type() == at::kInt && packed.dim() == 2,
+              "mi355q::w4a16_gemm packed weights must be a 2-D int32 tensor [K, N / 8], got ", packed.scalar_type(), " ", packed.sizes());
+  TORCH_CHECK(out_dtype == at::kFloat || out_dtype == at::kBFloat16, "mi355q::w4a16_gemm out_dtype must be float or bfloat16, got ", out_dtype);
+  TORCH_CHECK(A.dim() >= 1, "mi355q::w4a16_gemm A must have at least 1 dimension");
+  const int64_t K = packed.size(0), N = packed.size(1) * 8;
+  TORCH_CHECK(A.size(-1) == K, "Common dimension sizes of matmul inputs should be the same. Got ", A.size(-1), " and ", K);
+  TORCH_CHECK(scale.dim() == 2 && scale.size(1) == N && scale.size(0) > 0 && K % scale.size(0) == 0,
+              "mi355q::w4a16_gemm scale must be [K / group, N] = [*, ", N, "], got ", scale.sizes());
+  const int64_t groups = scale.size(0), group = K / groups;
+  const bool has_zp = zero_point.has_value() && zero_point->defined();
+  if (has_zp)
+    TORCH_CHECK(zero_point->scalar_type() == at::kInt && zero_point->dim() == 2 && zero_point->size(0) == groups &&
+                    zero_point->size(1) == N / 8,
+                "mi355q::w4a16_gemm zero_point must be packed int32 [K / group, N / 8], got ", zero_point->scalar_type(), " ",
+                zero_point->sizes());
+  const bool has_bias = bias.has_value() && bias->defined();
+  TORCH_CHECK(!has_bias || bias->numel() == N, "Bias must be size ", N, " but got ", has_bias ? bias->numel() : 0);
+  std::vector<int64_t> out_shape(A.sizes().begin(), A.sizes().end());
+  out_shape.back() = N;
+  TORCH_CHECK(A.device() == packed.device() && A.device() == scale.device(), "mi355q::w4a16_gemm operands must be on the same device");
+  TORCH_CHECK(!has_zp || zero_point->device() == A.device(), "mi355q::w4a16_gemm zero_point must be on the same device as A");
+  TORCH_CHECK(!has_bias || bias->device() == A.device(), "mi355q::w4a16_gemm bias must be on the same device as A");
+  if (A.is_meta()) return at::empty(out_shape, A.options().dtype(out_dtype));
+  DeviceGuard guard(A.device());
+  Tensor a = A.contiguous();
+  const int64_t M = K ? a.numel() / K : 0;
+  Tensor out = at::empty(out_shape, A.options().dtype(out_dtype));
+  if (out.numel() == 0) return out;
+  Tensor w = packed.contiguous(), s = scale.contiguous(), z, b;
+  if (has_zp) z = zero_point->contiguous();
+  if (has_bias) b = bias->to(out_dtype).contiguous();
+  MI355Q_OP_INFO("w4a16_gemm : A=" << A.sizes() << " packed=" << packed.sizes() << " group=" << group << " signed=" << is_signed);
+  const size_t bytes = mi355q_w4a16_gemm_workspace_bytes(M, N, K, group, to_mi355q_dtype(s.scalar_type()));
+  // the buffer kept per stream starts zero-filled, which the split over K needs; under graph capture a buffer of the
+  // graph's own, and K in one piece
+  Tensor ws = ticket_workspace(a, bytes, kWsW4a16);
+  const bool split = ws.defined();
+  if (!split) ws = at::empty({(int64_t)bytes}, A.options().dtype(at::kByte));
+  const int st = mi355q_w4a16_gemm(a.data_ptr(), MI355Q_BF16, K, w.data_ptr<int32_t>(), N / 8, s.data_ptr(),
+                                   to_mi355q_dtype(s.scalar_type()), has_zp ? z.data_ptr<int32_t>() : nullptr, is_signed ? 1 : 0, group,
+                                   out.data_ptr(), to_mi355q_dtype(out_dtype), N, M, N, K, has_bias ? b.data_ptr() : nullptr,
+                                   ws.data_ptr(), (size_t)ws.numel(), split ? 1 : 0, current_stream(a));
+  if (st != MI355Q_OK && split) drop_ticket_workspace(a, kWsW4a16);
+  TORCH_CHECK(st != MI355Q_ERR_UNSUPPORTED,
+              "mi355q::w4a16_gemm takes groups of 128 with bfloat16 scales, N a multiple of 32 and K a multiple of 16 (got group ", group,
+              ", ", s.scalar_type(), " scales, N ", N, ", K ", K, "); expand the weights with hpu::convert_from_", is_signed ? "int4" : "uint4",
+              " for other shapes");
+  check_status(st, "mi355q_w4a16_gemm");
   return out;
 }
 
@@ -1633,6 +1690,7 @@ TORCH_LIBRARY(mi355q, m) {
   m.def("mi355q::quantize_rows(Tensor input, ScalarType dtype) -> (Tensor, Tensor)");
   m.def("mi355q::silu_mul_quantize_rows(Tensor gate, Tensor up, ScalarType dtype) -> (Tensor, Tensor)");
   m.def("mi355q::w4a8_gemm(Tensor A, Tensor packed, Tensor scale, Tensor? zero_point, bool is_signed, ScalarType out_dtype, Tensor? A_scale_inv=None, Tensor? bias=None) -> Tensor");
+  m.def("mi355q::w4a16_gemm(Tensor A, Tensor packed, Tensor scale, Tensor? zero_point, bool is_signed, ScalarType out_dtype, Tensor? bias=None) -> Tensor");
   m.def("mi355q::scaled_mm(Tensor self, Tensor mat2, Tensor scale_a, Tensor scale_b, Tensor? bias=None, Tensor? scale_result=None, ScalarType? out_dtype=None, bool use_fast_accum=False) -> Tensor");
 }
 
@@ -1672,6 +1730,7 @@ TORCH_LIBRARY_IMPL(mi355q, CUDA, m) {
   m.impl("scaled_mm", scaled_mm);
   m.impl("silu_mul_quantize_rows", silu_mul_quantize_rows_op);
   m.impl("w4a8_gemm", w4a8_gemm);
+  m.impl("w4a16_gemm", w4a16_gemm);
 }
 TORCH_LIBRARY_IMPL(mi355q, Meta, m) {
   m.impl("amax", amax_op);
@@ -1680,4 +1739,5 @@ TORCH_LIBRARY_IMPL(mi355q, Meta, m) {
   m.impl("scaled_mm", scaled_mm);
   m.impl("silu_mul_quantize_rows", silu_mul_quantize_rows_op);
   m.impl("w4a8_gemm", w4a8_gemm);
+  m.impl("w4a16_gemm", w4a16_gemm);
 }

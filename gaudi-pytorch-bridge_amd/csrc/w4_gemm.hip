@@ -64,6 +64,9 @@ struct W4Args {
   int ksplit;
   uint32_t* tickets;       // one per strip, zero between launches
   float* partials;         // [ksplit][strips] partial sums of 32 x 256, in the consumers' register order
+  // 16-bit activations as two fp8 planes (wide kernel, A16): g.A holds the leading part of every value and a_lo,
+  // with the same pitch, 16 times what is left of it (split_rows_kernel); a = (A + a_lo / 16) / row scale
+  const uint8_t* a_lo;
 };
 
 template <int BM>
@@ -516,8 +519,8 @@ __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
 // first operand and column j of the second meet in lane j + 16 (i / 4), register i % 4.
 constexpr int kW4WideBN = 256;
 constexpr int kW4WidePacked = kBK * kW4WideBN / 2;
-constexpr int w4_wide_stage(int bm) { return bm * kBK + kW4WidePacked + kW4ScaleRow + kW4ZpRow; }
-constexpr int w4_wide_stages(int bm) { return (160 * 1024 - 1024) / w4_wide_stage(bm); }
+constexpr int w4_wide_stage(int bm, bool a16 = false) { return bm * kBK * (a16 ? 2 : 1) + kW4WidePacked + kW4ScaleRow + kW4ZpRow; }
+constexpr int w4_wide_stages(int bm, bool a16 = false) { return (160 * 1024 - 1024) / w4_wide_stage(bm, a16); }
 constexpr int w4_wide_partial_bytes(int bm) { return bm * kW4WideBN * 4; }  // per workgroup and part of K
 constexpr int kW4WideConsumers = 8;
 constexpr int kW4WideThreads = (kW4WideConsumers + kW4ColWaves) * 64;
@@ -531,17 +534,22 @@ __device__ __forceinline__ f32x4 w4_mfma16(const u32x4& plane, const i32x8& fa, 
 
 // ROWS: 16 (the 16x16x128 form), 32, or 64 (row blocks of 64 along grid.y; one set of accumulators, folded into
 // the totals at the start of the next stage, for the registers of three waves per SIMD).
-template <int FMT_A, bool HAS_Z, int ROWS>
+//
+// A16: the activations are 16-bit values handed over as two fp8 planes of the same shape (W4A16: see
+// split_rows_kernel): every stage carries both planes' tiles, and every product runs on both with the same weight
+// fragments, the second plane's MFMAs with a block scale of 2^-4.  Twice the matrix work, the weights still read once.
+template <int FMT_A, bool HAS_Z, int ROWS, bool A16 = false>
 __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
   constexpr bool M16 = ROWS == 16;
   constexpr int BM = ROWS == 64 ? 64 : 32, MT = BM / 32;
   constexpr int kConsumers = kW4WideConsumers;
-  constexpr int S = w4_wide_stages(BM), kStage = w4_wide_stage(BM);
-  constexpr int kOffPacked = BM * kBK, kOffScale = kOffPacked + kW4WidePacked, kOffZp = kOffScale + kW4ScaleRow;
+  constexpr int S = w4_wide_stages(BM, A16), kStage = w4_wide_stage(BM, A16);
+  constexpr int kOffLo = BM * kBK;  // the second plane's tile (A16)
+  constexpr int kOffPacked = BM * kBK * (A16 ? 2 : 1), kOffScale = kOffPacked + kW4WidePacked, kOffZp = kOffScale + kW4ScaleRow;
   constexpr int NV = M16 ? 8 : 16 * MT;  // results per consumer lane
   using LA = DmaLoader<true, BM, kBK, kW4ColWaves>;
   using GA = TileGeom<true, BM, kBK>;
-  constexpr int kOps = 4 + LA::kPerWave + 1;  // four 1 KiB regions of weights, A, and the scale or zero-point row
+  constexpr int kOps = 4 + LA::kPerWave * (A16 ? 2 : 1) + 1;  // four 1 KiB regions of weights, A, and the scale or zero-point row
   static_assert(S >= 3 && (S - 2) * kOps <= 63, "vmcnt holds 6 bits");
   static_assert(kStage % 1024 == 0, "stages stay 1 KiB aligned");
   static_assert(kConsumers * epilogue_stage_floats<MT, 1>() * 4 <= S * kStage, "epilogue area overlays the ring");
@@ -554,6 +562,7 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
   GemmArgs g = a.g;
   const int m_base = blockIdx.y * BM;
   g.A += (int64_t)m_base * g.lda;
+  const uint8_t* a_lo = A16 ? a.a_lo + (int64_t)m_base * g.lda : nullptr;
   g.C += (int64_t)m_base * g.ldc * (g.out_bf16 ? 2 : 4);
   if (g.sa_mode == MI355Q_GS_PER_ROW) g.sa += m_base;
   g.M = g.M - m_base < BM ? g.M - m_base : BM;
@@ -566,6 +575,7 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
   const int k_begin = kt0 * kBK;
   g.K = (g.K < kt1 * kBK ? g.K : kt1 * kBK) - k_begin;
   g.A += k_begin;
+  if constexpr (A16) a_lo += k_begin;
   const uint8_t* packed = a.packed + (int64_t)k_begin * a.ld_packed;
   const uint8_t* scale = a.scale + (int64_t)kt0 * g.N * 2;
   const uint8_t* zp = a.zp ? a.zp + (int64_t)kt0 * (g.N / 2) : nullptr;
@@ -579,10 +589,15 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
   for (int e = 0; e < NV; ++e) total[e] = 0.0f;
 
   if (producer) {
-    LA la;
+    LA la, la2;
     la.set_lane_offsets(g.lda, wq);
     la.set_tile(g.A, g.lda, 0, g.M, g.K);
     la.clamp_rows(g.lda, g.M);
+    if constexpr (A16) {
+      la2.set_lane_offsets(g.lda, wq);
+      la2.set_tile(a_lo, g.lda, 0, g.M, g.K);
+      la2.clamp_rows(g.lda, g.M);
+    }
     // Producer wq loads k-rows 32 wq .. 32 wq + 31, four regions of 8 rows of 128 bytes.  A lane writes
     // slot lane % 8 of row lane / 8 of its region; rows 8 r + lane / 8 have (row / 2) % 8 = 4 (r % 2) +
     // lane / 16, so that is what the lane's slot is XORed with on the memory side.
@@ -614,6 +629,10 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
       wp.step(packed_step);
       static_for<LA::kPerWave>([&](auto ic) { la.template issue_one<decltype(ic)::value, true>(lds + off, stage * kBK, g.K); });
       la.advance();
+      if constexpr (A16) {
+        static_for<LA::kPerWave>([&](auto ic) { la2.template issue_one<decltype(ic)::value, true>(lds + off + kOffLo, stage * kBK, g.K); });
+        la2.advance();
+      }
       w4_dma16(wr.rsrc(row_cap), lane * 16, base + row_dst);
       wr.step(row_step);
     };
@@ -638,7 +657,13 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         const u32x4 lo = *reinterpret_cast<const u32x4*>(st + GA::lds_offset(m, 2 * gk));
         const u32x4 hi = *reinterpret_cast<const u32x4*>(st + GA::lds_offset(m, 2 * gk + 1));
         const i32x8 fa = {(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-        const f32x4 r = w4_mfma16<FMT_A>(ones, fa, f32x4{0.f, 0.f, 0.f, 0.f}, 127);
+        f32x4 r = w4_mfma16<FMT_A>(ones, fa, f32x4{0.f, 0.f, 0.f, 0.f}, 127);
+        if constexpr (A16) {
+          const u32x4 lo2 = *reinterpret_cast<const u32x4*>(st + kOffLo + GA::lds_offset(m, 2 * gk));
+          const u32x4 hi2 = *reinterpret_cast<const u32x4*>(st + kOffLo + GA::lds_offset(m, 2 * gk + 1));
+          const i32x8 fb = {(int)lo2[0], (int)lo2[1], (int)lo2[2], (int)lo2[3], (int)hi2[0], (int)hi2[1], (int)hi2[2], (int)hi2[3]};
+          r = w4_mfma16<FMT_A>(ones, fb, r, 123);
+        }
         // every lane holds the sum of its row (lane % 16) and every lane stores it: a store under a lane mask would
         // take the MFMA, whose result only those lanes used, under the mask with it
         row_sums[slot][lane & 15] = r[0];
@@ -652,6 +677,13 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
           const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
           f32x16 r = w4_mfma<FMT_A, 127>(ones, fa[0], zero);
           r = w4_mfma<FMT_A, 127>(ones, fa[1], r);
+          if constexpr (A16) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+              static_for<2>([&](auto pc) { read_fragment_part<true, BM, decltype(pc)::value>(st + kOffLo, 32 * i, ks, fa[ks]); });
+            r = w4_mfma<FMT_A, 123>(ones, fa[0], r);
+            r = w4_mfma<FMT_A, 123>(ones, fa[1], r);
+          }
           row_sums[slot][32 * i + (lane & 31)] = r[0];  // by every lane, as above
         });
       }
@@ -740,6 +772,11 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
           for (int p = 0; p < 2; ++p)
             wt[t][p] = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LDS_AS i32x2*)((LDS_AS uint8_t*)st + poff[t][p]));
         const u32x4 alo = *reinterpret_cast<const u32x4*>(st + aoff0), ahi = *reinterpret_cast<const u32x4*>(st + aoff1);
+        u32x4 blo = alo, bhi = ahi;
+        if constexpr (A16) {
+          blo = *reinterpret_cast<const u32x4*>(st + kOffLo + aoff0);
+          bhi = *reinterpret_cast<const u32x4*>(st + kOffLo + aoff1);
+        }
         u32x2 snew[2];
         uint32_t znew[2] = {0u, 0u};
 #pragma unroll
@@ -760,6 +797,11 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
           }
           acc[B][t] = w4_mfma16<FMT_A>(hi, fa, f32x4{0.f, 0.f, 0.f, 0.f}, 130);
           acc[B][t] = w4_mfma16<FMT_A>(lo, fa, acc[B][t], 128);
+          if constexpr (A16) {
+            const i32x8 fb = {(int)blo[0], (int)blo[1], (int)blo[2], (int)blo[3], (int)bhi[0], (int)bhi[1], (int)bhi[2], (int)bhi[3]};
+            acc[B][t] = w4_mfma16<FMT_A>(hi, fb, acc[B][t], 126);
+            acc[B][t] = w4_mfma16<FMT_A>(lo, fb, acc[B][t], 124);
+          }
         }
         // the stage before this one, whose MFMAs finished long ago, behind the MFMAs just issued
         if constexpr (HAVE_PREV) fold(std::integral_constant<int, 1 - B>{}, (slot - 1) & (kW4SumRing - 1));
@@ -834,11 +876,13 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
           wt[j] = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LDS_AS i32x2*)((LDS_AS uint8_t*)st + poff[j]));
         // the A fragments of both halves of the stage up front, or (64 rows) of the second half behind the MFMAs of
         // the first, for the registers
-        i32x8 fa[2][MT];
+        i32x8 fa[2][MT], fb[A16 ? 2 : 1][MT];
         auto read_a = [&](int ks) {
           static_for<MT>([&](auto ic) {
             static_for<2>([&](auto pc) {
               read_fragment_part<true, BM, decltype(pc)::value>(st, 32 * decltype(ic)::value, ks, fa[MT == 1 ? ks : 0][decltype(ic)::value]);
+              if constexpr (A16)
+                read_fragment_part<true, BM, decltype(pc)::value>(st + kOffLo, 32 * decltype(ic)::value, ks, fb[MT == 1 ? ks : 0][decltype(ic)::value]);
             });
           });
         };
@@ -865,6 +909,10 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
             if (ks == 0) acc[B][i] = w4_mfma<FMT_A, 130>(hi, fa[f][i], zero);
             else acc[B][i] = w4_mfma<FMT_A, 130>(hi, fa[f][i], acc[B][i]);
             acc[B][i] = w4_mfma<FMT_A, 128>(lo, fa[f][i], acc[B][i]);
+            if constexpr (A16) {
+              acc[B][i] = w4_mfma<FMT_A, 126>(hi, fb[f][i], acc[B][i]);
+              acc[B][i] = w4_mfma<FMT_A, 124>(lo, fb[f][i], acc[B][i]);
+            }
           });
           if constexpr (MT == 2) {
             if (ks == 0) read_a(1);
@@ -1052,9 +1100,114 @@ void w4a8_launch_by_m(const W4Args& a, hipStream_t st) {
   }
 }
 
+// The wide kernel on two fp8 planes of 16-bit activations (always this kernel: K in one part where the plan would
+// rather use the 128-column strips, which have no two-plane form).
+inline void w4a16_launch(const W4Args& a, hipStream_t st) {
+  const bool z = a.zp != nullptr || a.is_signed;
+  const unsigned strips = (unsigned)((a.g.N + kW4WideBN - 1) / kW4WideBN);
+  constexpr int F = MI355Q_E4M3FN;
+  if (a.g.M <= 16) {
+    const dim3 grid(strips * (unsigned)a.ksplit);
+    if (z) w4a8_wide_kernel<F, true, 16, true><<<grid, kW4WideThreads, 0, st>>>(a);
+    else w4a8_wide_kernel<F, false, 16, true><<<grid, kW4WideThreads, 0, st>>>(a);
+  } else if (a.g.M <= 32) {
+    const dim3 grid(strips * (unsigned)a.ksplit);
+    if (z) w4a8_wide_kernel<F, true, 32, true><<<grid, kW4WideThreads, 0, st>>>(a);
+    else w4a8_wide_kernel<F, false, 32, true><<<grid, kW4WideThreads, 0, st>>>(a);
+  } else {
+    const dim3 grid(strips * (unsigned)a.ksplit, (unsigned)((a.g.M + 63) / 64));
+    if (z) w4a8_wide_kernel<F, true, 64, true><<<grid, kW4WideThreads, 0, st>>>(a);
+    else w4a8_wide_kernel<F, false, 64, true><<<grid, kW4WideThreads, 0, st>>>(a);
+  }
+}
+
+// Workspace of mi355q_w4a16_gemm: [arrival counters and partial sums of the K split, as for W4A8][plane 1][plane 2]
+// [1 / row scale], each part 256-byte aligned.
+struct W4A16Layout {
+  size_t split_bytes, plane_off, lo_off, scale_off, total;
+  int64_t ld;  // row pitch of the planes, a multiple of 16
+};
+inline W4A16Layout w4a16_layout(int64_t M, int64_t N, int64_t K, int64_t group, int scale_f32) {
+  const auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+  W4A16Layout l{};
+  const W4WidePlan plan = w4a8_wide_plan(M, N, K, group, scale_f32);
+  l.split_bytes = plan.parts >= 2 ? plan.workspace_bytes() : 0;
+  l.ld = (K + 15) & ~(int64_t)15;
+  l.plane_off = up(l.split_bytes);
+  l.lo_off = l.plane_off + up((size_t)(M * l.ld));
+  l.scale_off = l.lo_off + up((size_t)(M * l.ld));
+  l.total = l.scale_off + up((size_t)M * sizeof(float));
+  return l;
+}
+
 }  // namespace mi355q
 
 using namespace mi355q;
+
+extern "C" size_t mi355q_w4a16_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group, int scale_dtype) {
+  if (M <= 0 || N <= 0 || K <= 0 || group <= 0) return 0;
+  return w4a16_layout(M, N, K, group, scale_dtype == MI355Q_F32).total;
+}
+
+extern "C" int mi355q_w4a16_gemm(const void* A, int a_dtype, int64_t lda, const int32_t* packed, int64_t ld_packed,
+                                 const void* scale, int scale_dtype, const int32_t* zero_point, int is_signed,
+                                 int64_t group, void* C, int out_dtype, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                                 const void* bias, void* workspace, size_t workspace_bytes, int split_k, void* stream) {
+  if (a_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (out_dtype != MI355Q_F32 && out_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (scale_dtype != MI355Q_F32 && scale_dtype != MI355Q_BF16) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (M < 0 || N < 0 || K < 0 || group <= 0) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (M == 0 || N == 0) return MI355Q_OK;
+  if (C == nullptr || (K > 0 && (A == nullptr || packed == nullptr || scale == nullptr))) return MI355Q_ERR_INVALID_ARGUMENT;
+  if (K % group != 0 || lda < K || ld_packed < N / 8 || ldc < N) return MI355Q_ERR_INVALID_ARGUMENT;
+  const auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  const int es = 2;
+  // the two-plane kernel serves groups of 128 with bf16 scales; whole 16-byte pieces throughout
+  if (group != kBK || scale_dtype != MI355Q_BF16 || K == 0 || N % 32 != 0 || K % 16 != 0 || (lda * es) % 16 != 0 || (ld_packed * 4) % 16 != 0 ||
+      !al16(A) || !al16(packed) || !al16(scale) || (zero_point && !al16(zero_point)) ||
+      M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL || (M + 63) / 64 > 65535)
+    return MI355Q_ERR_UNSUPPORTED;
+  const W4A16Layout l = w4a16_layout(M, N, K, group, 0);
+  if (workspace == nullptr || !al16(workspace) || workspace_bytes < l.total) return MI355Q_ERR_WORKSPACE;
+  uint8_t* ws = static_cast<uint8_t*>(workspace);
+  float* sx_inv = reinterpret_cast<float*>(ws + l.scale_off);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int sp = mi355q_split_rows_fp8x2(A, a_dtype, lda, M, K, ws + l.plane_off, ws + l.lo_off, l.ld, sx_inv, stream);
+  if (sp != MI355Q_OK) return sp;
+  W4Args a{};
+  a.g.A = ws + l.plane_off;
+  a.a_lo = ws + l.lo_off;
+  a.g.C = static_cast<uint8_t*>(C);
+  a.g.lda = l.ld;
+  a.g.ldc = ldc;
+  a.g.M = (int)M;
+  a.g.N = (int)N;
+  a.g.K = (int)K;
+  a.g.sa = sx_inv;
+  a.g.sa_host = 1.0f;
+  a.g.sa_mode = MI355Q_GS_PER_ROW;
+  a.g.sb_mode = MI355Q_GS_NONE;
+  a.g.sb_host = 1.0f;
+  a.g.bias = static_cast<const uint8_t*>(bias);
+  a.g.bias_mode = bias ? MI355Q_BIAS_ROW_VECTOR : MI355Q_BIAS_NONE;
+  a.g.out_bf16 = out_dtype == MI355Q_BF16;
+  a.packed = reinterpret_cast<const uint8_t*>(packed);
+  a.ld_packed = ld_packed * 4;
+  a.scale = static_cast<const uint8_t*>(scale);
+  a.zp = reinterpret_cast<const uint8_t*>(zero_point);
+  a.scale_f32 = 0;
+  a.is_signed = is_signed != 0;
+  a.stages_per_group = 1;
+  const W4WidePlan plan = w4a8_wide_plan(M, N, K, group, 0);
+  a.ksplit = 1;
+  if (plan.parts >= 2 && split_k) {
+    a.ksplit = plan.parts;
+    a.tickets = reinterpret_cast<uint32_t*>(ws);
+    a.partials = reinterpret_cast<float*>(ws + plan.ticket_bytes());
+  }
+  w4a16_launch(a, st);
+  return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
+}
 
 extern "C" size_t mi355q_w4a8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group, int scale_dtype) {
   return w4a8_wide_plan(M, N, K, group, scale_dtype == MI355Q_F32).workspace_bytes();

@@ -327,6 +327,35 @@ int mi355q_softmax_fp8(const void* x, int x_dtype, int64_t rows, int64_t cols,
                        const int64_t* fused_add_row_strides, void* y, int y_dtype, void* stream);
 
 /*
+ * Fused int4-dequant GEMM on 16-bit activations (W4A16):
+ *   C[m, n] = out( sum_g s[g, n] * sum_{k in g} a[m, k] * (q[k, n] - z[g, n]) + bias[n] )
+ * with a bf16.  This is what the reference composes from convert_from_int4 / convert_from_uint4 to
+ * bf16 (Int4BaseOp::AddNode, hpu_ops/backend/int4_ops.cpp:40-56: nibble order, (q - z) * s, the
+ * group layout of its test, tests/pytest_working/any_mode/test_hpu_convert_from_int4.py:398-476)
+ * and a bf16 matmul; here the bf16 [K, N] matrix never exists.  The activations are first cut into
+ * two e4m3fn planes per row (mi355q_split_rows_fp8x2: a * s = hi + lo / 16 with a power-of-two row
+ * scale s, exact for every element within a factor 2^15 of the row's largest and to 3e-8 of that
+ * largest otherwise), and both planes meet the packed nibbles in the matrix unit as in
+ * mi355q_w4a8_gemm, so the integers (q - z) and the products enter the fp32 sums exactly.
+ * Serves groups of 128 with bf16 scales, N a multiple of 32 and K of 16 (MI355Q_ERR_UNSUPPORTED
+ * otherwise).  `workspace`: mi355q_w4a16_gemm_workspace_bytes(...) bytes of device memory, 16-byte
+ * aligned, for the planes, the row scales and, in front, the arrival counters and partial sums of
+ * the split over K: its first 1 KiB has to be zero before the first use and is left zero, so the
+ * buffer can be passed again (calls that may overlap need buffers of their own).  split_k = 0 keeps
+ * K in one piece (no counters are touched).  Nothing is allocated.
+ */
+size_t mi355q_w4a16_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group, int scale_dtype);
+int mi355q_w4a16_gemm(const void* A, int a_dtype, int64_t lda, const int32_t* packed, int64_t ld_packed,
+                      const void* scale, int scale_dtype, const int32_t* zero_point, int is_signed,
+                      int64_t group, void* C, int out_dtype, int64_t ldc, int64_t M, int64_t N, int64_t K,
+                      const void* bias, void* workspace, size_t workspace_bytes, int split_k, void* stream);
+/* The first step of mi355q_w4a16_gemm on its own: rows of bf16 x [rows, cols] (pitch ldx elements) as two
+ * e4m3fn planes hi, lo [rows, ld] (ld a multiple of 16, columns from cols on zero) and scale_inv[rows] =
+ * 1 / s with x * s = hi + lo / 16.  No counterpart in the reference. */
+int mi355q_split_rows_fp8x2(const void* x, int x_dtype, int64_t ldx, int64_t rows, int64_t cols, void* hi, void* lo,
+                            int64_t ld, float* scale_inv, void* stream);
+
+/*
  * Attention forward for inference on fp8 q, k, v:
  *   S   = (q d_scale_q) (k d_scale_k)^T softmax_scale  [+ float mask | -inf where a bool mask
  *         is 0 | -inf for key j > query i when is_causal]

@@ -327,6 +327,34 @@ def torch_w4a8_gemm(A8, packed, scale, zero_point, signed, out_dtype, A_scale_in
     return v.to(torch.float32).to(out_dtype)
 
 
+def torch_w4a16_gemm(A, packed, scale, zero_point, signed, out_dtype, bias=None):
+    """mi355q::w4a16_gemm: bf16 activations [M, K] times the same 4-bit weights,
+        C = out_dtype( A @ W + bias ),   W[k, n] = (q[k, n] - z[k / g, n]) * s[k / g, n],
+    i.e. hpu::convert_from_[u]int4 (int4_ops.cpp:40-56; layout of test_hpu_convert_from_int4.py:398-476) followed by
+    the matmul a bf16 model runs on its output, with W kept exact and the sums in float64 (the unfused route rounds W
+    to bf16 first)."""
+    assert A.dtype == torch.bfloat16
+    return torch_w4a8_gemm(A, packed, scale, zero_point, signed, out_dtype, None, bias)
+
+
+def split_rows_fp8x2(x):
+    """mi355q_split_rows_fp8x2: rows of a bf16 matrix as two e4m3fn planes and 1 / s per row, with
+    x s = hi + lo / 16: s is the largest power of two with max |x| s <= 448 (1 for a row of zeros),
+    hi = e4m3fn(x s) rounded to nearest even, lo = e4m3fn((x s - hi) 16).  Returns (hi, lo, scale_inv)."""
+    x = x.detach().cpu()
+    assert x.dtype == torch.bfloat16 and x.dim() == 2
+    xf = x.float()
+    amax = xf.abs().amax(dim=1, keepdim=True)
+    m, ea = torch.frexp(amax)                      # amax = m 2^ea, 0.5 <= m < 1
+    e = torch.where(m * 2 <= 1.75, 8, 7) - (ea - 1)
+    e = torch.where(amax > 0, e, torch.zeros_like(e)).clamp(-126, 126)
+    s = torch.exp2(e.float())
+    p = xf * s
+    hi = p.clamp(-448, 448).to(torch.float8_e4m3fn)
+    lo = ((p - hi.float()) * 16).clamp(-448, 448).to(torch.float8_e4m3fn)
+    return hi, lo, torch.exp2(-e.float()).reshape(-1)
+
+
 def c_silu_mul_bf16(gate, up):
     """bf16(bf16(silu(gate)) * up) with the oracle's spelled-out exp (ora_silu_mul_bf16)."""
     g = gate.detach().cpu().contiguous()
