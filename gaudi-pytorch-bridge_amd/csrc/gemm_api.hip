@@ -82,7 +82,7 @@ const char* mi355q_fp8_gemm_variant(int trans_a, int64_t lda, int trans_b, int64
   if (lda % 16 || ldb % 16 || !mi355q::k_chunks_ok(trans_a, trans_b, K)) return "simple";
   if (M > 128 && N > 128) {
     switch (mi355q::choose_tiles(M, N, 1)) {
-      case mi355q::TileChoice::k256x256: return "tile256x256x128_mfma32x32x64";
+      case mi355q::TileChoice::k256x256: return "tile256x256x128_mfma16x16x128";  // 32x32x64 with eight waves for epilogues beyond the fast bf16 one
       case mi355q::TileChoice::k256x128: return "tile256x128x128_mfma32x32x64";
       case mi355q::TileChoice::k128x128: return "tile128x128x128_mfma32x32x64";
     }

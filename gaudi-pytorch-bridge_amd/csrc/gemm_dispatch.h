@@ -22,6 +22,7 @@
 #pragma once
 #include "gemm_skinny.h"
 #include "gemm_tile.h"
+#include "gemm_tile16.h"
 
 namespace mi355q {
 
@@ -73,7 +74,8 @@ GemmArgs columns_from(const GemmArgs& g, int64_t n_off, int64_t batch) {
 
 template <bool AK, bool BK_, int FA, int FB>
 void launch_256x256(const GemmArgs& g, int64_t batch, hipStream_t st) {
-  if (g.fast_epi && g.D == nullptr) launch_tile<256, 256, 2, true, AK, BK_, FA, FB>(g, batch, st);
+  // the fast bf16 epilogue without an accumulate input: four waves on the 16x16x128 MFMA (gemm_tile16.h)
+  if (g.fast_epi && g.D == nullptr) launch_tile16<AK, BK_, FA, FB>(g, batch, st);
   else launch_tile<256, 256, 4, false, AK, BK_, FA, FB>(g, batch, st);
 }
 

@@ -113,7 +113,10 @@ constexpr int mfma_code() { return FMT == MI355Q_E5M2 ? 1 : 0; }
 //     8 slots of one parity and leaves the other parity to the adjacent chunk.
 //   MN-major, 128-byte rows: two rows per 256 bytes, so (row >> 1 & 3) << 1.
 //   K-major, 64-byte rows: four rows per 256 bytes, so (row >> 2) & 3.
-template <bool KMAJOR, int ROWS, int ROW_BYTES>
+//   MN-major, 256-byte rows, variant V = 1 (fragments of the 16x16x128 MFMA, gemm_tile16.h): the two 16-lane groups
+//     of a cycle read the same chunk of k-rows 32 apart, so bit 5 of the row goes into the XOR as well and sends
+//     the second group to the other parity.
+template <bool KMAJOR, int ROWS, int ROW_BYTES, int V = 0>
 struct TileGeom {
   static constexpr int kChunksPerRow = ROW_BYTES / 16;
   static constexpr int kChunks = ROWS * kChunksPerRow;
@@ -122,7 +125,7 @@ struct TileGeom {
   __device__ static __forceinline__ int swizzle(int row) {
     if constexpr (KMAJOR && ROW_BYTES == 128) return (row >> 1) & 7;
     else if constexpr (KMAJOR) return (row >> 2) & 3;
-    else if constexpr (ROW_BYTES == 256) return (row & 7) << 1;
+    else if constexpr (ROW_BYTES == 256) return V == 1 ? (((row & 7) << 1) | ((row >> 5) & 1)) : ((row & 7) << 1);
     else return ((row >> 1) & 3) << 1;
   }
   __device__ static __forceinline__ int lds_offset(int row, int chunk) {
@@ -161,14 +164,17 @@ __device__ __forceinline__ int lane_id_here() {
 //           descriptor; columns past the extent only feed outputs that are
 //           never stored.
 // EXT: tile extent along m/n; BK: bytes of K per stage; WAVES: waves of the workgroup
-template <bool KMAJOR, int EXT, int BK, int WAVES>
+// V: swizzle variant of TileGeom (1: the waves' shares must be whole blocks of 32 rows, inside which the swizzle
+// keeps its period of 8 rows)
+template <bool KMAJOR, int EXT, int BK, int WAVES, int V = 0>
 struct DmaLoader {
-  using G = TileGeom<KMAJOR, KMAJOR ? EXT : BK, KMAJOR ? BK : EXT>;
+  using G = TileGeom<KMAJOR, KMAJOR ? EXT : BK, KMAJOR ? BK : EXT, V>;
   static constexpr int kCPR = G::kChunksPerRow;
   static constexpr int kRowsPerRegion = 64 / kCPR;
   static constexpr int kRegions = G::kChunks / 64;
   static constexpr int kPerWave = kRegions / WAVES;
   static_assert(kRegions % WAVES == 0 && 64 % kCPR == 0, "tile does not split over the waves");
+  static_assert(V == 0 || KMAJOR || (EXT == 256 && kPerWave * kRowsPerRegion == 32), "variant 1: a wave loads whole blocks of 32 k-rows");
 
   // Raw buffer descriptor: base, stride 0, num_records (bytes), dword 3 flags.
   // The base walks along K, one stage per advance(), and num_records shrinks
