@@ -116,6 +116,12 @@ constexpr int mfma_code() { return FMT == MI355Q_E5M2 ? 1 : 0; }
 //   MN-major, 256-byte rows, variant V = 1 (fragments of the 16x16x128 MFMA, gemm_tile16.h): the two 16-lane groups
 //     of a cycle read the same chunk of k-rows 32 apart, so bit 5 of the row goes into the XOR as well and sends
 //     the second group to the other parity.
+//   K-major, 128-byte rows, variant V = 1 (the same fragments): lane group g = lane / 16 reads chunks 2 g, 2 g + 1 of
+//     16 consecutive rows, and with the XOR above every ds_read_b128 of that shape takes twice its four cycles
+//     (measured: SQ_LDS_BANK_CONFLICT half of SQ_LDS_IDX_ACTIVE, and 1.66 times the time of a conflict-free read in
+//     a loop that only reads).  Of the 4096 XORs that are linear in the row's low four bits, 1344 read at full
+//     rate; the one used swaps the two low bits of the XOR above: bit 0 from row bit 2, bit 1 from row bit 1,
+//     bit 2 from row bit 3.
 template <bool KMAJOR, int ROWS, int ROW_BYTES, int V = 0>
 struct TileGeom {
   static constexpr int kChunksPerRow = ROW_BYTES / 16;
@@ -123,7 +129,7 @@ struct TileGeom {
   static_assert(KMAJOR ? (ROW_BYTES == 128 || ROW_BYTES == 64) : (ROW_BYTES == 256 || ROW_BYTES == 128), "no swizzle defined");
   static constexpr int kSwizzlePeriod = KMAJOR ? 16 : 8;  // swizzle(row + kSwizzlePeriod) == swizzle(row)
   __device__ static __forceinline__ int swizzle(int row) {
-    if constexpr (KMAJOR && ROW_BYTES == 128) return (row >> 1) & 7;
+    if constexpr (KMAJOR && ROW_BYTES == 128) return V == 1 ? (((row >> 2) & 1) | (row & 2) | ((row >> 1) & 4)) : ((row >> 1) & 7);
     else if constexpr (KMAJOR) return (row >> 2) & 3;
     else if constexpr (ROW_BYTES == 256) return V == 1 ? (((row & 7) << 1) | ((row >> 5) & 1)) : ((row & 7) << 1);
     else return ((row >> 1) & 3) << 1;
