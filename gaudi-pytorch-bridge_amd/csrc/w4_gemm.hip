@@ -547,8 +547,10 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
   constexpr int kOffLo = BM * kBK;  // the second plane's tile (A16)
   constexpr int kOffPacked = BM * kBK * (A16 ? 2 : 1), kOffScale = kOffPacked + kW4WidePacked, kOffZp = kOffScale + kW4ScaleRow;
   constexpr int NV = M16 ? 8 : 16 * MT;  // results per consumer lane
-  using LA = DmaLoader<true, BM, kBK, kW4ColWaves>;
-  using GA = TileGeom<true, BM, kBK>;
+  // the 16-row form reads A fragments shaped for the 16x16x128 MFMA: the XOR of TileGeom's variant 1 keeps those off
+  // each other's banks
+  using LA = DmaLoader<true, BM, kBK, kW4ColWaves, ROWS == 16 ? 1 : 0>;
+  using GA = TileGeom<true, BM, kBK, ROWS == 16 ? 1 : 0>;
   constexpr int kOps = 4 + LA::kPerWave * (A16 ? 2 : 1) + 1;  // four 1 KiB regions of weights, A, and the scale or zero-point row
   static_assert(S >= 3 && (S - 2) * kOps <= 63, "vmcnt holds 6 bits");
   static_assert(kStage % 1024 == 0, "stages stay 1 KiB aligned");
