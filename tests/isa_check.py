@@ -153,3 +153,36 @@ def compile_to_isa(source, extra_flags=()):
     if r.returncode != 0:
         raise RuntimeError("hipcc failed: " + r.stderr[-2000:])
     return r.stdout
+
+
+def exchange_order(text):
+    """{kernel symbol: string} for kernels that draw a ticket (global_atomic_add), over
+    S / L (global store / load with the sc1 bit, what a device-scope atomic access compiles to), A (the atomic),
+    W (s_waitcnt vmcnt(0)), B (s_barrier, runs merged) and F (a cache-wide write-back or invalidate)."""
+    out = {}
+    for m in re.finditer(r"^(_Z\w+):\s*(?:;.*)?$", text, re.M):
+        end = text.find(".Lfunc_end", m.end())
+        if end < 0:
+            continue
+        body = text[m.end():end]
+        if "global_atomic_add" not in body:
+            continue
+        ev = []
+        for line in body.splitlines():
+            t = line.strip()
+            if not _is_instruction(line):
+                continue
+            if re.match(r"global_store\w*\s.*\bsc1\b", t):
+                ev.append("S")
+            elif re.match(r"global_load\w*\s.*\bsc1\b", t):
+                ev.append("L")
+            elif t.startswith("global_atomic_add"):
+                ev.append("A")
+            elif t.startswith("s_barrier"):
+                ev.append("B")
+            elif t.startswith("s_waitcnt") and "vmcnt(0)" in t:
+                ev.append("W")
+            elif re.match(r"buffer_wbl2|buffer_inv|global_wb|global_inv", t):
+                ev.append("F")
+        out[m.group(1)] = re.sub(r"B+", "B", "".join(ev))
+    return out

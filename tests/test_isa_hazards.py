@@ -142,3 +142,41 @@ def test_streaming_kernels_issue_their_loads_back_to_back():
         first_full_wait = seq.find("W") if "W" in seq else len(seq)
         assert seq[:first_full_wait].count("L") >= loads, (name, seq)
     assert seen >= 60
+
+
+def test_exchange_order_reads_a_kernel():
+    text = """
+_Z3barv:                                ; @_Z3barv
+	global_store_dwordx2 v[0:1], v[2:3], off sc1
+	s_waitcnt vmcnt(0)
+	s_barrier
+	global_atomic_add v4, v[0:1], v5, off sc0
+	s_waitcnt vmcnt(0)
+	s_barrier
+	s_barrier
+	global_load_dwordx2 v[6:7], v[0:1], off sc1
+	buffer_wbl2 sc1
+	s_endpgm
+.Lfunc_end0:
+"""
+    assert isa_check.exchange_order(text) == {"_Z3barv": "SWBAWBLF"}
+
+
+@pytest.mark.timeout(900)
+def test_partial_results_are_exchanged_by_device_scope_accesses_in_order():
+    """Workgroups that split one reduction (the K parts of the 4-bit GEMMs, the key splits of the decoding attention
+    kernel) hand their partial results over without a fence: device-scope relaxed atomic stores (sc1: written through
+    to where every XCD sees them), a wait until they are acknowledged, a workgroup barrier, the ticket; whoever draws
+    the last ticket passes a barrier and reads with device-scope loads (sc1).  The generated code has to keep that
+    order and those bits, and must hold no cache-wide write-back or invalidate."""
+    import re
+    with ThreadPoolExecutor(max_workers=2) as ex:
+        texts = list(ex.map(isa_check.compile_to_isa, ["w4_gemm.hip", "sdpa_kernels.hip"]))
+    for src, text, least in zip(["w4_gemm.hip", "sdpa_kernels.hip"], texts, [12, 2]):
+        orders = isa_check.exchange_order(text)
+        assert len(orders) >= least, src
+        for name, seq in orders.items():
+            assert "F" not in seq, name
+            assert seq.count("A") == 1, name
+            # partial results stored, acknowledged, barrier, ticket (and its return to zero by the last one), barrier, read
+            assert re.search(r"S+WBAW?S?BL+", seq), (name, seq)
