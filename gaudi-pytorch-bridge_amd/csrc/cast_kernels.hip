@@ -483,6 +483,70 @@ __global__ __launch_bounds__(kThreads) void split_rows_kernel(const uint16_t* __
   }
 }
 
+// The same split with the row held in registers (VPT 16-byte vectors of eight bf16 per thread): one pass
+// over the row, every load in flight before the first is used, 8-byte stores.  For rows that start 16-byte
+// aligned with cols a multiple of 8 and at most 8 * kThreads vectors; output columns from `cols` to ld
+// come from lanes whose load falls outside the row's descriptor and reads zeros.  Same bits as the kernel above.
+template <int VPT>
+__global__ __launch_bounds__(kThreads) void split_rows_vec_kernel(const uint16_t* __restrict__ x, int64_t ldx, int64_t cols,
+                                                                  uint8_t* __restrict__ hi, uint8_t* __restrict__ lo, int64_t ld,
+                                                                  float* __restrict__ scale_inv) {
+  __shared__ uint32_t wave_part[kThreads / 64];
+  const int64_t row = blockIdx.x;
+  const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(x) + row * ldx, 0, (int)cols * 2, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rhi = __builtin_amdgcn_make_buffer_rsrc(hi + row * ld, 0, (int)ld, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rlo = __builtin_amdgcn_make_buffer_rsrc(lo + row * ld, 0, (int)ld, 0x00020000);
+  u32x4 in[VPT];
+#pragma unroll
+  for (int u = 0; u < VPT; ++u)
+    in[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rin, ((int)threadIdx.x + u * kThreads) * 16, 0, 0));
+  uint32_t am = 0;
+#pragma unroll
+  for (int u = 0; u < VPT; ++u)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const u16x2 a = __builtin_bit_cast(u16x2, in[u][i] & 0x7fff7fffu);
+      am = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, __builtin_bit_cast(u16x2, am)));
+    }
+  {
+    const uint32_t l16 = am & 0xffffu, h16 = am >> 16;
+    am = (l16 > h16 ? l16 : h16) << 16;
+  }
+  am = wave_max_u32(am);
+  if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = am;
+  __syncthreads();
+  uint32_t r = wave_part[0];
+#pragma unroll
+  for (int w = 1; w < kThreads / 64; ++w) r = r > wave_part[w] ? r : wave_part[w];
+  int e = 0;
+  if (r != 0u && r < 0x7f800000u) {
+    const int ea = (int)(r >> 23) - 127;
+    e = ((r & 0x007fffffu) <= 0x00600000u ? 8 : 7) - (r >= 0x00800000u ? ea : -126);
+    e = e > 126 ? 126 : (e < -126 ? -126 : e);
+  }
+  const float s = __uint_as_float((uint32_t)(e + 127) << 23);
+  if (threadIdx.x == 0) scale_inv[row] = __uint_as_float((uint32_t)(127 - e) << 23);
+#pragma unroll
+  for (int u = 0; u < VPT; ++u) {
+    float p[8], q[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[2 * i] = __uint_as_float(in[u][i] << 16) * s;
+      p[2 * i + 1] = __uint_as_float(in[u][i] & 0xffff0000u) * s;
+    }
+    const u32x2 h = {cvt_fp8x4<MI355Q_E4M3FN>(p[0], p[1], p[2], p[3]), cvt_fp8x4<MI355Q_E4M3FN>(p[4], p[5], p[6], p[7])};
+    cvt_f32x4<MI355Q_E4M3FN>(h[0], q[0], q[1], q[2], q[3]);
+    cvt_f32x4<MI355Q_E4M3FN>(h[1], q[4], q[5], q[6], q[7]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) q[i] = (p[i] - q[i]) * 16.0f;
+    const u32x2 l = {cvt_fp8x4<MI355Q_E4M3FN>(q[0], q[1], q[2], q[3]), cvt_fp8x4<MI355Q_E4M3FN>(q[4], q[5], q[6], q[7])};
+    const int off = ((int)threadIdx.x + u * kThreads) * 8;
+    __builtin_amdgcn_raw_buffer_store_b64(h, rhi, off, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b64(l, rlo, off, 0, 0);
+  }
+}
+
 // ------------------------------------------------- dynamic per-row quantisation
 //
 // One pass of "per-row amax -> scale = target / amax -> cast with that scale":
@@ -1233,8 +1297,20 @@ int mi355q_split_rows_fp8x2(const void* x, int x_dtype, int64_t ldx, int64_t row
   if (rows == 0) return MI355Q_OK;
   if (x == nullptr || hi == nullptr || lo == nullptr || scale_inv == nullptr) return MI355Q_ERR_INVALID_ARGUMENT;
   if (ld % 16 != 0 || !aligned(hi, 16) || !aligned(lo, 16) || rows > 0x7fffffffLL) return MI355Q_ERR_UNSUPPORTED;
-  split_rows_kernel<<<(unsigned)rows, kThreads, 0, static_cast<hipStream_t>(stream)>>>(
-      static_cast<const uint16_t*>(x), ldx, cols, static_cast<uint8_t*>(hi), static_cast<uint8_t*>(lo), ld, scale_inv);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const uint16_t* xs = static_cast<const uint16_t*>(x);
+  uint8_t* h8 = static_cast<uint8_t*>(hi);
+  uint8_t* l8 = static_cast<uint8_t*>(lo);
+  const unsigned grid = (unsigned)rows;
+  const int64_t vpr = ld / 8;  // output vectors of a row
+  if (cols % 8 == 0 && ldx % 8 == 0 && aligned(x, 16) && vpr <= 8 * kThreads) {
+    if (vpr <= kThreads) split_rows_vec_kernel<1><<<grid, kThreads, 0, st>>>(xs, ldx, cols, h8, l8, ld, scale_inv);
+    else if (vpr <= 2 * kThreads) split_rows_vec_kernel<2><<<grid, kThreads, 0, st>>>(xs, ldx, cols, h8, l8, ld, scale_inv);
+    else if (vpr <= 4 * kThreads) split_rows_vec_kernel<4><<<grid, kThreads, 0, st>>>(xs, ldx, cols, h8, l8, ld, scale_inv);
+    else split_rows_vec_kernel<8><<<grid, kThreads, 0, st>>>(xs, ldx, cols, h8, l8, ld, scale_inv);
+  } else {
+    split_rows_kernel<<<grid, kThreads, 0, st>>>(xs, ldx, cols, h8, l8, ld, scale_inv);
+  }
   return launch_status();
 }
 

@@ -15,23 +15,32 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
-def test_split_rows_bit_exact(oracle, pkg, dev):
-    gen = torch.Generator().manual_seed(1)
-    x = (torch.randn(37, 1000, generator=gen) * torch.logspace(-6, 4, 37).reshape(-1, 1)).bfloat16()
-    x[3] = 0
-    x[5, ::7] *= 1e-5
+@pytest.mark.parametrize("rows,cols,ld", [
+    (37, 1000, 1008),      # one vector per thread, eight columns of padding
+    (9, 1003, 1008),       # cols not a multiple of 8: the element-wise kernel
+    (5, 8192, 8192),       # the benchmark's K: four vectors per thread
+    (3, 16384, 16384),     # eight vectors per thread
+    (2, 20000, 20000),     # longer than a workgroup's registers hold: the element-wise kernel
+    (4, 2056, 2064),       # two vectors per thread
+])
+def test_split_rows_bit_exact(oracle, pkg, dev, rows, cols, ld):
+    gen = torch.Generator().manual_seed(rows + cols)
+    x = (torch.randn(rows, cols, generator=gen) * torch.logspace(-6, 4, rows).reshape(-1, 1)).bfloat16()
+    if rows > 5:
+        x[3] = 0
+        x[5, ::7] *= 1e-5
+    x[0, ::5] *= 1e-4
     lib = pkg.capi()
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     xd = x.to(dev)
-    ld = 1008
-    hi = torch.full((37, ld), 0x7f, dtype=torch.uint8, device=dev)
-    lo = torch.full((37, ld), 0x7f, dtype=torch.uint8, device=dev)
-    sinv = torch.empty(37, device=dev)
-    assert lib.mi355q_split_rows_fp8x2(xd.data_ptr(), pkg.BF16, 1000, 37, 1000, hi.data_ptr(), lo.data_ptr(), ld, sinv.data_ptr(), st) == 0
+    hi = torch.full((rows, ld), 0x7f, dtype=torch.uint8, device=dev)
+    lo = torch.full((rows, ld), 0x7f, dtype=torch.uint8, device=dev)
+    sinv = torch.empty(rows, device=dev)
+    assert lib.mi355q_split_rows_fp8x2(xd.data_ptr(), pkg.BF16, cols, rows, cols, hi.data_ptr(), lo.data_ptr(), ld, sinv.data_ptr(), st) == 0
     rh, rl, rs = oracle.split_rows_fp8x2(x)
-    assert torch.equal(hi.cpu()[:, :1000], rh.view(torch.uint8)) and torch.equal(lo.cpu()[:, :1000], rl.view(torch.uint8))
+    assert torch.equal(hi.cpu()[:, :cols], rh.view(torch.uint8)) and torch.equal(lo.cpu()[:, :cols], rl.view(torch.uint8))
     assert torch.equal(sinv.cpu(), rs)
-    assert torch.count_nonzero(hi.cpu()[:, 1000:]) == 0 and torch.count_nonzero(lo.cpu()[:, 1000:]) == 0
+    assert torch.count_nonzero(hi.cpu()[:, cols:]) == 0 and torch.count_nonzero(lo.cpu()[:, cols:]) == 0
 
 
 @pytest.mark.parametrize("signed", [False, True])
