@@ -1147,12 +1147,24 @@ Tensor sdpa_valid_seq_len(const Tensor& t, const Tensor& q, const std::vector<in
   return t.reshape({nbatch}).to(at::kInt).contiguous();
 }
 
+// Elements of fp32 scores the bf16 / fp32 measurement pass of the attention ops holds at a time
+// (MI355Q_SDPA_MEASURE_SCORE_ELEMENTS overrides the default of 2^28, for tests).
+int64_t sdpa_measure_score_elements() {
+  if (const char* e = std::getenv("MI355Q_SDPA_MEASURE_SCORE_ELEMENTS")) {
+    const long long v = std::atoll(e);
+    if (v > 0) return (int64_t)v;
+  }
+  return (int64_t)1 << 28;
+}
+
 // Keys a query may attend to, as a boolean tensor that broadcasts against the scores [batch..., L, S]
 // (undefined: all of them): the triangular mask and the per-batch key window.
-Tensor sdpa_keep_mask(const Tensor& like, int64_t L, int64_t S, bool is_causal, const Tensor& valid, bool pad_left, int64_t batch_rank) {
+// Rows l0 .. l0 + L - 1 of the queries (l0 shifts the triangle).
+Tensor sdpa_keep_mask(const Tensor& like, int64_t L, int64_t S, bool is_causal, const Tensor& valid, bool pad_left, int64_t batch_rank,
+                      int64_t l0 = 0) {
   Tensor keep;
   auto bopts = like.options().dtype(at::kBool);
-  if (is_causal) keep = at::ones({L, S}, bopts).tril(0);
+  if (is_causal) keep = at::ones({L, S}, bopts).tril(l0);
   if (valid.defined()) {
     Tensor j = at::arange(S, like.options().dtype(at::kInt)).reshape({1, S});
     Tensor n = valid.reshape({-1, 1});
@@ -1169,15 +1181,19 @@ Tensor sdpa_keep_mask(const Tensor& like, int64_t L, int64_t S, bool is_causal, 
 
 // softmax(q k^T scale + masks) in fp32 on the device's own matmul and softmax: the route of the bf16 / fp32
 // measurement pass, where nothing is fp8.  A row with every key masked gives zeros.
+// q holds query rows l0 .. of the problem (a slice when the caller walks the queries in pieces); a mask with a row per
+// query is sliced the same way.
 Tensor sdpa_probabilities_unfused(const Tensor& q, const Tensor& k, const c10::optional<Tensor>& attention_mask, double scale,
-                                  bool is_causal, const Tensor& valid, bool pad_left, int64_t batch_rank) {
+                                  bool is_causal, const Tensor& valid, bool pad_left, int64_t batch_rank, int64_t l0 = 0) {
   const float ninf = -std::numeric_limits<float>::infinity();
   Tensor s = at::matmul(q, k.transpose(-2, -1)).to(at::kFloat) * scale;
   if (attention_mask.has_value() && attention_mask->defined()) {
-    if (attention_mask->scalar_type() == at::kBool) s = s.masked_fill(attention_mask->logical_not(), ninf);
-    else s = s + attention_mask->to(at::kFloat);
+    Tensor am = *attention_mask;
+    if (am.dim() >= 2 && am.size(-2) != 1 && am.size(-2) != q.size(-2)) am = am.narrow(-2, l0, q.size(-2));
+    if (am.scalar_type() == at::kBool) s = s.masked_fill(am.logical_not(), ninf);
+    else s = s + am.to(at::kFloat);
   }
-  Tensor keep = sdpa_keep_mask(q, q.size(-2), k.size(-2), is_causal, valid, pad_left, batch_rank);
+  Tensor keep = sdpa_keep_mask(q, q.size(-2), k.size(-2), is_causal, valid, pad_left, batch_rank, l0);
   if (keep.defined()) s = s.masked_fill(keep.logical_not(), ninf);
   return at::nan_to_num(at::softmax(s, -1), 0.0);
 }
@@ -1242,10 +1258,20 @@ SdpaOut fp8_sdpa_recomp_fwd_common(const Tensor& q, const Tensor& k, const Tenso
     // The measurement pass of the reference's flow: bf16 / fp32 q, k, v, no fp8 anywhere; only amax_s
     // (and amax_o) are wanted from it.  It runs on the device's own matmul and softmax.
     TORCH_CHECK(dt == at::kBFloat16 || dt == at::kFloat, "fp8_sdpa_recomp_fwd: q, k and v must be fp8, bfloat16 or float");
-    Tensor pr = sdpa_probabilities_unfused(q, k, attention_mask, scale, is_causal, valid, pad_left, (int64_t)bshape.size());
-    out.copy_(at::matmul(pr.to(dt), v));
-    if (pr.numel() > 0) amax_s.copy_(pr.max().reshape({1}));
-    else amax_s.zero_();
+    // The scores are a tensor [batch..., L, S] in fp32: the queries are walked in pieces that keep it below a fixed
+    // number of elements (1 GiB of fp32 by default), so that a long prompt does not ask for tens of gigabytes.
+    int64_t nbatch = 1;
+    for (int64_t b : bshape) nbatch *= b;
+    const int64_t per_row = std::max<int64_t>(nbatch * S, 1);
+    const int64_t rows_at_once = std::max<int64_t>(sdpa_measure_score_elements() / per_row, 1);
+    amax_s.zero_();
+    for (int64_t l0 = 0; l0 < L; l0 += rows_at_once) {
+      const int64_t len = std::min(rows_at_once, L - l0);
+      Tensor pr = sdpa_probabilities_unfused(q.narrow(-2, l0, len), k, attention_mask, scale, is_causal, valid, pad_left,
+                                             (int64_t)bshape.size(), l0);
+      out.narrow(-2, l0, len).copy_(at::matmul(pr.to(dt), v));
+      if (pr.numel() > 0) amax_s.copy_(at::maximum(amax_s, pr.max().reshape({1})));
+    }
     if (out.numel() > 0) amax_o.copy_(out.to(at::kFloat).abs().max().reshape({1}));
     else amax_o.zero_();
     return SdpaOut(out, m, linv, seed, amax_s, amax_o);

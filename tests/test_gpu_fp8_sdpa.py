@@ -400,6 +400,48 @@ def test_measurement_pass_with_bf16_inputs(dev):
     assert abs(float(amax_s.cpu()) - float(p.max())) <= 0.05
 
 
+@pytest.mark.parametrize("mask_kind", ["none", "bool_rows", "float_one_row"])
+def test_measurement_pass_walks_long_prompts_in_pieces(dev, monkeypatch, mask_kind):
+    """The bf16 measurement pass holds fp32 scores [batch, L, S]; beyond a fixed number of elements it walks the queries
+    in pieces.  With the limit forced down to 37 rows at a time the result equals the one-piece result (the triangle and
+    a per-query mask are shifted with the piece)."""
+    gen = torch.Generator().manual_seed(15)
+    B, H, L, S, D = 2, 3, 150, 200, 16
+    q = torch.randn(B, H, L, D, generator=gen).bfloat16().to(dev)
+    k = torch.randn(B, H, S, D, generator=gen).bfloat16().to(dev)
+    v = torch.randn(B, H, S, D, generator=gen).bfloat16().to(dev)
+    causal = mask_kind == "none"
+    mask = None
+    if mask_kind == "bool_rows":
+        mask = (torch.rand(B, 1, L, S, generator=gen) > 0.3)
+        mask[..., 0] = True
+        mask = mask.to(dev)
+    elif mask_kind == "float_one_row":
+        mask = (torch.randn(1, 1, 1, S, generator=gen)).bfloat16().to(dev)
+
+    def run():
+        out, _, _, _, amax_s, amax_o = torch.ops.hpu.fp8_sdpa_recomp_fwd(
+            q, k, v, mask, 0.0, 0.25, causal, False, "None", None, None, None, None, None, None, True, True, None, "left")
+        return out.cpu().float(), float(amax_s.cpu()), float(amax_o.cpu())
+
+    monkeypatch.delenv("MI355Q_SDPA_MEASURE_SCORE_ELEMENTS", raising=False)
+    whole = run()
+    monkeypatch.setenv("MI355Q_SDPA_MEASURE_SCORE_ELEMENTS", str(B * H * S * 37))
+    pieces = run()
+    assert torch.allclose(whole[0], pieces[0], atol=2e-2, rtol=1e-2)
+    assert abs(whole[1] - pieces[1]) <= 1e-3 and abs(whole[2] - pieces[2]) <= 2e-2
+    # and against plain attention
+    s = (q.cpu().float() @ k.cpu().float().transpose(-2, -1)) * 0.25
+    if causal:
+        s = s.masked_fill(~torch.ones(L, S, dtype=torch.bool).tril(), float("-inf"))
+    if mask_kind == "bool_rows":
+        s = s.masked_fill(~mask.cpu(), float("-inf"))
+    elif mask_kind == "float_one_row":
+        s = s + mask.cpu().float()
+    ref = torch.softmax(s, -1) @ v.cpu().float()
+    assert torch.allclose(pieces[0], ref, atol=0.08, rtol=1e-2)
+
+
 def test_c_entry_point_rejects_bad_arguments(pkg, dev):
     lib = pkg.capi()
     q = torch.zeros(16, 64, device=dev).to(E4)
