@@ -58,7 +58,7 @@ MEASURED_TRAFFIC = {
     "w4a8_gemm_M32": 140.25e6,
     "w4a8_gemm_M64": 158.58e6,
     "w4a8_gemm_M256": 283.02e6,     # four row blocks of 64 stream the weights; the caches catch half of it
-    "w4a16_gemm_M16": 131.96e6,     # split_rows_kernel + w4a8_wide_kernel<two planes>
+    "w4a16_gemm_M16": 131.98e6,     # split_rows_vec_kernel + w4a8_wide_kernel<two planes>
     "w4a16_gemm_M64": 164.56e6,
     "w4a16_gemm_M256": 316.05e6,
     "fp8_sdpa_B1_L8192": 124.63e6,
@@ -581,7 +581,7 @@ def bench_w4a16(oracle, dev, steps, warmup, cpu):
             c = {"value": round((K * cols_n // 2) / t / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
                  "sample": f"M=16, {cols_n} of the 28672 output columns: unpack, (q - z) * s in float64, matmul"}
         out.append(hbm_entry(f"w4a16_gemm_M{M}", f"w4a16_gemm M={M} K=8192 N=28672: uint4 weights (group 128, bf16 scales, packed zero points) "
-                                                 "x bf16 activations -> bf16", nbytes, ms, steps, "split_rows_kernel + w4a8_wide_kernel<two planes>", c,
+                                                 "x bf16 activations -> bf16", nbytes, ms, steps, "split_rows_vec_kernel + w4a8_wide_kernel<two planes>", c,
                              extra={"tflops": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 2)}))
     return out
 
