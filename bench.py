@@ -332,6 +332,22 @@ def bench_ceilings(pkg, dev, steps, warmup):
                              + (f", the rows in {parts} ranges" if parts > 1 else "") + (", nontemporal loads" if nt else ""),
                              pitch * rows, ms, k, "probe_strip_read_kernel"))
     del bufs
+    # the amax pass of C1 in the form that needs no zeroing launch (partial maxima, a ticket, the last workgroup
+    # reduces), beside the product's form (a one-thread fill and atomicMax), same buffers, same run
+    gen = torch.Generator().manual_seed(SEED)
+    x = c1_input(gen)
+    n = x.numel()
+    sets = n_sets(2 * n)
+    xs = [x.to(dev).clone() for _ in range(sets)]
+    am = torch.zeros((), dtype=torch.float32, device=dev)
+    k = max(steps, 50)
+    ms_ticket = time_gpu(lambda i: probe.mi355q_probe_amax_ticket(xs[i % sets].data_ptr(), n, am.data_ptr(), st), k, warmup)
+    assert float(am.cpu()) == float(x.abs().max().float())
+    ms_fill = time_gpu(lambda i: lib.mi355q_amax(xs[i % sets].data_ptr(), pkg.BF16, n, am.data_ptr(), st), k, warmup)
+    out.append(hbm_entry("probe_amax_ticket_form", "amax of bf16 [4096,4096] with partial maxima and a ticket instead of the zeroing launch",
+                         2 * n, ms_ticket, k, "probe_amax_ticket_kernel",
+                         extra={"product_form_ms_same_run": round(ms_fill, 5)}))
+    del xs
     return out
 
 

@@ -106,7 +106,8 @@ def probes():
     P.mi355q_probe_read.argtypes = [vp, i64, i32, vp, vp]
     P.mi355q_probe_coexec.argtypes = [i32, i32, i32, i32, i32, vp, vp]
     P.mi355q_probe_strip_read.argtypes = [vp, i64, i64, i32, i32, i32, vp, vp]
-    for name in ("mi355q_probe_mfma", "mi355q_probe_read", "mi355q_probe_strip_read", "mi355q_probe_coexec"):
+    P.mi355q_probe_amax_ticket.argtypes = [vp, i64, vp, vp]
+    for name in ("mi355q_probe_mfma", "mi355q_probe_read", "mi355q_probe_strip_read", "mi355q_probe_coexec", "mi355q_probe_amax_ticket"):
         getattr(P, name).restype = i32
     return P
 

@@ -16,6 +16,12 @@
 //                            MFMAs (mode bit 0), 32 x (v_exp_f32, v_mul_f32) in eight chains (bit 1), or both
 //                            dealt out in turns (3); the first wave of each SIMD takes mode_first, the second
 //                            mode_second
+//   mi355q_probe_amax_ticket the amax pass of mi355q_amax (bf16 input, the same loads and the same 256 workgroups of
+//                            1024 threads) without the launch that zeroes the result word: every workgroup stores
+//                            its maximum into a scratch array and draws a ticket, and the one that draws the last
+//                            ticket reduces the 256 values, writes the result and returns the ticket counter to
+//                            zero.  The form the product does not use: it is timed beside mi355q_amax so that the
+//                            comparison can be repeated
 // sink: a few bytes of device memory that are practically never written.
 #include "../device_common.h"
 
@@ -147,7 +153,77 @@ __global__ __launch_bounds__(256) void probe_strip_read_kernel(const uint8_t* ba
 
 using namespace mi355q;
 
+// ---- amax without the zeroing launch (see the head of the file)
+constexpr int kProbeAmaxThreads = 1024, kProbeAmaxBlocks = 256;
+static __device__ uint32_t probe_amax_part[kProbeAmaxBlocks];
+static __device__ uint32_t probe_amax_ticket;
+
+__global__ __launch_bounds__(kProbeAmaxThreads) void probe_amax_ticket_kernel(const uint8_t* __restrict__ x, int64_t nvec, uint32_t* __restrict__ out) {
+  constexpr int U = 4;
+  __shared__ uint32_t wave_part[kProbeAmaxThreads / 64];
+  __shared__ uint32_t last;
+  uint32_t am = 0;
+  const int64_t stride = (int64_t)gridDim.x * kProbeAmaxThreads;
+  for (int64_t v0 = (int64_t)blockIdx.x * kProbeAmaxThreads + threadIdx.x; v0 < nvec; v0 += stride * U) {
+    u32x4 in[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t v = v0 + (int64_t)u * stride;
+      ok[u] = v < nvec;
+      if (ok[u]) in[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x) + v);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (!ok[u]) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const u16x2 a = __builtin_bit_cast(u16x2, in[u][i] & 0x7fff7fffu);
+        am = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, __builtin_bit_cast(u16x2, am)));
+      }
+    }
+  }
+  {
+    const uint32_t lo = am & 0xffffu, hi = am >> 16;
+    am = (lo > hi ? lo : hi) << 16;
+  }
+  am = wave_max_u32(am);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) wave_part[wave] = am;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t r = wave_part[0];
+    for (int w = 1; w < kProbeAmaxThreads / 64; ++w) r = r > wave_part[w] ? r : wave_part[w];
+    __hip_atomic_store(&probe_amax_part[blockIdx.x], r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0);  // acknowledged before the ticket is drawn
+    const uint32_t t = __hip_atomic_fetch_add(&probe_amax_ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last = t == gridDim.x - 1;
+    if (last) __hip_atomic_store(&probe_amax_ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!last || wave != 0) return;
+  uint32_t r = 0;
+  for (int b = lane; b < (int)gridDim.x; b += 64) {
+    const uint32_t v = __hip_atomic_load(&probe_amax_part[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    r = r > v ? r : v;
+  }
+  r = wave_max_u32(r);
+  if (lane == 0) *out = r;
+}
+
 extern "C" {
+
+// x: bf16, 16-byte aligned, n a multiple of 8; out: one float (the bit pattern of the maximum of |x|).  One call at a
+// time per GPU (the scratch is shared).
+int mi355q_probe_amax_ticket(const void* x, int64_t n, float* out, void* stream) {
+  if (x == nullptr || out == nullptr || n <= 0 || n % 8 != 0 || reinterpret_cast<uintptr_t>(x) % 16 != 0) return MI355Q_ERR_INVALID_ARGUMENT;
+  const int64_t nvec = n / 8;
+  int64_t grid = (nvec + kProbeAmaxThreads * 4 - 1) / (kProbeAmaxThreads * 4);
+  if (grid > kProbeAmaxBlocks) grid = kProbeAmaxBlocks;
+  hipLaunchKernelGGL(probe_amax_ticket_kernel, dim3((unsigned)grid), dim3(kProbeAmaxThreads), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint8_t*>(x), nvec, reinterpret_cast<uint32_t*>(out));
+  return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
+}
 
 int mi355q_probe_mfma(int waves_per_simd, int mfma_per_wave, int workgroups, float* sink, void* stream) {
   if ((waves_per_simd != 1 && waves_per_simd != 2) || mfma_per_wave < 2 || workgroups <= 0 || sink == nullptr)
