@@ -348,6 +348,26 @@ def bench_ceilings(pkg, dev, steps, warmup):
                          2 * n, ms_ticket, k, "probe_amax_ticket_kernel",
                          extra={"product_form_ms_same_run": round(ms_fill, 5)}))
     del xs
+    # the column sum of [8192, 8192] e4m3fn as one kernel (the slices merged by the last arrival of each column block)
+    # beside the product's two kernels, same buffers, same run
+    m = 8192
+    codes = torch.tensor([0x00, 0x38, 0x40, 0x44, 0x48], dtype=torch.uint8)   # e4m3fn 0, 1, 2, 3, 4: every sum is exact
+    x8 = [codes[torch.randint(0, 5, (m, m), generator=gen)].to(dev) for _ in range(n_sets(m * m))]
+    res = torch.empty(m, dtype=torch.float32, device=dev)
+    ws_bytes = lib.mi355q_sum_fp8_workspace_bytes(1, m, m)
+    ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
+    k = max(steps, 50)
+    ms_ticket = time_gpu(lambda i: probe.mi355q_probe_sum_columns_ticket(x8[i % len(x8)].data_ptr(), m, m, res.data_ptr(), st), k, warmup)
+    ms_two = time_gpu(lambda i: lib.mi355q_sum_fp8(x8[i % len(x8)].data_ptr(), pkg.E4M3FN, 1, m, m, res.data_ptr(), pkg.F32,
+                                                   ws.data_ptr(), ws_bytes, st), k, warmup)
+    probe.mi355q_probe_sum_columns_ticket(x8[0].data_ptr(), m, m, res.data_ptr(), st)
+    got = res.clone()
+    lib.mi355q_sum_fp8(x8[0].data_ptr(), pkg.E4M3FN, 1, m, m, res.data_ptr(), pkg.F32, ws.data_ptr(), ws_bytes, st)
+    assert torch.equal(got, res) and torch.equal(res.cpu(), x8[0].cpu().view(E4).float().sum(0))
+    out.append(hbm_entry("probe_sum_columns_ticket_form", "sum_fp8 e4m3fn [8192,8192] over dim 0 as one kernel with a ticket merge",
+                         m * m + 4 * m, ms_ticket, k, "probe_sum_columns_ticket_kernel",
+                         extra={"product_form_ms_same_run": round(ms_two, 5)}))
+    del x8
     return out
 
 

@@ -107,7 +107,9 @@ def probes():
     P.mi355q_probe_coexec.argtypes = [i32, i32, i32, i32, i32, vp, vp]
     P.mi355q_probe_strip_read.argtypes = [vp, i64, i64, i32, i32, i32, vp, vp]
     P.mi355q_probe_amax_ticket.argtypes = [vp, i64, vp, vp]
-    for name in ("mi355q_probe_mfma", "mi355q_probe_read", "mi355q_probe_strip_read", "mi355q_probe_coexec", "mi355q_probe_amax_ticket"):
+    P.mi355q_probe_sum_columns_ticket.argtypes = [vp, i64, i64, vp, vp]
+    for name in ("mi355q_probe_mfma", "mi355q_probe_read", "mi355q_probe_strip_read", "mi355q_probe_coexec", "mi355q_probe_amax_ticket",
+                 "mi355q_probe_sum_columns_ticket"):
         getattr(P, name).restype = i32
     return P
 

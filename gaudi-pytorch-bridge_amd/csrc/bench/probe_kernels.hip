@@ -22,6 +22,10 @@
 //                            ticket reduces the 256 values, writes the result and returns the ticket counter to
 //                            zero.  The form the product does not use: it is timed beside mi355q_amax so that the
 //                            comparison can be repeated
+//   mi355q_probe_sum_columns_ticket  the column sum of mi355q_sum_fp8 (e4m3fn [R, C] over the rows, fp32 result; the same
+//                            loads, slices of 128 rows, 16 columns per lane) as one kernel: every slice stores its
+//                            partial sums and draws a ticket of its column block, and the workgroup that draws the
+//                            last one adds the slices in their order.  The product uses two kernels instead.
 // sink: a few bytes of device memory that are practically never written.
 #include "../device_common.h"
 
@@ -211,7 +215,101 @@ __global__ __launch_bounds__(kProbeAmaxThreads) void probe_amax_ticket_kernel(co
   if (lane == 0) *out = r;
 }
 
+// ---- column sum with the slices merged by the last arrival (see the head of the file)
+constexpr int kProbeSumMaxBlocks = 64, kProbeSumMaxSlices = 128;
+static __device__ __align__(256) float probe_sum_part[kProbeSumMaxSlices * kProbeSumMaxBlocks * 1024];  // [slice][column]
+static __device__ uint32_t probe_sum_ticket[kProbeSumMaxBlocks];
+
+__global__ __launch_bounds__(256) void probe_sum_columns_ticket_kernel(const uint8_t* __restrict__ x, int64_t R, int64_t C, int64_t per,
+                                                                       float* __restrict__ out) {
+  constexpr int WAVES = 4, VEC = 16;
+  __shared__ float part[WAVES - 1][64][VEC];
+  __shared__ uint32_t last;
+  const int s = blockIdx.y, splits = gridDim.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t c0 = ((int64_t)blockIdx.x * 64 + lane) * VEC;
+  const int64_t r0 = s * per, r1 = (r0 + per) < R ? (r0 + per) : R;
+  float acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
+  auto add = [&](const u32x4& t) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      float a, b, c, d;
+      cvt_f32x4<MI355Q_E4M3FN>(t[q], a, b, c, d);
+      acc[4 * q] += a; acc[4 * q + 1] += b; acc[4 * q + 2] += c; acc[4 * q + 3] += d;
+    }
+  };
+  {
+    const uint8_t* p = x + (r0 + wave) * C + c0;
+    const int64_t step = (int64_t)WAVES * C;
+    int64_t r = r0 + wave;
+    for (; r + 3 * WAVES < r1; r += 4 * WAVES) {
+      u32x4 w[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) w[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + u * step));
+#pragma unroll
+      for (int u = 0; u < 4; ++u) add(w[u]);
+      p += 4 * step;
+    }
+    for (; r < r1; r += WAVES, p += step) add(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)));
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) part[wave - 1][lane][e] = acc[e];
+  }
+  __syncthreads();
+  const int64_t ncol = (int64_t)gridDim.x * 1024;
+  if (wave == 0) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      float v = acc[e];
+#pragma unroll
+      for (int w = 0; w < WAVES - 1; ++w) v += part[w][lane][e];
+      __hip_atomic_store(&probe_sum_part[(int64_t)s * ncol + c0 + e], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_s_waitcnt(0);  // acknowledged before the ticket is drawn
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const uint32_t t = __hip_atomic_fetch_add(&probe_sum_ticket[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last = t == (uint32_t)splits - 1;
+    if (last) __hip_atomic_store(&probe_sum_ticket[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!last) return;
+  // 1024 columns, four per thread, the slices in their order
+  const int64_t c = (int64_t)blockIdx.x * 1024 + threadIdx.x * 4;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < splits; t += 4) {
+    float w[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        w[u][e] = t + u < splits ? __hip_atomic_load(&probe_sum_part[(int64_t)(t + u) * ncol + c + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] += w[u][e];
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) out[c + e] = v[e];
+}
+
 extern "C" {
+
+// x: e4m3fn [R, C] row-major, 16-byte aligned, C a multiple of 1024 and at most 65536, at most 128 slices of 128 rows;
+// out: C floats.  One call at a time per GPU (the scratch is shared).
+int mi355q_probe_sum_columns_ticket(const void* x, int64_t R, int64_t C, float* out, void* stream) {
+  const int64_t per = 128, splits = (R + per - 1) / per;
+  if (x == nullptr || out == nullptr || R <= 0 || C <= 0 || C % 1024 != 0 || C / 1024 > kProbeSumMaxBlocks || splits > kProbeSumMaxSlices ||
+      splits * C > (int64_t)kProbeSumMaxSlices * kProbeSumMaxBlocks * 1024 || reinterpret_cast<uintptr_t>(x) % 16 != 0)
+    return MI355Q_ERR_INVALID_ARGUMENT;
+  hipLaunchKernelGGL(probe_sum_columns_ticket_kernel, dim3((unsigned)(C / 1024), (unsigned)splits), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint8_t*>(x), R, C, per, out);
+  return hipGetLastError() == hipSuccess ? MI355Q_OK : MI355Q_ERR_LAUNCH;
+}
 
 // x: bf16, 16-byte aligned, n a multiple of 8; out: one float (the bit pattern of the maximum of |x|).  One call at a
 // time per GPU (the scratch is shared).
