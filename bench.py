@@ -628,11 +628,11 @@ def bench_sdpa(oracle, dev, steps, warmup, cpu):
     import math
     out = []
     gen = torch.Generator().manual_seed(SEED)
-    H, HK, D = 32, 8, 128
-    sc = 1.0 / math.sqrt(D)
-    for B, L in ((1, 8192), (4, 4096)):
-        if not want("sdpa", f"B{B}"):
+    H, HK = 32, 8
+    for B, L, D in ((1, 8192, 128), (4, 4096, 128), (1, 8192, 256)):
+        if not want("sdpa", f"B{B}" if D == 128 else f"D{D}"):
             continue
+        sc = 1.0 / math.sqrt(D)
         q = torch.randn(B, HK, H // HK, L, D, generator=gen).to(E4).to(dev)     # the grouped-query view of [B, H, L, D]
         k = torch.randn(B, HK, 1, L, D, generator=gen).to(E4).to(dev)
         v = torch.randn(B, HK, 1, L, D, generator=gen).to(E4).to(dev)
@@ -641,13 +641,14 @@ def bench_sdpa(oracle, dev, steps, warmup, cpu):
         ms = time_gpu(f, steps, warmup)
         flop = 4.0 * B * H * L * L * D * 0.5
         tf = flop / (ms * 1e-3) / 1e12
-        e = {"name": f"fp8_sdpa_B{B}_L{L}", "workload": f"fp8_sdpa_recomp_fwd causal, batch {B}, 32 query / 8 kv heads, "
-                                                        f"q_len = kv_len = {L}, head_dim 128, e4m3fn -> bf16",
+        name = f"fp8_sdpa_B{B}_L{L}" + ("" if D == 128 else f"_D{D}")
+        e = {"name": name, "workload": f"fp8_sdpa_recomp_fwd causal, batch {B}, 32 query / 8 kv heads, "
+                                       f"q_len = kv_len = {L}, head_dim {D}, e4m3fn -> bf16",
              "metric": "TFLOP/s", "value": round(tf, 1), "unit": "TFLOP/s", "ms_per_call": round(ms, 4), "steps": steps,
-             "roofline": {"bound": "mfma", "kernel": "fp8_sdpa_fwd_kernel<2,4,e4m3fn>", "achieved": round(tf, 1),
+             "roofline": {"bound": "mfma", "kernel": f"fp8_sdpa_fwd_kernel<{D // 64},{D // 32},e4m3fn>", "achieved": round(tf, 1),
                           "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / FP8_PEAK_TFLOPS, 4),
-                          "algorithmic_flop": flop, "traffic": MEASURED_TRAFFIC.get(f"fp8_sdpa_B{B}_L{L}")}}
-        if cpu and B == 1:
+                          "algorithmic_flop": flop, "traffic": MEASURED_TRAFFIC.get(name)}}
+        if cpu and B == 1 and D == 128:
             n = 1024    # a bounded sample: one head, the first 1024 queries and keys
             qc, kc, vc = q[0, 0, 0, :n].cpu(), k[0, 0, 0, :n].cpu(), v[0, 0, 0, :n].cpu()
             t = time_cpu(lambda: oracle.torch_fp8_sdpa(qc, kc, vc, is_causal=True, q_scale_s=128.0, d_scale_s=1 / 128.0), min_seconds=3.0)
@@ -655,6 +656,8 @@ def bench_sdpa(oracle, dev, steps, warmup, cpu):
                                  "kind": "port", "sample": f"one head, {n} queries x {n} keys, the float64 oracle"}
         out.append(e)
     # decoding: one query per head against a long cache; bound by reading k and v once
+    D = 128
+    sc = 1.0 / math.sqrt(D)
     for B, S in ((64, 4096), (8, 8192)):
         if not want("sdpa", f"decode_B{B}"):
             continue
@@ -744,7 +747,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", type=str, default="",
                     help="comma list of groups (gemm,cast,castlarge,int4,decode,mlp,reduce,w4a8,w4a16,sdpa,ceilings) or single workloads "
-                         "(decode_M16|M64|M256, w4a8_M16|M32|M64|M256, w4a16_M16|M64|M256, sdpa_B1|B4|decode_B64|decode_B8); "
+                         "(decode_M16|M64|M256, w4a8_M16|M32|M64|M256, w4a16_M16|M64|M256, sdpa_B1|B4|D256|decode_B64|decode_B8); "
                          "default: every group but ceilings (the measurement probes)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     args = ap.parse_args()

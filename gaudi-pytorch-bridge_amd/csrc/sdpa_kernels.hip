@@ -361,6 +361,11 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
 // chain of LDS reads, MFMAs, the softmax and MFMAs again) of which 1200 are vector work and 512 MFMA time, so a
 // SIMD is as busy as it has waves to switch between.
 constexpr bool sdpa_q_in_lds(int dkc, int dvt, bool dma) { return dma && dkc == 2 && dvt == 4; }
+// Workgroups per CU the kernel is compiled for.  Head dimension 256 (eight tiles of O: 128 registers) fits two with the
+// direct loads and a ring of two stages (255 registers, 64 KiB of LDS): 850 -> 1765 TFLOP/s at 32 / 8 heads and 8192
+// causal tokens against one workgroup with four stages.  Through registers (unaligned tensors) the same bound spills
+// 216 bytes per lane, so that form stays at one.
+constexpr int sdpa_workgroups_per_cu(int dkc, int dvt, bool dma) { return sdpa_q_in_lds(dkc, dvt, dma) ? 3 : (dvt <= 4 || dma) ? 2 : 1; }
 
 // DKC: 64-byte steps of the q.k depth (head_dim_qk <= 64 DKC); DVT: 32-column tiles of v
 // (head_dim_v <= 32 DVT).
@@ -370,7 +375,7 @@ constexpr bool sdpa_q_in_lds(int dkc, int dvt, bool dma) { return dma && dkc == 
 // puts there (vmcnt(0), in front of the first MFMA of every block) also waits for the blocks just requested
 // by the direct route.
 template <int DKC, int DVT, int FMT, bool DMA>
-__global__ __launch_bounds__(kSdpaThreads, (sdpa_q_in_lds(DKC, DVT, DMA) ? 3 : DVT <= 4 ? 2 : 1)) void fp8_sdpa_fwd_kernel(const SdpaArgs a) {
+__global__ __launch_bounds__(kSdpaThreads, sdpa_workgroups_per_cu(DKC, DVT, DMA)) void fp8_sdpa_fwd_kernel(const SdpaArgs a) {
   constexpr bool kQLds = sdpa_q_in_lds(DKC, DVT, DMA);
   constexpr int KROW = DKC * 64;
   constexpr int kVRow = DVT <= 4 ? 128 : 256;  // bytes of an LDS row of V
@@ -383,8 +388,9 @@ __global__ __launch_bounds__(kSdpaThreads, (sdpa_q_in_lds(DKC, DVT, DMA) ? 3 : D
   static_assert(KLOADS >= 1 && VLOADS >= 1, "block too small for the workgroup");
   // Direct loads run kStages - 1 blocks ahead of the arithmetic (a block's arithmetic takes about a
   // microsecond, less than a load from HBM under load; with the queries in LDS one block ahead, which the
-  // third workgroup on the CU covers); the route through registers uses two buffers.
-  constexpr int kStages = kQLds ? 2 : 4;
+  // third workgroup on the CU covers, and at head dimension 256, where two stages are what leaves room for a second
+  // workgroup); the route through registers uses two buffers.
+  constexpr int kStages = (kQLds || DVT > 4) ? 2 : 4;
   __shared__ __align__(1024) uint8_t lds[kStages * (KBYTES + VBYTES)];
   __shared__ __align__(16) uint8_t qlds[kQLds ? 4 * 4096 : 16];  // per wave: [depth chunk of 16 bytes][half-wave][row]
 

@@ -262,21 +262,24 @@ def test_long_sequence_properties(oracle, dev):
     assert (o1 - 1.0).abs().max() <= 2.0 ** -4
 
 
-def test_prefill_at_the_benchmark_shape(oracle, dev):
-    """32 query / 8 kv heads, q_len = kv_len = 8192, head_dim 128, causal, in the wrapper's grouped layout (what
-    bench.py times as fp8_sdpa_B1_L8192: 64 query blocks x 32 heads, kv broadcast along the heads of a group):
+@pytest.mark.parametrize("D", [128, 256])
+def test_prefill_at_the_benchmark_shape(oracle, dev, D):
+    """32 query / 8 kv heads, q_len = kv_len = 8192, head_dim 128 or 256, causal, in the wrapper's grouped layout (what
+    bench.py times as fp8_sdpa_B1_L8192 and fp8_sdpa_B1_L8192_D256: 64 query blocks x 32 heads, kv broadcast along the
+    heads of a group; at 256 two workgroups share a CU and the ring of two stages wraps 64 times):
     sampled rows of sampled heads against the oracle, every row of one head against the property that v = 1 gives 1."""
-    G, HG, L, D = 8, 4, 8192, 128
-    gen = torch.Generator().manual_seed(8192)
+    G, HG, L = 8, 4, 8192
+    gen = torch.Generator().manual_seed(8192 + D)
     q, k, v = make_qkv(gen, (1, G, HG, L, D), (1, G, 1, L, D), (1, G, 1, L, D))
     sc = (None, None, None, 128.0, None, 1 / 128.0)
     out = run_op(dev, q, k, v, causal=True, scales=sc)[0].cpu()
     assert out.shape == (1, G, HG, L, D)
     rows = [0, 1, 63, 64, 127, 128, 4095, 4096, 5000, 8063, 8064, 8191]
     for g, h in ((0, 0), (3, 2), (7, 3)):
-        for i in rows:
-            ref, _, _ = oracle.torch_fp8_sdpa(q[0, g, h, i:i + 1], k[0, g, 0, :i + 1], v[0, g, 0, :i + 1], q_scale_s=128.0, d_scale_s=1 / 128.0)
-            check_bf16(out[0, g, h, i:i + 1], ref, f"group {g} head {h} row {i}", vmax=float(v.float().abs().max()))
+        # the rows of a head are judged together: the bound allows 0.5 % of the values one flipped fp8 rounding
+        refs = [oracle.torch_fp8_sdpa(q[0, g, h, i:i + 1], k[0, g, 0, :i + 1], v[0, g, 0, :i + 1], q_scale_s=128.0, d_scale_s=1 / 128.0)[0]
+                for i in rows]
+        check_bf16(out[0, g, h, rows], torch.cat(refs), f"group {g} head {h}", vmax=float(v.float().abs().max()))
     # heads of one group differ (their queries do), groups read their own k / v
     assert not torch.equal(out[0, 0, 0], out[0, 0, 1]) and not torch.equal(out[0, 0, 0], out[0, 1, 0])
     o1 = run_op(dev, q, k, torch.ones_like(v.float()).to(E4), causal=True, scales=sc)[0].cpu().float()
