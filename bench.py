@@ -63,6 +63,7 @@ MEASURED_TRAFFIC = {
     "w4a16_gemm_M256": 316.05e6,
     "fp8_sdpa_B1_L8192": 124.63e6,
     "fp8_sdpa_B4_L4096": 235.55e6,
+    "fp8_sdpa_B1_L8192_D256": 347.00e6,   # k and v are re-read by the query blocks of a head group beyond L2
     "fp8_sdpa_decode_B64_S4096": 537.37e6,
     "fp8_sdpa_decode_B8_S8192": 143.15e6,   # fp8_sdpa_decode_kernel 138.81 + 4.34 written and read back by the merge
     "softmax_fp8": 1609.32e6,
