@@ -328,6 +328,29 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
   else exponentials(std::false_type{}, std::true_type{});
   l_run = l_run * alpha + psum;
 
+  // With the queries in LDS (three workgroups per CU, no registers for V fragments during the softmax) the V fragments
+  // are read here: the 32 score registers are dead, and the reads' latency passes under the rescaling of O instead of
+  // standing in front of each P V product.
+  constexpr bool kMidV = DVT <= 4 && QL;
+  i32x8 vfm[kMidV ? DVT : 1];
+  if constexpr (kMidV) {
+#pragma unroll
+    for (int t = 0; t < DVT; ++t) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const int krow = 32 * (p >> 1) + 8 * (2 * (p & 1) + (r8 >> 2)) + 4 * h + (r8 & 3);
+        const int off = v_lds_offset<kVRow>(krow, 2 * t + (g & 1)) + hh * 8;
+        const i32x2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((SDPA_LDS_AS i32x2*)((SDPA_LDS_AS uint8_t*)vb + off));
+        vfm[t][2 * p] = w[0];
+        vfm[t][2 * p + 1] = w[1];
+      }
+    }
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+    for (int t = 0; t < DVT; ++t) asm volatile("" : "+v"(vfm[t]));  // issued here, not sunk to their use
+#endif
+  }
+
   if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
     for (int t = 0; t < DVT; ++t)
@@ -340,6 +363,10 @@ __device__ __forceinline__ void sdpa_block(const SdpaArgs& a, const uint8_t* kb,
   for (int t = 0; t < DVT; ++t) {
     if constexpr (kEarlyV) {
       o[t] = sdpa_mfma<FMT>(vfe[t], pf, o[t]);
+      continue;
+    }
+    if constexpr (kMidV) {
+      o[t] = sdpa_mfma<FMT>(vfm[t], pf, o[t]);
       continue;
     }
     i32x8 vf;
