@@ -526,6 +526,33 @@ constexpr int kW4WideConsumers = 8;
 constexpr int kW4WideThreads = (kW4WideConsumers + kW4ColWaves) * 64;
 constexpr int kW4SumRing = 4;  // stages of row sums kept
 
+// The e4m3 codes 0 .. 15 are one linear ramp, q x 2^-9 (eight subnormals and the first binade): a nibble
+// zero-extended to a byte is an fp8 operand as it stands, and one MFMA with the block scale 2^9 accumulates
+// sum_k a q exactly.  Eight nibbles w become the bytes of w & 0x0f0f0f0f (nibbles 0, 2, 4, 6) and of
+// (w >> 4) & 0x0f0f0f0f (nibbles 1, 3, 5, 7): the transposing LDS read fills nibble i of a lane from the row
+// that lane i of its group of 16 addresses, so the lanes address the rows in the order that leaves k ascending
+// over the two registers (w4_nibble_row).
+constexpr int kW4ByteScale = 127 + 9;
+__device__ __forceinline__ int w4_nibble_row(int i) { return (i & 8) | ((i & 1) << 2) | ((i >> 1) & 3); }
+__device__ __forceinline__ i32x8 w4_bytes(const i32x2& w0, const i32x2& w1, uint32_t flip) {
+  i32x8 r;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t w = (uint32_t)(j < 2 ? w0[j & 1] : w1[j & 1]) ^ flip;
+    r[2 * j] = (int)(w & 0x0f0f0f0fu);
+    r[2 * j + 1] = (int)((w >> 4) & 0x0f0f0f0fu);
+  }
+  return r;
+}
+template <int FMT_A, int E>
+__device__ __forceinline__ f32x16 w4_mfma_bytes(const i32x8& w8, const i32x8& fa, const f32x16& c) {
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w8, fa, c, 0, mfma_code<FMT_A>(), 0, E, 0, 127);
+}
+template <int FMT_A, int E>
+__device__ __forceinline__ f32x4 w4_mfma16_bytes(const i32x8& w8, const i32x8& fa, const f32x4& c) {
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w8, fa, c, 0, mfma_code<FMT_A>(), 0, E, 0, 127);
+}
+
 template <int FMT_A>
 __device__ __forceinline__ f32x4 w4_mfma16(const u32x4& plane, const i32x8& fa, const f32x4& c, int e) {
   const i32x8 b = {(int)plane[0], (int)plane[1], (int)plane[2], (int)plane[3], 0, 0, 0, 0};
@@ -738,7 +765,7 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
       int poff[2][2];
 #pragma unroll
       for (int p = 0; p < 2; ++p) {
-        const int row = 16 * (4 * (gk & 1) + (gk >> 1) + 2 * p) + r16;
+        const int row = 32 * gk + 16 * p + w4_nibble_row(r16);  // the fp8 operand of lane group gk: k = 32 gk .. + 31
 #pragma unroll
         for (int t = 0; t < 2; ++t) poff[t][p] = kOffPacked + row * 128 + ((wq ^ ((row >> 1) & 7)) << 4) + t * 8;
       }
@@ -790,19 +817,11 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         const i32x8 fa = {(int)alo[0], (int)alo[1], (int)alo[2], (int)alo[3], (int)ahi[0], (int)ahi[1], (int)ahi[2], (int)ahi[3]};
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-          u32x4 hi, lo;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const uint32_t w = (uint32_t)wt[t][r >> 1][r & 1] ^ flip;
-            lo[r] = w & 0x33333333u;
-            hi[r] = (w >> 2) & 0x33333333u;
-          }
-          acc[B][t] = w4_mfma16<FMT_A>(hi, fa, f32x4{0.f, 0.f, 0.f, 0.f}, 130);
-          acc[B][t] = w4_mfma16<FMT_A>(lo, fa, acc[B][t], 128);
+          const i32x8 w8 = w4_bytes(wt[t][0], wt[t][1], flip);
+          acc[B][t] = w4_mfma16_bytes<FMT_A, kW4ByteScale>(w8, fa, f32x4{0.f, 0.f, 0.f, 0.f});
           if constexpr (A16) {
             const i32x8 fb = {(int)blo[0], (int)blo[1], (int)blo[2], (int)blo[3], (int)bhi[0], (int)bhi[1], (int)bhi[2], (int)bhi[3]};
-            acc[B][t] = w4_mfma16<FMT_A>(hi, fb, acc[B][t], 126);
-            acc[B][t] = w4_mfma16<FMT_A>(lo, fb, acc[B][t], 124);
+            acc[B][t] = w4_mfma16_bytes<FMT_A, kW4ByteScale - 4>(w8, fb, acc[B][t]);
           }
         }
         // the stage before this one, whose MFMAs finished long ago, behind the MFMAs just issued
@@ -837,7 +856,7 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
       int poff[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int row = 32 * j + 16 * th + tr;
+        const int row = 64 * (j >> 1) + 32 * th + 16 * (j & 1) + w4_nibble_row(tr);  // fp8 operand of lane half th: k = 32 th .. + 31
         poff[j] = kOffPacked + row * 128 + ((wq ^ ((row >> 1) & 7)) << 4) + (tg & 1) * 8;
       }
       const int soff = kOffScale + (wn + 4 * (lane >> 5)) * 2;
@@ -897,24 +916,14 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-          u32x4 hi, lo;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const uint32_t w = (uint32_t)wt[2 * ks + (r >> 1)][r & 1] ^ flip;
-            lo[r] = w & 0x33333333u;
-            hi[r] = (w >> 2) & 0x33333333u;
-          }
+          const i32x8 w8 = w4_bytes(wt[2 * ks], wt[2 * ks + 1], flip);
           const int f = MT == 1 ? ks : 0;
           static_for<MT>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            if (ks == 0) acc[B][i] = w4_mfma<FMT_A, 130>(hi, fa[f][i], zero);
-            else acc[B][i] = w4_mfma<FMT_A, 130>(hi, fa[f][i], acc[B][i]);
-            acc[B][i] = w4_mfma<FMT_A, 128>(lo, fa[f][i], acc[B][i]);
-            if constexpr (A16) {
-              acc[B][i] = w4_mfma<FMT_A, 126>(hi, fb[f][i], acc[B][i]);
-              acc[B][i] = w4_mfma<FMT_A, 124>(lo, fb[f][i], acc[B][i]);
-            }
+            if (ks == 0) acc[B][i] = w4_mfma_bytes<FMT_A, kW4ByteScale>(w8, fa[f][i], zero);
+            else acc[B][i] = w4_mfma_bytes<FMT_A, kW4ByteScale>(w8, fa[f][i], acc[B][i]);
+            if constexpr (A16) acc[B][i] = w4_mfma_bytes<FMT_A, kW4ByteScale - 4>(w8, fb[f][i], acc[B][i]);
           });
           if constexpr (MT == 2) {
             if (ks == 0) read_a(1);
