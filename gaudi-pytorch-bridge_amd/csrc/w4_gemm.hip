@@ -568,7 +568,9 @@ __device__ __forceinline__ f32x4 w4_mfma16(const u32x4& plane, const i32x8& fa, 
 template <int FMT_A, bool HAS_Z, int ROWS, bool A16 = false>
 __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
   constexpr bool M16 = ROWS == 16;
-  constexpr int BM = ROWS == 64 ? 64 : 32, MT = BM / 32;
+  constexpr bool F16 = ROWS == 16 || ROWS == 128;  // the 16x16x128 MFMA: one tile of 16 rows, or eight
+  constexpr int RT = ROWS == 128 ? 8 : 1;          // row tiles of 16 in that form
+  constexpr int BM = ROWS >= 64 ? ROWS : 32, MT = BM / 32;
   constexpr int kConsumers = kW4WideConsumers;
   constexpr int S = w4_wide_stages(BM, A16), kStage = w4_wide_stage(BM, A16);
   constexpr int kOffLo = BM * kBK;  // the second plane's tile (A16)
@@ -576,8 +578,8 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
   constexpr int NV = M16 ? 8 : 16 * MT;  // results per consumer lane
   // the 16-row form reads A fragments shaped for the 16x16x128 MFMA: the XOR of TileGeom's variant 1 keeps those off
   // each other's banks
-  using LA = DmaLoader<true, BM, kBK, kW4ColWaves, ROWS == 16 ? 1 : 0>;
-  using GA = TileGeom<true, BM, kBK, ROWS == 16 ? 1 : 0>;
+  using LA = DmaLoader<true, BM, kBK, kW4ColWaves, F16 ? 1 : 0>;
+  using GA = TileGeom<true, BM, kBK, F16 ? 1 : 0>;
   constexpr int kOps = 4 + LA::kPerWave * (A16 ? 2 : 1) + 1;  // four 1 KiB regions of weights, A, and the scale or zero-point row
   static_assert(S >= 3 && (S - 2) * kOps <= 63, "vmcnt holds 6 bits");
   static_assert(kStage % 1024 == 0, "stages stay 1 KiB aligned");
@@ -650,7 +652,7 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
       const i32x4 rp = wp.rsrc(0x7fffffffLL);
       // with tiles of 16 or 32 rows there is one row block: the weights are read once (with 64-row tiles further
       // row blocks read them again, out of the caches)
-      constexpr bool kOnce = ROWS != 64;
+      constexpr bool kOnce = ROWS < 64;
       w4_dma16<kOnce>(rp, vo_even, base + kOffPacked + (wq * 4) * 1024);
       w4_dma16<kOnce>(rp, vo_odd, base + kOffPacked + (wq * 4 + 1) * 1024);
       w4_dma16<kOnce>(rp, vo_even + 16 * ld, base + kOffPacked + (wq * 4 + 2) * 1024);
@@ -681,21 +683,26 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
     const u32x4 ones = {0x22222222u, 0x22222222u, 0x22222222u, 0x22222222u};  // e2m1 1.0
     auto sum_rows = [&](int off, int slot) {
       const uint8_t* st = lds + off;
-      if constexpr (M16) {
+      if constexpr (F16) {
         const int m = lane & 15, gk = lane >> 4;
-        const u32x4 lo = *reinterpret_cast<const u32x4*>(st + GA::lds_offset(m, 2 * gk));
-        const u32x4 hi = *reinterpret_cast<const u32x4*>(st + GA::lds_offset(m, 2 * gk + 1));
-        const i32x8 fa = {(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-        f32x4 r = w4_mfma16<FMT_A>(ones, fa, f32x4{0.f, 0.f, 0.f, 0.f}, 127);
-        if constexpr (A16) {
-          const u32x4 lo2 = *reinterpret_cast<const u32x4*>(st + kOffLo + GA::lds_offset(m, 2 * gk));
-          const u32x4 hi2 = *reinterpret_cast<const u32x4*>(st + kOffLo + GA::lds_offset(m, 2 * gk + 1));
-          const i32x8 fb = {(int)lo2[0], (int)lo2[1], (int)lo2[2], (int)lo2[3], (int)hi2[0], (int)hi2[1], (int)hi2[2], (int)hi2[3]};
-          r = w4_mfma16<FMT_A>(ones, fb, r, 123);
-        }
-        // every lane holds the sum of its row (lane % 16) and every lane stores it: a store under a lane mask would
-        // take the MFMA, whose result only those lanes used, under the mask with it
-        row_sums[slot][lane & 15] = r[0];
+        const int o0 = GA::lds_offset(m, 2 * gk), o1 = GA::lds_offset(m, 2 * gk + 1);  // rows 16 further on: + 2048
+        static_for<RT>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          const u32x4 lo = *reinterpret_cast<const u32x4*>(st + o0 + 2048 * i);
+          const u32x4 hi = *reinterpret_cast<const u32x4*>(st + o1 + 2048 * i);
+          const i32x8 fa = {(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+          f32x4 r = w4_mfma16<FMT_A>(ones, fa, f32x4{0.f, 0.f, 0.f, 0.f}, 127);
+          if constexpr (A16) {
+            const u32x4 lo2 = *reinterpret_cast<const u32x4*>(st + kOffLo + o0 + 2048 * i);
+            const u32x4 hi2 = *reinterpret_cast<const u32x4*>(st + kOffLo + o1 + 2048 * i);
+            const i32x8 fb = {(int)lo2[0], (int)lo2[1], (int)lo2[2], (int)lo2[3], (int)hi2[0], (int)hi2[1], (int)hi2[2], (int)hi2[3]};
+            r = w4_mfma16<FMT_A>(ones, fb, r, 123);
+          }
+          // every lane holds the sum of its row (lane % 16 of tile i) and every lane stores it: a store under a lane
+          // mask would take the MFMA, whose result only those lanes used, under the mask with it.  A consumer lane
+          // finds the sums of its RT rows side by side.
+          row_sums[slot][(lane & 15) * RT + i] = r[0];
+        });
       } else {
         static_for<MT>([&](auto ic) {
           constexpr int i = decltype(ic)::value;
@@ -850,6 +857,114 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         if (KT & 1) fold(std::integral_constant<int, 0>{}, (slot - 1) & (kW4SumRing - 1));
         else fold(std::integral_constant<int, 1>{}, (slot - 1) & (kW4SumRing - 1));
       }
+    } else if constexpr (ROWS == 128) {
+      // 128 rows as eight tiles of 16 on the 16x16x128 MFMA, which takes a whole stage of K in one instruction: the
+      // sixteen products of a stage (eight row tiles by two column tiles) are independent, and each is folded into
+      // the totals two products later, eight multiply-adds behind an MFMA that lasts as long as they do.  The scale
+      // term of a product uses its own stage's scales; the zero-point term, -(z x scale)[n] x (row sum of A)[m],
+      // whose factors the producers leave in LDS during a stage, follows one stage later.
+      // lane: rows m = 16 i + lane % 16 of A; columns wn + 16 t + 4 gk + e; product j = 2 i + t, total[4 j + e]
+      const int gk = lane >> 4, r16 = lane & 15;
+      int poff[2][2];
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        const int row = 32 * gk + 16 * p + w4_nibble_row(r16);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) poff[t][p] = kOffPacked + row * 128 + ((wq ^ ((row >> 1) & 7)) << 4) + t * 8;
+      }
+      const int aoff0 = GA::lds_offset(r16, 2 * gk), aoff1 = GA::lds_offset(r16, 2 * gk + 1);  // tile i: + 2048 i
+      const int soff = kOffScale + (wn + 4 * gk) * 2;  // + 32 t: four bf16
+      const int zsoff = wn + 4 * gk;                   // + 16 t: four fp32
+      constexpr int NB = 3, LAG = 2;
+      f32x4 acc[NB];
+      f32x4 sc[2], zsp[2];
+      float rsp[RT];
+      auto stage = [&](auto hpc) {
+        constexpr bool ZT = decltype(hpc)::value && HAS_Z;  // a stage before this one has left its zero-point term
+        __syncthreads();  // the stage is in LDS, and so are the row sums and zero-point row of the one before
+        const uint8_t* st = lds + rd_off;
+        i32x2 wt[2][2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int p = 0; p < 2; ++p)
+            wt[t][p] = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LDS_AS i32x2*)((LDS_AS uint8_t*)st + poff[t][p]));
+        i32x8 fa[2], fb[A16 ? 2 : 1];
+        auto read_a = [&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          const u32x4 lo = *reinterpret_cast<const u32x4*>(st + aoff0 + 2048 * i), hi = *reinterpret_cast<const u32x4*>(st + aoff1 + 2048 * i);
+          fa[i & 1] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+          if constexpr (A16) {
+            const u32x4 lo2 = *reinterpret_cast<const u32x4*>(st + kOffLo + aoff0 + 2048 * i);
+            const u32x4 hi2 = *reinterpret_cast<const u32x4*>(st + kOffLo + aoff1 + 2048 * i);
+            fb[i & 1] = i32x8{(int)lo2[0], (int)lo2[1], (int)lo2[2], (int)lo2[3], (int)hi2[0], (int)hi2[1], (int)hi2[2], (int)hi2[3]};
+          }
+        };
+        read_a(std::integral_constant<int, 0>{});
+        u32x2 snew[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) snew[t] = *reinterpret_cast<const u32x2*>(st + soff + 32 * t);
+        if constexpr (ZT) {
+          const int prev = slot - 1;
+#pragma unroll
+          for (int t = 0; t < 2; ++t) zsp[t] = *reinterpret_cast<const f32x4*>(&zs_rows[prev & 1][zsoff + 16 * t]);
+          const f32x4 r0 = *reinterpret_cast<const f32x4*>(&row_sums[prev & (kW4SumRing - 1)][r16 * RT]);
+          const f32x4 r1 = *reinterpret_cast<const f32x4*>(&row_sums[prev & (kW4SumRing - 1)][r16 * RT + 4]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            rsp[i] = r0[i];
+            rsp[4 + i] = r1[i];
+          }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          sc[t][0] = __uint_as_float(snew[t][0] << 16);
+          sc[t][1] = __uint_as_float(snew[t][0] & 0xffff0000u);
+          sc[t][2] = __uint_as_float(snew[t][1] << 16);
+          sc[t][3] = __uint_as_float(snew[t][1] & 0xffff0000u);
+        }
+        const i32x8 w8[2] = {w4_bytes(wt[0][0], wt[0][1], flip), w4_bytes(wt[1][0], wt[1][1], flip)};
+        auto fold = [&](auto jc) {
+          constexpr int j = decltype(jc)::value, t = j & 1, i = j >> 1, b = j % NB;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float v = __builtin_fmaf(acc[b][e], sc[t][e], total[4 * j + e]);
+            if constexpr (ZT) v = __builtin_fmaf(zsp[t][e], rsp[i], v);
+            total[4 * j + e] = v;
+          }
+        };
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<2 * RT>([&](auto jc) {
+          constexpr int j = decltype(jc)::value, t = j & 1, i = j >> 1, b = j % NB;
+          if constexpr (t == 0 && i + 1 < RT) read_a(std::integral_constant<int, i + 1>{});
+          acc[b] = w4_mfma16_bytes<FMT_A, kW4ByteScale>(w8[t], fa[i & 1], f32x4{0.f, 0.f, 0.f, 0.f});
+          if constexpr (A16) acc[b] = w4_mfma16_bytes<FMT_A, kW4ByteScale - 4>(w8[t], fb[i & 1], acc[b]);
+          if constexpr (j >= LAG) fold(std::integral_constant<int, j - LAG>{});
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        static_for<LAG>([&](auto lc) { fold(std::integral_constant<int, 2 * RT - LAG + decltype(lc)::value>{}); });
+        rd_off += kStage;
+        if (rd_off == S * kStage) rd_off = 0;
+        ++slot;
+      };
+      if (KT > 0) stage(F{});
+      for (int kt = 1; kt < KT; ++kt) stage(T{});
+      __syncthreads();  // the row sums and zero-point row of the last stage
+      if constexpr (HAS_Z) {
+        if (KT > 0) {
+          const int prev = slot - 1;
+#pragma unroll
+          for (int t = 0; t < 2; ++t) zsp[t] = *reinterpret_cast<const f32x4*>(&zs_rows[prev & 1][zsoff + 16 * t]);
+#pragma unroll
+          for (int i = 0; i < RT; ++i) {
+            const float rs = row_sums[prev & (kW4SumRing - 1)][r16 * RT + i];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) total[4 * (2 * i + t) + e] = __builtin_fmaf(zsp[t][e], rs, total[4 * (2 * i + t) + e]);
+          }
+        }
+      }
     } else {
       // lane: rows m = 32 i + lane % 32 of A (i < MT); columns wn + 8 q + 4 (lane / 32) + c, e = 4 q + c
       const int tg = lane >> 4, tr = lane & 15, th = tg >> 1;
@@ -1001,22 +1116,23 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
     }
   }
   if (producer) return;
-  if constexpr (M16) {
-    // C[m, n .. n + 3] for this lane's row and its two sets of four columns
-    const int gk = lane >> 4, m = lane & 15;
+  if constexpr (F16) {
+    // C[m, n .. n + 3] for this lane's rows (one per row tile) and its two sets of four columns
+    const int gk = lane >> 4;
     const ScalarScales scalars = load_scalar_scales(g);
-    if (m >= g.M) return;
-    const float sa = g.sa_mode == MI355Q_GS_PER_ROW ? g.sa[m] : scalars.sa;
     const int es = g.out_bf16 ? 2 : 4;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int j = 0; j < 2 * RT; ++j) {
+      const int t = j & 1, m = 16 * (j >> 1) + (lane & 15);
+      if (m >= g.M) continue;
+      const float sa = g.sa_mode == MI355Q_GS_PER_ROW ? g.sa[m] : scalars.sa;
       const int n = n0 + wq * 32 + 16 * t + 4 * gk;
       if (n >= g.N) continue;  // N is a multiple of 32: the four columns are inside or outside together
       float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float bias = g.bias_mode == MI355Q_BIAS_ROW_VECTOR ? load_out_as_f32(g.bias, n + e, g.out_bf16) : 0.0f;
-        v[e] = __fmul_rn(total[4 * t + e], sa) + bias;  // rounded as the other epilogues round
+        v[e] = __fmul_rn(total[4 * j + e], sa) + bias;  // rounded as the other epilogues round
       }
       uint8_t* cp = g.C + ((int64_t)m * g.ldc + n) * es;
       const bool vec_ok = (reinterpret_cast<uintptr_t>(cp) % (4 * es)) == 0;
@@ -1051,7 +1167,7 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
 // blocks, strips, and the parts K is walked in (0: the wide kernel does not apply).
 struct W4WidePlan {
   int rows, row_blocks, strips, parts;
-  int tile_rows() const { return rows == 64 ? 64 : 32; }
+  int tile_rows() const { return rows >= 64 ? rows : 32; }
   // The counters sit in front of the partial sums, in an area of a fixed size: a workspace that is used for
   // problems of different shapes then finds them zero whatever the last shape left in the partial sums.
   // K is only split for at most 128 strips (256 / groups >= 2 below).
@@ -1063,7 +1179,7 @@ struct W4WidePlan {
 inline W4WidePlan w4a8_wide_plan(int64_t M, int64_t N, int64_t K, int64_t group, int scale_f32) {
   W4WidePlan p{0, 0, 0, 0};
   if (group != kBK || scale_f32 || K <= 0 || M <= 0 || N <= 0) return p;
-  p.rows = M <= 16 ? 16 : (M <= 32 ? 32 : 64);
+  p.rows = M <= 16 ? 16 : (M <= 32 ? 32 : (M <= 64 ? 64 : 128));
   p.row_blocks = (int)((M + p.tile_rows() - 1) / p.tile_rows());
   p.strips = (int)((N + kW4WideBN - 1) / kW4WideBN);
   const int64_t kt = (K + kBK - 1) / kBK, groups = (int64_t)p.strips * p.row_blocks;
@@ -1099,10 +1215,14 @@ void w4a8_launch_by_m(const W4Args& a, hipStream_t st) {
       const dim3 grid(strips * (unsigned)a.ksplit);
       if (z) w4a8_wide_kernel<FMT_A, true, 32><<<grid, kW4WideThreads, 0, st>>>(a);
       else w4a8_wide_kernel<FMT_A, false, 32><<<grid, kW4WideThreads, 0, st>>>(a);
-    } else {
-      const dim3 grid(strips * (unsigned)a.ksplit, (unsigned)((a.g.M + 63) / 64));
+    } else if (a.g.M <= 64) {
+      const dim3 grid(strips * (unsigned)a.ksplit);
       if (z) w4a8_wide_kernel<FMT_A, true, 64><<<grid, kW4WideThreads, 0, st>>>(a);
       else w4a8_wide_kernel<FMT_A, false, 64><<<grid, kW4WideThreads, 0, st>>>(a);
+    } else {
+      const dim3 grid(strips * (unsigned)a.ksplit, (unsigned)((a.g.M + 127) / 128));
+      if (z) w4a8_wide_kernel<FMT_A, true, 128><<<grid, kW4WideThreads, 0, st>>>(a);
+      else w4a8_wide_kernel<FMT_A, false, 128><<<grid, kW4WideThreads, 0, st>>>(a);
     }
   } else if (a.g.M <= 32) {
     w4a8_launch<32, FMT_A>(a, st);
@@ -1125,10 +1245,14 @@ inline void w4a16_launch(const W4Args& a, hipStream_t st) {
     const dim3 grid(strips * (unsigned)a.ksplit);
     if (z) w4a8_wide_kernel<F, true, 32, true><<<grid, kW4WideThreads, 0, st>>>(a);
     else w4a8_wide_kernel<F, false, 32, true><<<grid, kW4WideThreads, 0, st>>>(a);
-  } else {
-    const dim3 grid(strips * (unsigned)a.ksplit, (unsigned)((a.g.M + 63) / 64));
+  } else if (a.g.M <= 64) {
+    const dim3 grid(strips * (unsigned)a.ksplit);
     if (z) w4a8_wide_kernel<F, true, 64, true><<<grid, kW4WideThreads, 0, st>>>(a);
     else w4a8_wide_kernel<F, false, 64, true><<<grid, kW4WideThreads, 0, st>>>(a);
+  } else {
+    const dim3 grid(strips * (unsigned)a.ksplit, (unsigned)((a.g.M + 127) / 128));
+    if (z) w4a8_wide_kernel<F, true, 128, true><<<grid, kW4WideThreads, 0, st>>>(a);
+    else w4a8_wide_kernel<F, false, 128, true><<<grid, kW4WideThreads, 0, st>>>(a);
   }
 }
 

@@ -160,7 +160,7 @@ def test_split_k_workspace_c_abi(oracle, pkg, dev):
     strips = (N + 255) // 256
     assert need == 1024 + 4 * strips * 32 * 256 * 4                       # 1 KiB of counters; K / 128 / 8 = 4 parts
     assert lib.mi355q_w4a8_gemm_workspace_bytes(33, N, K, group, pkg.BF16) == 1024 + 4 * strips * 64 * 256 * 4   # 64-row tiles
-    assert lib.mi355q_w4a8_gemm_workspace_bytes(130, N, K, group, pkg.BF16) == 1024 + 4 * strips * 3 * 64 * 256 * 4  # three row blocks
+    assert lib.mi355q_w4a8_gemm_workspace_bytes(130, N, K, group, pkg.BF16) == 1024 + 4 * strips * 2 * 128 * 256 * 4  # two row blocks of 128
     assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, 256, pkg.BF16) == 0       # groups of two stages
     assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, pkg.F32) == 0      # fp32 scales
     assert lib.mi355q_w4a8_gemm_workspace_bytes(M, N, 1024, group, pkg.BF16) == 0  # too few stages to split
