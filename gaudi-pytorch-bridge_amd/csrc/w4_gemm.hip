@@ -488,7 +488,7 @@ __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
 }
 
 // ---------------------------------------------------------------------------------- wide strips
-// For groups of 128 and bf16 scales (tiles of 16, 32 or 64 rows; more rows are further row blocks of 64).
+// For groups of 128 and bf16 scales (tiles of 16, 32, 64 or 128 rows; more rows are further row blocks of 128).
 // A workgroup takes 256 columns: a k-row
 // of its packed weights is a whole 128-byte line (the 64-byte rows of the 128-column strips move
 // at about 3.2 TB/s, whole lines at 4.3), and K is cut into `ksplit` parts walked by as many
@@ -502,21 +502,20 @@ __global__ __launch_bounds__(kW4Threads) void w4a8_gemm_kernel(W4Args a) {
 // columns and four producers.  The 16-byte slots of a packed row in LDS are XORed with
 // (row / 2) % 8, which spreads the 16 rows of a transposing read over all banks.
 //
-// The loads of this kernel run close to what HBM gives, and every MFMA costs time on top of them
-// (the chip clocks lower while the matrix units work): a stage with sixteen 32x32x64 MFMAs per SIMD
-// takes a third longer than one with none.  Two things keep their number down:
-//  * the zero-points are not two more planes: sum_k a (q - z) = sum_k a q - z sum_k a, and the row
-//    sums of the stage's A tile come from one producer wave (one MFMA against a plane of ones, the
-//    producers taking turns), which leaves them in a small ring in LDS for the consumers' fold of
-//    the next stage; in the 32- and 64-row forms another producer leaves -(z x scale) per column
-//    there as fp32, so that the fold is two multiply-adds per element
-//    (total += scale x acc; total += (-z x scale) x row sum);
-//  * with at most 16 rows (M16) the consumers use v_mfma_scale_f32_16x16x128_f8f6f4, half the
-//    matrix work of the 32x32x64 form, which would multiply 16 rows of padding.
-// In the 16x16x128 form with an fp4 first and an fp8 second operand, lane group g = lane / 16 of the
-// fp8 operand holds k = 32 g .. 32 g + 31 in its 32 bytes, and nibbles 16 p .. 16 p + 15 (p = 0, 1) of
-// the fp4 operand of lane group g pair with k = 16 (4 (g % 2) + g / 2 + 2 p) .. + 15.  Row i of the
-// first operand and column j of the second meet in lane j + 16 (i / 4), register i % 4.
+// The loads of this kernel run close to what HBM gives at 16 rows, and every vector or matrix instruction
+// costs time on top of them (both go through the same issue port of a SIMD).  What keeps their number down:
+//  * a nibble is an fp8 operand as it stands (w4_bytes below): one MFMA per product, not one per bit plane;
+//  * the zero-points are not more MFMAs: sum_k a (q - z) = sum_k a q - z sum_k a.  The row sums of a stage's A
+//    tile come from one MFMA against a plane of ones (by a producer wave with 16 rows, by the consumers with more:
+//    consumer w adds up row tile w), which leaves them in a small ring in LDS for every consumer's fold one stage
+//    later; with more than 16 rows a producer leaves -(z x scale) per column there as fp32, so that a fold is two
+//    multiply-adds per element (total += scale x acc; total += (-z x scale) x row sum);
+//  * every form multiplies on v_mfma_scale_f32_16x16x128_f8f6f4, which takes a whole stage of K in one
+//    instruction: a 16 x 16 product is complete after one MFMA and is folded while the next ones run.
+// In that MFMA with fp8 operands, lane group g = lane / 16 of either operand holds k = 32 g .. 32 g + 31 of its
+// row (column) lane % 16 in its 32 bytes; with an fp4 first operand (the plane of ones) nibbles 16 p .. 16 p + 15
+// (p = 0, 1) of lane group g pair with k = 16 (4 (g % 2) + g / 2 + 2 p) .. + 15.  Row i of the first operand and
+// column j of the second meet in lane j + 16 (i / 4), register i % 4.
 constexpr int kW4WideBN = 256;
 constexpr int kW4WidePacked = kBK * kW4WideBN / 2;
 constexpr int w4_wide_stage(int bm, bool a16 = false) { return bm * kBK * (a16 ? 2 : 1) + kW4WidePacked + kW4ScaleRow + kW4ZpRow; }
@@ -545,10 +544,6 @@ __device__ __forceinline__ i32x8 w4_bytes(const i32x2& w0, const i32x2& w1, uint
   return r;
 }
 template <int FMT_A, int E>
-__device__ __forceinline__ f32x16 w4_mfma_bytes(const i32x8& w8, const i32x8& fa, const f32x16& c) {
-  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w8, fa, c, 0, mfma_code<FMT_A>(), 0, E, 0, 127);
-}
-template <int FMT_A, int E>
 __device__ __forceinline__ f32x4 w4_mfma16_bytes(const i32x8& w8, const i32x8& fa, const f32x4& c) {
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w8, fa, c, 0, mfma_code<FMT_A>(), 0, E, 0, 127);
 }
@@ -559,8 +554,8 @@ __device__ __forceinline__ f32x4 w4_mfma16(const u32x4& plane, const i32x8& fa, 
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b, fa, c, 4, mfma_code<FMT_A>(), 0, e, 0, 127);
 }
 
-// ROWS: 16 (the 16x16x128 form), 32, or 64 (row blocks of 64 along grid.y; one set of accumulators, folded into
-// the totals at the start of the next stage, for the registers of three waves per SIMD).
+// ROWS: 16 (one row tile; a product is folded one stage late), or 32, 64, 128 (ROWS / 16 row tiles; row blocks of
+// 128 along grid.y; a product is folded two MFMAs late).
 //
 // A16: the activations are 16-bit values handed over as two fp8 planes of the same shape (W4A16: see
 // split_rows_kernel): every stage carries both planes' tiles, and every product runs on both with the same weight
@@ -568,25 +563,22 @@ __device__ __forceinline__ f32x4 w4_mfma16(const u32x4& plane, const i32x8& fa, 
 template <int FMT_A, bool HAS_Z, int ROWS, bool A16 = false>
 __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
   constexpr bool M16 = ROWS == 16;
-  constexpr bool F16 = ROWS == 16 || ROWS == 128;  // the 16x16x128 MFMA: one tile of 16 rows, or eight
-  constexpr int RT = ROWS == 128 ? 8 : 1;          // row tiles of 16 in that form
-  constexpr int BM = ROWS >= 64 ? ROWS : 32, MT = BM / 32;
+  constexpr int RT = ROWS / 16;             // row tiles of 16
+  constexpr int BM = M16 ? 32 : ROWS;       // rows of A per stage in LDS
   constexpr int kConsumers = kW4WideConsumers;
   constexpr int S = w4_wide_stages(BM, A16), kStage = w4_wide_stage(BM, A16);
   constexpr int kOffLo = BM * kBK;  // the second plane's tile (A16)
   constexpr int kOffPacked = BM * kBK * (A16 ? 2 : 1), kOffScale = kOffPacked + kW4WidePacked, kOffZp = kOffScale + kW4ScaleRow;
-  constexpr int NV = M16 ? 8 : 16 * MT;  // results per consumer lane
-  // the 16-row form reads A fragments shaped for the 16x16x128 MFMA: the XOR of TileGeom's variant 1 keeps those off
-  // each other's banks
-  using LA = DmaLoader<true, BM, kBK, kW4ColWaves, F16 ? 1 : 0>;
-  using GA = TileGeom<true, BM, kBK, F16 ? 1 : 0>;
+  constexpr int NV = 8 * RT;  // results per consumer lane: per row tile, two column tiles of four
+  // the A fragments are shaped for the 16x16x128 MFMA: the XOR of TileGeom's variant 1 keeps those off each other's banks
+  using LA = DmaLoader<true, BM, kBK, kW4ColWaves, 1>;
+  using GA = TileGeom<true, BM, kBK, 1>;
   constexpr int kOps = 4 + LA::kPerWave * (A16 ? 2 : 1) + 1;  // four 1 KiB regions of weights, A, and the scale or zero-point row
   static_assert(S >= 3 && (S - 2) * kOps <= 63, "vmcnt holds 6 bits");
   static_assert(kStage % 1024 == 0, "stages stay 1 KiB aligned");
-  static_assert(kConsumers * epilogue_stage_floats<MT, 1>() * 4 <= S * kStage, "epilogue area overlays the ring");
   __shared__ __attribute__((aligned(1024))) uint8_t lds[S * kStage];
   __shared__ float row_sums[kW4SumRing][BM];
-  // per stage (two kept) and column: minus the group's zero-point times its scale, fp32 (32- and 64-row forms)
+  // per stage (two kept) and column: minus the group's zero-point times its scale, fp32 (forms with row tiles)
   __shared__ __attribute__((aligned(16))) float zs_rows[2][(M16 || !HAS_Z) ? 4 : kW4WideBN];
   __shared__ uint32_t ticket_drawn;
 
@@ -650,9 +642,9 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
     auto issue_stage = [&](int off, int stage) {
       const uint32_t base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)(lds + off);
       const i32x4 rp = wp.rsrc(0x7fffffffLL);
-      // with tiles of 16 or 32 rows there is one row block: the weights are read once (with 64-row tiles further
-      // row blocks read them again, out of the caches)
-      constexpr bool kOnce = ROWS < 64;
+      // up to 128 rows there is one row block and the weights are read once; further row blocks read them again,
+      // out of the caches
+      constexpr bool kOnce = ROWS < 128;
       w4_dma16<kOnce>(rp, vo_even, base + kOffPacked + (wq * 4) * 1024);
       w4_dma16<kOnce>(rp, vo_odd, base + kOffPacked + (wq * 4 + 1) * 1024);
       w4_dma16<kOnce>(rp, vo_even + 16 * ld, base + kOffPacked + (wq * 4 + 2) * 1024);
@@ -679,53 +671,27 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         });
       }
     };
-    // sum_k a[m, k] over the stage at `off`, for the consumers' fold one stage later
+    // sum_k a[m, k] over the stage at `off`, for the consumers' fold one stage later (16-row form)
     const u32x4 ones = {0x22222222u, 0x22222222u, 0x22222222u, 0x22222222u};  // e2m1 1.0
     auto sum_rows = [&](int off, int slot) {
       const uint8_t* st = lds + off;
-      if constexpr (F16) {
-        const int m = lane & 15, gk = lane >> 4;
-        const int o0 = GA::lds_offset(m, 2 * gk), o1 = GA::lds_offset(m, 2 * gk + 1);  // rows 16 further on: + 2048
-        static_for<RT>([&](auto ic) {
-          constexpr int i = decltype(ic)::value;
-          const u32x4 lo = *reinterpret_cast<const u32x4*>(st + o0 + 2048 * i);
-          const u32x4 hi = *reinterpret_cast<const u32x4*>(st + o1 + 2048 * i);
-          const i32x8 fa = {(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-          f32x4 r = w4_mfma16<FMT_A>(ones, fa, f32x4{0.f, 0.f, 0.f, 0.f}, 127);
-          if constexpr (A16) {
-            const u32x4 lo2 = *reinterpret_cast<const u32x4*>(st + kOffLo + o0 + 2048 * i);
-            const u32x4 hi2 = *reinterpret_cast<const u32x4*>(st + kOffLo + o1 + 2048 * i);
-            const i32x8 fb = {(int)lo2[0], (int)lo2[1], (int)lo2[2], (int)lo2[3], (int)hi2[0], (int)hi2[1], (int)hi2[2], (int)hi2[3]};
-            r = w4_mfma16<FMT_A>(ones, fb, r, 123);
-          }
-          // every lane holds the sum of its row (lane % 16 of tile i) and every lane stores it: a store under a lane
-          // mask would take the MFMA, whose result only those lanes used, under the mask with it.  A consumer lane
-          // finds the sums of its RT rows side by side.
-          row_sums[slot][(lane & 15) * RT + i] = r[0];
-        });
-      } else {
-        static_for<MT>([&](auto ic) {
-          constexpr int i = decltype(ic)::value;
-          i32x8 fa[2];
-#pragma unroll
-          for (int ks = 0; ks < 2; ++ks)
-            static_for<2>([&](auto pc) { read_fragment_part<true, BM, decltype(pc)::value>(st, 32 * i, ks, fa[ks]); });
-          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          f32x16 r = w4_mfma<FMT_A, 127>(ones, fa[0], zero);
-          r = w4_mfma<FMT_A, 127>(ones, fa[1], r);
-          if constexpr (A16) {
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
-              static_for<2>([&](auto pc) { read_fragment_part<true, BM, decltype(pc)::value>(st + kOffLo, 32 * i, ks, fa[ks]); });
-            r = w4_mfma<FMT_A, 123>(ones, fa[0], r);
-            r = w4_mfma<FMT_A, 123>(ones, fa[1], r);
-          }
-          row_sums[slot][32 * i + (lane & 31)] = r[0];  // by every lane, as above
-        });
+      const int m = lane & 15, gk = lane >> 4;
+      const u32x4 lo = *reinterpret_cast<const u32x4*>(st + GA::lds_offset(m, 2 * gk));
+      const u32x4 hi = *reinterpret_cast<const u32x4*>(st + GA::lds_offset(m, 2 * gk + 1));
+      const i32x8 fa = {(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+      f32x4 r = w4_mfma16<FMT_A>(ones, fa, f32x4{0.f, 0.f, 0.f, 0.f}, 127);
+      if constexpr (A16) {
+        const u32x4 lo2 = *reinterpret_cast<const u32x4*>(st + kOffLo + GA::lds_offset(m, 2 * gk));
+        const u32x4 hi2 = *reinterpret_cast<const u32x4*>(st + kOffLo + GA::lds_offset(m, 2 * gk + 1));
+        const i32x8 fb = {(int)lo2[0], (int)lo2[1], (int)lo2[2], (int)lo2[3], (int)hi2[0], (int)hi2[1], (int)hi2[2], (int)hi2[3]};
+        r = w4_mfma16<FMT_A>(ones, fb, r, 123);
       }
+      // every lane holds the sum of its row (lane % 16) and every lane stores it: a store under a lane mask would
+      // take the MFMA, whose result only those lanes used, under the mask with it
+      row_sums[slot][lane & 15] = r[0];
     };
     // -(zero-point) x scale of the stage's group, four columns per lane, for the consumers' fold one stage later:
-    // what every consumer lane would otherwise work out for its sixteen columns in every stage.
+    // what every consumer lane would otherwise work out for its eight columns in every stage.
     const uint32_t pflip = a.is_signed ? 0x8888u : 0u, pzmask = a.zp ? 0xffffu : 0u;
     auto column_rows = [&](int off, int slot) {
       const uint8_t* st = lds + off;
@@ -751,7 +717,8 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
       if constexpr (!M16 && HAS_Z) {
         if (((kt + 2) & 3) == wq) column_rows(rd_off, kt & 1);
       }
-      if (HAS_Z && (kt & 3) == wq) sum_rows(rd_off, kt & (kW4SumRing - 1));
+      // (with more rows the consumers, which read every A fragment anyway, add the rows up)
+      if (HAS_Z && M16 && (kt & 3) == wq) sum_rows(rd_off, kt & (kW4SumRing - 1));
       wr_off += kStage;
       if (wr_off == S * kStage) wr_off = 0;
       rd_off += kStage;
@@ -857,12 +824,12 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         if (KT & 1) fold(std::integral_constant<int, 0>{}, (slot - 1) & (kW4SumRing - 1));
         else fold(std::integral_constant<int, 1>{}, (slot - 1) & (kW4SumRing - 1));
       }
-    } else if constexpr (ROWS == 128) {
-      // 128 rows as eight tiles of 16 on the 16x16x128 MFMA, which takes a whole stage of K in one instruction: the
-      // sixteen products of a stage (eight row tiles by two column tiles) are independent, and each is folded into
-      // the totals two products later, eight multiply-adds behind an MFMA that lasts as long as they do.  The scale
-      // term of a product uses its own stage's scales; the zero-point term, -(z x scale)[n] x (row sum of A)[m],
-      // whose factors the producers leave in LDS during a stage, follows one stage later.
+    } else {
+      // ROWS / 16 row tiles on the 16x16x128 MFMA, which takes a whole stage of K in one instruction: the products of
+      // a stage (row tiles by two column tiles) are independent, and each is folded into the totals two products
+      // later, eight multiply-adds behind an MFMA that lasts as long as they do.  The scale term of a product uses
+      // its own stage's scales; the zero-point term, -(z x scale)[n] x (row sum of A)[m], whose factors are left
+      // in LDS during a stage, follows one stage later.
       // lane: rows m = 16 i + lane % 16 of A; columns wn + 16 t + 4 gk + e; product j = 2 i + t, total[4 j + e]
       const int gk = lane >> 4, r16 = lane & 15;
       int poff[2][2];
@@ -875,45 +842,60 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
       const int aoff0 = GA::lds_offset(r16, 2 * gk), aoff1 = GA::lds_offset(r16, 2 * gk + 1);  // tile i: + 2048 i
       const int soff = kOffScale + (wn + 4 * gk) * 2;  // + 32 t: four bf16
       const int zsoff = wn + 4 * gk;                   // + 16 t: four fp32
-      constexpr int NB = 3, LAG = 2;
+      constexpr int NB = A16 ? 2 : 3, LAG = NB - 1;  // sets of partial sums; products between an MFMA and its fold
+      constexpr int NF = A16 ? 2 : 3;      // A fragments in registers: the one being multiplied and those on their way
+      const int sum_tile = wq & (RT - 1);  // the row tile this consumer adds up (with fewer tiles than consumers several do the same one)
+      const u32x4 ones = {0x22222222u, 0x22222222u, 0x22222222u, 0x22222222u};  // e2m1 1.0
       f32x4 acc[NB];
       f32x4 sc[2], zsp[2];
       float rsp[RT];
-      auto stage = [&](auto hpc) {
-        constexpr bool ZT = decltype(hpc)::value && HAS_Z;  // a stage before this one has left its zero-point term
-        __syncthreads();  // the stage is in LDS, and so are the row sums and zero-point row of the one before
-        const uint8_t* st = lds + rd_off;
-        i32x2 wt[2][2];
+      i32x2 wt[2][2];
+      i32x8 fa[NF], fb[A16 ? NF : 1];
+      u32x2 snew[2];
+      auto fragment = [&](const uint8_t* st, int tile) {
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(st + aoff0 + 2048 * tile), hi = *reinterpret_cast<const u32x4*>(st + aoff1 + 2048 * tile);
+        return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+      };
+      auto read_a = [&](const uint8_t* st, auto ic) {
+        constexpr int i = decltype(ic)::value;
+        fa[i % NF] = fragment(st, i);
+        if constexpr (A16) fb[i % NF] = fragment(st + kOffLo, i);
+      };
+      // what a stage starts with: the packed weights, the first A fragments, the scales
+      auto read_head = [&](const uint8_t* st) {
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int p = 0; p < 2; ++p)
             wt[t][p] = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LDS_AS i32x2*)((LDS_AS uint8_t*)st + poff[t][p]));
-        i32x8 fa[2], fb[A16 ? 2 : 1];
-        auto read_a = [&](auto ic) {
-          constexpr int i = decltype(ic)::value;
-          const u32x4 lo = *reinterpret_cast<const u32x4*>(st + aoff0 + 2048 * i), hi = *reinterpret_cast<const u32x4*>(st + aoff1 + 2048 * i);
-          fa[i & 1] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-          if constexpr (A16) {
-            const u32x4 lo2 = *reinterpret_cast<const u32x4*>(st + kOffLo + aoff0 + 2048 * i);
-            const u32x4 hi2 = *reinterpret_cast<const u32x4*>(st + kOffLo + aoff1 + 2048 * i);
-            fb[i & 1] = i32x8{(int)lo2[0], (int)lo2[1], (int)lo2[2], (int)lo2[3], (int)hi2[0], (int)hi2[1], (int)hi2[2], (int)hi2[3]};
-          }
-        };
-        read_a(std::integral_constant<int, 0>{});
-        u32x2 snew[2];
+        static_for<(NF - 1 < RT ? NF - 1 : RT)>([&](auto ic) { read_a(st, ic); });
 #pragma unroll
         for (int t = 0; t < 2; ++t) snew[t] = *reinterpret_cast<const u32x2*>(st + soff + 32 * t);
+      };
+      auto stage = [&](auto hpc) {
+        constexpr bool ZT = decltype(hpc)::value && HAS_Z;  // a stage before this one has left its zero-point term
+        const uint8_t* st = lds + rd_off;
+        rd_off += kStage;
+        if (rd_off == S * kStage) rd_off = 0;
+        i32x8 fs, fs2;  // the fragment of the row tile whose sums this consumer works out
+        if constexpr (HAS_Z) {
+          fs = fragment(st, sum_tile);
+          if constexpr (A16) fs2 = fragment(st + kOffLo, sum_tile);
+        }
         if constexpr (ZT) {
           const int prev = slot - 1;
 #pragma unroll
           for (int t = 0; t < 2; ++t) zsp[t] = *reinterpret_cast<const f32x4*>(&zs_rows[prev & 1][zsoff + 16 * t]);
-          const f32x4 r0 = *reinterpret_cast<const f32x4*>(&row_sums[prev & (kW4SumRing - 1)][r16 * RT]);
-          const f32x4 r1 = *reinterpret_cast<const f32x4*>(&row_sums[prev & (kW4SumRing - 1)][r16 * RT + 4]);
+          static_for<RT / 4>([&](auto hc) {
+            constexpr int h = decltype(hc)::value;
+            const f32x4 r = *reinterpret_cast<const f32x4*>(&row_sums[prev & (kW4SumRing - 1)][r16 * RT + 4 * h]);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            rsp[i] = r0[i];
-            rsp[4 + i] = r1[i];
+            for (int i = 0; i < 4; ++i) rsp[4 * h + i] = r[i];
+          });
+          if constexpr (RT == 2) {
+            const f32x2 r = *reinterpret_cast<const f32x2*>(&row_sums[prev & (kW4SumRing - 1)][r16 * RT]);
+            rsp[0] = r[0];
+            rsp[1] = r[1];
           }
         }
 #pragma unroll
@@ -933,23 +915,32 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
             total[4 * j + e] = v;
           }
         };
+        if constexpr (HAS_Z) {
+          // the row sums of that tile, for every consumer's fold of the next stage: one more MFMA, against a plane of
+          // ones.  Every lane holds the sum of its row and every lane stores it (a store under a lane mask would
+          // take the MFMA under the mask with it); a consumer lane finds the sums of its RT rows side by side.
+          f32x4 r = w4_mfma16<FMT_A>(ones, fs, f32x4{0.f, 0.f, 0.f, 0.f}, 127);
+          if constexpr (A16) r = w4_mfma16<FMT_A>(ones, fs2, r, 123);
+          row_sums[slot & (kW4SumRing - 1)][r16 * RT + sum_tile] = r[0];
+        }
         __builtin_amdgcn_sched_barrier(0);
         static_for<2 * RT>([&](auto jc) {
           constexpr int j = decltype(jc)::value, t = j & 1, i = j >> 1, b = j % NB;
-          if constexpr (t == 0 && i + 1 < RT) read_a(std::integral_constant<int, i + 1>{});
-          acc[b] = w4_mfma16_bytes<FMT_A, kW4ByteScale>(w8[t], fa[i & 1], f32x4{0.f, 0.f, 0.f, 0.f});
-          if constexpr (A16) acc[b] = w4_mfma16_bytes<FMT_A, kW4ByteScale - 4>(w8[t], fb[i & 1], acc[b]);
+          if constexpr (t == 0 && i + NF - 1 < RT) read_a(st, std::integral_constant<int, i + NF - 1>{});
+          acc[b] = w4_mfma16_bytes<FMT_A, kW4ByteScale>(w8[t], fa[i % NF], f32x4{0.f, 0.f, 0.f, 0.f});
+          if constexpr (A16) acc[b] = w4_mfma16_bytes<FMT_A, kW4ByteScale - 4>(w8[t], fb[i % NF], acc[b]);
           if constexpr (j >= LAG) fold(std::integral_constant<int, j - LAG>{});
           __builtin_amdgcn_sched_barrier(0);
         });
         static_for<LAG>([&](auto lc) { fold(std::integral_constant<int, 2 * RT - LAG + decltype(lc)::value>{}); });
-        rd_off += kStage;
-        if (rd_off == S * kStage) rd_off = 0;
         ++slot;
+        __syncthreads();  // the next stage is in LDS, and so are the row sums and the zero-point row of this one
+        read_head(lds + rd_off);  // (past the last stage: a slot of the ring whose contents are not used)
       };
+      __syncthreads();
+      read_head(lds);
       if (KT > 0) stage(F{});
       for (int kt = 1; kt < KT; ++kt) stage(T{});
-      __syncthreads();  // the row sums and zero-point row of the last stage
       if constexpr (HAS_Z) {
         if (KT > 0) {
           const int prev = slot - 1;
@@ -965,110 +956,6 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
           }
         }
       }
-    } else {
-      // lane: rows m = 32 i + lane % 32 of A (i < MT); columns wn + 8 q + 4 (lane / 32) + c, e = 4 q + c
-      const int tg = lane >> 4, tr = lane & 15, th = tg >> 1;
-      int poff[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int row = 64 * (j >> 1) + 32 * th + 16 * (j & 1) + w4_nibble_row(tr);  // fp8 operand of lane half th: k = 32 th .. + 31
-        poff[j] = kOffPacked + row * 128 + ((wq ^ ((row >> 1) & 7)) << 4) + (tg & 1) * 8;
-      }
-      const int soff = kOffScale + (wn + 4 * (lane >> 5)) * 2;
-      // two sets of partial sums, folded one stage late behind the next stage's MFMAs; with 64 rows there are
-      // registers for one set only, folded at the start of the next stage, before its MFMAs overwrite it
-      constexpr int NB = MT == 1 ? 2 : 1;
-      f32x16 acc[NB][MT];
-      float sc[16];
-      // total += scale x acc - (zero-point x scale) x (row sum of A): the second factor comes ready from a producer
-      const int zsoff = wn + 4 * (lane >> 5);
-      auto fold = [&](auto bc, int stage_no) {
-        constexpr int B = decltype(bc)::value % NB;
-        f32x4 zs[4];
-        if constexpr (HAS_Z) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) zs[q] = *reinterpret_cast<const f32x4*>(&zs_rows[stage_no & 1][zsoff + 8 * q]);
-        }
-        static_for<MT>([&](auto ic) {
-          constexpr int i = decltype(ic)::value;
-          float rs = 0.0f;
-          if constexpr (HAS_Z) rs = row_sums[stage_no & (kW4SumRing - 1)][32 * i + (lane & 31)];
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            float t = __builtin_fmaf(acc[B][i][e], sc[e], total[16 * i + e]);
-            if constexpr (HAS_Z) t = __builtin_fmaf(zs[e >> 2][e & 3], rs, t);
-            total[16 * i + e] = t;
-          }
-        });
-      };
-      auto stage = [&](auto bc, auto hpc) {
-        constexpr int B = decltype(bc)::value % NB;
-        constexpr bool HAVE_PREV = decltype(hpc)::value;
-        __syncthreads();  // the stage is in LDS, and so are the row sums of the one before
-        const uint8_t* st = lds + rd_off;
-        i32x2 wt[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          wt[j] = __builtin_amdgcn_ds_read_tr4_b64_v2i32((LDS_AS i32x2*)((LDS_AS uint8_t*)st + poff[j]));
-        // the A fragments of both halves of the stage up front, or (64 rows) of the second half behind the MFMAs of
-        // the first, for the registers
-        i32x8 fa[2][MT], fb[A16 ? 2 : 1][MT];
-        auto read_a = [&](int ks) {
-          static_for<MT>([&](auto ic) {
-            static_for<2>([&](auto pc) {
-              read_fragment_part<true, BM, decltype(pc)::value>(st, 32 * decltype(ic)::value, ks, fa[MT == 1 ? ks : 0][decltype(ic)::value]);
-              if constexpr (A16)
-                read_fragment_part<true, BM, decltype(pc)::value>(st + kOffLo, 32 * decltype(ic)::value, ks, fb[MT == 1 ? ks : 0][decltype(ic)::value]);
-            });
-          });
-        };
-        read_a(0);
-        if constexpr (MT == 1) read_a(1);
-        u32x2 snew[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) snew[q] = *reinterpret_cast<const u32x2*>(st + soff + q * 16);
-        if constexpr (HAVE_PREV && NB == 1) fold(std::integral_constant<int, 0>{}, (slot - 1) & (kW4SumRing - 1));
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-          const i32x8 w8 = w4_bytes(wt[2 * ks], wt[2 * ks + 1], flip);
-          const int f = MT == 1 ? ks : 0;
-          static_for<MT>([&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            if (ks == 0) acc[B][i] = w4_mfma_bytes<FMT_A, kW4ByteScale>(w8, fa[f][i], zero);
-            else acc[B][i] = w4_mfma_bytes<FMT_A, kW4ByteScale>(w8, fa[f][i], acc[B][i]);
-            if constexpr (A16) acc[B][i] = w4_mfma_bytes<FMT_A, kW4ByteScale - 4>(w8, fb[f][i], acc[B][i]);
-          });
-          if constexpr (MT == 2) {
-            if (ks == 0) read_a(1);
-          }
-        }
-        // the stage before this one, whose MFMAs finished long ago, behind the MFMAs just issued
-        if constexpr (HAVE_PREV && NB == 2) fold(std::integral_constant<int, 1 - B>{}, (slot - 1) & (kW4SumRing - 1));
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          sc[4 * q + 0] = __uint_as_float(snew[q][0] << 16);
-          sc[4 * q + 1] = __uint_as_float(snew[q][0] & 0xffff0000u);
-          sc[4 * q + 2] = __uint_as_float(snew[q][1] << 16);
-          sc[4 * q + 3] = __uint_as_float(snew[q][1] & 0xffff0000u);
-        }
-        rd_off += kStage;
-        if (rd_off == S * kStage) rd_off = 0;
-        ++slot;
-      };
-      int kt = 1;
-      if (KT > 0) stage(std::integral_constant<int, 0>{}, F{});
-      for (; kt + 1 < KT; kt += 2) {
-        stage(std::integral_constant<int, 1>{}, T{});
-        stage(std::integral_constant<int, 0>{}, T{});
-      }
-      if (kt < KT) stage(std::integral_constant<int, 1>{}, T{});
-      __syncthreads();  // the row sums of the last stage
-      if (KT > 0) {
-        if (KT & 1) fold(std::integral_constant<int, 0>{}, (slot - 1) & (kW4SumRing - 1));
-        else fold(std::integral_constant<int, 1>{}, (slot - 1) & (kW4SumRing - 1));
-      }
     }
   }
   __syncthreads();  // every load has landed and every stage is consumed: the ring is idle
@@ -1080,7 +967,7 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
     // which, done by every workgroup while the others still stream, costs more than the kernel).
     const int strips = gridDim.x / a.ksplit * gridDim.y;         // strips of all row blocks
     const int strip_rb = blockIdx.y * (gridDim.x / a.ksplit) + strip;
-    constexpr int kWords = 8 * MT * 64;  // per consumer wave (half of them used with 16 rows)
+    constexpr int kWords = BM * 16;  // per consumer wave (half of them used with 16 rows)
     unsigned long long* mine = reinterpret_cast<unsigned long long*>(a.partials) + ((int64_t)(part * strips + strip_rb) * kConsumers + wq) * kWords + lane;
     if (!producer) {
 #pragma unroll
@@ -1116,7 +1003,7 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
     }
   }
   if (producer) return;
-  if constexpr (F16) {
+  {
     // C[m, n .. n + 3] for this lane's rows (one per row tile) and its two sets of four columns
     const int gk = lane >> 4;
     const ScalarScales scalars = load_scalar_scales(g);
@@ -1152,18 +1039,10 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
         }
       }
     }
-  } else {
-    f32x16 out[MT][1];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) out[i][0][e] = total[16 * i + e];
-    float* stage_area = reinterpret_cast<float*>(lds) + wq * epilogue_stage_floats<MT, 1>();
-    epilogue<MT, 1>(g, 0, out, 0, n0 + wq * 32, stage_area);
   }
 }
 
-// How the wide kernel takes a problem: rows per workgroup (16 selects the 16x16x128 form of the 32-row tile), row
+// How the wide kernel takes a problem: rows per workgroup (16 rows sit in a 32-row tile of LDS), row
 // blocks, strips, and the parts K is walked in (0: the wide kernel does not apply).
 struct W4WidePlan {
   int rows, row_blocks, strips, parts;
