@@ -55,12 +55,12 @@ MEASURED_TRAFFIC = {
     "fp8_gemm_v2_decode_M64": 243.07e6,
     "fp8_gemm_v2_decode_M256": 266.45e6,
     "w4a8_gemm_M16": 130.86e6,      # the partial sums of the two K parts on top of the 124 MB of operands
-    "w4a8_gemm_M32": 140.25e6,
-    "w4a8_gemm_M64": 158.58e6,
-    "w4a8_gemm_M256": 283.02e6,     # four row blocks of 64 stream the weights; the caches catch half of it
-    "w4a16_gemm_M16": 131.98e6,     # split_rows_vec_kernel + w4a8_wide_kernel<two planes>
-    "w4a16_gemm_M64": 164.56e6,
-    "w4a16_gemm_M256": 316.05e6,
+    "w4a8_gemm_M32": 139.63e6,
+    "w4a8_gemm_M64": 157.22e6,
+    "w4a8_gemm_M256": 153.68e6,     # two row blocks of 128 on one XCD share a strip's weights in its L2
+    "w4a16_gemm_M16": 131.96e6,     # split_rows_vec_kernel + w4a8_wide_kernel<two planes>
+    "w4a16_gemm_M64": 161.49e6,
+    "w4a16_gemm_M256": 178.91e6,
     "fp8_sdpa_B1_L8192": 124.63e6,
     "fp8_sdpa_B4_L4096": 235.55e6,
     "fp8_sdpa_B1_L8192_D256": 347.00e6,   # k and v are re-read by the query blocks of a head group beyond L2

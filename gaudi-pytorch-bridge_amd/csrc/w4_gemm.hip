@@ -1,4 +1,4 @@
-// Fused int4-dequant GEMM for gfx950: fp8 activations times 4-bit weights (W4A8).
+// Fused int4-dequant GEMM for gfx950: fp8 activations times 4-bit weights (W4A8; 16-bit activations as two fp8 planes).
 //
 //   C[m, n] = out( sA[m] * sum_g s[g, n] * sum_{k in g} a[m, k] * (q[k, n] - z[g, n]) + bias[n] )
 //
@@ -8,21 +8,23 @@
 // nor as fp8: a weight stage travels from HBM to LDS as packed nibbles (half the bytes
 // of fp8 weights, a quarter of bf16) and goes from there into the MFMA as it is.
 //
-// How a nibble becomes an MFMA operand.  v_mfma_scale_f32_32x32x64_f8f6f4 multiplies an
-// fp8 operand by an fp4 (e2m1) one, and the e2m1 codes 0, 1, 2, 3 stand for 0, 0.5, 1,
-// 1.5: a two-bit integer v, zero-extended to four bits, is the e2m1 code of v / 2.  An
-// unsigned nibble q = 4 hi + lo therefore splits into two planes, (w >> 2) & 0x33333333
-// and w & 0x33333333 on eight nibbles at a time, and two MFMAs with the block scales 2^3
-// and 2^1 accumulate sum_k a q exactly.  The zero-point leaves the inner loop:
-// sum_k a (q - z) = sum_k a q - z sum_k a, and sum_k a comes from a third MFMA against
-// a plane of ones.  (A signed nibble s is q = s ^ 8 = s + 8 with z + 8.)  ds_read_b64_tr_b4
-// turns the packed rows (16 columns in 8 bytes) into the 16 consecutive k of one column
-// that an MFMA lane wants, so the only vector ALU work per 64 x 32 weights is the two
-// masks and a shift per register.
+// How a nibble becomes an MFMA operand.  Two ways, one per kernel below.
+//  * As an fp8 byte (the kernel for groups of 128, see w4_bytes): the e4m3 codes 0 .. 15 are one linear ramp,
+//    q x 2^-9, so a nibble zero-extended to a byte is an fp8 operand and one MFMA with the block scale 2^9
+//    accumulates sum_k a q exactly.
+//  * As two fp4 planes (the kernel for every other group size): v_mfma_scale_f32_32x32x64_f8f6f4 multiplies an
+//    fp8 operand by an fp4 (e2m1) one, and the e2m1 codes 0, 1, 2, 3 stand for 0, 0.5, 1, 1.5: a two-bit integer
+//    v, zero-extended to four bits, is the e2m1 code of v / 2.  An unsigned nibble q = 4 hi + lo therefore splits
+//    into two planes, (w >> 2) & 0x33333333 and w & 0x33333333 on eight nibbles at a time, and two MFMAs with
+//    the block scales 2^3 and 2^1 accumulate sum_k a q exactly.
+// In the first of these the zero-point leaves the inner loop: sum_k a (q - z) = sum_k a q - z sum_k a, and sum_k a
+// comes from one more MFMA against a plane of ones; in the second the zero-points are two more planes, the same
+// for every k of a group.  (A signed nibble s is q = s ^ 8 = s + 8 with z + 8.)  ds_read_b64_tr_b4 turns
+// the packed rows (16 columns in 8 bytes) into 16 k of one column, which is what an MFMA lane wants, so the only
+// vector ALU work per register of eight weights is two masks and a shift.
 //
-// Relative to an fp8 operand whose lane holds k = 32 h + j in byte j (h = lane / 32),
-// the fp4 operand of the same MFMA holds k = 16 h + j in nibble j < 16 and
-// k = 32 + 16 h + (j - 16) in nibble j >= 16.
+// Relative to an fp8 operand whose lane holds k = 32 h + j in byte j (h = lane / 32), the fp4 operand of the
+// 32x32x64 MFMA holds k = 16 h + j in nibble j < 16 and k = 32 + 16 h + (j - 16) in nibble j >= 16.
 //
 // Two kernels.  The first, below, is shaped like the strip kernel of gemm_skinny.h (the second, for groups of
 // 128 with bf16 scales, follows it: 256-column strips, K split over workgroups): the weights stream once through a deep LDS
