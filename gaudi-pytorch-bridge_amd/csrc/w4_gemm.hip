@@ -988,20 +988,31 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
     __syncthreads();
     if (ticket_drawn != (uint32_t)a.ksplit - 1) return;
     if (!producer) {
-#pragma unroll
-      for (int e = 0; e < NV; ++e) total[e] = 0.0f;
+      // part 0 + part 1 + part 2 + ..., whichever part comes last.  Part 0 or 1 keeps its own sums in its registers
+      // and adds the other of the two first (the same bits as the other way round, and no partial sum is -0); a
+      // later part starts from zero and reads its own with the rest.
       const unsigned long long* from = reinterpret_cast<const unsigned long long*>(a.partials) + ((int64_t)strip_rb * kConsumers + wq) * kWords + lane;
-      for (int p = 0; p < a.ksplit; ++p) {
+      const int64_t part_stride = (int64_t)strips * kConsumers * kWords;
+      auto add_part = [&](int p) {
+        const unsigned long long* src = from + p * part_stride;
         unsigned long long v[NV / 2];
 #pragma unroll
-        for (int h = 0; h < NV / 2; ++h) v[h] = __hip_atomic_load(from + h * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int h = 0; h < NV / 2; ++h) v[h] = __hip_atomic_load(src + h * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
         for (int h = 0; h < NV / 2; ++h) {
           total[2 * h] += __uint_as_float((uint32_t)v[h]);
           total[2 * h + 1] += __uint_as_float((uint32_t)(v[h] >> 32));
         }
-        from += (int64_t)strips * kConsumers * kWords;
+      };
+      int p = 0;
+      if (part <= 1) {
+        add_part(1 - part);
+        p = 2;
+      } else {
+#pragma unroll
+        for (int e = 0; e < NV; ++e) total[e] = 0.0f;
       }
+      for (; p < a.ksplit; ++p) add_part(p);
     }
   }
   if (producer) return;
