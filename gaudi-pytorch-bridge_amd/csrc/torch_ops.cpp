@@ -755,8 +755,10 @@ Tensor convert_from_uint4(const Tensor& input, const Tensor& scale,
 // queries do the same): one zero-filled buffer per (device, stream, op) is kept here and grown on
 // demand, so that a call launches one kernel and nothing else.  Calls on one stream run in order,
 // which is all the sharing the buffer allows; the two ops lay their counters out differently and
-// do not share.  While a stream is being captured into a graph no buffer is handed out (its memory
-// would belong to the graph's pool, and replays of two graphs could overlap).
+// do not share.  While a stream is being captured into a graph no kept buffer is handed out (its
+// memory would belong to the graph's pool, and replays of two graphs could overlap): the call takes
+// a buffer of the graph's own and clears its counters with a fill kernel that is part of the graph
+// (captured_ticket_workspace).
 enum TicketWorkspaceOp { kWsW4a8 = 0, kWsSdpa = 1, kWsW4a16 = 2 };
 struct TicketWorkspaceCache {
   std::mutex mu;
@@ -780,6 +782,15 @@ Tensor ticket_workspace(const Tensor& like, size_t bytes, TicketWorkspaceOp op) 
   if (!t.defined() || (size_t)t.numel() < bytes) t = at::zeros({(int64_t)bytes}, like.options().dtype(at::kByte));
   return t;
 }
+// While the stream is being captured: a buffer out of the graph's pool, its first KiB (the arrival counters of
+// every op that uses one) zeroed by a small fill kernel, which every replay runs again; the rest (partial sums
+// that are written before they are read) as it comes.
+Tensor captured_ticket_workspace(const Tensor& like, size_t bytes) {
+  Tensor t = at::empty({(int64_t)bytes}, like.options().dtype(at::kByte));
+  t.narrow(0, 0, std::min<int64_t>((int64_t)bytes, 1024)).zero_();
+  return t;
+}
+bool stream_is_capturing() { return c10::hip::currentStreamCaptureStatusMayInitCtx() != c10::hip::CaptureStatus::None; }
 // After a call that used the buffer has failed: its counters may be left non-zero (no workgroup then draws a
 // group's last ticket and the output stays unwritten), so the buffer is dropped and the next call starts from a
 // zero-filled one.
@@ -841,14 +852,16 @@ Tensor w4a8_gemm(const Tensor& A, const Tensor& packed, const Tensor& scale, con
     b = bias->to(out_dtype).contiguous();
   }
   MI355Q_OP_INFO("w4a8_gemm : A=" << A.sizes() << " packed=" << packed.sizes() << " group=" << group << " signed=" << is_signed);
-  // under graph capture: none, and the kernel then runs without the split
-  Tensor ws = ticket_workspace(a, mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, to_mi355q_dtype(s.scalar_type())), kWsW4a8);
+  // the buffer kept per stream, or under graph capture one of the graph's own with its counters cleared
+  const size_t ws_bytes = mi355q_w4a8_gemm_workspace_bytes(M, N, K, group, to_mi355q_dtype(s.scalar_type()));
+  const bool kept = !stream_is_capturing();
+  Tensor ws = kept ? ticket_workspace(a, ws_bytes, kWsW4a8) : (ws_bytes ? captured_ticket_workspace(a, ws_bytes) : Tensor());
   const int st = mi355q_w4a8_gemm(a.data_ptr(), to_mi355q_dtype(a.scalar_type()), K, w.data_ptr<int32_t>(), N / 8, s.data_ptr(),
                                   to_mi355q_dtype(s.scalar_type()), has_zp ? z.data_ptr<int32_t>() : nullptr, is_signed ? 1 : 0,
                                   group, out.data_ptr(), to_mi355q_dtype(out_dtype), N, M, N, K, sa_dev, 1.0f, sa_mode,
                                   b.defined() ? b.data_ptr() : nullptr, ws.defined() ? ws.data_ptr() : nullptr,
                                   ws.defined() ? (size_t)ws.numel() : 0, current_stream(a));
-  if (st != MI355Q_OK && ws.defined()) drop_ticket_workspace(a, kWsW4a8);
+  if (st != MI355Q_OK && ws.defined() && kept) drop_ticket_workspace(a, kWsW4a8);
   TORCH_CHECK(st != MI355Q_ERR_UNSUPPORTED,
               "mi355q::w4a8_gemm takes groups that are multiples of 128, N a multiple of 32 and K a multiple of 16 (got group ",
               group, ", N ", N, ", K ", K, "); expand the weights with hpu::convert_from_", is_signed ? "int4" : "uint4", " for other shapes");
@@ -896,15 +909,14 @@ Tensor w4a16_gemm(const Tensor& A, const Tensor& packed, const Tensor& scale, co
   MI355Q_OP_INFO("w4a16_gemm : A=" << A.sizes() << " packed=" << packed.sizes() << " group=" << group << " signed=" << is_signed);
   const size_t bytes = mi355q_w4a16_gemm_workspace_bytes(M, N, K, group, to_mi355q_dtype(s.scalar_type()));
   // the buffer kept per stream starts zero-filled, which the split over K needs; under graph capture a buffer of the
-  // graph's own, and K in one piece
-  Tensor ws = ticket_workspace(a, bytes, kWsW4a16);
-  const bool split = ws.defined();
-  if (!split) ws = at::empty({(int64_t)bytes}, A.options().dtype(at::kByte));
+  // graph's own with its counters cleared
+  const bool kept = !stream_is_capturing();
+  Tensor ws = kept ? ticket_workspace(a, bytes, kWsW4a16) : captured_ticket_workspace(a, bytes);
   const int st = mi355q_w4a16_gemm(a.data_ptr(), MI355Q_BF16, K, w.data_ptr<int32_t>(), N / 8, s.data_ptr(),
                                    to_mi355q_dtype(s.scalar_type()), has_zp ? z.data_ptr<int32_t>() : nullptr, is_signed ? 1 : 0, group,
                                    out.data_ptr(), to_mi355q_dtype(out_dtype), N, M, N, K, has_bias ? b.data_ptr() : nullptr,
-                                   ws.data_ptr(), (size_t)ws.numel(), split ? 1 : 0, current_stream(a));
-  if (st != MI355Q_OK && split) drop_ticket_workspace(a, kWsW4a16);
+                                   ws.data_ptr(), (size_t)ws.numel(), 1, current_stream(a));
+  if (st != MI355Q_OK && kept) drop_ticket_workspace(a, kWsW4a16);
   TORCH_CHECK(st != MI355Q_ERR_UNSUPPORTED,
               "mi355q::w4a16_gemm takes groups of 128 with bfloat16 scales, N a multiple of 32 and K a multiple of 16 (got group ", group,
               ", ", s.scalar_type(), " scales, N ", N, ", K ", K, "); expand the weights with hpu::convert_from_", is_signed ? "int4" : "uint4",

@@ -115,17 +115,19 @@ def test_graph_replays_of_the_reductions(dev):
 
 def decode_step(q, k, v, x8, pk, s, z):
     """Attention for one query per head against a long cache (the keys split over workgroups, which meet through
-    arrival counters in a workspace) and a W4A8 product (without its split while a graph is captured)."""
+    arrival counters in a workspace), a W4A8 product and a W4A16 product on the same weights (K split over
+    workgroups, which meet the same way)."""
     o = ops.fp8_sdpa_recomp_fwd(q, k, v, None, 0.0, 128 ** -0.5, False, False, "None", None, None, None, None, None, None,
                                 False, False, None, "left")[0]
     y = torch.ops.mi355q.w4a8_gemm(x8, pk, s, z, False, torch.bfloat16, None, None)
-    return o, y
+    y16 = torch.ops.mi355q.w4a16_gemm(x8.to(torch.bfloat16), pk, s, z, False, torch.bfloat16, None)
+    return o, y, y16
 
 
 def test_graph_replays_of_a_decode_step(dev):
-    """The key split's counters live in a zero-filled tensor of the graph's own while capturing (the fill is a
-    kernel of the graph, so every replay starts from zero) and in the stream's kept workspace in eager runs: same
-    bits either way, replay after replay, with eager calls in between."""
+    """The counters of the key split and of the W4A8 product's split over K live in a tensor of the graph's own while
+    capturing (cleared by a fill kernel of the graph, so every replay starts from zero) and in the stream's kept
+    workspace in eager runs: same bits either way, replay after replay, with eager calls in between."""
     g = torch.Generator().manual_seed(14)
     B, G, HG, S, D = 1, 2, 4, 4096, 128
     k = torch.randn(B, G, 1, S, D, generator=g).to(E4).to(dev)
@@ -156,8 +158,8 @@ def test_graph_replays_of_a_decode_step(dev):
         ref = decode_step(q, k, v, x, pk, s, z)
         torch.cuda.synchronize()
         assert torch.equal(got[0], ref[0]), rep
-        # the W4A8 product adds its K parts in another order with the split (eager) than without (captured)
-        assert torch.allclose(got[1].float(), ref[1].float(), rtol=2 ** -6, atol=2 ** -6 * float(ref[1].float().abs().max())), rep
+        assert torch.equal(got[1], ref[1]), rep   # the same kernel and the same split over K, captured or not
+        assert torch.equal(got[2], ref[2]), rep
 
 
 def test_ops_follow_the_current_stream(oracle, dev):
