@@ -1158,7 +1158,9 @@ inline W4A16Layout w4a16_layout(int64_t M, int64_t N, int64_t K, int64_t group, 
   const auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
   W4A16Layout l{};
   const W4WidePlan plan = w4a8_wide_plan(M, N, K, group, scale_f32);
-  l.split_bytes = plan.parts >= 2 ? plan.workspace_bytes() : 0;
+  // the arrival counters' KiB is set aside whether this shape splits K or not: a buffer that serves calls of several
+  // shapes must not find the planes of one call where the next one keeps its counters
+  l.split_bytes = plan.parts >= 2 ? plan.workspace_bytes() : W4WidePlan::ticket_bytes();
   l.ld = (K + 15) & ~(int64_t)15;
   l.plane_off = up(l.split_bytes);
   l.lo_off = l.plane_off + up((size_t)(M * l.ld));

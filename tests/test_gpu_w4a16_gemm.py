@@ -158,3 +158,25 @@ def test_batched_activations_c_abi_and_errors(oracle, pkg, dev):
         torch.ops.mi355q.w4a16_gemm(Ad[:, :K2], pkd, s.float().to(dev), None, True, torch.float32, None)
     with pytest.raises(RuntimeError, match="must be bfloat16"):
         torch.ops.mi355q.w4a16_gemm(Ad[:, :K2].float(), pkd, sd, None, True, torch.float32, None)
+
+
+def test_one_workspace_serves_shapes_with_and_without_a_split(oracle, pkg, dev):
+    """A buffer that is passed to calls of several shapes (the torch layer keeps one per stream): a shape that walks K
+    in one part leaves the first KiB alone, where a later shape that splits K keeps its arrival counters."""
+    lib = pkg.capi()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    gen = torch.Generator().manual_seed(21)
+    shapes = [(16, 512, 256), (32, 2048, 512), (16, 512, 256), (8, 4096, 512)]     # K in one part, in two, in one, in four
+    nbytes = max(lib.mi355q_w4a16_gemm_workspace_bytes(M, N, K, 128, pkg.BF16) for M, K, N in shapes)
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+    for M, K, N in shapes:
+        q, z, s, pk, pz = weights(oracle, gen, K, N, 128, False, True, pow2=True)
+        a = torch.randint(-255, 256, (M, K), generator=gen).float()
+        expect = a.double() @ ((q - z.repeat_interleave(128, 0)).double() * s.double().repeat_interleave(128, 0))
+        Ad, pkd, sd, pzd = a.bfloat16().to(dev), pk.to(dev), s.to(dev), pz.to(dev)
+        C = torch.full((M, N), -5.0, device=dev)
+        assert lib.mi355q_w4a16_gemm(Ad.data_ptr(), pkg.BF16, K, pkd.data_ptr(), N // 8, sd.data_ptr(), pkg.BF16, pzd.data_ptr(), 0, 128,
+                                     C.data_ptr(), pkg.F32, N, M, N, K, None, ws.data_ptr(), nbytes, 1, stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(C.cpu().double(), expect), (M, K, N)
+        assert torch.count_nonzero(ws[:1024]) == 0
