@@ -579,7 +579,7 @@ __global__ __launch_bounds__(kW4WideThreads) void w4a8_wide_kernel(W4Args a) {
   static_assert(S >= 3 && (S - 2) * kOps <= 63, "vmcnt holds 6 bits");
   static_assert(kStage % 1024 == 0, "stages stay 1 KiB aligned");
   __shared__ __attribute__((aligned(1024))) uint8_t lds[S * kStage];
-  __shared__ float row_sums[kW4SumRing][BM];
+  __shared__ __attribute__((aligned(16))) float row_sums[kW4SumRing][BM];  // (consumers read four of a row's sums at a time)
   // per stage (two kept) and column: minus the group's zero-point times its scale, fp32 (forms with row tiles)
   __shared__ __attribute__((aligned(16))) float zs_rows[2][(M16 || !HAS_Z) ? 4 : kW4WideBN];
   __shared__ uint32_t ticket_drawn;
