@@ -176,7 +176,12 @@ __device__ __forceinline__ void epilogue16_bf16_fast_any(const GemmArgs& g, int6
 }
 
 // Per-wave state of the K loop: 2 x 2 waves on a 256 x 256 tile, one per SIMD.
-template <bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
+// LEAN: K is a whole number of pairs of stages (K % 256 == 0), so that no stage has lanes past K, and each operand
+// spans less than DmaLoader::kNarrowBytes: the loads then need no per-lane test, four of them share a write of m0,
+// and a descriptor steps in four scalar instructions.  The K loop of the general form spends 93 instructions per
+// stage besides its 64 MFMAs and 48 LDS reads, this one 40; on a SIMD that issues for one wave that is 3.6 % of the
+// run time of a 8192 x 4096 x 14336 product.
+template <bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B, bool LEAN>
 struct TileCore16 {
   static constexpr int BM = 256, BN = 256, kWaves = 4;
   static constexpr int MT = 8, NT = 8;  // 16 x 16 MFMA tiles of the wave's 128 x 128
@@ -221,14 +226,22 @@ struct TileCore16 {
   template <int OP, int STAGE>
   __device__ __forceinline__ void dma_op(int kt) {
     constexpr int na = LoaderA::kPerWave;
-    if constexpr (OP < na) la.template issue_one<OP>(ring + STAGE * kStageA, kt * kBK, K);
-    else lb.template issue_one<OP - na>(ring + 2 * kStageA + STAGE * kStageB, kt * kBK, K);
+    if constexpr (OP < na) la.template issue_one<OP, false, false, !LEAN>(ring + STAGE * kStageA, kt * kBK, K);
+    else lb.template issue_one<OP - na, false, false, !LEAN>(ring + 2 * kStageA + STAGE * kStageB, kt * kBK, K);
+  }
+  __device__ __forceinline__ void step_descriptors() {
+    if constexpr (LEAN) {
+      la.advance_narrow();
+      lb.advance_narrow();
+    } else {
+      la.advance();
+      lb.advance();
+    }
   }
   template <int STAGE>
   __device__ __forceinline__ void issue_stage(int kt) {
     static_for<kDmaOps>([&](auto oc) { dma_op<decltype(oc)::value, STAGE>(kt); });
-    la.advance();
-    lb.advance();
+    step_descriptors();
   }
 
   static constexpr int kEpilogueStores = MT * 4;
@@ -276,14 +289,13 @@ struct TileCore16 {
         static_for<kPartsB>([&](auto pc) { rb.template read<j, decltype(pc)::value, NXT>(fb[j]); });
       __builtin_amdgcn_sched_barrier(0);
     });
-    la.advance();
-    lb.advance();
+    step_descriptors();
   }
 };
 
-template <bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B>
+template <bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B, bool LEAN>
 __global__ __launch_bounds__(256) void fp8_gemm_tile16_kernel(GemmArgs g) {
-  using Core = TileCore16<A_KMAJOR, B_KMAJOR, FMT_A, FMT_B>;
+  using Core = TileCore16<A_KMAJOR, B_KMAJOR, FMT_A, FMT_B, LEAN>;
   constexpr int BM = Core::BM, BN = Core::BN, MT = Core::MT, NT = Core::NT;
   __shared__ __attribute__((aligned(1024))) uint8_t lds_ring[Core::kRingBytes];
   __shared__ __attribute__((aligned(16))) float lds_epi[4 * epilogue_stage_floats<4, 4>()];
@@ -354,7 +366,13 @@ void launch_tile16(const GemmArgs& g, int64_t batch, hipStream_t st) {
   const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
   const int cus = compute_units();
   dim3 grid((unsigned)(tiles < cus ? tiles : cus), (unsigned)batch);
-  fp8_gemm_tile16_kernel<AK, BK_, FA, FB><<<grid, 256, 0, st>>>(a);
+  // bytes from an operand's first element to the end of what a descriptor on it may cover (see DmaLoader::set_tile)
+  const int64_t span_a = AK ? (int64_t)(g.M - 1) * g.lda + g.K : (int64_t)(g.K - 1) * g.lda + ((g.M + 15) & ~15);
+  const int64_t span_b = BK_ ? (int64_t)(g.N - 1) * g.ldb + g.K : (int64_t)(g.K - 1) * g.ldb + ((g.N + 15) & ~15);
+  constexpr int64_t narrow = DmaLoader<true, 256, kBK, 4, 1>::kNarrowBytes;
+  const bool lean = g.K % (2 * kBK) == 0 && span_a < narrow && span_b < narrow;
+  if (lean) fp8_gemm_tile16_kernel<AK, BK_, FA, FB, true><<<grid, 256, 0, st>>>(a);
+  else fp8_gemm_tile16_kernel<AK, BK_, FA, FB, false><<<grid, 256, 0, st>>>(a);
 }
 
 }  // namespace mi355q

@@ -113,6 +113,49 @@ def scan(text):
     return findings
 
 
+def m0_sharing(text):
+    """Global -> LDS loads that take the m0 a previous asm statement wrote (four loads of a group share one write, their
+    immediate offsets tell the regions apart): between such a load and the write of m0 it relies on there must be no
+    label (another path could arrive with another m0) and no other write of m0, and the write must be one of ours
+    (inside an asm statement).  Returns (number of loads that share, findings)."""
+    lines = text.splitlines()
+    findings, shared = [], 0
+    in_asm = False
+    block_writes_m0 = False
+    for n, l in enumerate(lines):
+        if "#ASMSTART" in l:
+            in_asm, block_writes_m0 = True, False
+            continue
+        if "#ASMEND" in l:
+            in_asm = False
+            continue
+        if not in_asm or not _is_instruction(l):
+            continue
+        if re.match(r"\s*s_mov_b32\s+m0\b", l):
+            block_writes_m0 = True
+        if _MEM.match(l) and " lds" in l and not block_writes_m0:
+            shared += 1
+            k = n - 1
+            inside = False
+            while k >= 0:
+                t = lines[k]
+                if "#ASMEND" in t:
+                    inside = True
+                elif "#ASMSTART" in t:
+                    inside = False
+                elif re.match(r"\s*\.?[A-Za-z_][\w.$]*:", t):
+                    findings.append(f"line {n + 1}: '{l.strip()}' takes m0 from before the label at line {k + 1}")
+                    break
+                elif _is_instruction(t) and re.match(r"\s*s_\w+\s+m0\b", t):
+                    if not (inside and re.match(r"\s*s_mov_b32\s+m0\b", t)):
+                        findings.append(f"line {n + 1}: '{l.strip()}' takes m0 from '{t.strip()}' (line {k + 1}), not from an asm statement")
+                    break
+                k -= 1
+            else:
+                findings.append(f"line {n + 1}: '{l.strip()}' has no write of m0 before it")
+    return shared, findings
+
+
 def memory_order(text):
     """{kernel symbol: string over L, S, W (s_waitcnt vmcnt(0)), w (s_waitcnt vmcnt(n > 0)), A (atomic)}"""
     out = {}

@@ -61,6 +61,8 @@ KERNEL_SHAPES = {
     "tile256_two_passes_and_tail_columns": (4000, 8208, 208),
     "tile256_two_passes_no_split": (4000, 7184, 144),
     "tile256_ten_k_stages": (4000, 4112, 1168),
+    "tile256_whole_stage_pairs_and_tail_columns": (4000, 4112, 512),   # K % 256 == 0: the kernel without per-lane K tests
+    "tile256_whole_stage_pairs_two_passes": (4000, 8208, 256),
     "tile256x128_more_tiles_than_cus": (1008, 12304, 208),
     "tile256x128_fewer_tiles_than_cus": (272, 10256, 272),
     "tile128_underfilled": (272, 4112, 400),

@@ -83,9 +83,33 @@ def test_gemm_kernels_have_no_uncovered_hazard():
     sources = ["gemm_inst_kk.hip", "gemm_inst_km.hip", "gemm_inst_mk.hip", "gemm_inst_mm.hip", "w4_gemm.hip", "sdpa_kernels.hip"]
     with ThreadPoolExecutor(max_workers=6) as ex:
         texts = list(ex.map(isa_check.compile_to_isa, sources))
+    sharing = 0
     for src, text in zip(sources, texts):
         assert text.count("#ASMSTART") > 100, f"{src}: the asm statements are gone?"
         assert isa_check.scan(text) == [], src
+        shared, findings = isa_check.m0_sharing(text)
+        assert findings == [], src
+        sharing += shared
+    assert sharing > 0, "the kernels whose loads share a write of m0 are gone?"
+
+
+def test_m0_sharing_scanner():
+    good = """
+	;;#ASMSTART
+	s_mov_b32 m0, s5
+	s_nop 0
+	buffer_load_dwordx4 v1, s[28:31], 0 offen lds
+	;;#ASMEND
+	v_mfma_f32_16x16x128_f8f6f4 a[0:3], v[2:9], v[10:17], a[0:3]
+	;;#ASMSTART
+	buffer_load_dwordx4 v2, s[28:31], 0 offen offset:1024 lds
+	;;#ASMEND
+"""
+    assert isa_check.m0_sharing(good) == (1, [])
+    across_a_label = good.replace("\tv_mfma", ".LBB0_3:\n\tv_mfma")
+    assert isa_check.m0_sharing(across_a_label)[1]
+    compiler_write = good.replace("\tv_mfma", "\ts_mov_b32 m0, s9\n\tv_mfma")
+    assert isa_check.m0_sharing(compiler_write)[1]
 
 
 @pytest.mark.timeout(600)
