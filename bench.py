@@ -49,8 +49,8 @@ MEASURED_TRAFFIC = {
     "cast_to_fp8_v2_large": 804.68e6,
     "convert_from_uint4": 43.36e6,
     "convert_from_int4": 43.10e6,
-    "fp8_gemm_v2": 939.92e6,
-    "fp8_gemm_v2_B_NK": 939.29e6,
+    "fp8_gemm_v2": 939.89e6,
+    "fp8_gemm_v2_B_NK": 939.33e6,
     "fp8_gemm_v2_decode_M16": 236.92e6,
     "fp8_gemm_v2_decode_M64": 243.07e6,
     "fp8_gemm_v2_decode_M256": 266.45e6,
