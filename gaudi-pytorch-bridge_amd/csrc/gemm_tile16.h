@@ -330,9 +330,13 @@ __global__ __launch_bounds__(256) void fp8_gemm_tile16_kernel(GemmArgs g) {
   bool stores_pending = false;
   // Only the first tile reads its first fragments here: the last K stage of a tile replaces its fragments, as they
   // die, by those of ring stage 0 like every other stage, and what sits there by then is the next tile's first stage.
-  core.first_fragments(false);
+  // (Not with both operands K-major: the registers do not hold the fragments across the epilogue there, and the
+  // spills cost more than reading them again.)
+  constexpr bool kKeepFragments = !(A_KMAJOR && B_KMAJOR);
+  if constexpr (kKeepFragments) core.first_fragments(false);
   for (;;) {
     const int m0 = tile_m * BM, n0 = tile_n * BN;
+    if constexpr (!kKeepFragments) core.first_fragments(stores_pending);
     auto k_pair = [&](auto first_c, int kt) {
       constexpr bool FIRST = decltype(first_c)::value;
       const bool last = kt + 2 == KT2;

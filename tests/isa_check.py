@@ -113,6 +113,16 @@ def scan(text):
     return findings
 
 
+def scratch_bytes(text):
+    """Kernels of a compiled source that use scratch memory (register spills): {mangled name: bytes per lane}."""
+    out = {}
+    for m in re.finditer(r"\.amdhsa_kernel (\S+)(.*?)\.end_amdhsa_kernel", text, re.S):
+        n = int(re.search(r"private_segment_fixed_size (\d+)", m.group(2)).group(1))
+        if n:
+            out[m.group(1)] = n
+    return out
+
+
 def m0_sharing(text):
     """Global -> LDS loads that take the m0 a previous asm statement wrote (four loads of a group share one write, their
     immediate offsets tell the regions apart): between such a load and the write of m0 it relies on there must be no
