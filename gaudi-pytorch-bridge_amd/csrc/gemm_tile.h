@@ -254,6 +254,7 @@ struct DmaLoader {
       step = (int64_t)BK * ld;
     }
     if (!valid) remaining = 0;
+    stage_offset = 0;
     const uint64_t b = reinterpret_cast<uint64_t>(base);
     rsrc[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
     rsrc[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((b >> 32) & 0xffffu));
@@ -270,11 +271,12 @@ struct DmaLoader {
   // which starts at k0.
   // NT: the nontemporal hint, for an operand that is read once (the weights of a decode-shaped call): a strip
   // read of a 235 MB matrix runs 8 % faster with it (41 against 45 us), through registers or into LDS alike.
-  // K_CHECK false: the caller's K is a whole number of the stages it walks, no lane is ever past K.
-  // Then (and without CLAMP_ROWS) a lane's offset does not depend on the stage, and four loads in a row share one
-  // write of m0: the instruction's immediate offset moves the LDS address and the memory address alike, so region
-  // I takes the m0 of region I - I % 4, the immediate (I % 4) KiB, and a lane offset lowered by as much.  The
-  // caller issues the regions of a group in order with nothing between them that writes m0.
+  // K_CHECK false: the caller's K is a whole number of the stages it walks, no lane is ever past K, and the
+  // operand is narrow (see advance_narrow()).  Then (and without CLAMP_ROWS) a lane's offset does not depend on the
+  // stage, the descriptor stays where set_tile() put it and the stage is the instruction's scalar offset; and four
+  // loads in a row share one write of m0: the instruction's immediate offset moves the LDS address and the memory
+  // address alike, so region I takes the m0 of region I - I % 4, the immediate (I % 4) KiB, and a lane offset
+  // lowered by as much.  The caller issues the regions of a group in order with nothing between them that writes m0.
   template <int I, bool CLAMP_ROWS = false, bool NT = false, bool K_CHECK = true>
   __device__ __forceinline__ void issue_one(uint8_t* lds_tile, int k0, int K) const {
     const uint32_t lds_base = (uint32_t)(uintptr_t)(LDS_AS uint8_t*)lds_tile;
@@ -283,12 +285,15 @@ struct DmaLoader {
       const int vo = voff[i % kStored] + (i / kStored) * region_step - r * 1024;
       if constexpr (r == 0) {
         const uint32_t dst = lds_base + (uint32_t)((wave * kPerWave + i) * 1024);
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                      :
-                     : "s"(dst), "v"(vo), "s"(rsrc)
+                     : "s"(dst), "v"(vo), "s"(rsrc), "s"(stage_offset)
                      : "memory", "m0");
       } else {
-        asm volatile("buffer_load_dwordx4 %0, %1, 0 offen offset:%2 lds" : : "v"(vo), "s"(rsrc), "n"(r * 1024) : "memory");
+        asm volatile("buffer_load_dwordx4 %0, %1, %3 offen offset:%2 lds"
+                     :
+                     : "v"(vo), "s"(rsrc), "n"(r * 1024), "s"(stage_offset)
+                     : "memory");
       }
     } else {
       constexpr int i = I;
@@ -333,19 +338,14 @@ struct DmaLoader {
   }
 
   // advance() for an operand whose whole extent, from its first byte to the last one the launch may address, is
-  // below kNarrowBytes, walked forwards only from set_tile() on: num_records then always is the number of bytes left
-  // and takes one subtraction and one max per stage.  (The clamps of the general form are 64-bit compares, which
-  // the compiler puts on the vector ALU, a dozen instructions per operand and stage: a wave that issues one MFMA
-  // after the other has no issue slot to spare for them.)  `remaining` is not kept up: set_tile() comes next.
+  // below kNarrowBytes, walked forwards only from set_tile() on and loaded with issue_one<.., K_CHECK = false>: the
+  // descriptor stays on the tile's first stage and the bytes walked so far go into the loads' scalar offset, one
+  // scalar addition per stage.  (The general form moves the base and clamps a 64-bit count of the bytes left with
+  // compares that the compiler puts on the vector ALU, a dozen instructions per operand and stage: a wave that
+  // issues one MFMA after the other has no issue slot to spare for them.)
   static constexpr int64_t kNarrowBytes = 0x40000000LL;
-  __device__ __forceinline__ void advance_narrow() {
-    uint64_t b = ((uint64_t)(uint32_t)rsrc[1] << 32) | (uint32_t)rsrc[0];
-    b += (uint64_t)step;
-    rsrc[0] = (int)(uint32_t)b;
-    rsrc[1] = (int)(uint32_t)(b >> 32);
-    const int r = rsrc[2] - (int)step;
-    rsrc[2] = r < 0 ? 0 : r;
-  }
+  int stage_offset = 0;
+  __device__ __forceinline__ void advance_narrow() { stage_offset += (int)step; }
 
   // Next K stage: scalar arithmetic on the descriptor only.
   __device__ __forceinline__ void advance() {

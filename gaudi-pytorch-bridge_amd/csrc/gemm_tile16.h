@@ -178,8 +178,8 @@ __device__ __forceinline__ void epilogue16_bf16_fast_any(const GemmArgs& g, int6
 // Per-wave state of the K loop: 2 x 2 waves on a 256 x 256 tile, one per SIMD.
 // LEAN: K is a whole number of pairs of stages (K % 256 == 0), so that no stage has lanes past K, and each operand
 // spans less than DmaLoader::kNarrowBytes: the loads then need no per-lane test, four of them share a write of m0,
-// and a descriptor steps in four scalar instructions.  The K loop of the general form spends 93 instructions per
-// stage besides its 64 MFMAs and 48 LDS reads, this one 40; on a SIMD that issues for one wave that is 3.6 % of the
+// and a step along K is one scalar addition per operand.  The K loop of the general form spends 93 instructions per
+// stage besides its 64 MFMAs and 48 LDS reads, this one 30; on a SIMD that issues for one wave that is 4 % of the
 // run time of a 8192 x 4096 x 14336 product.
 template <bool A_KMAJOR, bool B_KMAJOR, int FMT_A, int FMT_B, bool LEAN>
 struct TileCore16 {
